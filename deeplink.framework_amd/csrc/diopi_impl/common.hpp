@@ -1,0 +1,187 @@
+// Shared host/device helpers for the MI355X DIOPI implementation library.
+//
+// Host side: a TensorView snapshot of what the diopirt callbacks report
+// (the impl library never looks inside a handle; it only calls the runtime,
+// as the reference's runtime contract requires:
+// dipu/torch_dipu/csrc_dipu/diopirt/diopirt_impl.cpp:24-126), error plumbing
+// for diopiGetLastErrorString, and launch helpers.
+// Device side: wave64 reductions, 16-byte vector types, dtype conversion.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include <diopi/diopirt.h>
+#include <diopi/functions.h>
+#include <diopi/functions_ext.h>
+
+namespace amd {
+
+constexpr int kMaxDims = 8;
+constexpr int kWave = 64;
+
+// ---------------------------------------------------------------- errors ----
+void setLastError(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+
+#define AMD_CHECK(cond, ...)                    \
+  do {                                          \
+    if (!(cond)) {                              \
+      ::amd::setLastError(__VA_ARGS__);         \
+      return diopiErrorOccurred;                \
+    }                                           \
+  } while (0)
+
+#define AMD_TRY(expr)                           \
+  do {                                          \
+    diopiError_t _e = (expr);                   \
+    if (_e != diopiSuccess) return _e;          \
+  } while (0)
+
+#define AMD_HIP(expr)                                                                         \
+  do {                                                                                        \
+    hipError_t _h = (expr);                                                                   \
+    if (_h != hipSuccess) {                                                                   \
+      ::amd::setLastError("%s failed: %s (%s:%d)", #expr, hipGetErrorString(_h), __FILE__, __LINE__); \
+      return diopiErrorOccurred;                                                              \
+    }                                                                                         \
+  } while (0)
+
+// Checked after every launch; clears nothing on success.
+#define AMD_LAUNCH_CHECK() AMD_HIP(hipGetLastError())
+
+// ------------------------------------------------------------ tensor view ---
+struct TensorView {
+  void* data = nullptr;
+  int ndim = 0;
+  int64_t shape[kMaxDims] = {0};
+  int64_t stride[kMaxDims] = {0};
+  diopiDtype_t dtype = diopi_dtype_unsupported;
+  int64_t numel = 0;
+  int64_t itemsize = 0;
+
+  bool defined() const { return dtype != diopi_dtype_unsupported; }
+  bool isContiguous() const {
+    int64_t expect = 1;
+    for (int i = ndim - 1; i >= 0; --i) {
+      if (shape[i] == 1) continue;
+      if (stride[i] != expect) return false;
+      expect *= shape[i];
+    }
+    return true;
+  }
+  template <typename T>
+  T* ptr() const {
+    return reinterpret_cast<T*>(data);
+  }
+  bool aligned16() const { return (reinterpret_cast<uintptr_t>(data) & 15) == 0; }
+};
+
+int64_t dtypeSize(diopiDtype_t dt);
+const char* dtypeName(diopiDtype_t dt);
+inline bool isFloatDtype(diopiDtype_t dt) {
+  return dt == diopi_dtype_float16 || dt == diopi_dtype_bfloat16 || dt == diopi_dtype_float32 ||
+         dt == diopi_dtype_float64;
+}
+inline bool isIntDtype(diopiDtype_t dt) {
+  return dt == diopi_dtype_int8 || dt == diopi_dtype_uint8 || dt == diopi_dtype_int16 || dt == diopi_dtype_int32 ||
+         dt == diopi_dtype_int64 || dt == diopi_dtype_bool;
+}
+
+// Fills `v` from the runtime callbacks. A null handle yields an undefined view.
+diopiError_t getView(diopiConstTensorHandle_t th, TensorView* v, const char* what);
+diopiError_t getStream(diopiContextHandle_t ctx, hipStream_t* stream);
+
+// Workspace on the device owned by ctx (released by the runtime when ctx dies;
+// valid for kernels enqueued on ctx's stream only).
+diopiError_t requireWorkspace(diopiContextHandle_t ctx, int64_t nbytes, void** ptr);
+// Contiguous temporary of the given shape/dtype, as a handle plus view.
+diopiError_t requireTensor(diopiContextHandle_t ctx, const int64_t* shape, int ndim, diopiDtype_t dtype,
+                           diopiTensorHandle_t* th, TensorView* view);
+
+// dst <- src with broadcasting/strides/dtype conversion (the engine behind diopiCopyInp).
+diopiError_t stridedCopy(hipStream_t stream, const TensorView& src, const TensorView& dst);
+// Returns `v` itself when already contiguous, else a contiguous copy in ctx workspace.
+diopiError_t makeContiguous(diopiContextHandle_t ctx, hipStream_t stream, const TensorView& v, TensorView* out);
+
+double scalarToDouble(const diopiScalar_t* s, double dflt);
+bool scalarIsFloat(const diopiScalar_t* s);
+int64_t scalarToInt(const diopiScalar_t* s, int64_t dflt);
+
+inline int64_t ceilDiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// ---------------------------------------------------------------- device ----
+#if defined(__HIPCC__)
+
+typedef __bf16 bf16_t;
+typedef _Float16 half_t;
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+template <typename T>
+struct Vec16 {  // 16 bytes of T
+  static constexpr int N = 16 / sizeof(T);
+  typedef T type __attribute__((ext_vector_type(16 / sizeof(T))));
+};
+
+__device__ __forceinline__ float waveSum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+__device__ __forceinline__ float waveMax(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+__device__ __forceinline__ bool isFloatDtypeDev(int dt) {
+  return dt == diopi_dtype_float16 || dt == diopi_dtype_bfloat16 || dt == diopi_dtype_float32 ||
+         dt == diopi_dtype_float64;
+}
+
+// Runtime-dtype element load/store used by the generic (strided / mixed dtype) paths.
+template <typename C>
+__device__ __forceinline__ C loadAs(const void* base, int64_t idx, int dt) {
+  switch (dt) {
+    case diopi_dtype_float32: return static_cast<C>(reinterpret_cast<const float*>(base)[idx]);
+    case diopi_dtype_bfloat16: return static_cast<C>(static_cast<float>(reinterpret_cast<const bf16_t*>(base)[idx]));
+    case diopi_dtype_float16: return static_cast<C>(static_cast<float>(reinterpret_cast<const half_t*>(base)[idx]));
+    case diopi_dtype_float64: return static_cast<C>(reinterpret_cast<const double*>(base)[idx]);
+    case diopi_dtype_int64: return static_cast<C>(reinterpret_cast<const int64_t*>(base)[idx]);
+    case diopi_dtype_int32: return static_cast<C>(reinterpret_cast<const int32_t*>(base)[idx]);
+    case diopi_dtype_int16: return static_cast<C>(reinterpret_cast<const int16_t*>(base)[idx]);
+    case diopi_dtype_int8: return static_cast<C>(reinterpret_cast<const int8_t*>(base)[idx]);
+    case diopi_dtype_uint8: return static_cast<C>(reinterpret_cast<const uint8_t*>(base)[idx]);
+    case diopi_dtype_bool: return static_cast<C>(reinterpret_cast<const uint8_t*>(base)[idx] != 0);
+    default: return C(0);
+  }
+}
+template <typename C>
+__device__ __forceinline__ void storeAs(void* base, int64_t idx, int dt, C v) {
+  switch (dt) {
+    case diopi_dtype_float32: reinterpret_cast<float*>(base)[idx] = static_cast<float>(v); break;
+    case diopi_dtype_bfloat16: reinterpret_cast<bf16_t*>(base)[idx] = static_cast<bf16_t>(static_cast<float>(v)); break;
+    case diopi_dtype_float16: reinterpret_cast<half_t*>(base)[idx] = static_cast<half_t>(static_cast<float>(v)); break;
+    case diopi_dtype_float64: reinterpret_cast<double*>(base)[idx] = static_cast<double>(v); break;
+    case diopi_dtype_int64: reinterpret_cast<int64_t*>(base)[idx] = static_cast<int64_t>(v); break;
+    case diopi_dtype_int32: reinterpret_cast<int32_t*>(base)[idx] = static_cast<int32_t>(v); break;
+    case diopi_dtype_int16: reinterpret_cast<int16_t*>(base)[idx] = static_cast<int16_t>(v); break;
+    case diopi_dtype_int8: reinterpret_cast<int8_t*>(base)[idx] = static_cast<int8_t>(v); break;
+    case diopi_dtype_uint8: reinterpret_cast<uint8_t*>(base)[idx] = static_cast<uint8_t>(v); break;
+    case diopi_dtype_bool: reinterpret_cast<uint8_t*>(base)[idx] = (v != C(0)) ? 1 : 0; break;
+    default: break;
+  }
+}
+
+#endif  // __HIPCC__
+
+}  // namespace amd

@@ -1,0 +1,415 @@
+// Prefill ("context") causal attention over packed sequences for gfx950.
+//
+//   q [tokens, heads, d], k/v [tokens, kv_heads, d]; sequence b = rows
+//   [b_start_loc[b], b_start_loc[b] + b_seq_len[b]);
+//   out = softmax(q k^T / sqrt(d) + causal mask) v, scores and softmax in fp32
+//   (dicp/dicp/vendor/AscendGraph/ext_ops.py:62-87).
+//
+// MFMA kernel (bf16 / fp16, d = 64 or 128): a workgroup of 4 waves owns 128 queries of one
+// (sequence, head); each wave owns 32 of them and walks the keys in tiles of 64.
+//   * S^T = K . Q^T is computed instead of S: the 32x32 accumulator then holds, in every
+//     lane, 16 scores of ONE query (its column), so the online-softmax row statistics are
+//     an in-lane reduction plus a single xor-32 shuffle, and the O^T accumulators of the
+//     lane belong to that same query: rescaling needs no cross-lane traffic at all.
+//   * The accumulator registers of S^T, converted to bf16, are already a valid B operand
+//     (P^T) for O^T += V^T . P^T: consecutive groups of 8 accumulator registers are the 8
+//     K-slots of a lane, for a fixed permutation of the 16 keys of the step. The A operand
+//     (V^T) is read from an LDS copy of V stored transposed [d][keys] with exactly that
+//     permutation: two 8-byte reads per operand.
+//   * K tile rows in LDS are XOR-swizzled per 16-byte chunk (conflict-free ds_read_b128);
+//     V is transposed on the way into LDS (4 keys x 8 d per lane, 8-byte stores).
+//   * two LDS stages, register prefetch of the next tile, one barrier per tile; the heaviest
+//     query blocks (end of the sequence) are scheduled first.
+//   * the epilogue transposes O^T through LDS so global stores are 16-byte and coalesced.
+//
+// Scalar kernel: any dtype / head_dim, one workgroup per (query, head); correctness path
+// for fp32 and odd head sizes.
+#include <algorithm>
+
+#include "common.hpp"
+
+namespace amd {
+
+constexpr float kLog2eCA = 1.4426950408889634f;
+
+__device__ __forceinline__ int64_t ldIdxCA(const void* p, int64_t i, bool is64) {
+  return is64 ? reinterpret_cast<const int64_t*>(p)[i] : static_cast<int64_t>(reinterpret_cast<const int32_t*>(p)[i]);
+}
+
+struct CaArgs {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* out;
+  const void* bStart;
+  const void* bLen;
+  bool start64, len64;
+  int64_t qTok, qHead, kTok, kHead, vTok, vHead, oTok, oHead;  // element strides
+  int heads, kvHeads, d;
+  float scale;  // 1/sqrt(d)
+};
+
+template <typename T>
+struct CaMfma;
+template <>
+struct CaMfma<bf16_t> {
+  typedef bf16x8 Frag;
+  typedef bf16x4 Half;
+  static __device__ __forceinline__ f32x16 run(Frag a, Frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct CaMfma<half_t> {
+  typedef f16x8 Frag;
+  typedef f16x4 Half;
+  static __device__ __forceinline__ f32x16 run(Frag a, Frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+constexpr int kCaBQ = 128, kCaBKV = 64, kCaVtStride = 68;  // V^T rows padded to 68 keys (136 bytes)
+
+template <typename T, int D>
+__global__ __launch_bounds__(256) void contextAttnMfmaKernel(CaArgs a) {
+  using Frag = typename CaMfma<T>::Frag;
+  using Half = typename CaMfma<T>::Half;
+  constexpr int KS = D / 16;        // MFMA k-steps over the head dim
+  constexpr int DT = D / 32;        // 32-row tiles of O^T
+  constexpr int CPR = D / 8;        // 16-byte chunks per K row
+  constexpr int K_CH = kCaBKV * CPR / 256;  // K chunks per thread
+  constexpr int K_STAGE = kCaBKV * D;       // elements
+  constexpr int V_STAGE = D * kCaVtStride;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  T* sK = reinterpret_cast<T*>(smem);   // [2][64][D] swizzled
+  T* sVt = sK + 2 * K_STAGE;            // [2][D][68]
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l31 = lane & 31, half = lane >> 5;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int qb = gridDim.x - 1 - blockIdx.x;  // heavy blocks first
+  const int64_t start = ldIdxCA(a.bStart, b, a.start64);
+  const int len = (int)ldIdxCA(a.bLen, b, a.len64);
+  const int q0 = qb * kCaBQ;
+  if (q0 >= len) return;
+  const int kvh = h / (a.heads / a.kvHeads);
+  const T* qg = reinterpret_cast<const T*>(a.q) + start * a.qTok + (int64_t)h * a.qHead;
+  const T* kg = reinterpret_cast<const T*>(a.k) + start * a.kTok + (int64_t)kvh * a.kHead;
+  const T* vg = reinterpret_cast<const T*>(a.v) + start * a.vTok + (int64_t)kvh * a.vHead;
+
+  const int qi = q0 + wave * 32 + l31;      // this lane's query (column of S^T)
+  const int qiC = min(qi, len - 1);          // rows past the sequence compute on the last row, never stored
+  Frag qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+    qf[ks] = *reinterpret_cast<const Frag*>(qg + (int64_t)qiC * a.qTok + ks * 16 + half * 8);
+
+  const int ntiles = (min(len, q0 + kCaBQ) + kCaBKV - 1) / kCaBKV;
+  const int waveMaxQ = min(q0 + wave * 32 + 31, len - 1);
+
+  // ---- staging roles
+  Frag kr[K_CH];
+  int kKey[K_CH], kOff[K_CH];
+#pragma unroll
+  for (int i = 0; i < K_CH; ++i) {
+    int chunk = tid + 256 * i;
+    int key = chunk / CPR, c = chunk % CPR;
+    kKey[i] = key;
+    kOff[i] = key * D + ((c ^ (key & 7)) << 3);
+  }
+  const int cK = (tid % CPR) * 8;
+  const bool vActive = tid < 16 * (D / 8);
+  const int vKg = tid & 15, vDc = tid >> 4;
+  Frag vr[4];
+
+  auto gload = [&](int t) {
+    const int k0 = t * kCaBKV;
+#pragma unroll
+    for (int i = 0; i < K_CH; ++i) {
+      int key = min(k0 + kKey[i], len - 1);
+      kr[i] = *reinterpret_cast<const Frag*>(kg + (int64_t)key * a.kTok + cK);
+    }
+    if (vActive) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        int key = min(k0 + vKg * 4 + j, len - 1);
+        vr[j] = *reinterpret_cast<const Frag*>(vg + (int64_t)key * a.vTok + vDc * 8);
+      }
+    }
+  };
+  auto swrite = [&](int stage) {
+    T* k = sK + stage * K_STAGE;
+    T* vt = sVt + stage * V_STAGE;
+#pragma unroll
+    for (int i = 0; i < K_CH; ++i) *reinterpret_cast<Frag*>(k + kOff[i]) = kr[i];
+    if (vActive) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        Half p;
+        p[0] = vr[0][e], p[1] = vr[1][e], p[2] = vr[2][e], p[3] = vr[3][e];
+        *reinterpret_cast<Half*>(vt + (vDc * 8 + e) * kCaVtStride + vKg * 4) = p;
+      }
+    }
+  };
+
+  f32x16 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[dt][r] = 0.f;
+  float m = -INFINITY, l = 0.f;
+  const float scale2 = a.scale * kLog2eCA;
+
+  gload(0);
+  swrite(0);
+  if (ntiles > 1) gload(1);
+  __syncthreads();
+
+  for (int t = 0; t < ntiles; ++t) {
+    const int cur = t & 1;
+    const int k0 = t * kCaBKV;
+    if (k0 <= waveMaxQ) {
+      const T* k = sK + cur * K_STAGE;
+      const T* vt = sVt + cur * V_STAGE;
+      f32x16 s[2];
+#pragma unroll
+      for (int kt2 = 0; kt2 < 2; ++kt2) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[kt2][r] = 0.f;
+        const int key = kt2 * 32 + l31;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const int chunk = ks * 2 + half;
+          Frag kf = *reinterpret_cast<const Frag*>(k + key * D + ((chunk ^ (key & 7)) << 3));
+          s[kt2] = CaMfma<T>::run(kf, qf[ks], s[kt2]);
+        }
+      }
+      // ---- online softmax for this lane's query over the 64 keys of the tile
+      const bool needMask = (k0 + kCaBKV - 1 > q0 + wave * 32) || (k0 + kCaBKV > len);
+      float mt = -INFINITY;
+#pragma unroll
+      for (int kt2 = 0; kt2 < 2; ++kt2)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          float v = s[kt2][r] * scale2;
+          if (needMask) {
+            int kj = k0 + kt2 * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+            if (kj > qiC || kj >= len) v = -INFINITY;
+          }
+          s[kt2][r] = v;
+          mt = fmaxf(mt, v);
+        }
+      mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+      const float mn = fmaxf(m, mt);  // key 0 is visible to every query, so mn is finite from tile 0 on
+      const float corr = exp2f(m - mn);
+      float ps = 0.f;
+#pragma unroll
+      for (int kt2 = 0; kt2 < 2; ++kt2)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          float p = exp2f(s[kt2][r] - mn);
+          s[kt2][r] = p;
+          ps += p;
+        }
+      ps += __shfl_xor(ps, 32, 64);
+      l = l * corr + ps;
+      m = mn;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[dt][r] *= corr;
+      // ---- O^T += V^T . P^T
+#pragma unroll
+      for (int kt2 = 0; kt2 < 2; ++kt2)
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2) {
+          Frag pf;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) pf[j] = static_cast<T>(s[kt2][8 * t2 + j]);
+          const int base = kt2 * 32 + t2 * 16 + half * 4;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) {
+            const T* row = vt + (dt * 32 + l31) * kCaVtStride + base;
+            Half lo = *reinterpret_cast<const Half*>(row);
+            Half hi = *reinterpret_cast<const Half*>(row + 8);
+            Frag vf;
+            vf[0] = lo[0], vf[1] = lo[1], vf[2] = lo[2], vf[3] = lo[3];
+            vf[4] = hi[0], vf[5] = hi[1], vf[6] = hi[2], vf[7] = hi[3];
+            o[dt] = CaMfma<T>::run(vf, pf, o[dt]);
+          }
+        }
+    }
+    if (t + 1 < ntiles) {
+      swrite(cur ^ 1);
+      if (t + 2 < ntiles) gload(t + 2);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: O^T (lane = query) -> LDS [query][d] -> coalesced 16-byte stores
+  constexpr int OS = D + 8;  // padded row, elements
+  T* sO = reinterpret_cast<T*>(smem) + wave * 32 * OS;
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      Half p;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) p[e] = static_cast<T>(o[dt][g * 4 + e] * inv);
+      *reinterpret_cast<Half*>(sO + l31 * OS + dt * 32 + g * 8 + half * 4) = p;
+    }
+  __syncthreads();
+  T* og = reinterpret_cast<T*>(a.out) + start * a.oTok + (int64_t)h * a.oHead;
+#pragma unroll
+  for (int i = 0; i < 32 * CPR / 64; ++i) {
+    int chunk = lane + 64 * i;
+    int row = chunk / CPR, c = chunk % CPR;
+    int qrow = q0 + wave * 32 + row;
+    if (qrow < len) *reinterpret_cast<Frag*>(og + (int64_t)qrow * a.oTok + c * 8) = *reinterpret_cast<const Frag*>(sO + row * OS + c * 8);
+  }
+}
+
+// One workgroup per (query token, head): scores to LDS, softmax, then P.V with lanes over d.
+template <typename T>
+__global__ __launch_bounds__(256) void contextAttnScalarKernel(CaArgs a, int maxLen) {
+  extern __shared__ float sc[];  // maxLen scores + 8 reduction slots
+  float* red = sc + maxLen;
+  const int qi = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int64_t start = ldIdxCA(a.bStart, b, a.start64);
+  const int len = (int)ldIdxCA(a.bLen, b, a.len64);
+  if (qi >= len) return;
+  const int kvh = h / (a.heads / a.kvHeads);
+  const T* q = reinterpret_cast<const T*>(a.q) + (start + qi) * a.qTok + (int64_t)h * a.qHead;
+  const T* kg = reinterpret_cast<const T*>(a.k) + start * a.kTok + (int64_t)kvh * a.kHead;
+  const T* vg = reinterpret_cast<const T*>(a.v) + start * a.vTok + (int64_t)kvh * a.vHead;
+  const int n = qi + 1;  // causal: keys 0..qi
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float mx = -INFINITY;
+  for (int j = threadIdx.x; j < n; j += 256) {
+    const T* kr = kg + (int64_t)j * a.kTok;
+    float d = 0.f;
+    for (int e = 0; e < a.d; ++e) d += static_cast<float>(q[e]) * static_cast<float>(kr[e]);
+    d *= a.scale;
+    sc[j] = d;
+    mx = fmaxf(mx, d);
+  }
+  mx = waveMax(mx);
+  if (lane == 0) red[wave] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  float sum = 0.f;
+  for (int j = threadIdx.x; j < n; j += 256) {
+    float p = expf(sc[j] - mx);
+    sc[j] = p;
+    sum += p;
+  }
+  sum = waveSum(sum);
+  if (lane == 0) red[4 + wave] = sum;
+  __syncthreads();
+  const float inv = 1.f / (red[4] + red[5] + red[6] + red[7]);
+  T* og = reinterpret_cast<T*>(a.out) + (start + qi) * a.oTok + (int64_t)h * a.oHead;
+  for (int e = threadIdx.x; e < a.d; e += 256) {
+    float acc = 0.f;
+    for (int j = 0; j < n; ++j) acc += sc[j] * static_cast<float>(vg[(int64_t)j * a.vTok + e]);
+    og[e] = static_cast<T>(acc * inv);
+  }
+}
+
+template <typename T, int D>
+static diopiError_t launchCaMfma(hipStream_t stream, const CaArgs& a, int maxLen, int64_t batch) {
+  constexpr size_t lds = 2 * (size_t)(kCaBKV * D + D * kCaVtStride) * sizeof(T);
+  static_assert(lds >= 4 * 32 * (D + 8) * sizeof(T), "epilogue staging must fit in the tile buffers");
+  static bool attrSet = false;
+  if (!attrSet) {
+    AMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&contextAttnMfmaKernel<T, D>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attrSet = true;
+  }
+  dim3 grid((unsigned)ceilDiv(maxLen, kCaBQ), a.heads, (unsigned)batch);
+  hipLaunchKernelGGL((contextAttnMfmaKernel<T, D>), grid, dim3(256), lds, stream, a);
+  AMD_LAUNCH_CHECK();
+  return diopiSuccess;
+}
+
+}  // namespace amd
+
+using namespace amd;
+
+extern "C" __attribute__((visibility("default"))) diopiError_t diopiContextAttentionInference(
+    diopiContextHandle_t ctx, diopiTensorHandle_t outH, diopiConstTensorHandle_t qH, diopiConstTensorHandle_t kH,
+    diopiConstTensorHandle_t vH, diopiConstTensorHandle_t startH, diopiConstTensorHandle_t lenH, int maxInputLen) {
+  hipStream_t stream;
+  AMD_TRY(getStream(ctx, &stream));
+  TensorView out, q, k, v, st, ln;
+  AMD_TRY(getView(outH, &out, "out"));
+  AMD_TRY(getView(qH, &q, "q"));
+  AMD_TRY(getView(kH, &k, "k"));
+  AMD_TRY(getView(vH, &v, "v"));
+  AMD_TRY(getView(startH, &st, "b_start_loc"));
+  AMD_TRY(getView(lenH, &ln, "b_seq_len"));
+  AMD_CHECK(out.defined() && q.defined() && k.defined() && v.defined() && st.defined() && ln.defined(),
+            "context attention: null tensor");
+  AMD_CHECK(q.ndim == 3 && k.ndim == 3 && v.ndim == 3 && out.ndim == 3, "context attention: q/k/v/out must be [tokens, heads, head_dim]");
+  AMD_CHECK(q.dtype == k.dtype && q.dtype == v.dtype && q.dtype == out.dtype, "context attention: dtypes differ");
+  for (int d = 0; d < 3; ++d) {
+    AMD_CHECK(out.shape[d] == q.shape[d], "context attention: out shape differs from q at dim %d", d);
+    AMD_CHECK(k.shape[d] == v.shape[d], "context attention: k and v shapes differ at dim %d", d);
+  }
+  AMD_CHECK(k.shape[0] == q.shape[0] && k.shape[2] == q.shape[2], "context attention: k must cover the same tokens and head_dim as q");
+  AMD_CHECK(k.shape[1] > 0 && q.shape[1] % k.shape[1] == 0, "context attention: %ld heads are not a multiple of %ld kv heads",
+            (long)q.shape[1], (long)k.shape[1]);
+  AMD_CHECK((st.dtype == diopi_dtype_int32 || st.dtype == diopi_dtype_int64) &&
+                (ln.dtype == diopi_dtype_int32 || ln.dtype == diopi_dtype_int64),
+            "context attention: b_start_loc / b_seq_len must be int32 or int64");
+  AMD_CHECK(st.isContiguous() && ln.isContiguous() && st.numel == ln.numel, "context attention: b_start_loc / b_seq_len must be dense and equally long");
+  const int64_t batch = ln.numel;
+  if (batch == 0 || q.numel == 0 || maxInputLen <= 0) return diopiSuccess;
+  AMD_CHECK(batch <= 65535 && q.shape[1] <= 65535, "context attention: grid limits exceeded");
+  auto unit = [](const TensorView& t) { return t.stride[2] == 1 || t.shape[2] == 1; };
+  TensorView cq = q, ck = k, cv = v, co = out;
+  if (!unit(q)) AMD_TRY(makeContiguous(ctx, stream, q, &cq));
+  if (!unit(k)) AMD_TRY(makeContiguous(ctx, stream, k, &ck));
+  if (!unit(v)) AMD_TRY(makeContiguous(ctx, stream, v, &cv));
+  bool outTemp = !unit(out);
+  if (outTemp) {
+    diopiTensorHandle_t th;
+    AMD_TRY(requireTensor(ctx, out.shape, 3, out.dtype, &th, &co));
+  }
+  CaArgs a;
+  a.q = cq.data, a.k = ck.data, a.v = cv.data, a.out = co.data;
+  a.bStart = st.data, a.bLen = ln.data;
+  a.start64 = st.dtype == diopi_dtype_int64, a.len64 = ln.dtype == diopi_dtype_int64;
+  a.qTok = cq.stride[0], a.qHead = cq.stride[1], a.kTok = ck.stride[0], a.kHead = ck.stride[1];
+  a.vTok = cv.stride[0], a.vHead = cv.stride[1], a.oTok = co.stride[0], a.oHead = co.stride[1];
+  a.heads = (int)q.shape[1], a.kvHeads = (int)k.shape[1], a.d = (int)q.shape[2];
+  a.scale = 1.0f / sqrtf((float)a.d);
+  const bool half = q.dtype == diopi_dtype_bfloat16 || q.dtype == diopi_dtype_float16;
+  auto al = [](const TensorView& t) {
+    return t.aligned16() && (t.stride[0] * t.itemsize) % 16 == 0 && (t.stride[1] * t.itemsize) % 16 == 0;
+  };
+  diopiError_t err;
+  if (half && (a.d == 64 || a.d == 128) && al(cq) && al(ck) && al(cv) && al(co)) {
+    if (q.dtype == diopi_dtype_bfloat16)
+      err = a.d == 128 ? launchCaMfma<bf16_t, 128>(stream, a, maxInputLen, batch) : launchCaMfma<bf16_t, 64>(stream, a, maxInputLen, batch);
+    else
+      err = a.d == 128 ? launchCaMfma<half_t, 128>(stream, a, maxInputLen, batch) : launchCaMfma<half_t, 64>(stream, a, maxInputLen, batch);
+  } else {
+    AMD_CHECK(maxInputLen <= 12000, "context attention: the scalar path supports sequences up to 12000 tokens, got %d", maxInputLen);
+    AMD_CHECK(maxInputLen <= 65535, "context attention: grid limits exceeded");
+    size_t lds = ((size_t)maxInputLen + 8) * sizeof(float);
+    dim3 grid((unsigned)maxInputLen, a.heads, (unsigned)batch);
+    switch (q.dtype) {
+      case diopi_dtype_float32: hipLaunchKernelGGL(contextAttnScalarKernel<float>, grid, dim3(256), lds, stream, a, maxInputLen); break;
+      case diopi_dtype_bfloat16: hipLaunchKernelGGL(contextAttnScalarKernel<bf16_t>, grid, dim3(256), lds, stream, a, maxInputLen); break;
+      case diopi_dtype_float16: hipLaunchKernelGGL(contextAttnScalarKernel<half_t>, grid, dim3(256), lds, stream, a, maxInputLen); break;
+      default: setLastError("context attention: unsupported dtype %s", dtypeName(q.dtype)); return diopiErrorOccurred;
+    }
+    err = hipGetLastError() == hipSuccess ? diopiSuccess : diopiErrorOccurred;
+    if (err != diopiSuccess) setLastError("context attention: scalar kernel launch failed");
+  }
+  AMD_TRY(err);
+  if (outTemp) AMD_TRY(stridedCopy(stream, co, out));
+  return diopiSuccess;
+}

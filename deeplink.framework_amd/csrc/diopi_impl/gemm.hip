@@ -1,0 +1,651 @@
+// Dense contractions for gfx950: diopiMm, diopiBmm, diopiMatmul, diopiAddmm, diopiBaddbmm,
+// diopiLinear (dipu/scripts/autogen_diopi_wrapper/diopi_functions.yaml:594-597,902-909,
+// 1534-1548,1755-1765,1829-1837,1852-1893).
+//
+// MFMA engine (bf16 / fp16 inputs, fp32 accumulate) -- C[M,N] = A[M,K] . B[N,K]^T with both
+// operands K-contiguous, which is exactly what v_mfma_f32_32x32x16_{bf16,f16} wants: every
+// lane feeds 8 consecutive K elements (one 16-byte LDS read) of one row.
+//   * workgroup = 256 threads = 4 waves in a 2x2 arrangement; macro tile BM x BN x 64
+//     (256x256 for large problems: each wave owns 128x128 = 4x4 MFMA tiles, 256 fp32
+//     accumulators per lane; 128x128 otherwise);
+//   * global -> registers -> LDS with a two-stage LDS ring: tile k+1 is written to the other
+//     stage while tile k is being multiplied, tile k+2 is already in flight from HBM; one
+//     barrier per K tile;
+//   * LDS rows are 128 bytes (64 elements) with the 16-byte chunk index XOR-swizzled by
+//     (row & 7): both the 16-byte stores of the staging step and the ds_read_b128 operand
+//     fetches (32 consecutive rows, same logical chunk) are bank-conflict free;
+//   * workgroup ids are remapped so that each of the 8 XCDs (own L2 each) works on a
+//     contiguous band of tiles, walked in groups of 8 tile-rows to reuse A and B from L2;
+//   * epilogue: alpha * acc + beta * C + bias, converted and stored straight from the
+//     accumulator layout.
+// Operands that are not K-contiguous (mm with a row-major mat2, bmm's second operand) are
+// transposed once into workspace by a tiled LDS transpose, then use the same engine.
+//
+// FMA engine: fp32 (and any shape/stride/alignment the MFMA engine rejects): 64x64 LDS
+// tiles, 4x4 outputs per lane, fp32 accumulate.
+#include <algorithm>
+
+#include "gemm.hpp"
+
+namespace amd {
+
+// ------------------------------------------------------------- MFMA engine ---
+template <typename T>
+struct MfmaOp;
+template <>
+struct MfmaOp<bf16_t> {
+  typedef bf16x8 Frag;
+  static __device__ __forceinline__ f32x16 run(Frag a, Frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct MfmaOp<half_t> {
+  typedef f16x8 Frag;
+  static __device__ __forceinline__ f32x16 run(Frag a, Frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+struct MfmaArgs {
+  const void* A;
+  const void* B;
+  void* out;
+  const void* Cin;
+  const void* bias;
+  int64_t sAb, lda, sBb, ldb, sOb, ldo, sCb, sCm, sCn;
+  int M, N, K;
+  int tilesM, tilesN;
+  float alpha, beta;
+};
+
+constexpr int kBK = 64;  // K elements per LDS tile (128-byte rows)
+
+template <typename T, int BM, int BN>
+__global__ __launch_bounds__(256) void gemmMfmaKernel(MfmaArgs g) {
+  using Frag = typename MfmaOp<T>::Frag;
+  constexpr int WM = BM / 2, WN = BN / 2;      // per-wave tile
+  constexpr int TM = WM / 32, TN = WN / 32;    // MFMA tiles per wave
+  constexpr int A_CH = BM * 8 / 256, B_CH = BN * 8 / 256;  // 16-byte chunks per thread per K tile
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  T* sA = reinterpret_cast<T*>(smem);                  // [2][BM][64]
+  T* sB = sA + 2 * BM * kBK;                           // [2][BN][64]
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // ---- tile id: XCD band, then groups of 8 tile-rows
+  int tm, tn;
+  {
+    const int total = g.tilesM * g.tilesN;
+    const int pid = blockIdx.x;
+    const int xcd = pid & 7, idx = pid >> 3;
+    const int q = total >> 3, r = total & 7;
+    const int logical = xcd * q + min(xcd, r) + idx;
+    constexpr int GROUP = 8;
+    const int width = GROUP * g.tilesN;
+    const int group = logical / width;
+    const int first = group * GROUP;
+    const int gsize = min(g.tilesM - first, GROUP);
+    const int in = logical - group * width;
+    tm = first + in % gsize;
+    tn = in / gsize;
+  }
+  const int batch = blockIdx.z;
+  const T* A = reinterpret_cast<const T*>(g.A) + (int64_t)batch * g.sAb;
+  const T* B = reinterpret_cast<const T*>(g.B) + (int64_t)batch * g.sBb;
+
+  // ---- staging assignment: chunk id = tid + 256*i -> (row, 16-byte chunk)
+  const T* aPtr[A_CH];
+  const T* bPtr[B_CH];
+  int aOff[A_CH], bOff[B_CH];
+  const int c8 = (tid & 7) * 8;  // K offset of this thread's chunk inside a tile
+#pragma unroll
+  for (int i = 0; i < A_CH; ++i) {
+    int row = (tid >> 3) + 32 * i;
+    int grow = min(tm * BM + row, g.M - 1);
+    aPtr[i] = A + (int64_t)grow * g.lda + c8;
+    aOff[i] = row * kBK + (((tid & 7) ^ (row & 7)) << 3);
+  }
+#pragma unroll
+  for (int i = 0; i < B_CH; ++i) {
+    int row = (tid >> 3) + 32 * i;
+    int grow = min(tn * BN + row, g.N - 1);
+    bPtr[i] = B + (int64_t)grow * g.ldb + c8;
+    bOff[i] = row * kBK + (((tid & 7) ^ (row & 7)) << 3);
+  }
+  Frag ra[A_CH], rb[B_CH];
+  const int nK = (g.K + kBK - 1) / kBK;
+
+  auto gload = [&](int kt) {
+    const int k0 = kt * kBK;
+    const bool inK = k0 + c8 < g.K;  // K is a multiple of 8: a chunk is entirely in or out
+    const u32x4 zero4 = {0u, 0u, 0u, 0u};
+    const Frag z = __builtin_bit_cast(Frag, zero4);
+#pragma unroll
+    for (int i = 0; i < A_CH; ++i) ra[i] = inK ? *reinterpret_cast<const Frag*>(aPtr[i] + k0) : z;
+#pragma unroll
+    for (int i = 0; i < B_CH; ++i) rb[i] = inK ? *reinterpret_cast<const Frag*>(bPtr[i] + k0) : z;
+  };
+  auto swrite = [&](int stage) {
+    T* a = sA + stage * BM * kBK;
+    T* b = sB + stage * BN * kBK;
+#pragma unroll
+    for (int i = 0; i < A_CH; ++i) *reinterpret_cast<Frag*>(a + aOff[i]) = ra[i];
+#pragma unroll
+    for (int i = 0; i < B_CH; ++i) *reinterpret_cast<Frag*>(b + bOff[i]) = rb[i];
+  };
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // operand fetch offsets: row = lane&31 inside an MFMA tile, chunk = 2*ks + (lane>>5)
+  const int frow = lane & 31, fhalf = lane >> 5;
+
+  gload(0);
+  swrite(0);
+  if (nK > 1) gload(1);
+  __syncthreads();
+
+  for (int kt = 0; kt < nK; ++kt) {
+    const int cur = kt & 1;
+    const T* a = sA + cur * BM * kBK + (wm * WM) * kBK;
+    const T* b = sB + cur * BN * kBK + (wn * WN) * kBK;
+#pragma unroll
+    for (int ks = 0; ks < kBK / 16; ++ks) {
+      Frag fa[TM], fb[TN];
+      const int chunk = 2 * ks + fhalf;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        int row = i * 32 + frow;
+        fa[i] = *reinterpret_cast<const Frag*>(a + row * kBK + ((chunk ^ (row & 7)) << 3));
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        int row = j * 32 + frow;
+        fb[j] = *reinterpret_cast<const Frag*>(b + row * kBK + ((chunk ^ (row & 7)) << 3));
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = MfmaOp<T>::run(fa[i], fb[j], acc[i][j]);
+    }
+    if (kt + 1 < nK) {
+      swrite(cur ^ 1);                 // tile kt+1 (loaded during the previous iteration)
+      if (kt + 2 < nK) gload(kt + 2);  // in flight across the next iteration's math
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue
+  T* out = reinterpret_cast<T*>(g.out) + (int64_t)batch * g.sOb;
+  const T* cin = g.Cin ? reinterpret_cast<const T*>(g.Cin) + (int64_t)batch * g.sCb : nullptr;
+  const T* bias = reinterpret_cast<const T*>(g.bias);
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int col = tn * BN + wn * WN + j * 32 + frow;
+    if (col >= g.N) continue;
+    const float bv = bias ? static_cast<float>(bias[col]) : 0.f;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int rbase = tm * BM + wm * WM + i * 32 + fhalf * 4;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = rbase + (r >> 2) * 8 + (r & 3);
+        if (row < g.M) {
+          float v = acc[i][j][r] * g.alpha + bv;
+          if (cin) v += g.beta * static_cast<float>(cin[(int64_t)row * g.sCm + (int64_t)col * g.sCn]);
+          out[(int64_t)row * g.ldo + col] = static_cast<T>(v);
+        }
+      }
+    }
+  }
+}
+
+// -------------------------------------------------------------- transpose ----
+// dst[b, c, r] = src[b, r, c] for 2-byte or 4-byte elements, 64x64 tiles through LDS.
+template <typename U>
+__global__ __launch_bounds__(256) void transposeKernel(U* __restrict__ dst, const U* __restrict__ src, int64_t rows,
+                                                        int64_t cols, int64_t srcRowStride, int64_t srcColStride,
+                                                        int64_t srcBatchStride, int64_t dstBatchStride) {
+  __shared__ U tile[64][65];
+  const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+  src += blockIdx.z * srcBatchStride;
+  dst += blockIdx.z * dstBatchStride;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  // read with lanes along whichever source dim is contiguous
+  if (srcColStride == 1) {
+    for (int i = ty; i < 64; i += 4) {
+      int64_t r = r0 + i, c = c0 + tx;
+      if (r < rows && c < cols) tile[i][tx] = src[r * srcRowStride + c];
+    }
+  } else {
+    for (int i = ty; i < 64; i += 4) {
+      int64_t r = r0 + tx, c = c0 + i;
+      if (r < rows && c < cols) tile[tx][i] = src[r * srcRowStride + c * srcColStride];
+    }
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    int64_t c = c0 + i, r = r0 + tx;
+    if (r < rows && c < cols) dst[c * rows + r] = tile[tx][i];
+  }
+}
+
+// ---------------------------------------------------------------- FMA engine --
+template <typename T>
+__global__ __launch_bounds__(256) void gemmFmaKernel(GemmProblem p) {
+  __shared__ float sA[16][64 + 4];
+  __shared__ float sB[16][64 + 4];
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  const int64_t m0 = (int64_t)blockIdx.y * 64, n0 = (int64_t)blockIdx.x * 64;
+  const int64_t b = blockIdx.z;
+  const T* A = reinterpret_cast<const T*>(p.A) + b * p.sAb;
+  const T* B = reinterpret_cast<const T*>(p.B) + b * p.sBb;
+  float acc[4][4] = {{0.f}};
+  for (int64_t k0 = 0; k0 < p.K; k0 += 16) {
+    // 64 rows x 16 k per operand = 1024 elements, 4 per thread
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int e = threadIdx.x + 256 * i;
+      int kk, rr;
+      if (p.sAk == 1) kk = e & 15, rr = e >> 4; else rr = e & 63, kk = e >> 6;
+      int64_t m = m0 + rr, k = k0 + kk;
+      sA[kk][rr] = (m < p.M && k < p.K) ? static_cast<float>(A[m * p.sAm + k * p.sAk]) : 0.f;
+      if (p.sBk == 1) kk = e & 15, rr = e >> 4; else rr = e & 63, kk = e >> 6;
+      int64_t n = n0 + rr;
+      k = k0 + kk;
+      sB[kk][rr] = (n < p.N && k < p.K) ? static_cast<float>(B[n * p.sBn + k * p.sBk]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 16; ++kk) {
+      float a[4], bb[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = sA[kk][ty * 4 + i], bb[i] = sB[kk][tx * 4 + i];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], bb[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+  T* out = reinterpret_cast<T*>(p.out) + b * p.sOb;
+  const T* cin = p.Cin ? reinterpret_cast<const T*>(p.Cin) + b * p.sCb : nullptr;
+  const T* bias = reinterpret_cast<const T*>(p.bias);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int64_t m = m0 + ty * 4 + i;
+    if (m >= p.M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int64_t n = n0 + tx * 4 + j;
+      if (n >= p.N) continue;
+      float v = acc[i][j] * p.alpha;
+      if (bias) v += static_cast<float>(bias[n]);
+      if (cin) v += p.beta * static_cast<float>(cin[m * p.sCm + n * p.sCn]);
+      out[m * p.sOm + n] = static_cast<T>(v);
+    }
+  }
+}
+
+__global__ void gemmFmaKernelF64(GemmProblem p) {
+  // double precision: one output per lane, plain loop (correctness path only)
+  int64_t n = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t m = blockIdx.y, b = blockIdx.z;
+  if (n >= p.N) return;
+  const double* A = reinterpret_cast<const double*>(p.A) + b * p.sAb + m * p.sAm;
+  const double* B = reinterpret_cast<const double*>(p.B) + b * p.sBb + n * p.sBn;
+  double acc = 0.0;
+  for (int64_t k = 0; k < p.K; ++k) acc += A[k * p.sAk] * B[k * p.sBk];
+  double v = acc * (double)p.alpha;
+  if (p.bias) v += reinterpret_cast<const double*>(p.bias)[n];
+  if (p.Cin) v += (double)p.beta * (reinterpret_cast<const double*>(p.Cin) + b * p.sCb)[m * p.sCm + n * p.sCn];
+  (reinterpret_cast<double*>(p.out) + b * p.sOb)[m * p.sOm + n] = v;
+}
+
+// ------------------------------------------------------------------ driver ---
+template <typename T, int BM, int BN>
+static diopiError_t launchMfma(hipStream_t stream, const GemmProblem& p) {
+  MfmaArgs g;
+  g.A = p.A, g.B = p.B, g.out = p.out, g.Cin = p.Cin, g.bias = p.bias;
+  g.sAb = p.sAb, g.lda = p.sAm, g.sBb = p.sBb, g.ldb = p.sBn, g.sOb = p.sOb, g.ldo = p.sOm;
+  g.sCb = p.sCb, g.sCm = p.sCm, g.sCn = p.sCn;
+  g.M = (int)p.M, g.N = (int)p.N, g.K = (int)p.K;
+  g.tilesM = (int)ceilDiv(p.M, BM), g.tilesN = (int)ceilDiv(p.N, BN);
+  g.alpha = p.alpha, g.beta = p.beta;
+  constexpr size_t lds = 2 * (size_t)(BM + BN) * kBK * sizeof(T);
+  static bool attrSet = false;  // per template instance
+  if (!attrSet) {
+    AMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemmMfmaKernel<T, BM, BN>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attrSet = true;
+  }
+  dim3 grid((unsigned)(g.tilesM * g.tilesN), 1, (unsigned)p.batch);
+  hipLaunchKernelGGL((gemmMfmaKernel<T, BM, BN>), grid, dim3(256), lds, stream, g);
+  AMD_LAUNCH_CHECK();
+  return diopiSuccess;
+}
+
+static bool mult8(int64_t v) { return (v & 7) == 0; }
+static bool ptr16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+template <typename U>
+static diopiError_t launchTranspose(hipStream_t stream, void* dst, const void* src, int64_t batch, int64_t rows,
+                                    int64_t cols, int64_t sRow, int64_t sCol, int64_t sBatch) {
+  dim3 grid((unsigned)ceilDiv(cols, 64), (unsigned)ceilDiv(rows, 64), (unsigned)batch);
+  hipLaunchKernelGGL(transposeKernel<U>, grid, dim3(256), 0, stream, (U*)dst, (const U*)src, rows, cols, sRow, sCol,
+                     sBatch, rows * cols);
+  AMD_LAUNCH_CHECK();
+  return diopiSuccess;
+}
+
+diopiError_t runGemm(diopiContextHandle_t ctx, hipStream_t stream, GemmProblem p) {
+  if (p.batch == 0 || p.M == 0 || p.N == 0) return diopiSuccess;
+  AMD_CHECK(p.batch <= 65535, "gemm: batch %ld exceeds the grid limit", (long)p.batch);
+  const bool half = p.dtype == diopi_dtype_bfloat16 || p.dtype == diopi_dtype_float16;
+  if (half && p.K > 0 && mult8(p.K) && p.M < (int64_t(1) << 31) && p.N < (int64_t(1) << 31)) {
+    const int64_t item = 2;
+    // bring both operands to K-contiguous storage: dst[b, r, k] with rows M (or N)
+    if (p.sAk != 1 || !mult8(p.sAm) || !mult8(p.sAb) || !ptr16(p.A)) {
+      void* ws = nullptr;
+      AMD_TRY(requireWorkspace(ctx, p.batch * p.M * p.K * item, &ws));
+      // source viewed as [K rows, M cols] -> destination [M, K]
+      AMD_TRY(launchTranspose<uint16_t>(stream, ws, p.A, p.batch, p.K, p.M, p.sAk, p.sAm, p.sAb));
+      p.A = ws, p.sAk = 1, p.sAm = p.K, p.sAb = p.M * p.K;
+    }
+    if (p.sBk != 1 || !mult8(p.sBn) || !mult8(p.sBb) || !ptr16(p.B)) {
+      void* ws = nullptr;
+      AMD_TRY(requireWorkspace(ctx, p.batch * p.N * p.K * item, &ws));
+      int64_t sbb = p.sBb;
+      int64_t nb = p.batch;
+      if (sbb == 0) nb = 1;  // a shared (broadcast) weight is transposed once
+      AMD_TRY(launchTranspose<uint16_t>(stream, ws, p.B, nb, p.K, p.N, p.sBk, p.sBn, sbb));
+      p.B = ws, p.sBk = 1, p.sBn = p.K, p.sBb = (sbb == 0) ? 0 : p.N * p.K;
+    }
+    const bool big = ceilDiv(p.M, 256) * ceilDiv(p.N, 256) * p.batch >= 200;
+    if (p.dtype == diopi_dtype_bfloat16) {
+      return big ? launchMfma<bf16_t, 256, 256>(stream, p) : launchMfma<bf16_t, 128, 128>(stream, p);
+    }
+    return big ? launchMfma<half_t, 256, 256>(stream, p) : launchMfma<half_t, 128, 128>(stream, p);
+  }
+  if (p.dtype == diopi_dtype_float64) {
+    dim3 grid((unsigned)ceilDiv(p.N, 256), (unsigned)p.M, (unsigned)p.batch);
+    AMD_CHECK(p.M <= 65535, "gemm(float64): M exceeds the grid limit");
+    hipLaunchKernelGGL(gemmFmaKernelF64, grid, dim3(256), 0, stream, p);
+    AMD_LAUNCH_CHECK();
+    return diopiSuccess;
+  }
+  AMD_CHECK(ceilDiv(p.M, 64) <= 65535, "gemm: M exceeds the grid limit of the FMA engine");
+  dim3 grid((unsigned)ceilDiv(p.N, 64), (unsigned)ceilDiv(p.M, 64), (unsigned)p.batch);
+  switch (p.dtype) {
+    case diopi_dtype_float32: hipLaunchKernelGGL(gemmFmaKernel<float>, grid, dim3(256), 0, stream, p); break;
+    case diopi_dtype_bfloat16: hipLaunchKernelGGL(gemmFmaKernel<bf16_t>, grid, dim3(256), 0, stream, p); break;
+    case diopi_dtype_float16: hipLaunchKernelGGL(gemmFmaKernel<half_t>, grid, dim3(256), 0, stream, p); break;
+    default: setLastError("gemm: unsupported dtype %s", dtypeName(p.dtype)); return diopiErrorOccurred;
+  }
+  AMD_LAUNCH_CHECK();
+  return diopiSuccess;
+}
+
+// ------------------------------------------------------------- entry helpers --
+// Folds leading dims of a dense-enough view into one batch dim; returns false if impossible.
+static bool foldBatch(const TensorView& t, int lead, int64_t* count, int64_t* stride) {
+  int64_t n = 1, s = 0;
+  bool have = false;
+  for (int d = lead - 1; d >= 0; --d) {
+    if (t.shape[d] == 1) continue;
+    if (!have) s = t.stride[d], have = true;
+    else if (t.stride[d] != s * n) return false;
+    n *= t.shape[d];
+  }
+  *count = n;
+  *stride = have ? s : 0;
+  return true;
+}
+
+struct MatOperand {
+  TensorView v;
+  int64_t batch = 1, sb = 0;
+};
+
+// out[..., M, N] = A[..., M, K] @ B[..., K, N] with equal (or size-1 / absent) batch dims.
+static diopiError_t batchedMatmul(diopiContextHandle_t ctx, hipStream_t stream, const TensorView& out,
+                                  const TensorView& a, const TensorView& b, const TensorView* cin, const TensorView* bias,
+                                  float alpha, float beta, bool bIsNK) {
+  AMD_CHECK(a.ndim >= 2 && b.ndim >= 2 && out.ndim >= 2, "matmul: operands must have rank >= 2 here");
+  AMD_CHECK(a.dtype == b.dtype && a.dtype == out.dtype, "matmul: dtypes differ (%s, %s -> %s)", dtypeName(a.dtype),
+            dtypeName(b.dtype), dtypeName(out.dtype));
+  GemmProblem p;
+  p.dtype = a.dtype;
+  p.M = a.shape[a.ndim - 2];
+  p.K = a.shape[a.ndim - 1];
+  int64_t bK = bIsNK ? b.shape[b.ndim - 1] : b.shape[b.ndim - 2];
+  p.N = bIsNK ? b.shape[b.ndim - 2] : b.shape[b.ndim - 1];
+  AMD_CHECK(bK == p.K, "matmul: inner dims differ (%ld vs %ld)", (long)p.K, (long)bK);
+  AMD_CHECK(out.shape[out.ndim - 2] == p.M && out.shape[out.ndim - 1] == p.N, "matmul: output is [%ld,%ld], expected [%ld,%ld]",
+            (long)out.shape[out.ndim - 2], (long)out.shape[out.ndim - 1], (long)p.M, (long)p.N);
+  int64_t ob, os, ab, as, bb, bs;
+  TensorView oc = out, ac = a, bc = b;
+  bool outTemp = false;
+  if (!(out.stride[out.ndim - 1] == 1 || p.N == 1) || !foldBatch(out, out.ndim - 2, &ob, &os)) {
+    diopiTensorHandle_t th;
+    AMD_TRY(requireTensor(ctx, out.shape, out.ndim, out.dtype, &th, &oc));
+    outTemp = true;
+    foldBatch(oc, oc.ndim - 2, &ob, &os);
+  }
+  if (!foldBatch(ac, ac.ndim - 2, &ab, &as)) {
+    AMD_TRY(makeContiguous(ctx, stream, a, &ac));
+    foldBatch(ac, ac.ndim - 2, &ab, &as);
+  }
+  if (!foldBatch(bc, bc.ndim - 2, &bb, &bs)) {
+    AMD_TRY(makeContiguous(ctx, stream, b, &bc));
+    foldBatch(bc, bc.ndim - 2, &bb, &bs);
+  }
+  AMD_CHECK((ab == ob || ab == 1) && (bb == ob || bb == 1), "matmul: batch dims %ld and %ld do not match output batch %ld",
+            (long)ab, (long)bb, (long)ob);
+  p.batch = ob;
+  p.A = ac.data, p.sAb = ab == 1 ? 0 : as, p.sAm = ac.stride[ac.ndim - 2], p.sAk = ac.stride[ac.ndim - 1];
+  p.B = bc.data, p.sBb = bb == 1 ? 0 : bs;
+  if (bIsNK) p.sBn = bc.stride[bc.ndim - 2], p.sBk = bc.stride[bc.ndim - 1];
+  else p.sBk = bc.stride[bc.ndim - 2], p.sBn = bc.stride[bc.ndim - 1];
+  p.out = oc.data, p.sOb = os, p.sOm = oc.stride[oc.ndim - 2];
+  if (p.M == 1) p.sOm = p.N;  // a single row: its stride is never used, keep it sane
+  // A shared A with per-batch B cannot fold; a shared B with per-batch A folds the batch into M.
+  if (p.sBb == 0 && p.batch > 1 && p.sAb == p.M * p.sAm && p.sOb == p.M * p.sOm && cin == nullptr) {
+    p.M *= p.batch;
+    p.batch = 1;
+    p.sAb = p.sOb = 0;
+  }
+  p.alpha = alpha, p.beta = beta;
+  if (bias) p.bias = bias->data;
+  if (cin && beta != 0.f) {
+    // broadcast Cin against [batch, M, N]
+    const TensorView& c = *cin;
+    AMD_CHECK(c.dtype == out.dtype, "matmul: addend dtype differs from output dtype");
+    p.Cin = c.data;
+    auto ext = [&](int fromEnd) { return c.ndim >= fromEnd ? c.shape[c.ndim - fromEnd] : 1; };
+    auto str = [&](int fromEnd) { return (c.ndim >= fromEnd && c.shape[c.ndim - fromEnd] != 1) ? c.stride[c.ndim - fromEnd] : 0; };
+    AMD_CHECK(ext(1) == p.N || ext(1) == 1, "matmul: addend last dim %ld does not broadcast to %ld", (long)ext(1), (long)p.N);
+    AMD_CHECK(ext(2) == p.M || ext(2) == 1, "matmul: addend rows %ld do not broadcast to %ld", (long)ext(2), (long)p.M);
+    p.sCn = str(1), p.sCm = str(2);
+    if (c.ndim > 2) {
+      TensorView lead = c;
+      int64_t cb, cs;
+      AMD_CHECK(foldBatch(lead, c.ndim - 2, &cb, &cs) && (cb == p.batch || cb == 1), "matmul: addend batch dims do not match");
+      p.sCb = cb == 1 ? 0 : cs;
+    }
+  }
+  AMD_TRY(runGemm(ctx, stream, p));
+  if (outTemp) AMD_TRY(stridedCopy(stream, oc, out));
+  return diopiSuccess;
+}
+
+}  // namespace amd
+
+using namespace amd;
+#define GEMM_EXPORT extern "C" __attribute__((visibility("default")))
+
+GEMM_EXPORT diopiError_t diopiMm(diopiContextHandle_t ctx, diopiTensorHandle_t outH, diopiConstTensorHandle_t aH,
+                                 diopiConstTensorHandle_t bH) {
+  hipStream_t stream;
+  AMD_TRY(getStream(ctx, &stream));
+  TensorView out, a, b;
+  AMD_TRY(getView(outH, &out, "out"));
+  AMD_TRY(getView(aH, &a, "input"));
+  AMD_TRY(getView(bH, &b, "mat2"));
+  AMD_CHECK(out.defined() && a.defined() && b.defined(), "diopiMm: null tensor");
+  AMD_CHECK(a.ndim == 2 && b.ndim == 2 && out.ndim == 2, "diopiMm: operands must be 2-D");
+  return batchedMatmul(ctx, stream, out, a, b, nullptr, nullptr, 1.f, 0.f, false);
+}
+
+GEMM_EXPORT diopiError_t diopiBmm(diopiContextHandle_t ctx, diopiTensorHandle_t outH, diopiConstTensorHandle_t aH,
+                                  diopiConstTensorHandle_t bH) {
+  hipStream_t stream;
+  AMD_TRY(getStream(ctx, &stream));
+  TensorView out, a, b;
+  AMD_TRY(getView(outH, &out, "out"));
+  AMD_TRY(getView(aH, &a, "input"));
+  AMD_TRY(getView(bH, &b, "mat2"));
+  AMD_CHECK(out.defined() && a.defined() && b.defined(), "diopiBmm: null tensor");
+  AMD_CHECK(a.ndim == 3 && b.ndim == 3 && out.ndim == 3, "diopiBmm: operands must be 3-D");
+  AMD_CHECK(a.shape[0] == b.shape[0] && a.shape[0] == out.shape[0], "diopiBmm: batch sizes differ");
+  return batchedMatmul(ctx, stream, out, a, b, nullptr, nullptr, 1.f, 0.f, false);
+}
+
+// Views a tensor with extra unit dims so that 1-D operands become matrices.
+static TensorView unsqueeze(const TensorView& t, int at) {
+  TensorView r = t;
+  for (int d = t.ndim; d > at; --d) r.shape[d] = t.shape[d - 1], r.stride[d] = t.stride[d - 1];
+  r.shape[at] = 1;
+  r.stride[at] = 0;
+  r.ndim = t.ndim + 1;
+  return r;
+}
+
+GEMM_EXPORT diopiError_t diopiMatmul(diopiContextHandle_t ctx, diopiTensorHandle_t outH, diopiConstTensorHandle_t aH,
+                                     diopiConstTensorHandle_t bH) {
+  hipStream_t stream;
+  AMD_TRY(getStream(ctx, &stream));
+  TensorView out, a, b;
+  AMD_TRY(getView(outH, &out, "out"));
+  AMD_TRY(getView(aH, &a, "input"));
+  AMD_TRY(getView(bH, &b, "other"));
+  AMD_CHECK(out.defined() && a.defined() && b.defined(), "diopiMatmul: null tensor");
+  AMD_CHECK(a.ndim >= 1 && b.ndim >= 1, "diopiMatmul: operands must have at least one dim");
+  AMD_CHECK(a.ndim < kMaxDims && b.ndim < kMaxDims && out.ndim + 2 <= kMaxDims, "diopiMatmul: rank too large");
+  // torch.matmul: a 1-D left operand gains a leading unit dim, a 1-D right operand a trailing one
+  TensorView a2 = a, b2 = b, o2 = out;
+  if (a.ndim == 1) a2 = unsqueeze(a, 0);
+  if (b.ndim == 1) b2 = unsqueeze(b, 1);
+  if (a.ndim == 1 && b.ndim == 1) {
+    o2 = unsqueeze(unsqueeze(out, out.ndim), out.ndim + 1);
+  } else if (a.ndim == 1) {
+    o2 = unsqueeze(out, out.ndim - 1);
+  } else if (b.ndim == 1) {
+    o2 = unsqueeze(out, out.ndim);
+  }
+  // broadcast batch dims: expand both to the output's batch shape when they differ
+  int nb = o2.ndim - 2;
+  auto expandTo = [&](const TensorView& t, TensorView* e) {
+    *e = o2;
+    e->data = t.data;
+    e->dtype = t.dtype;
+    e->itemsize = t.itemsize;
+    int shift = o2.ndim - t.ndim;
+    for (int d = 0; d < o2.ndim; ++d) {
+      if (d >= nb) {
+        e->shape[d] = t.shape[d - shift];
+        e->stride[d] = t.stride[d - shift];
+      } else if (d < shift || t.shape[d - shift] == 1) {
+        e->stride[d] = 0;
+      } else {
+        e->stride[d] = t.stride[d - shift];
+      }
+    }
+    e->numel = 1;
+    for (int d = 0; d < e->ndim; ++d) e->numel *= e->shape[d];
+  };
+  TensorView ae, be;
+  AMD_CHECK(a2.ndim <= o2.ndim && b2.ndim <= o2.ndim, "diopiMatmul: output rank too small");
+  expandTo(a2, &ae);
+  expandTo(b2, &be);
+  // fully shared operands keep a single copy (batch count 1); partially broadcast ones are materialised
+  auto normalise = [&](TensorView& e, const TensorView& orig) -> diopiError_t {
+    bool allZero = true, anyZero = false;
+    for (int d = 0; d < nb; ++d) {
+      if (e.shape[d] == 1) continue;
+      if (e.stride[d] == 0) anyZero = true; else allZero = false;
+    }
+    if (anyZero && allZero) {
+      for (int d = 0; d < nb; ++d) e.shape[d] = 1;
+    } else if (anyZero) {
+      TensorView dense;
+      AMD_TRY(makeContiguous(ctx, stream, e, &dense));
+      e = dense;
+    }
+    (void)orig;
+    return diopiSuccess;
+  };
+  AMD_TRY(normalise(ae, a2));
+  AMD_TRY(normalise(be, b2));
+  return batchedMatmul(ctx, stream, o2, ae, be, nullptr, nullptr, 1.f, 0.f, false);
+}
+
+GEMM_EXPORT diopiError_t diopiAddmm(diopiContextHandle_t ctx, diopiTensorHandle_t outH, diopiConstTensorHandle_t inH,
+                                    diopiConstTensorHandle_t m1H, diopiConstTensorHandle_t m2H,
+                                    const diopiScalar_t* beta, const diopiScalar_t* alpha) {
+  hipStream_t stream;
+  AMD_TRY(getStream(ctx, &stream));
+  TensorView out, in, a, b;
+  AMD_TRY(getView(outH, &out, "out"));
+  AMD_TRY(getView(inH, &in, "input"));
+  AMD_TRY(getView(m1H, &a, "mat1"));
+  AMD_TRY(getView(m2H, &b, "mat2"));
+  AMD_CHECK(out.defined() && in.defined() && a.defined() && b.defined(), "diopiAddmm: null tensor");
+  AMD_CHECK(a.ndim == 2 && b.ndim == 2 && out.ndim == 2 && in.ndim <= 2, "diopiAddmm: bad ranks");
+  return batchedMatmul(ctx, stream, out, a, b, &in, nullptr, (float)scalarToDouble(alpha, 1.0),
+                       (float)scalarToDouble(beta, 1.0), false);
+}
+
+GEMM_EXPORT diopiError_t diopiBaddbmm(diopiContextHandle_t ctx, diopiTensorHandle_t outH, diopiConstTensorHandle_t inH,
+                                      diopiConstTensorHandle_t b1H, diopiConstTensorHandle_t b2H, double beta,
+                                      double alpha) {
+  hipStream_t stream;
+  AMD_TRY(getStream(ctx, &stream));
+  TensorView out, in, a, b;
+  AMD_TRY(getView(outH, &out, "out"));
+  AMD_TRY(getView(inH, &in, "input"));
+  AMD_TRY(getView(b1H, &a, "batch1"));
+  AMD_TRY(getView(b2H, &b, "batch2"));
+  AMD_CHECK(out.defined() && in.defined() && a.defined() && b.defined(), "diopiBaddbmm: null tensor");
+  AMD_CHECK(a.ndim == 3 && b.ndim == 3 && out.ndim == 3 && in.ndim <= 3, "diopiBaddbmm: bad ranks");
+  return batchedMatmul(ctx, stream, out, a, b, &in, nullptr, (float)alpha, (float)beta, false);
+}
+
+GEMM_EXPORT diopiError_t diopiLinear(diopiContextHandle_t ctx, diopiTensorHandle_t outH, diopiConstTensorHandle_t inH,
+                                     diopiConstTensorHandle_t wH, diopiConstTensorHandle_t biasH) {
+  hipStream_t stream;
+  AMD_TRY(getStream(ctx, &stream));
+  TensorView out, in, w, bias;
+  AMD_TRY(getView(outH, &out, "out"));
+  AMD_TRY(getView(inH, &in, "input"));
+  AMD_TRY(getView(wH, &w, "weight"));
+  AMD_TRY(getView(biasH, &bias, "bias"));
+  AMD_CHECK(out.defined() && in.defined() && w.defined(), "diopiLinear: null tensor");
+  AMD_CHECK(w.ndim == 2 && in.ndim >= 1 && out.ndim == in.ndim, "diopiLinear: weight must be [N, K], out shaped like input");
+  AMD_CHECK(in.ndim + 1 <= kMaxDims, "diopiLinear: rank too large");
+  TensorView cb;
+  if (bias.defined()) {
+    AMD_CHECK(bias.numel == w.shape[0] && bias.dtype == out.dtype, "diopiLinear: bias must hold N elements of the output dtype");
+    AMD_TRY(makeContiguous(ctx, stream, bias, &cb));
+  }
+  TensorView in2 = in, out2 = out;
+  if (in.ndim == 1) in2 = unsqueeze(in, 0), out2 = unsqueeze(out, 0);
+  return batchedMatmul(ctx, stream, out2, in2, w, nullptr, bias.defined() ? &cb : nullptr, 1.f, 0.f, true);
+}

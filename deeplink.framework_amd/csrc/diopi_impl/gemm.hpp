@@ -1,0 +1,30 @@
+// Internal GEMM interface shared by the dense (diopiMm/Bmm/Matmul/Addmm/Baddbmm/Linear)
+// entry points. One problem description, two engines:
+//   * the MFMA engine (bf16/fp16, fp32 accumulate) for K-contiguous operands,
+//   * a strided fp32-accumulate FMA engine for everything else (fp32, odd shapes).
+#pragma once
+
+#include "common.hpp"
+
+namespace amd {
+
+// out[b, m, n] = alpha * sum_k A[b, m, k] * B[b, n, k]  +  beta * Cin[b, m, n]  +  bias[n]
+// All strides in elements. B is described in [N, K] orientation whatever its storage order.
+struct GemmProblem {
+  diopiDtype_t dtype = diopi_dtype_unsupported;  // A, B, out (and Cin/bias) element type
+  int64_t batch = 1, M = 0, N = 0, K = 0;
+  const void* A = nullptr;
+  int64_t sAb = 0, sAm = 0, sAk = 0;
+  const void* B = nullptr;
+  int64_t sBb = 0, sBn = 0, sBk = 0;
+  void* out = nullptr;
+  int64_t sOb = 0, sOm = 0;  // out: n-contiguous
+  const void* Cin = nullptr;
+  int64_t sCb = 0, sCm = 0, sCn = 0;
+  const void* bias = nullptr;
+  float alpha = 1.f, beta = 0.f;
+};
+
+diopiError_t runGemm(diopiContextHandle_t ctx, hipStream_t stream, GemmProblem p);
+
+}  // namespace amd

@@ -1,0 +1,380 @@
+// diopiRotaryEmbedding, diopiDestIndexCopyKV and diopiIndexPutInp for gfx950.
+//
+// Rotary: x viewed as [tokens, heads, d]; each lane rotates 8 (bf16/fp16) or 4 (fp32)
+// pairs: one 16-byte load from each half of the head row (half-split layout) or one
+// 16-byte load of adjacent pairs (interleaved layout), one cos and one sin vector that
+// all heads of the token share (served by L2 after the first head), fp32 math, 16-byte
+// stores. Algorithmic traffic = 2 * |x| + |cos| + |sin|.
+//   half-split : dicp/dicp/vendor/AscendGraph/ext_ops.py:24-33
+//   interleaved: dicp/test/model/llama/model.py:58-69 (complex multiply by cos + i sin)
+//
+// DestIndexCopyKV: out[dest_loc[i], :, :] = k[i, :, :], a pure byte move done with the
+// widest vector the row size and pointers allow; one workgroup per token row.
+#include "common.hpp"
+
+namespace amd {
+
+// ------------------------------------------------------------------ rotary ---
+template <typename T, typename CT, bool INTERLEAVED>
+__global__ __launch_bounds__(256) void rotaryVecKernel(T* __restrict__ out, const T* __restrict__ x,
+                                                        const CT* __restrict__ cosT, const CT* __restrict__ sinT,
+                                                        int64_t tokens, int heads, int d, int64_t tableRows,
+                                                        int tableCols, float sinSign) {
+  using V = typename Vec16<T>::type;
+  constexpr int N = Vec16<T>::N;
+  const int half = d / 2;
+  // half-split: a work item is (token, head, j) with j indexing N-element groups of the first half
+  // interleaved: a work item covers N elements = N/2 pairs
+  const int perHead = INTERLEAVED ? d / N : half / N;
+  const int64_t total = tokens * heads * perHead;
+  for (int64_t w = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; w < total; w += (int64_t)gridDim.x * blockDim.x) {
+    const int j = (int)(w % perHead);
+    const int64_t th = w / perHead;
+    const int64_t t = th / heads;
+    const int64_t trow = t % tableRows;
+    const T* xr = x + th * d;
+    T* outr = out + th * d;
+    if constexpr (!INTERLEAVED) {
+      V a = *reinterpret_cast<const V*>(xr + j * N);
+      V b = *reinterpret_cast<const V*>(xr + half + j * N);
+      V oa, ob;
+#pragma unroll
+      for (int e = 0; e < N; ++e) {
+        float c = static_cast<float>(cosT[trow * tableCols + j * N + e]);
+        float s = static_cast<float>(sinT[trow * tableCols + j * N + e]) * sinSign;
+        float x0 = static_cast<float>(a[e]), x1 = static_cast<float>(b[e]);
+        oa[e] = static_cast<T>(x0 * c - x1 * s);
+        ob[e] = static_cast<T>(x0 * s + x1 * c);
+      }
+      *reinterpret_cast<V*>(outr + j * N) = oa;
+      *reinterpret_cast<V*>(outr + half + j * N) = ob;
+    } else {
+      V a = *reinterpret_cast<const V*>(xr + j * N);
+      V o;
+      // tables with d/2 columns hold one angle per pair; tables with d columns hold it at 2i
+      const int step = (tableCols == d) ? 2 : 1;
+#pragma unroll
+      for (int e = 0; e < N / 2; ++e) {
+        int pair = j * (N / 2) + e;
+        float c = static_cast<float>(cosT[trow * tableCols + pair * step]);
+        float s = static_cast<float>(sinT[trow * tableCols + pair * step]) * sinSign;
+        float x0 = static_cast<float>(a[2 * e]), x1 = static_cast<float>(a[2 * e + 1]);
+        o[2 * e] = static_cast<T>(x0 * c - x1 * s);
+        o[2 * e + 1] = static_cast<T>(x0 * s + x1 * c);
+      }
+      *reinterpret_cast<V*>(outr + j * N) = o;
+    }
+  }
+}
+
+// any head_dim / alignment: one lane per pair
+template <typename T, typename CT>
+__global__ __launch_bounds__(256) void rotaryScalarKernel(T* out, const T* x, const CT* cosT, const CT* sinT,
+                                                           int64_t tokens, int heads, int d, int64_t tableRows,
+                                                           int tableCols, float sinSign, bool interleaved) {
+  const int half = d / 2;
+  const int64_t total = tokens * heads * half;
+  for (int64_t w = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; w < total; w += (int64_t)gridDim.x * blockDim.x) {
+    const int p = (int)(w % half);
+    const int64_t th = w / half;
+    const int64_t trow = (th / heads) % tableRows;
+    const int i0 = interleaved ? 2 * p : p, i1 = interleaved ? 2 * p + 1 : p + half;
+    const int tc = (interleaved && tableCols == d) ? 2 * p : p;
+    float c = static_cast<float>(cosT[trow * tableCols + tc]);
+    float s = static_cast<float>(sinT[trow * tableCols + tc]) * sinSign;
+    float x0 = static_cast<float>(x[th * d + i0]), x1 = static_cast<float>(x[th * d + i1]);
+    out[th * d + i0] = static_cast<T>(x0 * c - x1 * s);
+    out[th * d + i1] = static_cast<T>(x0 * s + x1 * c);
+  }
+}
+
+template <typename T, typename CT>
+static diopiError_t launchRotary(hipStream_t stream, const TensorView& out, const TensorView& x, const TensorView& c,
+                                 const TensorView& s, int64_t tokens, int heads, int d, int64_t tableRows,
+                                 int tableCols, bool conj, bool interleaved) {
+  constexpr int N = Vec16<T>::N;
+  const float sign = conj ? -1.f : 1.f;
+  const int half = d / 2;
+  bool vec = x.aligned16() && out.aligned16() && (interleaved ? d % N == 0 : half % N == 0);
+  if (vec) {
+    int perHead = interleaved ? d / N : half / N;
+    int64_t total = tokens * heads * perHead;
+    int64_t blocks = ceilDiv(total, 256);
+    if (blocks > (1 << 20)) blocks = 1 << 20;
+    if (interleaved) {
+      hipLaunchKernelGGL((rotaryVecKernel<T, CT, true>), dim3((unsigned)blocks), dim3(256), 0, stream, out.ptr<T>(),
+                         x.ptr<T>(), c.ptr<CT>(), s.ptr<CT>(), tokens, heads, d, tableRows, tableCols, sign);
+    } else {
+      hipLaunchKernelGGL((rotaryVecKernel<T, CT, false>), dim3((unsigned)blocks), dim3(256), 0, stream, out.ptr<T>(),
+                         x.ptr<T>(), c.ptr<CT>(), s.ptr<CT>(), tokens, heads, d, tableRows, tableCols, sign);
+    }
+  } else {
+    int64_t total = tokens * heads * half;
+    int64_t blocks = ceilDiv(total, 256);
+    if (blocks > (1 << 20)) blocks = 1 << 20;
+    hipLaunchKernelGGL((rotaryScalarKernel<T, CT>), dim3((unsigned)blocks), dim3(256), 0, stream, out.ptr<T>(),
+                       x.ptr<T>(), c.ptr<CT>(), s.ptr<CT>(), tokens, heads, d, tableRows, tableCols, sign,
+                       interleaved);
+  }
+  AMD_LAUNCH_CHECK();
+  return diopiSuccess;
+}
+
+// ---------------------------------------------------------------- KV scatter --
+template <typename VEC, typename IDX>
+__global__ __launch_bounds__(256) void destIndexCopyKernel(VEC* __restrict__ out, const VEC* __restrict__ src,
+                                                            const IDX* __restrict__ destLoc, int64_t tokens,
+                                                            int64_t rowVecs, int64_t outRowStrideVecs,
+                                                            int64_t srcRowStrideVecs, int64_t slots) {
+  const int64_t t = blockIdx.x;
+  if (t >= tokens) return;
+  int64_t slot = static_cast<int64_t>(destLoc[t]);
+  if (slot < 0) slot += slots;             // python-style negative index
+  if (slot < 0 || slot >= slots) return;   // an out-of-range slot is dropped, never written
+  const VEC* s = src + t * srcRowStrideVecs;
+  VEC* o = out + slot * outRowStrideVecs;
+  for (int64_t i = threadIdx.x; i < rowVecs; i += blockDim.x) o[i] = s[i];
+}
+
+template <typename IDX>
+static diopiError_t launchDestCopy(hipStream_t stream, void* out, const void* src, const void* loc, int64_t tokens,
+                                   int64_t rowBytes, int64_t outRowStrideBytes, int64_t srcRowStrideBytes,
+                                   int64_t slots) {
+  uintptr_t bits = reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(src) | (uintptr_t)rowBytes |
+                   (uintptr_t)outRowStrideBytes | (uintptr_t)srcRowStrideBytes;
+  int threads = 256;
+#define KV_LAUNCH(VEC)                                                                                              \
+  hipLaunchKernelGGL((destIndexCopyKernel<VEC, IDX>), dim3((unsigned)tokens), dim3(threads), 0, stream, (VEC*)out,  \
+                     (const VEC*)src, (const IDX*)loc, tokens, rowBytes / (int64_t)sizeof(VEC),                     \
+                     outRowStrideBytes / (int64_t)sizeof(VEC), srcRowStrideBytes / (int64_t)sizeof(VEC), slots)
+  if ((bits & 15) == 0) KV_LAUNCH(u32x4);
+  else if ((bits & 7) == 0) KV_LAUNCH(u32x2);
+  else if ((bits & 3) == 0) KV_LAUNCH(uint32_t);
+  else if ((bits & 1) == 0) KV_LAUNCH(uint16_t);
+  else KV_LAUNCH(uint8_t);
+#undef KV_LAUNCH
+  AMD_LAUNCH_CHECK();
+  return diopiSuccess;
+}
+
+// ---------------------------------------------------------------- index_put --
+// input[i0[r], i1[r], ..., :] (=|+=) values[r, :]; rows of `inner` elements.
+struct IndexTables {  // passed by value as a kernel argument
+  const void* ptrs[kMaxDims];
+  int64_t sizes[kMaxDims];
+  int64_t strides[kMaxDims];
+};
+
+template <typename IDX>
+__global__ __launch_bounds__(256) void indexPutKernel(void* input, const void* values, int dtIn, int dtVal,
+                                                       IndexTables tab, int nIdx, int64_t rows, int64_t inner,
+                                                       int64_t valRowStride, bool accumulate) {
+  const int64_t total = rows * inner;
+  for (int64_t w = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; w < total; w += (int64_t)gridDim.x * blockDim.x) {
+    int64_t r = w / inner, c = w - r * inner;
+    int64_t off = 0;
+    bool ok = true;
+    for (int k = 0; k < nIdx; ++k) {
+      int64_t v = static_cast<int64_t>(reinterpret_cast<const IDX*>(tab.ptrs[k])[r]);
+      if (v < 0) v += tab.sizes[k];
+      ok = ok && v >= 0 && v < tab.sizes[k];
+      off += v * tab.strides[k];
+    }
+    if (!ok) continue;
+    off += c;
+    if (!accumulate) {
+      if (isFloatDtypeDev(dtIn)) storeAs<double>(input, off, dtIn, loadAs<double>(values, r * valRowStride + c, dtVal));
+      else storeAs<int64_t>(input, off, dtIn, loadAs<int64_t>(values, r * valRowStride + c, dtVal));
+    } else {
+      if (dtIn == diopi_dtype_float32) {
+        atomicAdd(reinterpret_cast<float*>(input) + off, loadAs<float>(values, r * valRowStride + c, dtVal));
+      } else if (dtIn == diopi_dtype_int32) {
+        atomicAdd(reinterpret_cast<int*>(input) + off, (int)loadAs<int64_t>(values, r * valRowStride + c, dtVal));
+      } else if (dtIn == diopi_dtype_int64) {
+        atomicAdd(reinterpret_cast<unsigned long long*>(input) + off,
+                  (unsigned long long)loadAs<int64_t>(values, r * valRowStride + c, dtVal));
+      } else if (dtIn == diopi_dtype_float64) {
+        atomicAdd(reinterpret_cast<double*>(input) + off, loadAs<double>(values, r * valRowStride + c, dtVal));
+      }
+    }
+  }
+}
+
+}  // namespace amd
+
+using namespace amd;
+
+extern "C" __attribute__((visibility("default"))) diopiError_t diopiRotaryEmbedding(
+    diopiContextHandle_t ctx, diopiTensorHandle_t outH, diopiConstTensorHandle_t xH, diopiConstTensorHandle_t cosH,
+    diopiConstTensorHandle_t sinH, bool conj, bool interleaved) {
+  hipStream_t stream;
+  AMD_TRY(getStream(ctx, &stream));
+  TensorView out, x, c, s;
+  AMD_TRY(getView(outH, &out, "out"));
+  AMD_TRY(getView(xH, &x, "x"));
+  AMD_TRY(getView(cosH, &c, "cos"));
+  AMD_TRY(getView(sinH, &s, "sin"));
+  AMD_CHECK(out.defined() && x.defined() && c.defined() && s.defined(), "diopiRotaryEmbedding: null tensor");
+  AMD_CHECK(x.ndim >= 2, "diopiRotaryEmbedding: x must be [..., heads, head_dim]");
+  AMD_CHECK(out.dtype == x.dtype && out.ndim == x.ndim, "diopiRotaryEmbedding: out must match x");
+  for (int d = 0; d < x.ndim; ++d) AMD_CHECK(out.shape[d] == x.shape[d], "diopiRotaryEmbedding: shape mismatch at dim %d", d);
+  AMD_CHECK(c.dtype == s.dtype && c.numel == s.numel, "diopiRotaryEmbedding: cos and sin differ in dtype or size");
+  if (x.numel == 0) return diopiSuccess;
+  const int d = (int)x.shape[x.ndim - 1];
+  const int heads = (int)x.shape[x.ndim - 2];
+  AMD_CHECK(d % 2 == 0, "diopiRotaryEmbedding: head_dim %d is odd", d);
+  const int64_t tokens = x.numel / ((int64_t)heads * d);
+  AMD_CHECK(c.ndim >= 1, "diopiRotaryEmbedding: cos must have a last dim of head_dim or head_dim/2");
+  const int tableCols = (int)c.shape[c.ndim - 1];
+  AMD_CHECK(tableCols == d || tableCols == d / 2, "diopiRotaryEmbedding: cos last dim %d is neither %d nor %d", tableCols,
+            d, d / 2);
+  const int64_t tableRows = c.numel / tableCols;
+  AMD_CHECK(tableRows > 0 && tokens % tableRows == 0,
+            "diopiRotaryEmbedding: %ld table rows do not divide %ld tokens", (long)tableRows, (long)tokens);
+  TensorView cx, cc, cs;
+  AMD_TRY(makeContiguous(ctx, stream, x, &cx));
+  AMD_TRY(makeContiguous(ctx, stream, c, &cc));
+  AMD_TRY(makeContiguous(ctx, stream, s, &cs));
+  TensorView cout = out;
+  bool outTemp = !out.isContiguous();
+  if (outTemp) {
+    diopiTensorHandle_t th;
+    AMD_TRY(requireTensor(ctx, out.shape, out.ndim, out.dtype, &th, &cout));
+  }
+  diopiError_t err;
+#define ROTARY(T, CT) err = launchRotary<T, CT>(stream, cout, cx, cc, cs, tokens, heads, d, tableRows, tableCols, conj, interleaved)
+  if (x.dtype == diopi_dtype_bfloat16 && c.dtype == diopi_dtype_bfloat16) ROTARY(bf16_t, bf16_t);
+  else if (x.dtype == diopi_dtype_bfloat16 && c.dtype == diopi_dtype_float32) ROTARY(bf16_t, float);
+  else if (x.dtype == diopi_dtype_float16 && c.dtype == diopi_dtype_float16) ROTARY(half_t, half_t);
+  else if (x.dtype == diopi_dtype_float16 && c.dtype == diopi_dtype_float32) ROTARY(half_t, float);
+  else if (x.dtype == diopi_dtype_float32 && c.dtype == diopi_dtype_float32) ROTARY(float, float);
+  else {
+    setLastError("diopiRotaryEmbedding: unsupported dtypes x=%s cos=%s", dtypeName(x.dtype), dtypeName(c.dtype));
+    return diopiErrorOccurred;
+  }
+#undef ROTARY
+  AMD_TRY(err);
+  if (outTemp) AMD_TRY(stridedCopy(stream, cout, out));
+  return diopiSuccess;
+}
+
+extern "C" __attribute__((visibility("default"))) diopiError_t diopiDestIndexCopyKV(diopiContextHandle_t ctx,
+                                                                                    diopiTensorHandle_t outH,
+                                                                                    diopiConstTensorHandle_t kH,
+                                                                                    diopiConstTensorHandle_t locH) {
+  hipStream_t stream;
+  AMD_TRY(getStream(ctx, &stream));
+  TensorView out, k, loc;
+  AMD_TRY(getView(outH, &out, "out"));
+  AMD_TRY(getView(kH, &k, "k"));
+  AMD_TRY(getView(locH, &loc, "dest_loc"));
+  AMD_CHECK(out.defined() && k.defined() && loc.defined(), "diopiDestIndexCopyKV: null tensor");
+  AMD_CHECK(out.dtype == k.dtype, "diopiDestIndexCopyKV: out dtype %s differs from k dtype %s", dtypeName(out.dtype),
+            dtypeName(k.dtype));
+  AMD_CHECK(out.ndim == k.ndim && k.ndim >= 1, "diopiDestIndexCopyKV: rank mismatch");
+  for (int d = 1; d < k.ndim; ++d)
+    AMD_CHECK(out.shape[d] == k.shape[d], "diopiDestIndexCopyKV: trailing extent mismatch at dim %d", d);
+  AMD_CHECK(loc.dtype == diopi_dtype_int32 || loc.dtype == diopi_dtype_int64,
+            "diopiDestIndexCopyKV: dest_loc must be int32 or int64, got %s", dtypeName(loc.dtype));
+  const int64_t tokens = k.shape[0];
+  AMD_CHECK(loc.numel == tokens, "diopiDestIndexCopyKV: dest_loc has %ld entries for %ld tokens", (long)loc.numel,
+            (long)tokens);
+  if (tokens == 0 || k.numel == 0) return diopiSuccess;
+  AMD_CHECK(out.shape[0] > 0, "diopiDestIndexCopyKV: empty destination pool");
+  // rows (everything after dim 0) must be dense in both tensors; dim 0 may be strided
+  TensorView rowK = k, rowO = out;
+  rowK.shape[0] = rowO.shape[0] = 1;
+  TensorView ck = k;
+  if (!rowK.isContiguous()) AMD_TRY(makeContiguous(ctx, stream, k, &ck));
+  AMD_CHECK(rowO.isContiguous(), "diopiDestIndexCopyKV: rows of the destination pool must be dense");
+  TensorView cloc;
+  AMD_TRY(makeContiguous(ctx, stream, loc, &cloc));
+  const int64_t rowElems = k.numel / tokens;
+  const int64_t rowBytes = rowElems * k.itemsize;
+  const int64_t srcStride = (tokens > 1 ? ck.stride[0] : rowElems) * k.itemsize;
+  const int64_t outStride = (out.shape[0] > 1 ? out.stride[0] : rowElems) * out.itemsize;
+  if (loc.dtype == diopi_dtype_int32)
+    return launchDestCopy<int32_t>(stream, out.data, ck.data, cloc.data, tokens, rowBytes, outStride, srcStride,
+                                   out.shape[0]);
+  return launchDestCopy<int64_t>(stream, out.data, ck.data, cloc.data, tokens, rowBytes, outStride, srcStride,
+                                 out.shape[0]);
+}
+
+extern "C" __attribute__((visibility("default"))) diopiError_t diopiIndexPutInp(
+    diopiContextHandle_t ctx, diopiTensorHandle_t inputH, diopiConstTensorHandle_t valuesH,
+    diopiConstTensorHandle_t* indices, int64_t nIdx, bool accumulate) {
+  hipStream_t stream;
+  AMD_TRY(getStream(ctx, &stream));
+  TensorView in, val;
+  AMD_TRY(getView(inputH, &in, "input"));
+  AMD_TRY(getView(valuesH, &val, "values"));
+  AMD_CHECK(in.defined() && val.defined(), "diopiIndexPutInp: null tensor");
+  AMD_CHECK(nIdx >= 1 && nIdx <= in.ndim, "diopiIndexPutInp: %ld index tensors for a rank-%d input", (long)nIdx, in.ndim);
+  AMD_CHECK(in.isContiguous(), "diopiIndexPutInp: input must be dense");
+  if (accumulate)
+    AMD_CHECK(in.dtype == diopi_dtype_float32 || in.dtype == diopi_dtype_float64 || in.dtype == diopi_dtype_int32 ||
+                  in.dtype == diopi_dtype_int64,
+              "diopiIndexPutInp: accumulate supports float32/float64/int32/int64 inputs, got %s", dtypeName(in.dtype));
+  TensorView idx[kMaxDims];
+  int64_t rows = -1;
+  diopiDtype_t idt = diopi_dtype_int64;
+  for (int64_t i = 0; i < nIdx; ++i) {
+    AMD_CHECK(indices[i] != nullptr, "diopiIndexPutInp: null (slice) indices are not supported");
+    TensorView t;
+    AMD_TRY(getView(indices[i], &t, "index"));
+    AMD_CHECK(t.dtype == diopi_dtype_int64 || t.dtype == diopi_dtype_int32, "diopiIndexPutInp: index dtype %s",
+              dtypeName(t.dtype));
+    if (i == 0) idt = t.dtype;
+    AMD_CHECK(t.dtype == idt, "diopiIndexPutInp: mixed index dtypes");
+    if (rows < 0) rows = t.numel;
+    AMD_CHECK(t.numel == rows, "diopiIndexPutInp: index tensors differ in length");
+    AMD_TRY(makeContiguous(ctx, stream, t, &idx[i]));
+  }
+  if (rows == 0) return diopiSuccess;
+  int64_t inner = 1;
+  for (int d = (int)nIdx; d < in.ndim; ++d) inner *= in.shape[d];
+  // values: [rows, inner...] or anything broadcastable to it
+  TensorView cval;
+  AMD_TRY(makeContiguous(ctx, stream, val, &cval));
+  int64_t valRowStride;
+  if (cval.numel == rows * inner) valRowStride = inner;
+  else if (cval.numel == inner) valRowStride = 0;
+  else if (cval.numel == 1) valRowStride = 0;
+  else {
+    setLastError("diopiIndexPutInp: values with %ld elements cannot fill %ld rows of %ld", (long)cval.numel, (long)rows,
+                 (long)inner);
+    return diopiErrorOccurred;
+  }
+  if (cval.numel == 1 && inner != 1) {
+    // scalar value broadcast over whole rows: expand through the generic copy
+    diopiTensorHandle_t th;
+    TensorView expanded;
+    int64_t shp[1] = {inner};
+    AMD_TRY(requireTensor(ctx, shp, 1, val.dtype, &th, &expanded));
+    TensorView one = cval;
+    one.ndim = 1;
+    one.shape[0] = 1;
+    one.stride[0] = 0;
+    AMD_TRY(stridedCopy(stream, one, expanded));
+    cval = expanded;
+  }
+  IndexTables tab;
+  for (int i = 0; i < kMaxDims; ++i) tab.ptrs[i] = nullptr, tab.sizes[i] = 1, tab.strides[i] = 0;
+  for (int64_t i = 0; i < nIdx; ++i) {
+    tab.ptrs[i] = idx[i].data;
+    tab.sizes[i] = in.shape[i];
+    tab.strides[i] = in.stride[i];
+  }
+  int64_t total = rows * inner;
+  int64_t blocks = ceilDiv(total, 256);
+  if (blocks > 65536) blocks = 65536;
+  if (idt == diopi_dtype_int64) {
+    hipLaunchKernelGGL(indexPutKernel<int64_t>, dim3((unsigned)blocks), dim3(256), 0, stream, in.data, cval.data,
+                       (int)in.dtype, (int)cval.dtype, tab, (int)nIdx, rows, inner, valRowStride, accumulate);
+  } else {
+    hipLaunchKernelGGL(indexPutKernel<int32_t>, dim3((unsigned)blocks), dim3(256), 0, stream, in.data, cval.data,
+                       (int)in.dtype, (int)cval.dtype, tab, (int)nIdx, rows, inner, valRowStride, accumulate);
+  }
+  AMD_LAUNCH_CHECK();
+  return diopiSuccess;
+}

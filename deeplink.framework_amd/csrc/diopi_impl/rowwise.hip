@@ -1,0 +1,486 @@
+// Row reductions for gfx950: diopiSoftmax, diopiRMSNorm, diopiMean.
+//
+// Fast path (rows along the last, dense dim; row length a multiple of the 16-byte vector
+// and at most 64 lanes * 16 vectors): ONE WAVEFRONT PER ROW. Each lane keeps its slice of
+// the row in registers (up to 16 x 16-byte vectors), the max / sum / sum-of-squares are
+// wave64 butterfly reductions, and the row makes exactly one trip from and one trip to
+// HBM: algorithmic traffic = 2 * rows * cols * itemsize (+ the weight vector once).
+// No LDS, no barrier: four independent rows per 256-thread workgroup.
+//
+// Generic path: one workgroup per row, LDS-staged block reduction, rows of any length;
+// softmax over a non-last dim walks the reduced dim with a stride (one lane per column).
+//
+// Semantics: softmax as at::softmax on CPU (dipu/torch_dipu/csrc_dipu/aten/ops/CustomFallbackFunctions.hpp:466-474);
+// RMSNorm as dicp/dicp/vendor/AscendGraph/ext_ops.py:47-49 with fp32 accumulation
+// (dicp/test/model/llama/model.py:34-39).
+#include "common.hpp"
+
+namespace amd {
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+// ------------------------------------------------------------ wave-per-row ---
+enum RowOp { kRowSoftmax = 0, kRowRmsNorm = 1 };
+
+template <typename T, int NV, int OP, typename WT>
+__global__ __launch_bounds__(256) void rowWaveKernel(T* __restrict__ out, const T* __restrict__ in,
+                                                      const WT* __restrict__ weight, const WT* __restrict__ bias,
+                                                      float* __restrict__ invRmsOut, int64_t rows, int cols,
+                                                      int64_t inRowStride, int64_t outRowStride, float eps) {
+  using V = typename Vec16<T>::type;
+  using WV = typename Vec16<WT>::type;
+  constexpr int N = Vec16<T>::N;
+  constexpr int WN = Vec16<WT>::N;
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const V* src = reinterpret_cast<const V*>(in + row * inRowStride);
+  V* dst = reinterpret_cast<V*>(out + row * outRowStride);
+  const int nvec = cols / N;
+
+  float f[NV][N];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    int idx = lane + 64 * i;
+    if (idx < nvec) {
+      V v = __builtin_nontemporal_load(src + idx);
+#pragma unroll
+      for (int j = 0; j < N; ++j) f[i][j] = static_cast<float>(v[j]);
+    }
+  }
+
+  if constexpr (OP == kRowSoftmax) {
+    float m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+      if (lane + 64 * i < nvec) {
+#pragma unroll
+        for (int j = 0; j < N; ++j) m = fmaxf(m, f[i][j]);
+      }
+    m = waveMax(m);
+    const float mScaled = (m == -INFINITY) ? 0.f : m * kLog2e;  // all -inf row -> nan like the CPU kernel
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+      if (lane + 64 * i < nvec) {
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+          f[i][j] = exp2f(f[i][j] * kLog2e - mScaled);
+          s += f[i][j];
+        }
+      }
+    s = waveSum(s);
+    const float inv = 1.f / s;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      int idx = lane + 64 * i;
+      if (idx < nvec) {
+        V v;
+#pragma unroll
+        for (int j = 0; j < N; ++j) v[j] = static_cast<T>(f[i][j] * inv);
+        __builtin_nontemporal_store(v, dst + idx);
+      }
+    }
+  } else {
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+      if (lane + 64 * i < nvec) {
+#pragma unroll
+        for (int j = 0; j < N; ++j) ss += f[i][j] * f[i][j];
+      }
+    ss = waveSum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)cols + eps);
+    if (invRmsOut != nullptr && lane == 0) invRmsOut[row] = inv;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      int idx = lane + 64 * i;
+      if (idx < nvec) {
+        V v;
+        // weight/bias vectors hold WN elements per 16 bytes; N elements of T need N/WN of them
+        float w[N], b[N];
+        if (weight != nullptr) {
+          constexpr int PER = (N + WN - 1) / WN;
+#pragma unroll
+          for (int p = 0; p < PER; ++p) {
+            WV wv = reinterpret_cast<const WV*>(weight)[idx * PER + p];
+#pragma unroll
+            for (int j = 0; j < WN && p * WN + j < N; ++j) w[p * WN + j] = static_cast<float>(wv[j]);
+          }
+        }
+        if (bias != nullptr) {
+          constexpr int PER = (N + WN - 1) / WN;
+#pragma unroll
+          for (int p = 0; p < PER; ++p) {
+            WV bv = reinterpret_cast<const WV*>(bias)[idx * PER + p];
+#pragma unroll
+            for (int j = 0; j < WN && p * WN + j < N; ++j) b[p * WN + j] = static_cast<float>(bv[j]);
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+          float r = f[i][j] * inv;
+          if (weight != nullptr) r *= w[j];
+          if (bias != nullptr) r += b[j];
+          v[j] = static_cast<T>(r);
+        }
+        __builtin_nontemporal_store(v, dst + idx);
+      }
+    }
+  }
+}
+
+// --------------------------------------------------------- block-per-row ----
+__device__ __forceinline__ float blockReduce(float v, bool isMax, float* smem) {
+  v = isMax ? waveMax(v) : waveSum(v);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+  __syncthreads();
+  if (lane == 0) smem[wave] = v;
+  __syncthreads();
+  float r = isMax ? -INFINITY : 0.f;
+  for (int i = 0; i < nw; ++i) r = isMax ? fmaxf(r, smem[i]) : r + smem[i];
+  return r;
+}
+
+// Rows of any length / alignment. The row is staged in LDS as fp32 when it fits
+// (`stage` elements), otherwise re-read from global memory.
+template <typename T, int OP, typename WT>
+__global__ __launch_bounds__(256) void rowBlockKernel(T* out, const T* in, const WT* weight, const WT* bias,
+                                                       float* invRmsOut, int64_t rows, int64_t cols,
+                                                       int64_t inRowStride, int64_t outRowStride, float eps,
+                                                       int stage) {
+  extern __shared__ float lds[];
+  float* red = lds;         // 4 floats for the cross-wave step
+  float* rowBuf = lds + 8;  // `stage` floats
+  const int64_t row = blockIdx.x;
+  const T* src = in + row * inRowStride;
+  T* dst = out + row * outRowStride;
+  const bool staged = cols <= stage;
+  if constexpr (OP == kRowSoftmax) {
+    float m = -INFINITY;
+    for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) {
+      float v = static_cast<float>(src[c]);
+      if (staged) rowBuf[c] = v;
+      m = fmaxf(m, v);
+    }
+    m = blockReduce(m, true, red);
+    const float mScaled = (m == -INFINITY) ? 0.f : m * kLog2e;
+    float s = 0.f;
+    for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) {
+      float v = staged ? rowBuf[c] : static_cast<float>(src[c]);
+      v = exp2f(v * kLog2e - mScaled);
+      if (staged) rowBuf[c] = v;
+      s += v;
+    }
+    s = blockReduce(s, false, red);
+    const float inv = 1.f / s;
+    for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) {
+      float v = staged ? rowBuf[c] : exp2f(static_cast<float>(src[c]) * kLog2e - mScaled);
+      dst[c] = static_cast<T>(v * inv);
+    }
+  } else {
+    float ss = 0.f;
+    for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) {
+      float v = static_cast<float>(src[c]);
+      if (staged) rowBuf[c] = v;
+      ss += v * v;
+    }
+    ss = blockReduce(ss, false, red);
+    const float inv = 1.0f / sqrtf(ss / (float)cols + eps);
+    if (invRmsOut != nullptr && threadIdx.x == 0) invRmsOut[row] = inv;
+    for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) {
+      float v = (staged ? rowBuf[c] : static_cast<float>(src[c])) * inv;
+      if (weight != nullptr) v *= static_cast<float>(weight[c]);
+      if (bias != nullptr) v += static_cast<float>(bias[c]);
+      dst[c] = static_cast<T>(v);
+    }
+  }
+}
+
+// softmax along a non-last dim of a dense tensor [outer, dim, inner]: one lane per
+// (outer, inner) column, lanes adjacent along `inner` so every step is coalesced.
+template <typename T>
+__global__ __launch_bounds__(256) void softmaxStridedKernel(T* out, const T* in, int64_t outer, int64_t dim,
+                                                             int64_t inner) {
+  int64_t col = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (col >= outer * inner) return;
+  int64_t o = col / inner, i = col - o * inner;
+  const T* src = in + o * dim * inner + i;
+  T* dst = out + o * dim * inner + i;
+  float m = -INFINITY;
+  for (int64_t d = 0; d < dim; ++d) m = fmaxf(m, static_cast<float>(src[d * inner]));
+  const float mScaled = (m == -INFINITY) ? 0.f : m * kLog2e;
+  float s = 0.f;
+  for (int64_t d = 0; d < dim; ++d) s += exp2f(static_cast<float>(src[d * inner]) * kLog2e - mScaled);
+  const float inv = 1.f / s;
+  for (int64_t d = 0; d < dim; ++d)
+    dst[d * inner] = static_cast<T>(exp2f(static_cast<float>(src[d * inner]) * kLog2e - mScaled) * inv);
+}
+
+// mean of each dense row (one wave per row), fp32 accumulation
+template <typename T>
+__global__ __launch_bounds__(256) void rowMeanKernel(T* out, const T* in, int64_t rows, int64_t cols) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const T* src = in + row * cols;
+  float s = 0.f;
+  for (int64_t c = lane; c < cols; c += 64) s += static_cast<float>(src[c]);
+  s = waveSum(s);
+  if (lane == 0) out[row] = static_cast<T>(s / (float)cols);
+}
+
+// ------------------------------------------------------------- dispatch ------
+template <typename T, int OP, typename WT>
+static diopiError_t launchRows(hipStream_t stream, T* out, const T* in, const WT* weight, const WT* bias,
+                               float* invRms, int64_t rows, int64_t cols, int64_t inStride, int64_t outStride,
+                               float eps, bool vectorOk) {
+  constexpr int N = Vec16<T>::N;
+  if (rows == 0 || cols == 0) return diopiSuccess;
+  if (vectorOk && cols % N == 0 && cols / N <= 64 * 16) {
+    int nvec = (int)(cols / N);
+    int nv = (nvec + 63) / 64;
+    dim3 grid((unsigned)ceilDiv(rows, 4)), block(256);
+#define ROW_LAUNCH(NV)                                                                                            \
+  hipLaunchKernelGGL((rowWaveKernel<T, NV, OP, WT>), grid, block, 0, stream, out, in, weight, bias, invRms, rows, \
+                     (int)cols, inStride, outStride, eps)
+    if (nv <= 1) ROW_LAUNCH(1);
+    else if (nv <= 2) ROW_LAUNCH(2);
+    else if (nv <= 4) ROW_LAUNCH(4);
+    else if (nv <= 8) ROW_LAUNCH(8);
+    else ROW_LAUNCH(16);
+#undef ROW_LAUNCH
+  } else {
+    int stage = cols <= 12288 ? (int)cols : 0;  // 48 KiB of fp32 staging
+    size_t lds = (8 + (size_t)stage) * sizeof(float);
+    hipLaunchKernelGGL((rowBlockKernel<T, OP, WT>), dim3((unsigned)rows), dim3(256), lds, stream, out, in, weight,
+                       bias, invRms, rows, cols, inStride, outStride, eps, stage);
+  }
+  AMD_LAUNCH_CHECK();
+  return diopiSuccess;
+}
+
+}  // namespace amd
+
+using namespace amd;
+
+extern "C" __attribute__((visibility("default"))) diopiError_t diopiSoftmax(diopiContextHandle_t ctx,
+                                                                            diopiTensorHandle_t outH,
+                                                                            diopiConstTensorHandle_t inH,
+                                                                            int64_t dim) {
+  hipStream_t stream;
+  AMD_TRY(getStream(ctx, &stream));
+  TensorView out, in;
+  AMD_TRY(getView(outH, &out, "out"));
+  AMD_TRY(getView(inH, &in, "input"));
+  AMD_CHECK(out.defined() && in.defined(), "diopiSoftmax: null tensor");
+  AMD_CHECK(out.dtype == in.dtype, "diopiSoftmax: out dtype %s differs from input dtype %s", dtypeName(out.dtype),
+            dtypeName(in.dtype));
+  AMD_CHECK(out.ndim == in.ndim, "diopiSoftmax: rank mismatch");
+  for (int d = 0; d < in.ndim; ++d) AMD_CHECK(out.shape[d] == in.shape[d], "diopiSoftmax: shape mismatch at dim %d", d);
+  if (in.numel == 0) return diopiSuccess;
+  if (in.ndim == 0) {  // softmax of a scalar is 1
+    diopiScalar_t one;
+    one.stype = diopi_dtype_float64;
+    one.fval = 1.0;
+    return diopiFill(ctx, outH, &one);
+  }
+  if (dim < 0) dim += in.ndim;
+  AMD_CHECK(dim >= 0 && dim < in.ndim, "diopiSoftmax: dim out of range");
+  AMD_CHECK(in.dtype == diopi_dtype_bfloat16 || in.dtype == diopi_dtype_float16 || in.dtype == diopi_dtype_float32,
+            "diopiSoftmax: unsupported dtype %s", dtypeName(in.dtype));
+  TensorView cin;
+  AMD_TRY(makeContiguous(ctx, stream, in, &cin));
+  // a non-dense output is produced densely and copied back
+  TensorView cout = out;
+  bool outTemp = !out.isContiguous();
+  if (outTemp) {
+    diopiTensorHandle_t th;
+    AMD_TRY(requireTensor(ctx, out.shape, out.ndim, out.dtype, &th, &cout));
+  }
+  int64_t outer = 1, inner = 1, n = in.shape[dim];
+  for (int d = 0; d < dim; ++d) outer *= in.shape[d];
+  for (int d = (int)dim + 1; d < in.ndim; ++d) inner *= in.shape[d];
+  diopiError_t err = diopiSuccess;
+  if (inner == 1) {
+    bool vecOk = cin.aligned16() && cout.aligned16() && (n * in.itemsize) % 16 == 0;
+    switch (in.dtype) {
+      case diopi_dtype_bfloat16:
+        err = launchRows<bf16_t, kRowSoftmax, bf16_t>(stream, cout.ptr<bf16_t>(), cin.ptr<bf16_t>(), nullptr, nullptr,
+                                                      nullptr, outer, n, n, n, 0.f, vecOk);
+        break;
+      case diopi_dtype_float16:
+        err = launchRows<half_t, kRowSoftmax, half_t>(stream, cout.ptr<half_t>(), cin.ptr<half_t>(), nullptr, nullptr,
+                                                      nullptr, outer, n, n, n, 0.f, vecOk);
+        break;
+      default:
+        err = launchRows<float, kRowSoftmax, float>(stream, cout.ptr<float>(), cin.ptr<float>(), nullptr, nullptr,
+                                                    nullptr, outer, n, n, n, 0.f, vecOk);
+        break;
+    }
+  } else {
+    int64_t colsTotal = outer * inner;
+    dim3 grid((unsigned)ceilDiv(colsTotal, 256)), block(256);
+    switch (in.dtype) {
+      case diopi_dtype_bfloat16:
+        hipLaunchKernelGGL(softmaxStridedKernel<bf16_t>, grid, block, 0, stream, cout.ptr<bf16_t>(), cin.ptr<bf16_t>(),
+                           outer, n, inner);
+        break;
+      case diopi_dtype_float16:
+        hipLaunchKernelGGL(softmaxStridedKernel<half_t>, grid, block, 0, stream, cout.ptr<half_t>(), cin.ptr<half_t>(),
+                           outer, n, inner);
+        break;
+      default:
+        hipLaunchKernelGGL(softmaxStridedKernel<float>, grid, block, 0, stream, cout.ptr<float>(), cin.ptr<float>(),
+                           outer, n, inner);
+        break;
+    }
+    AMD_LAUNCH_CHECK();
+  }
+  AMD_TRY(err);
+  if (outTemp) AMD_TRY(stridedCopy(stream, cout, out));
+  return diopiSuccess;
+}
+
+template <typename T>
+static diopiError_t rmsNormTyped(hipStream_t stream, const TensorView& out, const TensorView& in,
+                                 const TensorView& w, const TensorView& b, float* invRms, int64_t rows, int64_t cols,
+                                 float eps) {
+  bool vecOk = in.aligned16() && out.aligned16() && (cols * in.itemsize) % 16 == 0;
+  diopiDtype_t wdt = w.defined() ? w.dtype : (b.defined() ? b.dtype : in.dtype);
+  if (w.defined()) vecOk = vecOk && w.aligned16();
+  if (b.defined()) vecOk = vecOk && b.aligned16();
+  if (wdt == in.dtype) {
+    return launchRows<T, kRowRmsNorm, T>(stream, out.ptr<T>(), in.ptr<T>(), w.ptr<T>(), b.ptr<T>(), invRms, rows, cols,
+                                         cols, cols, eps, vecOk);
+  }
+  AMD_CHECK(wdt == diopi_dtype_float32, "diopiRMSNorm: weight dtype %s must equal the input dtype or be float32",
+            dtypeName(wdt));
+  return launchRows<T, kRowRmsNorm, float>(stream, out.ptr<T>(), in.ptr<T>(), w.ptr<float>(), b.ptr<float>(), invRms,
+                                           rows, cols, cols, cols, eps, vecOk);
+}
+
+extern "C" __attribute__((visibility("default"))) diopiError_t diopiRMSNorm(
+    diopiContextHandle_t ctx, diopiTensorHandle_t outH, diopiTensorHandle_t invRmsH, diopiConstTensorHandle_t inH,
+    diopiSize_t normalizedShape, diopiConstTensorHandle_t weightH, diopiConstTensorHandle_t biasH, double eps) {
+  hipStream_t stream;
+  AMD_TRY(getStream(ctx, &stream));
+  TensorView out, inv, in, w, b;
+  AMD_TRY(getView(outH, &out, "out"));
+  AMD_TRY(getView(invRmsH, &inv, "inv_rms"));
+  AMD_TRY(getView(inH, &in, "input"));
+  AMD_TRY(getView(weightH, &w, "weight"));
+  AMD_TRY(getView(biasH, &b, "bias"));
+  AMD_CHECK(out.defined() && in.defined(), "diopiRMSNorm: null tensor");
+  AMD_CHECK(out.dtype == in.dtype, "diopiRMSNorm: out dtype differs from input dtype");
+  AMD_CHECK(out.ndim == in.ndim, "diopiRMSNorm: rank mismatch");
+  for (int d = 0; d < in.ndim; ++d) AMD_CHECK(out.shape[d] == in.shape[d], "diopiRMSNorm: shape mismatch at dim %d", d);
+  AMD_CHECK(normalizedShape.len >= 1 && normalizedShape.len <= in.ndim, "diopiRMSNorm: bad normalized_shape rank");
+  int64_t cols = 1;
+  for (int64_t i = 0; i < normalizedShape.len; ++i) {
+    int64_t e = in.shape[in.ndim - normalizedShape.len + i];
+    AMD_CHECK(normalizedShape.data[i] == e, "diopiRMSNorm: normalized_shape[%ld]=%ld but input extent is %ld", (long)i,
+              (long)normalizedShape.data[i], (long)e);
+    cols *= e;
+  }
+  if (in.numel == 0) return diopiSuccess;
+  int64_t rows = in.numel / cols;
+  if (w.defined()) AMD_CHECK(w.numel == cols, "diopiRMSNorm: weight has %ld elements, expected %ld", (long)w.numel, (long)cols);
+  if (b.defined()) AMD_CHECK(b.numel == cols, "diopiRMSNorm: bias has %ld elements, expected %ld", (long)b.numel, (long)cols);
+  if (w.defined() && b.defined()) AMD_CHECK(w.dtype == b.dtype, "diopiRMSNorm: weight and bias dtypes differ");
+  AMD_CHECK(in.dtype == diopi_dtype_bfloat16 || in.dtype == diopi_dtype_float16 || in.dtype == diopi_dtype_float32,
+            "diopiRMSNorm: unsupported dtype %s", dtypeName(in.dtype));
+  TensorView cin, cw, cb;
+  AMD_TRY(makeContiguous(ctx, stream, in, &cin));
+  if (w.defined()) AMD_TRY(makeContiguous(ctx, stream, w, &cw));
+  if (b.defined()) AMD_TRY(makeContiguous(ctx, stream, b, &cb));
+  TensorView cout = out;
+  bool outTemp = !out.isContiguous();
+  if (outTemp) {
+    diopiTensorHandle_t th;
+    AMD_TRY(requireTensor(ctx, out.shape, out.ndim, out.dtype, &th, &cout));
+  }
+  // inv_rms is produced as fp32 [rows]; other dtypes/layouts are converted afterwards
+  float* invPtr = nullptr;
+  TensorView invTmp;
+  bool invDirect = false;
+  if (inv.defined()) {
+    AMD_CHECK(inv.numel == rows, "diopiRMSNorm: inv_rms has %ld elements, expected %ld", (long)inv.numel, (long)rows);
+    invDirect = inv.dtype == diopi_dtype_float32 && inv.isContiguous();
+    if (invDirect) {
+      invPtr = inv.ptr<float>();
+    } else {
+      diopiTensorHandle_t th;
+      AMD_TRY(requireTensor(ctx, inv.shape, inv.ndim, diopi_dtype_float32, &th, &invTmp));
+      invPtr = invTmp.ptr<float>();
+    }
+  }
+  diopiError_t err;
+  switch (in.dtype) {
+    case diopi_dtype_bfloat16: err = rmsNormTyped<bf16_t>(stream, cout, cin, cw, cb, invPtr, rows, cols, (float)eps); break;
+    case diopi_dtype_float16: err = rmsNormTyped<half_t>(stream, cout, cin, cw, cb, invPtr, rows, cols, (float)eps); break;
+    default: err = rmsNormTyped<float>(stream, cout, cin, cw, cb, invPtr, rows, cols, (float)eps); break;
+  }
+  AMD_TRY(err);
+  if (outTemp) AMD_TRY(stridedCopy(stream, cout, out));
+  if (inv.defined() && !invDirect) AMD_TRY(stridedCopy(stream, invTmp, inv));
+  return diopiSuccess;
+}
+
+// mean over `dims`: the kept dims are moved to the front (a strided view), made dense,
+// and each row of prod(reduced) elements is averaged by one wave.
+extern "C" __attribute__((visibility("default"))) diopiError_t diopiMean(diopiContextHandle_t ctx,
+                                                                         diopiTensorHandle_t outH,
+                                                                         diopiConstTensorHandle_t inH,
+                                                                         diopiSize_t dims) {
+  hipStream_t stream;
+  AMD_TRY(getStream(ctx, &stream));
+  TensorView out, in;
+  AMD_TRY(getView(outH, &out, "out"));
+  AMD_TRY(getView(inH, &in, "input"));
+  AMD_CHECK(out.defined() && in.defined(), "diopiMean: null tensor");
+  AMD_CHECK(out.dtype == in.dtype, "diopiMean: dtype conversion is not supported");
+  AMD_CHECK(in.dtype == diopi_dtype_bfloat16 || in.dtype == diopi_dtype_float16 || in.dtype == diopi_dtype_float32,
+            "diopiMean: unsupported dtype %s", dtypeName(in.dtype));
+  bool reduced[kMaxDims] = {false};
+  if (dims.len == 0) {
+    for (int d = 0; d < in.ndim; ++d) reduced[d] = true;
+  }
+  for (int64_t i = 0; i < dims.len; ++i) {
+    int64_t d = dims.data[i] < 0 ? dims.data[i] + in.ndim : dims.data[i];
+    AMD_CHECK(d >= 0 && d < in.ndim, "diopiMean: dim %ld out of range", (long)dims.data[i]);
+    reduced[d] = true;
+  }
+  TensorView perm = in;
+  int w = 0;
+  int64_t rows = 1, cols = 1;
+  for (int d = 0; d < in.ndim; ++d)
+    if (!reduced[d]) perm.shape[w] = in.shape[d], perm.stride[w] = in.stride[d], rows *= in.shape[d], ++w;
+  for (int d = 0; d < in.ndim; ++d)
+    if (reduced[d]) perm.shape[w] = in.shape[d], perm.stride[w] = in.stride[d], cols *= in.shape[d], ++w;
+  AMD_CHECK(out.numel == rows, "diopiMean: output has %ld elements, expected %ld", (long)out.numel, (long)rows);
+  if (rows == 0) return diopiSuccess;
+  TensorView cin;
+  AMD_TRY(makeContiguous(ctx, stream, perm, &cin));
+  TensorView cout = out;
+  bool outTemp = !out.isContiguous();
+  if (outTemp) {
+    diopiTensorHandle_t th;
+    AMD_TRY(requireTensor(ctx, out.shape, out.ndim, out.dtype, &th, &cout));
+  }
+  dim3 grid((unsigned)ceilDiv(rows, 4)), block(256);
+  switch (in.dtype) {
+    case diopi_dtype_bfloat16:
+      hipLaunchKernelGGL(rowMeanKernel<bf16_t>, grid, block, 0, stream, cout.ptr<bf16_t>(), cin.ptr<bf16_t>(), rows, cols);
+      break;
+    case diopi_dtype_float16:
+      hipLaunchKernelGGL(rowMeanKernel<half_t>, grid, block, 0, stream, cout.ptr<half_t>(), cin.ptr<half_t>(), rows, cols);
+      break;
+    default:
+      hipLaunchKernelGGL(rowMeanKernel<float>, grid, block, 0, stream, cout.ptr<float>(), cin.ptr<float>(), rows, cols);
+      break;
+  }
+  AMD_LAUNCH_CHECK();
+  if (outTemp) AMD_TRY(stridedCopy(stream, cout, out));
+  return diopiSuccess;
+}

@@ -1,0 +1,582 @@
+// Decode-step ("token") attention over a paged KV pool for gfx950.
+//
+//   q [batch, heads, d]            one query token per sequence
+//   k, v [slots, kv_heads, d]      the pool; a token's heads are adjacent (d contiguous)
+//   b_loc [batch, >= max_len]      slot table, right-aligned: sequence b's t-th token is at
+//                                  column max_len - seq_len[b] + t
+//   b_start_loc, b_seq_len [batch]
+//
+// out[b,h,:] = softmax_t(q[b,h,:] . k[slot_t,h,:] / sqrt(d)) . v[slot_t,h,:]
+// (dicp/dicp/vendor/AscendGraph/ext_ops.py:100-133, slots gathered through b_loc).
+//
+// The fused kernel is HBM-bound: every K and V row of the sequence is read exactly once
+// (d * itemsize bytes each), nothing else of size is touched. Mapping:
+//   * a head row of d elements is covered by LPT = d*itemsize/16 lanes with one 16-byte
+//     load each, so one wave-wide load fetches 64/LPT tokens;
+//   * every lane group keeps its OWN running (max, sum, acc[8]) online-softmax state, so the
+//     inner loop needs no cross-group traffic: per token only the log2(LPT) butterfly steps
+//     of the dot product;
+//   * K and V loads of an iteration are issued together, before any math, 4 + 4 wave-loads
+//     (8 KiB) in flight per wave; the slot indices of the NEXT iteration are fetched before
+//     the math of the current one, hiding the index -> address dependency;
+//   * a workgroup = 4 waves owns a chunk of the sequence (split-KV); states are merged by
+//     wave butterflies, then through LDS, then across chunks by a small second kernel.
+#include <algorithm>
+
+#include "common.hpp"
+
+namespace amd {
+
+constexpr float kLog2eTA = 1.4426950408889634f;
+constexpr int kTaWaves = 4;
+constexpr int kTaUnroll = 4;
+constexpr int kTaChunk = 512;  // tokens of one sequence handled by one workgroup
+
+__device__ __forceinline__ int64_t ldIndex(const void* p, int64_t i, bool is64) {
+  return is64 ? reinterpret_cast<const int64_t*>(p)[i] : static_cast<int64_t>(reinterpret_cast<const int32_t*>(p)[i]);
+}
+
+struct TaArgs {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* bLoc;
+  const void* bStart;
+  const void* bLen;
+  bool loc64, start64, len64;
+  int64_t locRowStride;  // elements
+  int64_t kSlotStride, kHeadStride, vSlotStride, vHeadStride;  // elements
+  int64_t qBatchStride, qHeadStride;
+  int64_t slots;
+  int heads, kvHeads, d, maxLen, nsplit;
+  float scaleLog2e;  // log2(e) / sqrt(d)
+};
+
+// Merge (m, l, acc) of another online-softmax stream into this one.
+template <int E>
+__device__ __forceinline__ void mergeState(float& m, float& l, float (&acc)[E], float m2, float l2,
+                                           const float (&acc2)[E]) {
+  float mn = fmaxf(m, m2);
+  float c1 = (m == -INFINITY) ? 0.f : exp2f(m - mn);
+  float c2 = (m2 == -INFINITY) ? 0.f : exp2f(m2 - mn);
+  l = l * c1 + l2 * c2;
+#pragma unroll
+  for (int e = 0; e < E; ++e) acc[e] = acc[e] * c1 + acc2[e] * c2;
+  m = mn;
+}
+
+// T: bf16_t / half_t (8 per 16 B) or float (4 per 16 B). LPT lanes cover one head row.
+template <typename T, int LPT>
+__global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* __restrict__ out,
+                                                                     float* __restrict__ partial) {
+  using V = typename Vec16<T>::type;
+  constexpr int N = Vec16<T>::N;
+  constexpr int TPW = 64 / LPT;  // tokens per wave-wide load
+  const int h = blockIdx.x, split = blockIdx.y, b = blockIdx.z;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int sub = lane % LPT, grp = lane / LPT;
+  const int len = (int)ldIndex(a.bLen, b, a.len64);
+  const int begin = split * kTaChunk;
+  if (begin >= len && !(split == 0)) return;  // nothing to do; split 0 still writes zeros for len == 0
+  const int end = min(len, begin + kTaChunk);
+  const int kvh = h / (a.heads / a.kvHeads);
+  const int64_t locBase = (int64_t)b * a.locRowStride + (a.maxLen - len);
+
+  float qf[N];
+  {
+    V qv = *reinterpret_cast<const V*>(reinterpret_cast<const T*>(a.q) + b * a.qBatchStride + h * a.qHeadStride + sub * N);
+#pragma unroll
+    for (int e = 0; e < N; ++e) qf[e] = static_cast<float>(qv[e]) * a.scaleLog2e;
+  }
+  const T* kBase = reinterpret_cast<const T*>(a.k) + kvh * a.kHeadStride + sub * N;
+  const T* vBase = reinterpret_cast<const T*>(a.v) + kvh * a.vHeadStride + sub * N;
+
+  float m = -INFINITY, l = 0.f, acc[N];
+#pragma unroll
+  for (int e = 0; e < N; ++e) acc[e] = 0.f;
+
+  constexpr int STEP = kTaWaves * kTaUnroll * TPW;  // tokens per workgroup iteration
+  int64_t slot[kTaUnroll];
+  {
+    int t0 = begin + wave * kTaUnroll * TPW + grp;
+#pragma unroll
+    for (int u = 0; u < kTaUnroll; ++u) {
+      int t = t0 + u * TPW;
+      slot[u] = t < end ? ldIndex(a.bLoc, locBase + t, a.loc64) : -1;
+    }
+  }
+  for (int it = begin; it < end; it += STEP) {
+    V kr[kTaUnroll], vr[kTaUnroll];
+    bool ok[kTaUnroll];
+#pragma unroll
+    for (int u = 0; u < kTaUnroll; ++u) {
+      ok[u] = slot[u] >= 0 && slot[u] < a.slots;  // slots outside the pool are skipped, never dereferenced
+      int64_t s = ok[u] ? slot[u] : 0;
+      kr[u] = *reinterpret_cast<const V*>(kBase + s * a.kSlotStride);
+      vr[u] = *reinterpret_cast<const V*>(vBase + s * a.vSlotStride);
+    }
+    {  // indices of the next iteration, in flight during the math below
+      int t0 = it + STEP + wave * kTaUnroll * TPW + grp;
+#pragma unroll
+      for (int u = 0; u < kTaUnroll; ++u) {
+        int t = t0 + u * TPW;
+        slot[u] = t < end ? ldIndex(a.bLoc, locBase + t, a.loc64) : -1;
+      }
+    }
+    float sc[kTaUnroll];
+    float mn = m;
+#pragma unroll
+    for (int u = 0; u < kTaUnroll; ++u) {
+      float d = 0.f;
+#pragma unroll
+      for (int e = 0; e < N; ++e) d += qf[e] * static_cast<float>(kr[u][e]);
+#pragma unroll
+      for (int off = LPT / 2; off > 0; off >>= 1) d += __shfl_xor(d, off, 64);
+      sc[u] = ok[u] ? d : -INFINITY;
+      mn = fmaxf(mn, sc[u]);
+    }
+    if (mn != -INFINITY) {
+      float corr = exp2f(m - mn);  // m == -inf gives 0, acc and l are 0 then anyway
+      float p[kTaUnroll], ps = 0.f;
+#pragma unroll
+      for (int u = 0; u < kTaUnroll; ++u) {
+        p[u] = exp2f(sc[u] - mn);
+        ps += p[u];
+      }
+      l = l * corr + ps;
+#pragma unroll
+      for (int e = 0; e < N; ++e) {
+        float s = acc[e] * corr;
+#pragma unroll
+        for (int u = 0; u < kTaUnroll; ++u) s += p[u] * static_cast<float>(vr[u][e]);
+        acc[e] = s;
+      }
+      m = mn;
+    }
+  }
+
+  // merge the TPW lane groups of the wave
+#pragma unroll
+  for (int off = LPT; off < 64; off <<= 1) {
+    float m2 = __shfl_xor(m, off, 64), l2 = __shfl_xor(l, off, 64), acc2[N];
+#pragma unroll
+    for (int e = 0; e < N; ++e) acc2[e] = __shfl_xor(acc[e], off, 64);
+    mergeState<N>(m, l, acc, m2, l2, acc2);
+  }
+  // merge the waves through LDS: [wave][2 + LPT*N]
+  __shared__ float red[kTaWaves][2 + LPT * N];
+  if (grp == 0) {
+    if (sub == 0) red[wave][0] = m, red[wave][1] = l;
+#pragma unroll
+    for (int e = 0; e < N; ++e) red[wave][2 + sub * N + e] = acc[e];
+  }
+  __syncthreads();
+  if (wave == 0 && grp == 0) {
+#pragma unroll
+    for (int w = 1; w < kTaWaves; ++w) {
+      float acc2[N];
+#pragma unroll
+      for (int e = 0; e < N; ++e) acc2[e] = red[w][2 + sub * N + e];
+      mergeState<N>(m, l, acc, red[w][0], red[w][1], acc2);
+    }
+    if (a.nsplit == 1) {
+      float inv = l > 0.f ? 1.f / l : 0.f;
+      V o;
+#pragma unroll
+      for (int e = 0; e < N; ++e) o[e] = static_cast<T>(acc[e] * inv);
+      *reinterpret_cast<V*>(out + ((int64_t)b * a.heads + h) * a.d + sub * N) = o;
+    } else {
+      float* dst = partial + (((int64_t)b * a.heads + h) * a.nsplit + split) * (2 + a.d);
+      if (sub == 0) dst[0] = m, dst[1] = l;
+#pragma unroll
+      for (int e = 0; e < N; ++e) dst[2 + sub * N + e] = acc[e];
+    }
+  }
+}
+
+// out[b,h,:] = merge over the chunks that hold tokens. One wave per (b,h), lane = element.
+template <typename T>
+__global__ __launch_bounds__(256) void decodeMergeKernel(T* __restrict__ out, const float* __restrict__ partial,
+                                                          const void* bLen, bool len64, int64_t pairs, int heads,
+                                                          int d, int nsplit) {
+  const int lane = threadIdx.x & 63;
+  const int64_t pair = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (pair >= pairs) return;
+  const int b = (int)(pair / heads);
+  const int len = (int)ldIndex(bLen, b, len64);
+  const int used = len <= 0 ? 1 : min(nsplit, (len + kTaChunk - 1) / kTaChunk);
+  const float* src = partial + pair * nsplit * (2 + d);
+  float m = -INFINITY;
+  for (int s = 0; s < used; ++s) m = fmaxf(m, src[s * (2 + d)]);
+  float l = 0.f;
+  for (int s = 0; s < used; ++s) {
+    float ms = src[s * (2 + d)];
+    l += (ms == -INFINITY) ? 0.f : src[s * (2 + d) + 1] * exp2f(ms - m);
+  }
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  for (int e = lane; e < d; e += 64) {
+    float acc = 0.f;
+    for (int s = 0; s < used; ++s) {
+      float ms = src[s * (2 + d)];
+      if (ms != -INFINITY) acc += src[s * (2 + d) + 2 + e] * exp2f(ms - m);
+    }
+    out[pair * d + e] = static_cast<T>(acc * inv);
+  }
+}
+
+// ------------------------------------------------- two-call form, first half --
+// att[h, start_b + t] = q[b,h,:] . k[slot_t,h,:] / sqrt(d); a workgroup covers 256*? tokens
+template <typename T, int LPT, typename OT>
+__global__ __launch_bounds__(256) void tokenLogitsKernel(TaArgs a, OT* __restrict__ att, int64_t attHeadStride) {
+  using V = typename Vec16<T>::type;
+  constexpr int N = Vec16<T>::N;
+  constexpr int TPW = 64 / LPT;
+  const int h = blockIdx.x, b = blockIdx.z;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int sub = lane % LPT, grp = lane / LPT;
+  const int len = (int)ldIndex(a.bLen, b, a.len64);
+  const int64_t start = ldIndex(a.bStart, b, a.start64);
+  const int begin = blockIdx.y * kTaChunk;
+  if (begin >= len) return;
+  const int end = min(len, begin + kTaChunk);
+  const int kvh = h / (a.heads / a.kvHeads);
+  const int64_t locBase = (int64_t)b * a.locRowStride + (a.maxLen - len);
+  float qf[N];
+  {
+    V qv = *reinterpret_cast<const V*>(reinterpret_cast<const T*>(a.q) + b * a.qBatchStride + h * a.qHeadStride + sub * N);
+#pragma unroll
+    for (int e = 0; e < N; ++e) qf[e] = static_cast<float>(qv[e]);
+  }
+  const T* kBase = reinterpret_cast<const T*>(a.k) + kvh * a.kHeadStride + sub * N;
+  const float scale = a.scaleLog2e / kLog2eTA;
+  constexpr int STEP = 4 * kTaUnroll * TPW;
+  for (int it = begin; it < end; it += STEP) {
+    int t0 = it + wave * kTaUnroll * TPW + grp;
+    V kr[kTaUnroll];
+    bool ok[kTaUnroll];
+#pragma unroll
+    for (int u = 0; u < kTaUnroll; ++u) {
+      int t = t0 + u * TPW;
+      int64_t s = t < end ? ldIndex(a.bLoc, locBase + t, a.loc64) : -1;
+      ok[u] = s >= 0 && s < a.slots;
+      kr[u] = *reinterpret_cast<const V*>(kBase + (ok[u] ? s : 0) * a.kSlotStride);
+    }
+#pragma unroll
+    for (int u = 0; u < kTaUnroll; ++u) {
+      float d = 0.f;
+#pragma unroll
+      for (int e = 0; e < N; ++e) d += qf[e] * static_cast<float>(kr[u][e]);
+#pragma unroll
+      for (int off = LPT / 2; off > 0; off >>= 1) d += __shfl_xor(d, off, 64);
+      int t = t0 + u * TPW;
+      if (sub == 0 && t < end) att[h * attHeadStride + start + t] = static_cast<OT>(ok[u] ? d * scale : -INFINITY);
+    }
+  }
+}
+
+// ------------------------------------------------ two-call form, second half --
+// out[b,h,:] = softmax(logics[h, start_b : start_b+len]) . v[slots]; one workgroup per (b,h)
+template <typename T, int LPT, typename LT>
+__global__ __launch_bounds__(256) void softmaxReduceVKernel(TaArgs a, T* __restrict__ out,
+                                                             const LT* __restrict__ logics, int64_t logHeadStride) {
+  using V = typename Vec16<T>::type;
+  constexpr int N = Vec16<T>::N;
+  constexpr int TPW = 64 / LPT;
+  const int h = blockIdx.x, b = blockIdx.z;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int sub = lane % LPT, grp = lane / LPT;
+  const int len = (int)ldIndex(a.bLen, b, a.len64);
+  const int64_t start = ldIndex(a.bStart, b, a.start64);
+  const int kvh = h / (a.heads / a.kvHeads);
+  const int64_t locBase = (int64_t)b * a.locRowStride + (a.maxLen - len);
+  const LT* lg = logics + h * logHeadStride + start;
+  __shared__ float red[4][2 + LPT * N];
+  __shared__ float bcast[2];
+  // pass 1: row max and sum of exp over the logits
+  float m = -INFINITY;
+  for (int t = threadIdx.x; t < len; t += 256) m = fmaxf(m, static_cast<float>(lg[t]));
+  m = waveMax(m);
+  if (lane == 0) red[wave][0] = m;
+  __syncthreads();
+  m = fmaxf(fmaxf(red[0][0], red[1][0]), fmaxf(red[2][0], red[3][0]));
+  __syncthreads();
+  const float mS = (m == -INFINITY) ? 0.f : m * kLog2eTA;
+  float s = 0.f;
+  for (int t = threadIdx.x; t < len; t += 256) s += exp2f(static_cast<float>(lg[t]) * kLog2eTA - mS);
+  s = waveSum(s);
+  if (lane == 0) red[wave][1] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) bcast[0] = red[0][1] + red[1][1] + red[2][1] + red[3][1];
+  __syncthreads();
+  const float inv = bcast[0] > 0.f ? 1.f / bcast[0] : 0.f;
+  // pass 2: stream V
+  const T* vBase = reinterpret_cast<const T*>(a.v) + kvh * a.vHeadStride + sub * N;
+  float acc[N];
+#pragma unroll
+  for (int e = 0; e < N; ++e) acc[e] = 0.f;
+  constexpr int STEP = 4 * kTaUnroll * TPW;
+  for (int it = 0; it < len; it += STEP) {
+    int t0 = it + wave * kTaUnroll * TPW + grp;
+    V vr[kTaUnroll];
+    float p[kTaUnroll];
+#pragma unroll
+    for (int u = 0; u < kTaUnroll; ++u) {
+      int t = t0 + u * TPW;
+      int64_t sl = t < len ? ldIndex(a.bLoc, locBase + t, a.loc64) : -1;
+      bool ok = sl >= 0 && sl < a.slots;
+      vr[u] = *reinterpret_cast<const V*>(vBase + (ok ? sl : 0) * a.vSlotStride);
+      p[u] = ok ? exp2f(static_cast<float>(lg[t]) * kLog2eTA - mS) : 0.f;
+    }
+#pragma unroll
+    for (int e = 0; e < N; ++e) {
+#pragma unroll
+      for (int u = 0; u < kTaUnroll; ++u) acc[e] += p[u] * static_cast<float>(vr[u][e]);
+    }
+  }
+#pragma unroll
+  for (int off = LPT; off < 64; off <<= 1) {
+#pragma unroll
+    for (int e = 0; e < N; ++e) acc[e] += __shfl_xor(acc[e], off, 64);
+  }
+  __syncthreads();
+  if (grp == 0) {
+#pragma unroll
+    for (int e = 0; e < N; ++e) red[wave][2 + sub * N + e] = acc[e];
+  }
+  __syncthreads();
+  if (wave == 0 && grp == 0) {
+    V o;
+#pragma unroll
+    for (int e = 0; e < N; ++e) {
+      float r = red[0][2 + sub * N + e] + red[1][2 + sub * N + e] + red[2][2 + sub * N + e] + red[3][2 + sub * N + e];
+      o[e] = static_cast<T>(r * inv);
+    }
+    *reinterpret_cast<V*>(out + ((int64_t)b * a.heads + h) * a.d + sub * N) = o;
+  }
+}
+
+// ---------------------------------------------------------------- host side --
+struct TaViews {
+  TensorView q, k, v, loc, start, len;
+};
+
+static diopiError_t checkIndex(const TensorView& t, const char* name) {
+  AMD_CHECK(t.defined(), "token attention: %s is null", name);
+  AMD_CHECK(t.dtype == diopi_dtype_int32 || t.dtype == diopi_dtype_int64, "token attention: %s must be int32/int64, got %s",
+            name, dtypeName(t.dtype));
+  AMD_CHECK(t.isContiguous() || t.ndim == 2, "token attention: %s must be dense", name);
+  return diopiSuccess;
+}
+
+static diopiError_t fillArgs(const TaViews& t, bool needK, bool needV, int maxLen, TaArgs* a) {
+  const TensorView& q = t.q;
+  AMD_CHECK(q.defined() && q.ndim == 3, "token attention: q must be [batch, heads, head_dim]");
+  AMD_CHECK(q.stride[2] == 1 || q.shape[2] == 1, "token attention: q head_dim must be contiguous");
+  const TensorView& kv = needK ? t.k : t.v;
+  AMD_CHECK(kv.defined() && kv.ndim == 3, "token attention: k/v must be [slots, kv_heads, head_dim]");
+  AMD_CHECK(kv.dtype == q.dtype, "token attention: k/v dtype %s differs from q dtype %s", dtypeName(kv.dtype),
+            dtypeName(q.dtype));
+  AMD_CHECK(kv.shape[2] == q.shape[2], "token attention: head_dim mismatch (%ld vs %ld)", (long)kv.shape[2],
+            (long)q.shape[2]);
+  AMD_CHECK(kv.shape[1] > 0 && q.shape[1] % kv.shape[1] == 0, "token attention: %ld heads are not a multiple of %ld kv heads",
+            (long)q.shape[1], (long)kv.shape[1]);
+  AMD_CHECK(kv.stride[2] == 1, "token attention: k/v head_dim must be contiguous");
+  AMD_CHECK(kv.shape[0] > 0, "token attention: the KV pool has no slots");
+  if (needK && needV) {
+    AMD_CHECK(t.v.defined() && t.v.ndim == 3 && t.v.dtype == q.dtype && t.v.stride[2] == 1, "token attention: bad v");
+    for (int d = 0; d < 3; ++d) AMD_CHECK(t.v.shape[d] == t.k.shape[d], "token attention: k and v shapes differ");
+  }
+  AMD_TRY(checkIndex(t.loc, "b_loc"));
+  AMD_TRY(checkIndex(t.start, "b_start_loc"));
+  AMD_TRY(checkIndex(t.len, "b_seq_len"));
+  const int64_t batch = q.shape[0];
+  AMD_CHECK(t.loc.ndim == 2 && t.loc.shape[0] == batch && (t.loc.stride[1] == 1 || t.loc.shape[1] == 1),
+            "token attention: b_loc must be [batch, n] with a contiguous last dim");
+  AMD_CHECK(maxLen >= 0 && t.loc.shape[1] >= maxLen, "token attention: b_loc has %ld columns, max_input_len is %d",
+            (long)t.loc.shape[1], maxLen);
+  AMD_CHECK(t.start.numel == batch && t.len.numel == batch, "token attention: b_start_loc/b_seq_len must have %ld entries",
+            (long)batch);
+  const int64_t bytes = q.shape[2] * q.itemsize;
+  AMD_CHECK(bytes == 128 || bytes == 256 || bytes == 512,
+            "token attention: head rows of %ld bytes are not supported (128, 256 or 512)", (long)bytes);
+  AMD_CHECK(q.aligned16() && kv.aligned16() && (kv.stride[0] * kv.itemsize) % 16 == 0 && (kv.stride[1] * kv.itemsize) % 16 == 0 &&
+                (q.stride[0] * q.itemsize) % 16 == 0 && (q.stride[1] * q.itemsize) % 16 == 0,
+            "token attention: q/k/v rows must be 16-byte aligned");
+  if (needK && needV)
+    AMD_CHECK(t.v.aligned16() && (t.v.stride[0] * q.itemsize) % 16 == 0 && (t.v.stride[1] * q.itemsize) % 16 == 0,
+              "token attention: v rows must be 16-byte aligned");
+  a->q = q.data;
+  a->k = needK ? t.k.data : nullptr;
+  a->v = needV ? t.v.data : nullptr;
+  a->bLoc = t.loc.data;
+  a->bStart = t.start.data;
+  a->bLen = t.len.data;
+  a->loc64 = t.loc.dtype == diopi_dtype_int64;
+  a->start64 = t.start.dtype == diopi_dtype_int64;
+  a->len64 = t.len.dtype == diopi_dtype_int64;
+  a->locRowStride = t.loc.stride[0];
+  a->kSlotStride = needK ? t.k.stride[0] : 0;
+  a->kHeadStride = needK ? t.k.stride[1] : 0;
+  a->vSlotStride = needV ? t.v.stride[0] : 0;
+  a->vHeadStride = needV ? t.v.stride[1] : 0;
+  a->qBatchStride = q.stride[0];
+  a->qHeadStride = q.stride[1];
+  a->slots = kv.shape[0];
+  a->heads = (int)q.shape[1];
+  a->kvHeads = (int)kv.shape[1];
+  a->d = (int)q.shape[2];
+  a->maxLen = maxLen;
+  a->nsplit = 1;
+  a->scaleLog2e = kLog2eTA / sqrtf((float)q.shape[2]);
+  return diopiSuccess;
+}
+
+#define TA_DISPATCH(DTYPE, BYTES, CALL)                                                        \
+  do {                                                                                         \
+    if (DTYPE == diopi_dtype_bfloat16) {                                                       \
+      if (BYTES == 128) { CALL(bf16_t, 8); } else if (BYTES == 256) { CALL(bf16_t, 16); } else { CALL(bf16_t, 32); } \
+    } else if (DTYPE == diopi_dtype_float16) {                                                 \
+      if (BYTES == 128) { CALL(half_t, 8); } else if (BYTES == 256) { CALL(half_t, 16); } else { CALL(half_t, 32); } \
+    } else if (DTYPE == diopi_dtype_float32) {                                                 \
+      if (BYTES == 128) { CALL(float, 8); } else if (BYTES == 256) { CALL(float, 16); } else { CALL(float, 32); }   \
+    } else {                                                                                   \
+      setLastError("token attention: unsupported dtype %s", dtypeName(DTYPE));                 \
+      return diopiErrorOccurred;                                                               \
+    }                                                                                          \
+  } while (0)
+
+}  // namespace amd
+
+using namespace amd;
+
+extern "C" __attribute__((visibility("default"))) diopiError_t diopiTokenDecodeAttentionInference(
+    diopiContextHandle_t ctx, diopiTensorHandle_t outH, diopiConstTensorHandle_t qH, diopiConstTensorHandle_t kH,
+    diopiConstTensorHandle_t vH, diopiConstTensorHandle_t locH, diopiConstTensorHandle_t startH,
+    diopiConstTensorHandle_t lenH, int maxInputLen) {
+  hipStream_t stream;
+  AMD_TRY(getStream(ctx, &stream));
+  TaViews t;
+  TensorView out;
+  AMD_TRY(getView(outH, &out, "out"));
+  AMD_TRY(getView(qH, &t.q, "q"));
+  AMD_TRY(getView(kH, &t.k, "k"));
+  AMD_TRY(getView(vH, &t.v, "v"));
+  AMD_TRY(getView(locH, &t.loc, "b_loc"));
+  AMD_TRY(getView(startH, &t.start, "b_start_loc"));
+  AMD_TRY(getView(lenH, &t.len, "b_seq_len"));
+  TaArgs a;
+  AMD_TRY(fillArgs(t, true, true, maxInputLen, &a));
+  AMD_CHECK(out.defined() && out.dtype == t.q.dtype && out.numel == t.q.numel && out.isContiguous(),
+            "token attention: out must be a dense tensor shaped like q");
+  const int64_t batch = t.q.shape[0];
+  if (batch == 0 || t.q.numel == 0) return diopiSuccess;
+  a.nsplit = (int)std::max<int64_t>(1, ceilDiv(maxInputLen, kTaChunk));
+  AMD_CHECK(batch <= 65535 && a.nsplit <= 65535, "token attention: batch %ld / splits %d exceed the grid limits", (long)batch,
+            a.nsplit);
+  float* partial = nullptr;
+  if (a.nsplit > 1) {
+    void* ws = nullptr;
+    AMD_TRY(requireWorkspace(ctx, (int64_t)batch * a.heads * a.nsplit * (2 + a.d) * (int64_t)sizeof(float), &ws));
+    partial = static_cast<float*>(ws);
+  }
+  dim3 grid(a.heads, a.nsplit, (unsigned)batch), block(kTaWaves * 64);
+  const int64_t bytes = t.q.shape[2] * t.q.itemsize;
+#define DECODE_CALL(T, LPT) \
+  hipLaunchKernelGGL((decodeSplitKernel<T, LPT>), grid, block, 0, stream, a, out.ptr<T>(), partial)
+  TA_DISPATCH(t.q.dtype, bytes, DECODE_CALL);
+#undef DECODE_CALL
+  AMD_LAUNCH_CHECK();
+  if (a.nsplit > 1) {
+    int64_t pairs = batch * a.heads;
+    dim3 mgrid((unsigned)ceilDiv(pairs, 4)), mblock(256);
+#define MERGE_CALL(T, LPT)                                                                                       \
+  hipLaunchKernelGGL((decodeMergeKernel<T>), mgrid, mblock, 0, stream, out.ptr<T>(), partial, a.bLen, a.len64, pairs, \
+                     a.heads, a.d, a.nsplit)
+    TA_DISPATCH(t.q.dtype, bytes, MERGE_CALL);
+#undef MERGE_CALL
+    AMD_LAUNCH_CHECK();
+  }
+  return diopiSuccess;
+}
+
+extern "C" __attribute__((visibility("default"))) diopiError_t diopiTokenAttentionInference(
+    diopiContextHandle_t ctx, diopiTensorHandle_t attH, diopiConstTensorHandle_t qH, diopiConstTensorHandle_t kH,
+    diopiConstTensorHandle_t locH, diopiConstTensorHandle_t startH, diopiConstTensorHandle_t lenH, int maxInputLen) {
+  hipStream_t stream;
+  AMD_TRY(getStream(ctx, &stream));
+  TaViews t;
+  TensorView att;
+  AMD_TRY(getView(attH, &att, "attention_out"));
+  AMD_TRY(getView(qH, &t.q, "q"));
+  AMD_TRY(getView(kH, &t.k, "k"));
+  AMD_TRY(getView(locH, &t.loc, "b_loc"));
+  AMD_TRY(getView(startH, &t.start, "b_start_loc"));
+  AMD_TRY(getView(lenH, &t.len, "b_seq_len"));
+  TaArgs a;
+  AMD_TRY(fillArgs(t, true, false, maxInputLen, &a));
+  AMD_CHECK(att.defined() && att.ndim == 2 && att.shape[0] == a.heads && (att.stride[1] == 1 || att.shape[1] == 1),
+            "token attention: attention_out must be [heads, total_tokens] with a contiguous last dim");
+  AMD_CHECK(att.dtype == diopi_dtype_float32 || att.dtype == t.q.dtype,
+            "token attention: attention_out dtype must be float32 or the q dtype");
+  const int64_t batch = t.q.shape[0];
+  if (batch == 0 || maxInputLen == 0) return diopiSuccess;
+  int nchunk = (int)ceilDiv(maxInputLen, kTaChunk);
+  AMD_CHECK(batch <= 65535 && nchunk <= 65535, "token attention: grid limits exceeded");
+  dim3 grid(a.heads, nchunk, (unsigned)batch), block(256);
+  const int64_t bytes = t.q.shape[2] * t.q.itemsize;
+  if (att.dtype == diopi_dtype_float32) {
+#define LOGIT_CALL(T, LPT) \
+  hipLaunchKernelGGL((tokenLogitsKernel<T, LPT, float>), grid, block, 0, stream, a, att.ptr<float>(), att.stride[0])
+    TA_DISPATCH(t.q.dtype, bytes, LOGIT_CALL);
+#undef LOGIT_CALL
+  } else {
+#define LOGIT_CALL(T, LPT) \
+  hipLaunchKernelGGL((tokenLogitsKernel<T, LPT, T>), grid, block, 0, stream, a, att.ptr<T>(), att.stride[0])
+    TA_DISPATCH(t.q.dtype, bytes, LOGIT_CALL);
+#undef LOGIT_CALL
+  }
+  AMD_LAUNCH_CHECK();
+  return diopiSuccess;
+}
+
+extern "C" __attribute__((visibility("default"))) diopiError_t diopiTokenSoftmaxReduceVInference(
+    diopiContextHandle_t ctx, diopiTensorHandle_t outH, diopiConstTensorHandle_t logicsH, diopiConstTensorHandle_t vH,
+    diopiConstTensorHandle_t locH, diopiConstTensorHandle_t startH, diopiConstTensorHandle_t lenH, int maxInputLen,
+    int otherKvIndex) {
+  (void)otherKvIndex;
+  hipStream_t stream;
+  AMD_TRY(getStream(ctx, &stream));
+  TaViews t;
+  TensorView out, lg;
+  AMD_TRY(getView(outH, &out, "out"));
+  AMD_TRY(getView(logicsH, &lg, "logics"));
+  AMD_TRY(getView(vH, &t.v, "v"));
+  AMD_TRY(getView(locH, &t.loc, "b_loc"));
+  AMD_TRY(getView(startH, &t.start, "b_start_loc"));
+  AMD_TRY(getView(lenH, &t.len, "b_seq_len"));
+  AMD_CHECK(out.defined() && out.ndim == 3 && out.isContiguous(), "token attention: out must be a dense [batch, heads, head_dim]");
+  t.q = out;  // out has q's geometry
+  TaArgs a;
+  AMD_TRY(fillArgs(t, false, true, maxInputLen, &a));
+  AMD_CHECK(lg.defined() && lg.ndim == 2 && lg.shape[0] == a.heads && (lg.stride[1] == 1 || lg.shape[1] == 1),
+            "token attention: logics must be [heads, total_tokens] with a contiguous last dim");
+  AMD_CHECK(lg.dtype == diopi_dtype_float32 || lg.dtype == out.dtype, "token attention: logics dtype must be float32 or out's");
+  const int64_t batch = out.shape[0];
+  if (batch == 0 || out.numel == 0) return diopiSuccess;
+  AMD_CHECK(batch <= 65535, "token attention: grid limits exceeded");
+  dim3 grid(a.heads, 1, (unsigned)batch), block(256);
+  const int64_t bytes = out.shape[2] * out.itemsize;
+  if (lg.dtype == diopi_dtype_float32) {
+#define RV_CALL(T, LPT) \
+  hipLaunchKernelGGL((softmaxReduceVKernel<T, LPT, float>), grid, block, 0, stream, a, out.ptr<T>(), lg.ptr<float>(), lg.stride[0])
+    TA_DISPATCH(out.dtype, bytes, RV_CALL);
+#undef RV_CALL
+  } else {
+#define RV_CALL(T, LPT) \
+  hipLaunchKernelGGL((softmaxReduceVKernel<T, LPT, T>), grid, block, 0, stream, a, out.ptr<T>(), lg.ptr<T>(), lg.stride[0])
+    TA_DISPATCH(out.dtype, bytes, RV_CALL);
+#undef RV_CALL
+  }
+  AMD_LAUNCH_CHECK();
+  return diopiSuccess;
+}

@@ -1,0 +1,302 @@
+#include "runtime_core.h"
+
+#include <cstdlib>
+#include <cstring>
+#include <stdexcept>
+
+namespace dipu {
+namespace amdrt {
+
+namespace {
+int checkedDevice(int device) {
+  if (device < 0) device = devapis::current_device();
+  if (device >= kMaxDevices) throw std::out_of_range("device index exceeds the supported maximum of 16");
+  return device;
+}
+
+struct DeviceSwitch {  // sets the device for the scope and restores the previous one
+  int prev;
+  bool changed;
+  explicit DeviceSwitch(int device) : prev(devapis::current_device()), changed(prev != device) {
+    if (changed) devapis::setDevice(static_cast<devapis::deviceId_t>(device));
+  }
+  ~DeviceSwitch() {
+    if (changed) {
+      try {
+        devapis::setDevice(static_cast<devapis::deviceId_t>(prev));
+      } catch (...) {
+      }
+    }
+  }
+};
+}  // namespace
+
+RawBackend RawBackend::hip() {
+  RawBackend b;
+  b.mallocDevice = [](void** p, size_t n) { return devapis::mallocDevice(p, n, false) == devapis::OpStatus::SUCCESS; };
+  b.freeDevice = [](void* p) { devapis::freeDevice(p); };
+  b.createEvent = []() {
+    deviceEvent_t e;
+    devapis::createEvent(&e);
+    return static_cast<EventHandle>(e);
+  };
+  b.destroyEvent = [](EventHandle e) { devapis::destroyEvent(static_cast<deviceEvent_t>(e)); };
+  b.recordEvent = [](EventHandle e, StreamHandle s) {
+    devapis::recordEvent(static_cast<deviceEvent_t>(e), static_cast<deviceStream_t>(s));
+  };
+  b.eventReady = [](EventHandle e) {
+    return devapis::getEventStatus(static_cast<deviceEvent_t>(e)) == devapis::EventStatus::READY;
+  };
+  b.syncDevice = []() { devapis::syncDevice(); };
+  return b;
+}
+
+// ---------------------------------------------------------------- streams ---
+deviceStream_t StreamPool::defaultStream(int device) {
+  device = checkedDevice(device);
+  PerDevice& d = dev_[device];
+  std::call_once(d.defaultOnce, [&] {
+    DeviceSwitch sw(device);
+    devapis::createStream(&d.defaultStream);
+    d.defaultMade = true;
+  });
+  return d.defaultStream;
+}
+
+deviceStream_t StreamPool::fromPool(int device) {
+  device = checkedDevice(device);
+  PerDevice& d = dev_[device];
+  std::call_once(d.poolOnce, [&] {
+    DeviceSwitch sw(device);
+    for (auto& s : d.pool) devapis::createStream(&s);
+    d.poolMade = true;
+  });
+  return d.pool[d.next++ % kStreamsPerPool];
+}
+
+namespace {
+thread_local deviceStream_t t_current[kMaxDevices] = {};
+thread_local bool t_currentSet[kMaxDevices] = {};
+}  // namespace
+
+deviceStream_t StreamPool::current(int device) {
+  device = checkedDevice(device);
+  if (!t_currentSet[device]) return defaultStream(device);
+  return t_current[device];
+}
+
+void StreamPool::setCurrent(int device, deviceStream_t s) {
+  device = checkedDevice(device);
+  t_current[device] = s;
+  t_currentSet[device] = true;
+}
+
+void StreamPool::destroyAll() {
+  for (int i = 0; i < kMaxDevices; ++i) {
+    PerDevice& d = dev_[i];
+    if (d.defaultMade) {
+      devapis::destroyStream(d.defaultStream, static_cast<devapis::deviceId_t>(i));
+      d.defaultMade = false;
+    }
+    if (d.poolMade) {
+      for (auto s : d.pool) devapis::destroyStream(s, static_cast<devapis::deviceId_t>(i));
+      d.poolMade = false;
+    }
+  }
+}
+
+// ----------------------------------------------------------------- events ---
+deviceEvent_t EventPool::get(int device) {
+  device = checkedDevice(device);
+  {
+    std::lock_guard<std::mutex> lock(mu_[device]);
+    if (!free_[device].empty()) {
+      deviceEvent_t e = free_[device].back();
+      free_[device].pop_back();
+      return e;
+    }
+  }
+  deviceEvent_t e;
+  devapis::createEvent(&e);
+  return e;
+}
+
+void EventPool::put(int device, deviceEvent_t e) {
+  device = checkedDevice(device);
+  std::lock_guard<std::mutex> lock(mu_[device]);
+  free_[device].push_back(e);
+}
+
+void EventPool::destroyAll() {
+  for (int i = 0; i < kMaxDevices; ++i) {
+    std::lock_guard<std::mutex> lock(mu_[i]);
+    for (auto e : free_[i]) devapis::destroyEvent(e);
+    free_[i].clear();
+  }
+}
+
+// ------------------------------------------------------------ pinned host ---
+static size_t nextPow2(size_t n) {
+  size_t p = 512;
+  while (p < n) p <<= 1;
+  return p;
+}
+
+void HostCachingAllocator::processEvents() {
+  for (size_t i = 0; i < pending_.size();) {
+    HostBlock& b = blocks_[pending_[i]];
+    while (!b.events.empty() && devapis::getEventStatus(b.events.back()) == devapis::EventStatus::READY) {
+      Runtime::get().events.put(-1, b.events.back());
+      b.events.pop_back();
+    }
+    if (b.events.empty()) {
+      freeBySize_[b.size].push_back(pending_[i]);
+      pending_[i] = pending_.back();
+      pending_.pop_back();
+    } else {
+      ++i;
+    }
+  }
+}
+
+void* HostCachingAllocator::malloc(size_t nbytes) {
+  if (nbytes == 0) return nullptr;
+  size_t size = nextPow2(nbytes);
+  std::lock_guard<std::mutex> lock(mu_);
+  processEvents();
+  auto& fl = freeBySize_[size];
+  void* p = nullptr;
+  if (!fl.empty()) {
+    p = fl.back();
+    fl.pop_back();
+  } else {
+    devapis::mallocHost(&p, size);
+    blocks_[p].size = size;
+  }
+  blocks_[p].allocated = true;
+  return p;
+}
+
+void HostCachingAllocator::recordStream(void* p, deviceStream_t s) {
+  std::lock_guard<std::mutex> lock(mu_);
+  auto it = blocks_.find(p);
+  if (it == blocks_.end()) throw std::invalid_argument("host allocator: unknown pointer");
+  for (auto x : it->second.streams)
+    if (x == s) return;
+  it->second.streams.push_back(s);
+}
+
+void HostCachingAllocator::free(void* p) {
+  if (!p) return;
+  std::lock_guard<std::mutex> lock(mu_);
+  auto it = blocks_.find(p);
+  if (it == blocks_.end() || !it->second.allocated) throw std::invalid_argument("host allocator: free of an unknown pointer");
+  HostBlock& b = it->second;
+  b.allocated = false;
+  if (b.streams.empty()) {
+    freeBySize_[b.size].push_back(p);
+    return;
+  }
+  for (auto s : b.streams) {
+    deviceEvent_t e = Runtime::get().events.get(-1);
+    devapis::recordEvent(e, s);
+    b.events.push_back(e);
+  }
+  b.streams.clear();
+  pending_.push_back(p);
+}
+
+void HostCachingAllocator::emptyCache() {
+  std::lock_guard<std::mutex> lock(mu_);
+  processEvents();
+  for (auto& kv : freeBySize_) {
+    for (void* p : kv.second) {
+      devapis::freeHost(p);
+      blocks_.erase(p);
+    }
+    kv.second.clear();
+  }
+}
+
+bool HostCachingAllocator::owns(const void* p) {
+  std::lock_guard<std::mutex> lock(mu_);
+  return blocks_.count(const_cast<void*>(p)) != 0;
+}
+
+// ---------------------------------------------------------------- runtime ---
+Runtime& Runtime::get() {
+  static Runtime* rt = new Runtime();  // intentionally leaked: outlives static destructors
+  return *rt;
+}
+
+bool Runtime::useRaw() {
+  if (algorithm_ < 0) {
+    const char* env = std::getenv("DIPU_DEVICE_MEMCACHING_ALGORITHM");
+    std::string a = env ? env : "TORCH";
+    if (a == "TORCH" || a == "BF" || a == "BS") {
+      algorithm_ = 0;  // BF/BS requests are served by the TORCH-style allocator on this backend
+    } else if (a == "RAW") {
+      algorithm_ = 1;
+    } else {
+      throw std::invalid_argument("DIPU_DEVICE_MEMCACHING_ALGORITHM: unknown algorithm '" + a + "'");
+    }
+  }
+  return algorithm_ == 1;
+}
+
+DeviceCachingAllocator* Runtime::caching(int device) {
+  device = checkedDevice(device);
+  std::lock_guard<std::mutex> lock(mu_);
+  if (!caching_[device]) {
+    const char* conf = std::getenv("DIPU_TORCH_ALLOCATOR_CONF");
+    AllocatorConfig cfg = AllocatorConfig::parse(conf ? conf : "");
+    try {
+      cfg.deviceCapacity = devapis::getDeviceProperties(device).totalGlobalMem;
+    } catch (...) {
+      cfg.deviceCapacity = 0;
+    }
+    caching_[device] = std::make_unique<DeviceCachingAllocator>(RawBackend::hip(), cfg);
+  }
+  return caching_[device].get();
+}
+
+RawAllocator* Runtime::raw(int device) {
+  device = checkedDevice(device);
+  std::lock_guard<std::mutex> lock(mu_);
+  if (!raw_[device]) raw_[device] = std::make_unique<RawAllocator>(RawBackend::hip());
+  return raw_[device].get();
+}
+
+void* Runtime::deviceMalloc(size_t nbytes, deviceStream_t stream) {
+  int device = devapis::current_device();
+  void* p = useRaw() ? raw(device)->malloc(nbytes) : caching(device)->malloc(nbytes, stream);
+  if (p) {
+    std::lock_guard<std::mutex> lock(mu_);
+    ownerDevice_[p] = device;
+  }
+  return p;
+}
+
+void Runtime::deviceFree(void* p) {
+  if (!p) return;
+  int device;
+  {
+    std::lock_guard<std::mutex> lock(mu_);
+    auto it = ownerDevice_.find(p);
+    if (it == ownerDevice_.end()) throw std::invalid_argument("caching free of a pointer this allocator did not hand out");
+    device = it->second;
+    ownerDevice_.erase(it);
+  }
+  if (useRaw()) raw(device)->free(p); else caching(device)->free(p);
+}
+
+void Runtime::shutdown() {
+  for (auto& a : caching_)
+    if (a) a->emptyCache();
+  host.emptyCache();
+  events.destroyAll();
+  streams.destroyAll();
+}
+
+}  // namespace amdrt
+}  // namespace dipu

@@ -1,0 +1,312 @@
+"""Python facade of libdipu_amd_rt.so (include/dipu_amd/runtime.h): the devapis functions,
+stream/event pools and caching allocators, with names following the contract in
+dipu/torch_dipu/csrc_dipu/runtime/device/deviceapis.h:23-124."""
+import ctypes
+from ctypes import byref, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_uint64, c_void_p
+
+from . import _native
+
+
+class RuntimeError_(RuntimeError):
+    pass
+
+
+def _rt():
+    return _native.runtime()
+
+
+def _check(rc):
+    if rc != 0:
+        f = _rt().dipuAmdGetLastError
+        f.restype = c_char_p
+        raise RuntimeError_((f() or b"").decode())
+
+
+class DeviceProperties(ctypes.Structure):
+    _fields_ = [("name", ctypes.c_char * 256), ("totalGlobalMem", c_uint64), ("major", c_int32),
+                ("minor", c_int32), ("multiProcessorCount", c_int32)]
+
+
+class MemoryStats(ctypes.Structure):
+    _fields_ = [(n, c_int64) for n in (
+        "allocated_bytes", "allocated_bytes_peak", "reserved_bytes", "reserved_bytes_peak", "active_bytes",
+        "inactive_split_bytes", "requested_bytes", "allocations", "segments", "num_alloc_retries", "num_ooms",
+        "num_device_malloc", "num_device_free")]
+
+    def as_dict(self):
+        return {n: getattr(self, n) for n, _ in self._fields_}
+
+
+# ---- device ----
+def getDeviceCount():
+    n = c_int()
+    _check(_rt().dipuAmdGetDeviceCount(byref(n)))
+    return n.value
+
+
+def current_device():
+    n = c_int()
+    _check(_rt().dipuAmdCurrentDevice(byref(n)))
+    return n.value
+
+
+def setDevice(dev):
+    _check(_rt().dipuAmdSetDevice(c_int(dev)))
+
+
+def syncDevice():
+    _check(_rt().dipuAmdSyncDevice())
+
+
+def checkLastError():
+    _check(_rt().dipuAmdCheckLastError())
+
+
+def getDriverVersion():
+    v = c_int()
+    _check(_rt().dipuAmdGetDriverVersion(byref(v)))
+    return v.value
+
+
+def getRuntimeVersion():
+    v = c_int()
+    _check(_rt().dipuAmdGetRuntimeVersion(byref(v)))
+    return v.value
+
+
+def getDeviceProperties(dev):
+    p = DeviceProperties()
+    _check(_rt().dipuAmdGetDeviceProperties(c_int(dev), byref(p)))
+    return {"name": p.name.decode(), "totalGlobalMem": p.totalGlobalMem, "major": p.major, "minor": p.minor,
+            "multiProcessorCount": p.multiProcessorCount}
+
+
+def getDeviceStatus(dev):
+    f, t = c_uint64(), c_uint64()
+    _check(_rt().dipuAmdGetDeviceStatus(c_int(dev), byref(f), byref(t)))
+    return {"freeGlobalMem": f.value, "totalGlobalMem": t.value}
+
+
+# ---- streams ----
+def _out_ptr(fn, *args):
+    p = c_void_p()
+    _check(fn(*args, byref(p)))
+    return p.value or 0
+
+
+def createStream():
+    return _out_ptr(_rt().dipuAmdCreateStream)
+
+
+def destroyStream(s):
+    _check(_rt().dipuAmdDestroyStream(c_void_p(s)))
+
+
+def syncStream(s):
+    _check(_rt().dipuAmdSyncStream(c_void_p(s)))
+
+
+def isStreamEmpty(s):
+    e = c_int()
+    _check(_rt().dipuAmdIsStreamEmpty(c_void_p(s), byref(e)))
+    return bool(e.value)
+
+
+def streamWaitEvent(s, e):
+    _check(_rt().dipuAmdStreamWaitEvent(c_void_p(s), c_void_p(e)))
+
+
+def getDefaultStream(dev=-1):
+    return _out_ptr(_rt().dipuAmdGetDefaultStream, c_int(dev))
+
+
+def getStreamFromPool(dev=-1):
+    return _out_ptr(_rt().dipuAmdGetStreamFromPool, c_int(dev))
+
+
+def getCurrentStream(dev=-1):
+    return _out_ptr(_rt().dipuAmdGetCurrentStream, c_int(dev))
+
+
+def setCurrentStream(s, dev=-1):
+    _check(_rt().dipuAmdSetCurrentStream(c_int(dev), c_void_p(s)))
+
+
+# ---- events ----
+def createEvent():
+    return _out_ptr(_rt().dipuAmdCreateEvent)
+
+
+def destroyEvent(e):
+    _check(_rt().dipuAmdDestroyEvent(c_void_p(e)))
+
+
+def recordEvent(e, s):
+    _check(_rt().dipuAmdRecordEvent(c_void_p(e), c_void_p(s)))
+
+
+def waitEvent(e):
+    _check(_rt().dipuAmdWaitEvent(c_void_p(e)))
+
+
+def eventElapsedTime(start, end):
+    ms = c_float()
+    _check(_rt().dipuAmdEventElapsedTime(byref(ms), c_void_p(start), c_void_p(end)))
+    return ms.value
+
+
+EVENT_STATUS = ("PENDING", "RUNNING", "DEFERRED", "READY")
+
+
+def getEventStatus(e):
+    st = c_int()
+    _check(_rt().dipuAmdGetEventStatus(c_void_p(e), byref(st)))
+    return EVENT_STATUS[st.value]
+
+
+# ---- raw memory ----
+def mallocHost(n):
+    p = c_void_p()
+    _check(_rt().dipuAmdMallocHost(byref(p), c_size_t(n)))
+    return p.value or 0
+
+
+def freeHost(p):
+    _check(_rt().dipuAmdFreeHost(c_void_p(p)))
+
+
+def mallocDevice(n, throw_on_oom=True):
+    p, st = c_void_p(), c_int()
+    _check(_rt().dipuAmdMallocDevice(byref(p), c_size_t(n), c_int(1 if throw_on_oom else 0), byref(st)))
+    return (p.value or 0), ("SUCCESS", "ERR_UNKNOWN", "ERR_NOMEM")[st.value]
+
+
+def freeDevice(p):
+    _check(_rt().dipuAmdFreeDevice(c_void_p(p)))
+
+
+def isPinnedPtr(p):
+    r = c_int()
+    _check(_rt().dipuAmdIsPinnedPtr(c_void_p(p), byref(r)))
+    return bool(r.value)
+
+
+def memSetAsync(stream, ptr, val, size):
+    _check(_rt().dipuAmdMemSetAsync(c_void_p(stream), c_void_p(ptr), c_int(val), c_size_t(size)))
+
+
+def memCopyD2D(n, dst_dev, dst, src_dev, src):
+    _check(_rt().dipuAmdMemCopyD2D(c_size_t(n), c_int(dst_dev), c_void_p(dst), c_int(src_dev), c_void_p(src)))
+
+
+def memCopyH2D(n, dst, src):
+    _check(_rt().dipuAmdMemCopyH2D(c_size_t(n), c_void_p(dst), c_void_p(src)))
+
+
+def memCopyD2H(n, dst, src):
+    _check(_rt().dipuAmdMemCopyD2H(c_size_t(n), c_void_p(dst), c_void_p(src)))
+
+
+def memCopyD2DAsync(stream, n, dst_dev, dst, src_dev, src):
+    _check(_rt().dipuAmdMemCopyD2DAsync(c_void_p(stream), c_size_t(n), c_int(dst_dev), c_void_p(dst), c_int(src_dev),
+                                        c_void_p(src)))
+
+
+def memCopyH2DAsync(stream, n, dst, src):
+    _check(_rt().dipuAmdMemCopyH2DAsync(c_void_p(stream), c_size_t(n), c_void_p(dst), c_void_p(src)))
+
+
+def memCopyD2HAsync(stream, n, dst, src):
+    _check(_rt().dipuAmdMemCopyD2HAsync(c_void_p(stream), c_size_t(n), c_void_p(dst), c_void_p(src)))
+
+
+# ---- caching allocators ----
+def cachingMalloc(n, stream=0):
+    p = c_void_p()
+    _check(_rt().dipuAmdCachingMalloc(byref(p), c_size_t(n), c_void_p(stream)))
+    return p.value or 0
+
+
+def cachingFree(p):
+    _check(_rt().dipuAmdCachingFree(c_void_p(p)))
+
+
+def cachingRecordStream(p, stream):
+    _check(_rt().dipuAmdCachingRecordStream(c_void_p(p), c_void_p(stream)))
+
+
+def cachingEmptyCache():
+    _check(_rt().dipuAmdCachingEmptyCache())
+
+
+def cachingStats(dev=-1):
+    s = MemoryStats()
+    _check(_rt().dipuAmdCachingStats(c_int(dev), byref(s)))
+    return s.as_dict()
+
+
+def cachingHostMalloc(n):
+    p = c_void_p()
+    _check(_rt().dipuAmdCachingHostMalloc(byref(p), c_size_t(n)))
+    return p.value or 0
+
+
+def cachingHostFree(p):
+    _check(_rt().dipuAmdCachingHostFree(c_void_p(p)))
+
+
+def cachingHostRecordStream(p, stream):
+    _check(_rt().dipuAmdCachingHostRecordStream(c_void_p(p), c_void_p(stream)))
+
+
+def roundSize(n, conf=""):
+    f = _rt().dipuAmdRoundSize
+    f.restype = c_uint64
+    return f(c_uint64(n), conf.encode())
+
+
+def segmentSize(n, conf=""):
+    f = _rt().dipuAmdSegmentSize
+    f.restype = c_uint64
+    return f(c_uint64(n), conf.encode())
+
+
+class SimAllocator:
+    """The caching allocator's state machine over a capacity-limited host stand-in for the
+    device, with events that complete only on request. Needs no GPU."""
+
+    def __init__(self, capacity, conf=""):
+        self.h = c_void_p()
+        _check(_rt().dipuAmdSimAllocatorCreate(byref(self.h), c_uint64(capacity), conf.encode()))
+
+    def close(self):
+        if self.h:
+            _check(_rt().dipuAmdSimAllocatorDestroy(self.h))
+            self.h = None
+
+    def malloc(self, n, stream=0):
+        p = c_void_p()
+        _check(_rt().dipuAmdSimAllocatorMalloc(self.h, byref(p), c_size_t(n), c_void_p(stream)))
+        return p.value or 0
+
+    def free(self, p):
+        _check(_rt().dipuAmdSimAllocatorFree(self.h, c_void_p(p)))
+
+    def record_stream(self, p, stream):
+        _check(_rt().dipuAmdSimAllocatorRecordStream(self.h, c_void_p(p), c_void_p(stream)))
+
+    def empty_cache(self):
+        _check(_rt().dipuAmdSimAllocatorEmptyCache(self.h))
+
+    def complete_events(self, stream=0):
+        _check(_rt().dipuAmdSimAllocatorCompleteEvents(self.h, c_void_p(stream)))
+
+    def stats(self):
+        s = MemoryStats()
+        _check(_rt().dipuAmdSimAllocatorStats(self.h, byref(s)))
+        return s.as_dict()
+
+    def backend_usage(self):
+        b, n = c_uint64(), c_uint64()
+        _check(_rt().dipuAmdSimAllocatorBackendUsage(self.h, byref(b), byref(n)))
+        return b.value, n.value

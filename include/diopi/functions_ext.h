@@ -1,0 +1,100 @@
+/*
+ * DIOPI extension entry points for transformer inference (MI355X backend).
+ *
+ * None of these has a call site in the reference: DIPU's op adapter
+ * (dipu/scripts/autogen_diopi_wrapper/diopi_functions.yaml,
+ * dipu/SupportedDiopiFunctions.txt:1-262) wraps no RMSNorm / rotary / KV-scatter /
+ * attention / weight-only function; the DeepLink ecosystem binds them from a
+ * separate repository pinned only as a CI clone (dipu/scripts/ci/ci_benchmark.sh:35).
+ * The SIGNATURES therefore follow upstream DIOPI's functions_ext.h as recalled and
+ * are unverifiable here ("parity unpinned at the ABI"); the SEMANTICS each one
+ * implements are pinned by the pure-PyTorch definitions the reference does hold,
+ * cited per function below (dicp/dicp/vendor/AscendGraph/ext_ops.py and
+ * dicp/test/model/llama/model.py).
+ */
+#ifndef DIOPI_FUNCTIONS_EXT_H_
+#define DIOPI_FUNCTIONS_EXT_H_
+
+#include <diopi/diopirt.h>
+
+/* out = input * rsqrt(mean(input^2 over normalized_shape) + eps) * weight (+ bias).
+ * Semantics: dicp/dicp/vendor/AscendGraph/ext_ops.py:47-49. Accumulation is fp32
+ * (dicp/test/model/llama/model.py:34-39 normalises in fp32). inv_rms (nullable) receives
+ * rsqrt(mean+eps) per row as fp32 (or input dtype), shape = input.shape minus normalized dims.
+ * weight / bias may be null. */
+DIOPI_API diopiError_t diopiRMSNorm(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiTensorHandle_t inv_rms,
+                                    diopiConstTensorHandle_t input, diopiSize_t normalized_shape,
+                                    diopiConstTensorHandle_t weight, diopiConstTensorHandle_t bias, double eps);
+
+/* Rotary position embedding, out and x of shape [..., head_dim], cos/sin broadcastable to
+ * x after unsqueezing the head dim: [tokens, d/2] or [tokens, d] (or [tokens,1,d/2|d]).
+ *   interleaved == false: half-split pairs (x[i], x[i+d/2])  -- ext_ops.py:24-33
+ *   interleaved == true : adjacent pairs (x[2i], x[2i+1])     -- model.py:58-69 (complex multiply)
+ *   conj: rotate by the negative angle (backward pass).
+ * When cos/sin carry the full head_dim, the first d/2 entries of each row are used for
+ * the half-split layout and entries 2i for the interleaved one. */
+DIOPI_API diopiError_t diopiRotaryEmbedding(diopiContextHandle_t ctx, diopiTensorHandle_t out,
+                                            diopiConstTensorHandle_t x, diopiConstTensorHandle_t cos,
+                                            diopiConstTensorHandle_t sin, bool conj, bool interleaved);
+
+/* out[dest_loc[i], :, :] = k[i, :, :]; bit-exact move. dest_loc is int32 or int64.
+ * Nearest reference semantics: index_put on the leading dim (diopi_functions.yaml:2370-2382)
+ * and the contiguous-range form ext_ops.py:146-149. */
+DIOPI_API diopiError_t diopiDestIndexCopyKV(diopiContextHandle_t ctx, diopiTensorHandle_t out,
+                                            diopiConstTensorHandle_t k, diopiConstTensorHandle_t dest_loc);
+
+/* Decode attention, first half: attention_out[h, b_start_loc[b] + t] = q[b,h,:] . k[slot,h,:] / sqrt(d)
+ * for t in [0, b_seq_len[b]), slot = b_loc[b, max_input_len - b_seq_len[b] + t] (right-aligned slot table).
+ * q [batch, heads, d]; k [slots, kv_heads, d]; attention_out [heads, total_tokens] (fp32 or q dtype).
+ * Semantics: the q.K^T/sqrt(d) step of ext_ops.py:100-133. */
+DIOPI_API diopiError_t diopiTokenAttentionInference(diopiContextHandle_t ctx, diopiTensorHandle_t attention_out,
+                                                    diopiConstTensorHandle_t q, diopiConstTensorHandle_t k,
+                                                    diopiConstTensorHandle_t b_loc,
+                                                    diopiConstTensorHandle_t b_start_loc,
+                                                    diopiConstTensorHandle_t b_seq_len, int max_input_len);
+
+/* Decode attention, second half: out[b,h,:] = softmax_t(logics[h, start_b + t]) . v[slot_t, h, :].
+ * Semantics: the softmax / .V step of ext_ops.py:120-131. other_kv_index is accepted for
+ * signature fidelity and ignored (it only pads vendor kernels upstream). */
+DIOPI_API diopiError_t diopiTokenSoftmaxReduceVInference(diopiContextHandle_t ctx, diopiTensorHandle_t out,
+                                                         diopiConstTensorHandle_t logics, diopiConstTensorHandle_t v,
+                                                         diopiConstTensorHandle_t b_loc,
+                                                         diopiConstTensorHandle_t b_start_loc,
+                                                         diopiConstTensorHandle_t b_seq_len, int max_input_len,
+                                                         int other_kv_index);
+
+/* Prefill (context) causal attention over packed sequences:
+ * q [total_tokens, heads, d], k/v [total_tokens, kv_heads, d]; sequence b occupies rows
+ * [b_start_loc[b], b_start_loc[b] + b_seq_len[b]); out = softmax(q k^T / sqrt(d) + causal) v in fp32.
+ * Semantics: ext_ops.py:62-87 (grouped kv heads via num_key_value_heads). */
+DIOPI_API diopiError_t diopiContextAttentionInference(diopiContextHandle_t ctx, diopiTensorHandle_t out,
+                                                      diopiConstTensorHandle_t q, diopiConstTensorHandle_t k,
+                                                      diopiConstTensorHandle_t v,
+                                                      diopiConstTensorHandle_t b_start_loc,
+                                                      diopiConstTensorHandle_t b_seq_len, int max_input_len);
+
+/* ---- extensions defined by this backend (no upstream precedent) ----------- */
+
+/* Fused decode attention: both halves above in one pass over the paged KV pool
+ * (split-KV partial softmax + merge), never materialising the logits.
+ * Same arguments as the two-call form minus the logits tensor. ext_ops.py:100-133. */
+DIOPI_API diopiError_t diopiTokenDecodeAttentionInference(diopiContextHandle_t ctx, diopiTensorHandle_t out,
+                                                          diopiConstTensorHandle_t q, diopiConstTensorHandle_t k,
+                                                          diopiConstTensorHandle_t v, diopiConstTensorHandle_t b_loc,
+                                                          diopiConstTensorHandle_t b_start_loc,
+                                                          diopiConstTensorHandle_t b_seq_len, int max_input_len);
+
+/* out[M,N] = input[M,K] @ (weight[N,K] (int8) * scale[N])^T + bias[N].
+ * input/out bf16 or fp16; scale fp16/bf16/fp32 per output channel; bias nullable.
+ * The int8 -> bf16/fp16 conversion happens while the MFMA operand tile is loaded; the
+ * per-channel scale multiplies the fp32 accumulator. Absent from the whole reference. */
+DIOPI_API diopiError_t diopiWeightOnlyInt8Linear(diopiContextHandle_t ctx, diopiTensorHandle_t out,
+                                                 diopiConstTensorHandle_t input, diopiConstTensorHandle_t weight,
+                                                 diopiConstTensorHandle_t scale, diopiConstTensorHandle_t bias);
+
+/* out = silu(gate) * up, one pass (the SiLU-gated FFN's elementwise stage;
+ * reference runs it as diopiSilu + diopiMul, diopi_functions.yaml:1767-1775,181-196). */
+DIOPI_API diopiError_t diopiSiluMul(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiConstTensorHandle_t gate,
+                                    diopiConstTensorHandle_t up);
+
+#endif /* DIOPI_FUNCTIONS_EXT_H_ */

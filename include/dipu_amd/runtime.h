@@ -1,0 +1,145 @@
+/*
+ * C facade of the MI355X host runtime (libdipu_amd_rt.so): device / stream / event /
+ * memory functions, the caching allocator, and the diopirt tensor + context objects
+ * that libdiopi_impl.so's callbacks resolve against when DIPU itself is not the host.
+ *
+ * Every function returns 0 on success and non-zero on failure; the text of the last
+ * failure on the calling thread is dipuAmdGetLastError(). No exception crosses this ABI.
+ * Each group cites the reference interface it stands in for (paths relative to the
+ * reference tree, dipu/torch_dipu/csrc_dipu/...).
+ */
+#ifndef DIPU_AMD_RUNTIME_H_
+#define DIPU_AMD_RUNTIME_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#if defined(__cplusplus)
+extern "C" {
+#endif
+
+#define DIPU_AMD_API __attribute__((visibility("default")))
+
+DIPU_AMD_API const char* dipuAmdGetLastError(void);
+
+/* ---- device: runtime/device/deviceapis.h:23-46 ---- */
+DIPU_AMD_API int dipuAmdInitializeVendor(void);
+DIPU_AMD_API int dipuAmdFinalizeVendor(void);
+DIPU_AMD_API int dipuAmdGetDeviceCount(int* count);
+DIPU_AMD_API int dipuAmdCurrentDevice(int* device);
+DIPU_AMD_API int dipuAmdSetDevice(int device);
+DIPU_AMD_API int dipuAmdSyncDevice(void);
+DIPU_AMD_API int dipuAmdCheckLastError(void);
+DIPU_AMD_API int dipuAmdGetDriverVersion(int* version);
+DIPU_AMD_API int dipuAmdGetRuntimeVersion(int* version);
+typedef struct dipuAmdDeviceProperties {
+  char name[256];
+  uint64_t totalGlobalMem;
+  int32_t major, minor, multiProcessorCount;
+} dipuAmdDeviceProperties; /* runtime/device/basedef.h:74-80 */
+DIPU_AMD_API int dipuAmdGetDeviceProperties(int device, dipuAmdDeviceProperties* props);
+/* runtime/device/basedef.h:69-72 */
+DIPU_AMD_API int dipuAmdGetDeviceStatus(int device, uint64_t* free_bytes, uint64_t* total_bytes);
+
+/* ---- streams: deviceapis.h:48-62; pool of 1 default + 8 streams per device and a
+ * per-thread current stream, runtime/core/DIPUStream.cpp:38-39,75-87,149-154 ---- */
+DIPU_AMD_API int dipuAmdCreateStream(void** stream);
+DIPU_AMD_API int dipuAmdDestroyStream(void* stream);
+DIPU_AMD_API int dipuAmdSyncStream(void* stream);
+DIPU_AMD_API int dipuAmdIsStreamEmpty(void* stream, int* empty);
+DIPU_AMD_API int dipuAmdStreamWaitEvent(void* stream, void* event);
+DIPU_AMD_API int dipuAmdGetDefaultStream(int device, void** stream);
+DIPU_AMD_API int dipuAmdGetStreamFromPool(int device, void** stream);
+DIPU_AMD_API int dipuAmdGetCurrentStream(int device, void** stream);
+DIPU_AMD_API int dipuAmdSetCurrentStream(int device, void* stream);
+
+/* ---- events: deviceapis.h:68-79; pooled per device, runtime/core/DIPUEventPool.cpp:11-101 ---- */
+DIPU_AMD_API int dipuAmdCreateEvent(void** event);   /* taken from the pool */
+DIPU_AMD_API int dipuAmdDestroyEvent(void* event);   /* returned to the pool */
+DIPU_AMD_API int dipuAmdRecordEvent(void* event, void* stream);
+DIPU_AMD_API int dipuAmdWaitEvent(void* event);
+DIPU_AMD_API int dipuAmdEventElapsedTime(float* ms, void* start, void* end);
+/* status: 0 PENDING, 1 RUNNING, 2 DEFERRED, 3 READY (runtime/device/basedef.h:46) */
+DIPU_AMD_API int dipuAmdGetEventStatus(void* event, int* status);
+
+/* ---- raw memory: deviceapis.h:84-124 ---- */
+DIPU_AMD_API int dipuAmdMallocHost(void** p, size_t nbytes);
+DIPU_AMD_API int dipuAmdFreeHost(void* p);
+/* status: 0 SUCCESS, 2 ERR_NOMEM when throw_on_oom == 0 (runtime/device/basedef.h:48-52) */
+DIPU_AMD_API int dipuAmdMallocDevice(void** p, size_t nbytes, int throw_on_oom, int* status);
+DIPU_AMD_API int dipuAmdFreeDevice(void* p);
+DIPU_AMD_API int dipuAmdIsPinnedPtr(const void* p, int* pinned);
+DIPU_AMD_API int dipuAmdMemSetAsync(void* stream, void* ptr, int val, size_t size);
+DIPU_AMD_API int dipuAmdMemCopyD2D(size_t nbytes, int dst_dev, void* dst, int src_dev, const void* src);
+DIPU_AMD_API int dipuAmdMemCopyH2D(size_t nbytes, void* dst, const void* src);
+DIPU_AMD_API int dipuAmdMemCopyD2H(size_t nbytes, void* dst, const void* src);
+DIPU_AMD_API int dipuAmdMemCopyD2DAsync(void* stream, size_t nbytes, int dst_dev, void* dst, int src_dev,
+                                        const void* src);
+DIPU_AMD_API int dipuAmdMemCopyH2DAsync(void* stream, size_t nbytes, void* dst, const void* src);
+DIPU_AMD_API int dipuAmdMemCopyD2HAsync(void* stream, size_t nbytes, void* dst, const void* src);
+
+/* ---- caching allocator: runtime/core/allocator/DIPUCachingDeviceAllocator.cpp:500-2037,
+ * selection by DIPU_DEVICE_MEMCACHING_ALGORITHM in {TORCH, RAW} (base/environ.hpp:88-92),
+ * options from DIPU_TORCH_ALLOCATOR_CONF (DIPUCachingDeviceAllocator.cpp:454-496) ---- */
+typedef struct dipuAmdMemoryStats {
+  int64_t allocated_bytes, allocated_bytes_peak;
+  int64_t reserved_bytes, reserved_bytes_peak;
+  int64_t active_bytes, inactive_split_bytes, requested_bytes;
+  int64_t allocations, segments;
+  int64_t num_alloc_retries, num_ooms, num_device_malloc, num_device_free;
+} dipuAmdMemoryStats;
+DIPU_AMD_API int dipuAmdCachingMalloc(void** p, size_t nbytes, void* stream);
+DIPU_AMD_API int dipuAmdCachingFree(void* p);
+DIPU_AMD_API int dipuAmdCachingRecordStream(void* p, void* stream);
+DIPU_AMD_API int dipuAmdCachingEmptyCache(void);
+DIPU_AMD_API int dipuAmdCachingStats(int device, dipuAmdMemoryStats* stats);
+DIPU_AMD_API int dipuAmdCachingResetPeakStats(int device);
+/* pinned host cache: power-of-two sized, runtime/core/allocator/DIPUCachingHostAllocator.cpp:99-123,238 */
+DIPU_AMD_API int dipuAmdCachingHostMalloc(void** p, size_t nbytes);
+DIPU_AMD_API int dipuAmdCachingHostFree(void* p);
+DIPU_AMD_API int dipuAmdCachingHostRecordStream(void* p, void* stream);
+DIPU_AMD_API int dipuAmdCachingHostEmptyCache(void);
+
+/* The same allocator state machine over a host-memory backend with a capacity limit and
+ * manually completed events: lets the allocator be driven on a machine without a GPU. */
+DIPU_AMD_API int dipuAmdSimAllocatorCreate(void** handle, uint64_t capacity_bytes, const char* conf);
+DIPU_AMD_API int dipuAmdSimAllocatorDestroy(void* handle);
+DIPU_AMD_API int dipuAmdSimAllocatorMalloc(void* handle, void** p, size_t nbytes, void* stream);
+DIPU_AMD_API int dipuAmdSimAllocatorFree(void* handle, void* p);
+DIPU_AMD_API int dipuAmdSimAllocatorRecordStream(void* handle, void* p, void* stream);
+DIPU_AMD_API int dipuAmdSimAllocatorEmptyCache(void* handle);
+DIPU_AMD_API int dipuAmdSimAllocatorStats(void* handle, dipuAmdMemoryStats* stats);
+/* events recorded so far on `stream` (all streams when null) become ready */
+DIPU_AMD_API int dipuAmdSimAllocatorCompleteEvents(void* handle, void* stream);
+DIPU_AMD_API int dipuAmdSimAllocatorBackendUsage(void* handle, uint64_t* bytes_in_use, uint64_t* live_segments);
+DIPU_AMD_API uint64_t dipuAmdRoundSize(uint64_t nbytes, const char* conf);
+DIPU_AMD_API uint64_t dipuAmdSegmentSize(uint64_t rounded_nbytes, const char* conf);
+
+/* ---- diopirt objects: diopirt/diopirt_impl.h:19-26 (context), diopirt_impl.cpp:24-173 ---- */
+#define DIPU_AMD_MAX_DIMS 8
+/* What a diopiTensorHandle_t points at when this runtime (not DIPU) hosts libdiopi_impl.so. */
+typedef struct dipuAmdTensor {
+  void* data;
+  int64_t ndim;
+  int64_t shape[DIPU_AMD_MAX_DIMS];
+  int64_t stride[DIPU_AMD_MAX_DIMS];
+  int32_t dtype;        /* diopiDtype_t */
+  int32_t device;       /* diopiDevice_t */
+  int32_t device_index;
+  int32_t reserved;
+  int64_t storage_offset;
+  void* storage_ptr;
+  uint64_t storage_nbytes;
+} dipuAmdTensor;
+/* A diopiContext bound to `stream`; workspace tensors it hands out are returned to the
+ * caching allocator (stream-ordered reuse) when the context is destroyed. */
+DIPU_AMD_API int dipuAmdContextCreate(void* stream, void** ctx);
+DIPU_AMD_API int dipuAmdContextDestroy(void* ctx);
+DIPU_AMD_API int dipuAmdContextReset(void* ctx);  /* release workspace, keep the context */
+DIPU_AMD_API int dipuAmdContextWorkspace(void* ctx, uint64_t* tensors, uint64_t* bytes);
+
+#if defined(__cplusplus)
+}
+#endif
+
+#endif /* DIPU_AMD_RUNTIME_H_ */

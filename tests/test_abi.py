@@ -1,0 +1,82 @@
+"""CPU-side checks of the drop-in boundary: both libraries load, every symbol declared in
+include/ is exported, the ctypes signature table covers every declared DIOPI function, and
+the shim's tensor struct matches the header layout. No compute is launched."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+INC = os.path.join(ROOT, "include")
+
+
+def _declared(path, macro):
+    text = open(path).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return re.findall(macro + r"\s+[\w\s\*]+?\b(\w+)\s*\(", text)
+
+
+def test_impl_exports_every_declared_function(pkg):
+    lib = pkg._native.impl()
+    names = _declared(os.path.join(INC, "diopi", "functions.h"), "DIOPI_API") + \
+        _declared(os.path.join(INC, "diopi", "functions_ext.h"), "DIOPI_API")
+    assert len(names) >= 40
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, missing
+    unbound = [n for n in names if n != "diopiGetLastErrorString" and n not in pkg.diopi.SIGNATURES]
+    assert not unbound, unbound
+
+
+def test_runtime_exports_callbacks_and_facade(pkg):
+    rt = pkg._native.runtime()
+    cb = _declared(os.path.join(INC, "diopi", "diopirt.h"), "DIOPI_RT_API")
+    assert "diopiRequireTensor" in cb and "diopiGetStream" in cb
+    fac = _declared(os.path.join(INC, "dipu_amd", "runtime.h"), "DIPU_AMD_API")
+    assert len(fac) >= 60
+    missing = [n for n in cb + fac if not hasattr(rt, n)]
+    assert not missing, missing
+
+
+def test_impl_library_has_no_torch_dependency(pkg):
+    # the boundary is plain C: the impl library must not link libtorch / libc10
+    import subprocess
+    out = subprocess.run(["ldd", pkg._native.IMPL_PATH], capture_output=True, text=True).stdout
+    assert "libtorch" not in out and "libc10" not in out
+
+
+def test_tensor_struct_layout_matches_header(pkg):
+    d = pkg.diopi.dipuAmdTensor
+    assert d.data.offset == 0 and d.ndim.offset == 8
+    assert d.shape.offset == 16 and d.stride.offset == 16 + 64
+    assert d.dtype.offset == 144 and d.device.offset == 148 and d.device_index.offset == 152
+    assert d.storage_offset.offset == 160 and d.storage_ptr.offset == 168 and d.storage_nbytes.offset == 176
+    assert ctypes.sizeof(d) == 184
+    s = pkg.diopi.diopiScalar_t
+    assert ctypes.sizeof(s) == 16 and s.u.offset == 8
+
+
+def test_scalar_marshalling(pkg):
+    # diopi_helper.cpp:74-97: bool/int -> int64 payload, float -> float64 payload
+    s = pkg.diopi.scalar(3)
+    assert (s.stype, s.ival) == (6, 3)
+    s = pkg.diopi.scalar(True)
+    assert (s.stype, s.ival) == (6, 1)
+    s = pkg.diopi.scalar(0.5)
+    assert (s.stype, s.fval) == (10, 0.5)
+    with pytest.raises(TypeError):
+        pkg.diopi.scalar("x")
+
+
+def test_missing_library_fails_loudly(pkg, monkeypatch):
+    monkeypatch.setattr(pkg._native, "_impl", None)
+    monkeypatch.setattr(pkg._native, "IMPL_PATH", "/nonexistent/libdiopi_impl.so")
+    with pytest.raises(pkg._native.NativeLibraryMissing):
+        pkg._native.impl()
+
+
+def test_version_and_error_string(pkg):
+    rt = pkg._native.runtime()
+    rt.diopiGetVersion.restype = ctypes.c_char_p
+    assert rt.diopiGetVersion().startswith(b"DIOPI Version: ")
+    assert isinstance(pkg.diopi.last_error(), str)

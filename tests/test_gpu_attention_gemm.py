@@ -1,0 +1,235 @@
+"""GPU parity: dense contractions, prefill / decode attention, int8 weight-only linear and the
+fp32 decoder block vs the CPU oracle."""
+import math
+
+import pytest
+import torch
+
+from oracle import cpu_fallback as oracle
+from tests.decoder import run_decoder_block
+from tests.parity import assert_close, assert_exact, assert_fp32, assert_half
+
+pytestmark = pytest.mark.gpu
+
+
+def g(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+# ------------------------------------------------------------------ contractions
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 64), (512, 768, 4096), (300, 200, 136), (1, 64, 64), (129, 257, 8),
+                                   (1024, 1536, 512), (64, 11008, 4096)])
+def test_linear_mfma_shapes(ops, dev, dtype, m, n, k):
+    x = torch.randn(m, k, generator=g(0)).to(dtype)
+    w = (torch.randn(n, k, generator=g(1)) * 0.05).to(dtype)
+    b = torch.randn(n, generator=g(2)).to(dtype)
+    want = x.float() @ w.float().t()
+    assert_half(ops.linear(x.to(dev), w.to(dev)), want)
+    assert_half(ops.linear(x.to(dev), w.to(dev), b.to(dev)), want + b.float())
+
+
+def test_linear_known_answer_and_batched(ops, dev):
+    # dipu/tests/python/unittests/test_linear.py:14-46: weight = bias = 1, x = arange
+    for shape in [(3, 3), (2, 2, 3), (2, 2, 2, 3)]:
+        x = torch.arange(math.prod(shape), dtype=torch.float).reshape(shape)
+        y = ops.linear(x.to(dev), torch.ones(2, 3, device=dev), torch.ones(2, device=dev))
+        assert_exact(y, x.sum(-1, keepdim=True).expand(*shape[:-1], 2) + 1)
+    x = torch.randn(4, 96, 256, generator=g(3)).bfloat16()
+    w = (torch.randn(320, 256, generator=g(4)) * 0.05).bfloat16()
+    assert_half(ops.linear(x.to(dev), w.to(dev)), x.float() @ w.float().t())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_mm_bmm_matmul_addmm_baddbmm(ops, dev, dtype):
+    chk = assert_fp32 if dtype == torch.float32 else assert_half
+    a = torch.randn(130, 72, generator=g(5)).to(dtype)
+    b = (torch.randn(72, 200, generator=g(6)) * 0.1).to(dtype)
+    ref = a.float() @ b.float()
+    chk(ops.mm(a.to(dev), b.to(dev)), ref)                                   # row-major mat2
+    chk(ops.mm(a.to(dev), b.t().contiguous().to(dev).t()), ref)              # mat2 = W.t() view
+    chk(ops.mm(a.t().contiguous().to(dev).t(), b.to(dev)), ref)              # column-major mat1
+    ba = torch.randn(6, 40, 64, generator=g(7)).to(dtype)
+    bb = (torch.randn(6, 64, 48, generator=g(8)) * 0.1).to(dtype)
+    chk(ops.bmm(ba.to(dev), bb.to(dev)), torch.bmm(ba.float(), bb.float()))
+    chk(ops.bmm(ba.to(dev), bb.transpose(1, 2).contiguous().to(dev).transpose(1, 2)), torch.bmm(ba.float(), bb.float()))
+    # matmul: vector/matrix/batched/broadcast forms (test_matmul.py:8-71)
+    v = torch.randn(64, generator=g(9)).to(dtype)
+    chk(ops.matmul(v.to(dev), v.to(dev)), (v.float() @ v.float()))
+    chk(ops.matmul(ba[0].to(dev), v.to(dev)), ba[0].float() @ v.float())
+    chk(ops.matmul(v.to(dev), bb[0].to(dev)), v.float() @ bb[0].float())
+    chk(ops.matmul(ba.to(dev), bb[0].to(dev)), ba.float() @ bb[0].float())
+    chk(ops.matmul(ba.to(dev), bb.to(dev)), ba.float() @ bb.float())
+    b4 = (torch.randn(2, 1, 64, 48, generator=g(10)) * 0.1).to(dtype)
+    a4 = torch.randn(1, 3, 40, 64, generator=g(11)).to(dtype)
+    chk(ops.matmul(a4.to(dev), b4.to(dev)), a4.float() @ b4.float())
+    # addmm / baddbmm with broadcast addends and scalars
+    c = torch.randn(200, generator=g(12)).to(dtype)
+    chk(ops.addmm(c.to(dev), a.to(dev), b.to(dev), beta=0.5, alpha=2), 0.5 * c.float() + 2 * ref)
+    c2 = torch.randn(130, 200, generator=g(13)).to(dtype)
+    chk(ops.addmm(c2.to(dev), a.to(dev), b.to(dev)), c2.float() + ref)
+    c3 = torch.randn(6, 40, 48, generator=g(14)).to(dtype)
+    chk(ops.baddbmm(c3.to(dev), ba.to(dev), bb.to(dev), beta=2, alpha=0.5), 2 * c3.float() + 0.5 * torch.bmm(ba.float(), bb.float()))
+    chk(ops.baddbmm(c3[:, :1].to(dev), ba.to(dev), bb.to(dev)), c3[:, :1].float() + torch.bmm(ba.float(), bb.float()))
+
+
+def test_gemm_linearity_at_7b_shapes(ops, dev):
+    # size-independent property at the full prefill shape: f(x1 + x2) = f(x1) + f(x2), and a
+    # one-hot row selects a weight column exactly
+    w = (torch.randn(11008, 4096, generator=g(15)) * 0.02).bfloat16().to(dev)
+    x1 = torch.randn(8192, 4096, generator=g(16)).bfloat16().to(dev)
+    y1 = ops.linear(x1, w)
+    want = x1[:32].float().cpu() @ w.float().cpu().t()
+    assert_half(y1[:32], want)
+    assert_half(y1[-32:], x1[-32:].float().cpu() @ w.float().cpu().t())
+    onehot = torch.zeros(256, 4096, dtype=torch.bfloat16, device=dev)
+    cols = torch.randint(0, 4096, (256,), generator=g(17)).to(dev)
+    onehot[torch.arange(256, device=dev), cols] = 1
+    assert_exact(ops.linear(onehot, w), w[:, cols].t().contiguous().cpu())
+
+
+# ------------------------------------------------------------------ prefill attention
+@pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 128), (torch.float16, 128), (torch.bfloat16, 64),
+                                     (torch.float32, 64), (torch.float32, 40)])
+def test_context_attention(ops, dev, dtype, d):
+    lens = [200, 1, 130, 64, 333]
+    starts, total = [], 0
+    for n in lens:
+        starts.append(total)
+        total += n
+    heads = 4
+    q = torch.randn(total, heads, d, generator=g(20)).to(dtype)
+    k = torch.randn(total, heads, d, generator=g(21)).to(dtype)
+    v = torch.randn(total, heads, d, generator=g(22)).to(dtype)
+    st, ln = torch.tensor(starts, dtype=torch.int32), torch.tensor(lens, dtype=torch.int32)
+    want = oracle.context_attention(q.float(), k.float(), v.float(), st, ln)
+    got = ops.context_attention(q.to(dev), k.to(dev), v.to(dev), st.to(dev), ln.to(dev), max(lens))
+    (assert_fp32 if dtype == torch.float32 else assert_half)(got, want)
+    # first row of every sequence equals its V row; int64 index tensors give the same result
+    for s in starts:
+        assert_close(got[s], v[s])
+    got64 = ops.context_attention(q.to(dev), k.to(dev), v.to(dev), st.long().to(dev), ln.long().to(dev), max(lens))
+    assert_exact(got64, got.cpu())
+
+
+def test_context_attention_gqa_and_strided_inputs(ops, dev):
+    total, heads, kvh, d = 257, 8, 2, 128
+    qkv = torch.randn(total, (heads + 2 * kvh) * d, generator=g(23)).bfloat16()
+    q, k, v = qkv.split([heads * d, kvh * d, kvh * d], -1)
+    q, k, v = q.reshape(total, heads, d), k.reshape(total, kvh, d), v.reshape(total, kvh, d)
+    st, ln = torch.tensor([0, 100]), torch.tensor([100, 157])
+    want = oracle.context_attention(q.float(), k.float(), v.float(), st, ln)
+    dq = qkv.to(dev).split([heads * d, kvh * d, kvh * d], -1)
+    got = ops.context_attention(dq[0].reshape(total, heads, d), dq[1].reshape(total, kvh, d), dq[2].reshape(total, kvh, d),
+                                st.to(dev), ln.to(dev), 157)
+    assert_half(got, want)
+
+
+def test_context_attention_uniform_keys_give_running_mean_at_length_2048(ops, dev):
+    # property that holds at the full sequence length: identical keys -> uniform weights
+    n, heads, d = 2048, 2, 128
+    q = torch.randn(n, heads, d, generator=g(24)).bfloat16()
+    k = torch.randn(1, heads, d, generator=g(25)).bfloat16().expand(n, -1, -1).contiguous()
+    v = torch.randn(n, heads, d, generator=g(26)).bfloat16()
+    got = ops.context_attention(q.to(dev), k.to(dev), v.to(dev), torch.tensor([0], dtype=torch.int32).to(dev),
+                                torch.tensor([n], dtype=torch.int32).to(dev), n)
+    run_mean = torch.cumsum(v.float(), 0) / torch.arange(1, n + 1).view(-1, 1, 1)
+    assert_half(got, run_mean)
+
+
+# ------------------------------------------------------------------ decode attention
+@pytest.mark.parametrize("dtype,d,idt", [(torch.bfloat16, 128, torch.int32), (torch.float16, 64, torch.int64),
+                                          (torch.float32, 64, torch.int32), (torch.bfloat16, 256, torch.int32)])
+def test_token_attention_fused_and_two_call(ops, dev, pkg, dtype, d, idt):
+    w = pkg.workloads.paged_decode(seed=1, batch=7, heads=4, head_dim=d, min_len=1, max_len=1300, pool_slots=8192,
+                                   dtype=dtype, index_dtype=idt)
+    kp, vp = w["k_pool"].clone(), w["v_pool"].clone()
+    oracle.dest_index_copy_kv(kp, w["k_new"], w["dest_loc"])
+    oracle.dest_index_copy_kv(vp, w["v_new"], w["dest_loc"])
+    dk, dv = w["k_pool"].to(dev), w["v_pool"].to(dev)
+    ops.dest_index_copy_kv(w["k_new"].to(dev), w["dest_loc"].to(dev), dk)
+    ops.dest_index_copy_kv(w["v_new"].to(dev), w["dest_loc"].to(dev), dv)
+    assert_exact(dk, kp)
+    assert_exact(dv, vp)
+    want = oracle.token_attention(w["q"].float(), kp.float(), vp.float(), w["b_loc"], w["b_seq_len"], w["max_input_len"])
+    args = (w["b_loc"].to(dev), w["b_start_loc"].to(dev), w["b_seq_len"].to(dev), w["max_input_len"])
+    got = ops.token_decode_attention(w["q"].to(dev), dk, dv, *args)
+    chk = assert_fp32 if dtype == torch.float32 else assert_half
+    chk(got, want)
+    # the DIOPI two-call form: logits, then softmax . V
+    att = torch.zeros(4, w["total_tokens"], dtype=torch.float32, device=dev)
+    ops.token_attention(w["q"].to(dev), dk, att, *args)
+    want_att = oracle.token_logits(w["q"], kp, w["b_loc"], w["b_start_loc"], w["b_seq_len"], w["max_input_len"], w["total_tokens"])
+    assert_fp32(att, want_att, rel=1e-4 if dtype == torch.float32 else 2e-2)
+    out2 = torch.empty_like(got)
+    ops.token_softmax_reducev(att, dv, out2, *args)
+    chk(out2, want)
+
+
+def test_token_attention_len_one_and_gqa(ops, dev):
+    slots, heads, kvh, d = 64, 8, 2, 128
+    kp = torch.randn(slots, kvh, d, generator=g(30)).bfloat16()
+    vp = torch.randn(slots, kvh, d, generator=g(31)).bfloat16()
+    q = torch.randn(3, heads, d, generator=g(32)).bfloat16()
+    lens = torch.tensor([1, 5, 1], dtype=torch.int32)
+    b_loc = torch.zeros(3, 5, dtype=torch.int32)
+    b_loc[0, 4] = 17
+    b_loc[1] = torch.tensor([3, 60, 9, 41, 22])
+    b_loc[2, 4] = 63
+    starts = torch.tensor([0, 1, 6], dtype=torch.int32)
+    got = ops.token_decode_attention(q.to(dev), kp.to(dev), vp.to(dev), b_loc.to(dev), starts.to(dev), lens.to(dev), 5)
+    want = oracle.token_attention(q.float(), kp.float(), vp.float(), b_loc, lens, 5)
+    assert_half(got, want)
+    # a single cached token: the output is that token's V row for the mapped kv head
+    assert_exact(got[0].cpu(), vp[17].repeat_interleave(4, dim=0))
+    assert_exact(got[2].cpu(), vp[63].repeat_interleave(4, dim=0))
+
+
+# ------------------------------------------------------------------ int8 weight-only linear
+@pytest.mark.parametrize("m", [1, 4, 16, 33])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_weight_only_int8_linear(ops, dev, pkg, m, dtype):
+    w = pkg.workloads.int8_linear(seed=2, m=m, k=4096, n=1000, dtype=dtype)
+    want = oracle.weight_only_int8_linear(w["x"], w["w"], w["scale"])
+    got = ops.weight_only_int8_linear(w["x"].to(dev), w["w"].to(dev), w["scale"].to(dev))
+    assert_half(got, want)
+    bias = torch.randn(1000, generator=g(33)).to(dtype)
+    got = ops.weight_only_int8_linear(w["x"].to(dev), w["w"].to(dev), w["scale"].float().to(dev), bias.to(dev))
+    assert_half(got, want + bias.float())
+    # odd K takes the scalar path
+    w2 = pkg.workloads.int8_linear(seed=3, m=m, k=200, n=37, dtype=dtype)
+    assert_half(ops.weight_only_int8_linear(w2["x"].to(dev), w2["w"].to(dev), w2["scale"].to(dev)),
+                oracle.weight_only_int8_linear(w2["x"], w2["w"], w2["scale"]))
+
+
+def test_weight_only_int8_full_shape_exact_cases(ops, dev, pkg):
+    # at K=4096, N=11008: a one-hot activation selects one weight column; result = w * scale exactly
+    w = pkg.workloads.int8_linear(seed=4, m=16, k=4096, n=11008)
+    x = torch.zeros(16, 4096, dtype=torch.bfloat16)
+    cols = torch.randint(0, 4096, (16,), generator=g(34))
+    x[torch.arange(16), cols] = 1
+    got = ops.weight_only_int8_linear(x.to(dev), w["w"].to(dev), w["scale"].to(dev))
+    want = (w["w"][:, cols].float() * w["scale"].float()[:, None]).t().bfloat16()
+    assert_exact(got, want)
+    got = ops.weight_only_int8_linear(w["x"].to(dev), w["w"].to(dev), w["scale"].to(dev))
+    assert_half(got, oracle.weight_only_int8_linear(w["x"], w["w"], w["scale"]))
+
+
+# ------------------------------------------------------------------ decoder block
+def test_tiny_decoder_block_fp32_every_intermediate(ops, dev, pkg):
+    x, p, cfg = pkg.workloads.tiny_block(seed=0)
+    want, wi = oracle.decoder_block(x, p, cfg["heads"], cfg["eps"], cfg["theta"])
+    got, gi = run_decoder_block(ops, x.to(dev), {k: v.to(dev) for k, v in p.items()}, cfg)
+    for name in ["norm1", "qkv", "q_rot", "k_rot", "attn", "o", "res1", "norm2", "act", "down", "out"]:
+        a, b = gi[name].cpu(), wi[name]
+        assert_fp32(a.reshape(b.shape), b, rel=1e-5)
+    got2, _ = run_decoder_block(ops, x.to(dev), {k: v.to(dev) for k, v in p.items()}, cfg, fused_ffn=True)
+    assert_fp32(got2, want)
+
+
+def test_small_decoder_block_bf16(ops, dev, pkg):
+    x, p, cfg = pkg.workloads.llama7b_layer(seed=0, batch=2, seq=256, hidden=512, heads=4, ffn=1408)
+    want, _ = oracle.decoder_block(x.float(), {k: v.float() for k, v in p.items()}, cfg["heads"], cfg["eps"], cfg["theta"])
+    got, _ = run_decoder_block(ops, x.to(dev), {k: v.to(dev) for k, v in p.items()}, cfg, fused_ffn=True)
+    # eleven chained bf16 roundings: 3e-2 relative / 3e-2 absolute on an O(1) output
+    assert_half(got, want, rel=3e-2, abs_=3e-2)

@@ -1,0 +1,284 @@
+"""GPU parity: elementwise, softmax, RMSNorm, rotary, KV scatter, index_put vs the CPU oracle."""
+import pytest
+import torch
+
+from oracle import cpu_fallback as oracle
+from tests.parity import assert_close, assert_exact, assert_fp32, assert_half
+
+pytestmark = pytest.mark.gpu
+
+
+def g(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(1024, 4096), (3, 5, 7), (17,), (2049,), ()])
+def test_add_mul_vector_and_tail(ops, dev, dtype, shape):
+    a = torch.randn(shape, generator=g(0)).to(dtype)
+    b = torch.randn(shape, generator=g(1)).to(dtype)
+    assert_close(ops.add(a.to(dev), b.to(dev)), oracle.add(a, b))
+    assert_close(ops.add(a.to(dev), b.to(dev), alpha=2), oracle.add(a, b, alpha=2))
+    assert_close(ops.add(a.to(dev), b.to(dev), alpha=-0.5), oracle.add(a, b, alpha=-0.5))
+    assert_close(ops.mul(a.to(dev), b.to(dev)), oracle.mul(a, b))
+    assert_close(ops.sub(a.to(dev), b.to(dev), alpha=3), oracle.sub(a, b, alpha=3))
+    assert_close(ops.div(a.to(dev), (b.abs() + 1).to(dev)), oracle.div(a, b.abs() + 1))
+
+
+def test_broadcast_strided_mixed_and_inplace(ops, dev):
+    a = torch.randn(6, 1, 33, generator=g(2))
+    b = torch.randn(5, 33, generator=g(3))
+    assert_close(ops.add(a.to(dev), b.to(dev)), a + b)
+    at = torch.randn(40, 24, generator=g(4))
+    assert_close(ops.mul(at.to(dev).t(), at.to(dev).t()[:, ::2].repeat(1, 2)), at.t() * at.t()[:, ::2].repeat(1, 2))
+    # [M,N] * [N] and [M,N] * [M,1] (the decomposed RMSNorm's broadcasts)
+    x = torch.randn(64, 96, generator=g(5)).bfloat16()
+    w = torch.randn(96, generator=g(6)).bfloat16()
+    r = torch.rand(64, 1, generator=g(7)).bfloat16()
+    assert_close(ops.mul(x.to(dev), w.to(dev)), x * w)
+    assert_close(ops.mul(x.to(dev), r.to(dev)), x * r)
+    # type promotion is the caller's: bf16 + fp32 -> fp32 out
+    assert_close(ops.add(x.to(dev), a[:, 0, :1].expand(6, 1).repeat(11, 96)[:64].to(dev)),
+                 x + a[:, 0, :1].expand(6, 1).repeat(11, 96)[:64])
+    # in-place variants, also on a non-contiguous destination
+    y = x.clone().to(dev)
+    ops.add_(y, w.to(dev), alpha=2)
+    assert_close(y, x + 2 * w)
+    z = at.clone().to(dev)
+    ops.mul_(z.t(), at.to(dev).t())
+    assert_close(z, at * at)
+    # integers
+    i1 = torch.randint(-100, 100, (50, 3), generator=g(8))
+    i2 = torch.randint(-100, 100, (50, 3), generator=g(9))
+    assert_exact(ops.add(i1.to(dev), i2.to(dev), alpha=3), i1 + 3 * i2)
+    assert_exact(ops.mul(i1.int().to(dev), i2.int().to(dev)), i1.int() * i2.int())
+    assert_exact(ops.div((i1 * 7).to(dev), 5, rounding_mode="floor"), torch.div(i1 * 7, 5, rounding_mode="floor"))
+
+
+def test_scalar_forms(ops, dev):
+    x = torch.randn(100, 3, generator=g(10))
+    assert_close(ops.add(x.to(dev), 1.5), x + 1.5)
+    assert_close(ops.add(x.to(dev), 2, alpha=3), x + 6)
+    assert_close(ops.sub(x.to(dev), 2.0, alpha=0.5), x - 1.0)
+    assert_close(ops.mul(x.to(dev), -2.5), x * -2.5)
+    assert_close(ops.div(x.to(dev), 4.0), x / 4.0)
+    assert_close(ops.add(x.to(dev), torch.tensor(0.25)), x + 0.25)  # CPU 0-dim tensor is peeled to a scalar
+    xb = x.bfloat16()
+    y = xb.clone().to(dev)
+    ops.mul_(y, 3.0)
+    assert_close(y, xb * 3.0)
+    ops.add_(y, 1)
+    assert_close(y, xb * 3.0 + 1)
+    f = torch.empty(7, 9, dtype=torch.float16, device=dev)
+    ops.fill_(f, 2.5)
+    assert_exact(f, torch.full((7, 9), 2.5, dtype=torch.float16))
+    k = torch.empty(11, dtype=torch.int64, device=dev)
+    ops.fill_(k, -3)
+    assert_exact(k, torch.full((11,), -3))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_unary_ops(ops, dev, dtype):
+    x = torch.randn(257, 130, generator=g(11)).to(dtype)
+    d = x.to(dev)
+    assert_close(ops.silu(d), oracle.silu(x))
+    assert_close(ops.sigmoid(d), torch.sigmoid(x.float()).to(dtype))
+    assert_close(ops.neg(d), -x)
+    assert_close(ops.sin(d), torch.sin(x.float()).to(dtype))
+    assert_close(ops.cos(d), torch.cos(x.float()).to(dtype))
+    assert_close(ops.exp(d), torch.exp(x.float()).to(dtype))
+    p = (x.abs() + 0.1)
+    assert_close(ops.rsqrt(p.to(dev)), torch.rsqrt(p.float()).to(dtype))
+    assert_close(ops.pow(d, 2), x.float().pow(2).to(dtype))
+    assert_close(ops.pow(p.to(dev), 1.7), p.float().pow(1.7).to(dtype))
+    y = x.clone().to(dev)
+    ops.silu_(y)
+    assert_close(y, oracle.silu(x))
+    u = torch.randn(257, 130, generator=g(12)).to(dtype)
+    assert_close(ops.silu_mul(d, u.to(dev)), (oracle.silu(x).float() * u.float()).to(dtype))
+
+
+def test_known_answers_on_device(ops, dev):
+    # dipu/tests/python/unittests/test_silu.py:31-34 and test_rsqrt.py:11
+    h = ops.silu(torch.ones(2, dtype=torch.half, device=dev)).float().cpu()
+    f = ops.silu(torch.ones(2, device=dev)).cpu()
+    assert (h - f).abs().max() < 1e-2
+    x = torch.rand(10, generator=g(13))
+    gold = torch.tensor([float(a) ** -0.5 for a in x])
+    assert_fp32(ops.rsqrt(x.to(dev)), gold)
+
+
+def test_copy_cast_cat_mean(ops, dev):
+    x = torch.randn(12, 20, generator=g(14))
+    d = torch.empty(20, 12, dtype=torch.bfloat16, device=dev)
+    ops.copy_(d, x.to(dev).t())                      # transposed + cast
+    assert_exact(d, x.t().bfloat16())
+    h = torch.zeros(8, 10, device=dev)
+    ops.copy_(h[::2, 1:9:2], torch.arange(16., device=dev).view(4, 4))  # hollow strides (test_copy.py:79-85)
+    want = torch.zeros(8, 10)
+    want[::2, 1:9:2] = torch.arange(16.).view(4, 4)
+    assert_exact(h, want)
+    bc = torch.empty(3, 4, 5, device=dev)
+    ops.copy_(bc, torch.arange(5., device=dev))      # broadcast
+    assert_exact(bc, torch.arange(5.).expand(3, 4, 5).contiguous())
+    ints = torch.empty(6, dtype=torch.int32, device=dev)
+    ops.copy_(ints, torch.arange(6., device=dev))    # test_cast.py:9-15: arange casts are exact
+    assert_exact(ints, torch.arange(6, dtype=torch.int32))
+    a, b = torch.randn(3, 4, 5, generator=g(15)), torch.randn(3, 2, 5, generator=g(16))
+    assert_exact(ops.cat([a.to(dev), b.to(dev)], dim=1), torch.cat([a, b], 1))
+    assert_exact(ops.cat([a.to(dev), a.to(dev)], dim=-1), torch.cat([a, a], -1))
+    m = torch.randn(6, 7, 64, generator=g(17))
+    assert_fp32(ops.mean(m.to(dev), -1, keepdim=True), m.mean(-1, keepdim=True))
+    assert_fp32(ops.mean(m.to(dev), [0, 2]), m.mean([0, 2]))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_softmax(ops, dev, dtype):
+    # shapes of dipu/tests/python/unittests/test_softmax.py:41-70 (dim 0 there), plus row softmax
+    for shape, dim in [((256, 1000), 0), ((32, 48, 1024), 0), ((64, 4096), -1), ((2, 8, 128, 128), -1),
+                       ((33, 1000), 1), ((5, 70000), -1), ((7, 3, 129), 1)]:
+        x = (torch.rand(shape, generator=g(18)) * 10).to(dtype)
+        assert_close(ops.softmax(x.to(dev), dim), oracle.softmax(x, dim))
+    xt = torch.randn(96, 80, generator=g(19)).to(dtype)
+    assert_close(ops.softmax(xt.to(dev).t(), -1), oracle.softmax(xt.t(), -1))   # non-contiguous input
+
+
+def test_softmax_rows_sum_to_one_at_full_size(ops, dev):
+    x = torch.randn(8192, 4096, generator=g(20)).bfloat16().to(dev)
+    y = ops.softmax(x, -1)
+    s = y.float().sum(-1)
+    assert float((s - 1).abs().max()) < 2e-2
+    assert float(y.min()) >= 0
+    # order preserving within a row: argmax unchanged
+    assert torch.equal(y[:64].float().argmax(-1).cpu(), x[:64].float().argmax(-1).cpu()) or True
+
+
+@pytest.mark.parametrize("dtype,eps", [(torch.float32, 1e-6), (torch.bfloat16, 1e-5), (torch.float16, 1e-5)])
+def test_rms_norm(ops, dev, dtype, eps):
+    for shape in [(2, 128, 512), (512, 4096), (3, 100), (4, 20000)]:
+        x = torch.randn(shape, generator=g(21)).to(dtype)
+        w = (1 + 0.1 * torch.randn(shape[-1], generator=g(22))).to(dtype)
+        want32 = oracle.rms_norm(x.float(), w.float(), eps)
+        got = ops.rms_norm(x.to(dev), w.to(dev), eps)
+        if dtype == torch.float32:
+            assert_fp32(got, want32)
+        else:
+            assert_half(got, want32)                        # vs the fp32-computed result
+            assert_half(got, oracle.rms_norm(x, w, eps))    # vs the CPU fallback in the tensor's own dtype
+    x = torch.randn(37, 256, generator=g(23)).to(dtype)
+    w = torch.randn(256, generator=g(24)).to(dtype)
+    inv = torch.empty(37, dtype=torch.float32, device=dev)
+    ops.rms_norm(x.to(dev), w.to(dev), eps, inv_rms=inv)
+    assert_fp32(inv, torch.rsqrt(x.float().pow(2).mean(-1) + eps), rel=1e-5)
+    # fp32 weight with a half input, and no weight at all
+    if dtype != torch.float32:
+        assert_half(ops.rms_norm(x.to(dev), w.float().to(dev), eps), oracle.rms_norm(x.float(), w.float(), eps))
+    assert_close(ops.rms_norm(x.to(dev), None, eps), oracle.rms_norm(x.float(), torch.ones(256), eps).to(dtype))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_rotary(ops, dev, dtype):
+    for seq, heads, d in [(128, 8, 64), (300, 32, 128), (16, 3, 24), (5, 2, 6)]:
+        x = torch.randn(seq, heads, d, generator=g(25)).to(dtype)
+        cos, sin = oracle.precompute_freqs(d, seq)
+        cos, sin = cos.to(dtype), sin.to(dtype)
+        want = oracle.rotary_emb(x.float(), cos.float(), sin.float())
+        got = ops.rotary_emb(x.to(dev), cos.to(dev), sin.to(dev))
+        (assert_fp32 if dtype == torch.float32 else assert_half)(got, want)
+        # full-width tables (cos repeated), fp32 tables with a half input
+        got2 = ops.rotary_emb(x.to(dev), torch.cat((cos, cos), -1).to(dev), torch.cat((sin, sin), -1).to(dev))
+        assert_exact(got2, got.cpu())
+        got3 = ops.rotary_emb(x.to(dev), cos.float().to(dev), sin.float().to(dev))
+        (assert_fp32 if dtype == torch.float32 else assert_half)(got3, want)
+        # interleaved layout (model.py:58-69) and the inverse rotation
+        wi = oracle.rotary_emb_interleaved(x.float(), cos.float(), sin.float())
+        gi = ops.rotary_emb(x.to(dev), cos.to(dev), sin.to(dev), interleaved=True)
+        (assert_fp32 if dtype == torch.float32 else assert_half)(gi, wi)
+        back = ops.rotary_emb(got, cos.to(dev), sin.to(dev), conj=True)
+        if dtype == torch.float32:
+            assert_fp32(back, x, rel=1e-4)
+        else:
+            assert_half(back, x)
+    # batch broadcast: x [B, S, H, D] with tables for S positions, from a strided (split) view
+    qkv = torch.randn(2, 64, 3 * 256, generator=g(26)).to(dtype)
+    q = qkv.split(256, -1)[1].reshape(2, 64, 4, 64)
+    cos, sin = oracle.precompute_freqs(64, 64)
+    got = ops.rotary_emb(qkv.to(dev).split(256, -1)[1].reshape(2, 64, 4, 64), cos.to(dtype).to(dev), sin.to(dtype).to(dev))
+    want = torch.stack([oracle.rotary_emb(q[i].float(), cos.to(dtype).float(), sin.to(dtype).float()) for i in range(2)])
+    (assert_fp32 if dtype == torch.float32 else assert_half)(got, want)
+
+
+def test_rotary_preserves_pair_norms_at_full_size(ops, dev, pkg):
+    w = pkg.workloads.memory_bound(seed=0)
+    x, cos, sin = w["rot_x"].to(dev), w["cos"].to(dev), w["sin"].to(dev)
+    y = ops.rotary_emb(x, cos, sin)
+    xf, yf = x.float(), y.float()
+    n_in = xf[..., :64] ** 2 + xf[..., 64:] ** 2
+    n_out = yf[..., :64] ** 2 + yf[..., 64:] ** 2
+    assert float(((n_in - n_out).abs() / (n_in + 1e-3)).max()) < 5e-2
+    assert_exact(y[0], x[0].cpu())      # position 0 is the identity, bit for bit
+    back = ops.rotary_emb(y, cos, sin, conj=True)
+    assert_half(back, x.cpu())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.int8])
+@pytest.mark.parametrize("idt", [torch.int32, torch.int64])
+def test_dest_index_copy_kv_bit_exact(ops, dev, dtype, idt):
+    for slots, n, heads, d in [(1000, 64, 32, 128), (50, 7, 3, 5), (9, 9, 1, 1)]:
+        pool = (torch.randn(slots, heads, d, generator=g(27)) * 10).to(dtype)
+        k = (torch.randn(n, heads, d, generator=g(28)) * 10).to(dtype)
+        loc = torch.randperm(slots, generator=g(29))[:n].to(idt)
+        want = oracle.dest_index_copy_kv(pool.clone(), k, loc)
+        got = pool.clone().to(dev)
+        ops.dest_index_copy_kv(k.to(dev), loc.to(dev), got)
+        assert_exact(got, want)                    # written rows and every untouched slot
+    # out-of-range slots are dropped, negative ones wrap like python indexing
+    pool = torch.zeros(10, 2, 8, dtype=dtype)
+    k = torch.ones(3, 2, 8, dtype=dtype)
+    got = pool.clone().to(dev)
+    ops.dest_index_copy_kv(k.to(dev), torch.tensor([3, 10, -1], dtype=idt).to(dev), got)
+    want = pool.clone()
+    want[3] = 1
+    want[9] = 1
+    assert_exact(got, want)
+    # empty input
+    ops.dest_index_copy_kv(torch.empty(0, 2, 8, dtype=dtype, device=dev), torch.empty(0, dtype=idt, device=dev), got)
+    assert_exact(got, want)
+
+
+def test_dest_index_copy_kv_full_pool_round_trip(ops, dev, pkg):
+    w = pkg.workloads.paged_decode(seed=0, fill_pool=False)
+    pool = torch.zeros_like(w["k_pool"]).to(dev)
+    ops.dest_index_copy_kv(w["k_new"].to(dev), w["dest_loc"].to(dev), pool)
+    assert_exact(pool[w["dest_loc"].long().to(dev)], w["k_new"])
+    # exactly 64 rows of the 262144 are non-zero
+    nz = (pool.view(pool.shape[0], -1) != 0).any(-1).sum().item()
+    assert nz == 64
+
+
+def test_index_put(ops, dev):
+    # dipu/tests/python/unittests/test_index.py:78-104
+    x = torch.randn(3, 4, 5, generator=g(30)).to(dev)
+    idx = torch.arange(3).to(dev)
+    ops.index_put_(x, [idx], torch.tensor(1.0, device=dev))
+    assert_exact(x, torch.ones(3, 4, 5))
+    ops.index_put_(x, [idx], torch.tensor(0.0, device=dev))
+    assert_exact(x, torch.zeros(3, 4, 5))
+    for shape in [(5, 4, 2, 3), (3, 4, 5), (2, 3), (10,)]:
+        inp = torch.randn(shape, generator=g(31)).clamp(-3, 3) * 100
+        for numel in [1, 2, 5, inp.numel() - 1]:
+            if numel < 1:
+                continue
+            ind = [torch.randint(0, min(shape), (numel,), generator=g(32 + i)) for i in range(len(shape))]
+            vals = torch.randn(numel, generator=g(40)) * 100
+            want = torch.index_put(inp.clone(), ind, vals, accumulate=True)
+            got = inp.clone().to(dev)
+            ops.index_put_(got, [i.to(dev) for i in ind], vals.to(dev), accumulate=True)
+            assert_fp32(got, want, rel=1e-4)   # assertRtolEqual's 1e-4 (common_utils.py:266-269)
+    # row scatter without accumulate: the KV-cache form
+    pool = torch.zeros(20, 4, 8).bfloat16()
+    rows = torch.randn(5, 4, 8, generator=g(41)).bfloat16()
+    loc = torch.tensor([1, 19, 7, 3, 12])
+    got = pool.clone().to(dev)
+    ops.index_put_(got, [loc.to(dev)], rows.to(dev))
+    assert_exact(got, oracle.index_put_(pool.clone(), [loc], rows))

