@@ -1,0 +1,346 @@
+#!/usr/bin/env python3
+"""Benchmark of the DIOPI inference hot path on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-ops]
+
+One "step" is one pass of a Llama-2-7B-shaped decoder layer (prefill, batch 4 x seq 2048,
+hidden 4096, 32 heads x 128, FFN 11008, bf16, random weights, synthetic activations) through
+the DIOPI C ABI of libdiopi_impl.so: RMSNorm -> QKV linear -> rotary(q,k) -> causal context
+attention -> out linear -> residual add -> RMSNorm -> gate/up linears -> SiLU*mul -> down linear
+-> residual add. Inputs and weights are resident in HBM before the timed region.
+
+Prints ONE JSON line: tokens/s for the layer (whole job = the one GPU), the roofline of the
+dominant kernel (the bf16 MFMA GEMM) measured with device events on the launch stream inside the
+timed region, the CPU baseline (the oracle timed on the host cores on a bounded sample), and,
+under "ops", the HBM-roofline figures of the memory-bound ops (add, mul, softmax, RMSNorm,
+rotary on bf16 [8192, 4096]; the paged decode step; the int8 weight-only linear).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+MFMA_BF16_PEAK_TF = 2500.0   # MI355X dense bf16, published
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-ops", action="store_true", help="skip the per-op HBM microbenchmarks")
+    ap.add_argument("--only-layer", action="store_true", help="alias for --no-cpu --no-ops")
+    return ap.parse_args()
+
+
+class Prepared:
+    """A DIOPI call with its arguments marshalled once: per launch it costs two C calls
+    (the op and the release of the context's workspace), so short kernels are not host-bound."""
+
+    def __init__(self, pkg, name, *args):
+        d = pkg.diopi
+        self.keep = []
+        self.cargs = []
+        for a in args:
+            if a is None or hasattr(a, "data_ptr"):
+                h, p = d.handle(a)
+                self.keep.append(h)
+                self.cargs.append(p)
+            elif isinstance(a, d.diopiScalar_t):
+                import ctypes
+                self.keep.append(a)
+                self.cargs.append(ctypes.byref(a))
+            else:
+                self.cargs.append(a)
+        self.ctx = d.Context()
+        self.fn = d.fn(name)
+        self.name = name
+        self.reset = pkg._native.runtime().dipuAmdContextReset
+        self.err = d.last_error
+
+    def __call__(self):
+        rc = self.fn(self.ctx.ptr, *self.cargs)
+        if rc != 0:
+            raise RuntimeError(f"{self.name} failed: {self.err()}")
+        self.reset(self.ctx.ptr)
+
+
+def layer_plan(pkg, torch, dev, x, p, cfg):
+    """Preallocates every intermediate and returns the ordered list of (label, Prepared)."""
+    d = pkg.diopi
+    b, s, hidden = x.shape
+    heads = cfg["heads"]
+    hd = hidden // heads
+    ffn = p["wgate"].shape[0]
+    T = b * s
+    bf = x.dtype
+    new = lambda *shape: torch.empty(*shape, dtype=bf, device=dev)
+    h1, qkv, attn, o, x1, h2 = new(T, hidden), new(T, 3 * hidden), new(T, heads, hd), new(T, hidden), new(T, hidden), new(T, hidden)
+    qr, kr = new(T, heads, hd), new(T, heads, hd)
+    gate, up, act, down, out = new(T, ffn), new(T, ffn), new(T, ffn), new(T, hidden), new(T, hidden)
+    cos, sin = pkg.workloads.rotary_tables(hd, s, cfg["theta"], dtype=bf)
+    cos, sin = cos.to(dev), sin.to(dev)
+    starts = (torch.arange(b, dtype=torch.int32) * s).to(dev)
+    lens = torch.full((b,), s, dtype=torch.int32).to(dev)
+    x2 = x.reshape(T, hidden)
+    q, k, v = qkv.split(hidden, dim=-1)
+    q4, k4 = q.reshape(b, s, heads, hd), k.reshape(b, s, heads, hd)
+    v3 = v.reshape(T, heads, hd)
+    one = d.scalar(1)
+    P = lambda name, *a: Prepared(pkg, name, *a)
+    plan = [
+        ("rms_norm", P("diopiRMSNorm", h1, None, x2, d.size([hidden]), p["norm1"], None, float(cfg["eps"]))),
+        ("gemm_qkv", P("diopiLinear", qkv, h1, p["wqkv"], None)),
+        ("rotary_q", P("diopiRotaryEmbedding", qr.view(b, s, heads, hd), q4, cos, sin, False, False)),
+        ("rotary_k", P("diopiRotaryEmbedding", kr.view(b, s, heads, hd), k4, cos, sin, False, False)),
+        ("context_attention", P("diopiContextAttentionInference", attn, qr, kr, v3, starts, lens, int(s))),
+        ("gemm_o", P("diopiLinear", o, attn.view(T, hidden), p["wo"], None)),
+        ("add", P("diopiAdd", x1, x2, o, one)),
+        ("rms_norm", P("diopiRMSNorm", h2, None, x1, d.size([hidden]), p["norm2"], None, float(cfg["eps"]))),
+        ("gemm_gate", P("diopiLinear", gate, h2, p["wgate"], None)),
+        ("gemm_up", P("diopiLinear", up, h2, p["wup"], None)),
+        ("silu_mul", P("diopiSiluMul", act, gate, up)),
+        ("gemm_down", P("diopiLinear", down, act, p["wdown"], None)),
+        ("add", P("diopiAdd", out, x1, down, one)),
+    ]
+    keep = [h1, qkv, attn, o, x1, h2, qr, kr, gate, up, act, down, out, cos, sin, starts, lens, x2]
+    flops = {"gemm_qkv": 2 * T * 3 * hidden * hidden, "gemm_o": 2 * T * hidden * hidden, "gemm_gate": 2 * T * ffn * hidden,
+             "gemm_up": 2 * T * ffn * hidden, "gemm_down": 2 * T * hidden * ffn}
+    return plan, keep, flops, out
+
+
+def time_ops(rt, stream, calls, iters, warm):
+    """Average device time per launch of each prepared call (events on the launch stream)."""
+    out = []
+    for call in calls:
+        for _ in range(warm):
+            call()
+        e0, e1 = rt.createEvent(), rt.createEvent()
+        rt.syncStream(stream)
+        rt.recordEvent(e0, stream)
+        for _ in range(iters):
+            call()
+        rt.recordEvent(e1, stream)
+        rt.waitEvent(e1)
+        out.append(rt.eventElapsedTime(e0, e1) / iters * 1e3)  # us
+        rt.destroyEvent(e0)
+        rt.destroyEvent(e1)
+    return out
+
+
+def op_microbench(pkg, torch, dev, rt, stream):
+    """HBM-bound ops: algorithmic bytes / measured device time. `cold` rotates through enough
+    buffer sets to exceed the 256 MB Infinity Cache; `hot` reuses one set."""
+    d = pkg.diopi
+    wl = pkg.workloads
+    res = []
+    w = wl.memory_bound(seed=0)
+    E = w["a"].numel()
+    nset = 6  # 6 x (3 x 64 MiB) = 1.1 GiB of distinct buffers in rotation
+    A = [w["a"].to(dev).clone() for _ in range(nset)]
+    B = [w["b"].to(dev).clone() for _ in range(nset)]
+    O = [torch.empty_like(A[0]) for _ in range(nset)]
+    rw = w["rms_weight"].to(dev)
+    one = d.scalar(1)
+
+    def rotating(mk):
+        calls = [mk(i) for i in range(nset)]
+        state = {"i": 0}
+
+        def run():
+            calls[state["i"] % nset]()
+            state["i"] += 1
+        return run
+
+    specs = [
+        ("diopiAdd", 3 * E * 2, lambda i: Prepared(pkg, "diopiAdd", O[i], A[i], B[i], one)),
+        ("diopiMul", 3 * E * 2, lambda i: Prepared(pkg, "diopiMul", O[i], A[i], B[i])),
+        ("diopiSoftmax", 2 * E * 2, lambda i: Prepared(pkg, "diopiSoftmax", O[i], A[i], -1)),
+        ("diopiRMSNorm", 2 * E * 2 + 8192, lambda i: Prepared(pkg, "diopiRMSNorm", O[i], None, A[i], d.size([4096]), rw, None, 1e-5)),
+        ("diopiSiluMul", 3 * E * 2, lambda i: Prepared(pkg, "diopiSiluMul", O[i], A[i], B[i])),
+    ]
+    for name, nbytes, mk in specs:
+        hot, cold = time_ops(rt, stream, [mk(0), rotating(mk)], 60, 12)
+        res.append({"op": name, "workload": "bf16 [8192,4096]", "bytes": nbytes, "us_hot": round(hot, 2), "us_cold": round(cold, 2),
+                    "GBs_hot": round(nbytes / hot / 1e3, 1), "GBs_cold": round(nbytes / cold / 1e3, 1),
+                    "frac_hot": round(nbytes / hot / 1e3 / HBM_PEAK_GBS, 3), "frac_cold": round(nbytes / cold / 1e3 / HBM_PEAK_GBS, 3)})
+    del A, B, O
+    X = [w["rot_x"].to(dev).clone() for _ in range(nset)]
+    RO = [torch.empty_like(X[0]) for _ in range(nset)]
+    cos, sin = w["cos"].to(dev), w["sin"].to(dev)
+    nbytes = 2 * X[0].numel() * 2 + 2 * cos.numel() * 2
+    mk = lambda i: Prepared(pkg, "diopiRotaryEmbedding", RO[i], X[i], cos, sin, False, False)
+    hot, cold = time_ops(rt, stream, [mk(0), rotating(mk)], 60, 12)
+    res.append({"op": "diopiRotaryEmbedding", "workload": "bf16 [8192,32,128], tables [8192,64]", "bytes": nbytes,
+                "us_hot": round(hot, 2), "us_cold": round(cold, 2), "GBs_hot": round(nbytes / hot / 1e3, 1),
+                "GBs_cold": round(nbytes / cold / 1e3, 1), "frac_hot": round(nbytes / hot / 1e3 / HBM_PEAK_GBS, 3),
+                "frac_cold": round(nbytes / cold / 1e3 / HBM_PEAK_GBS, 3)})
+    del X, RO
+    # paged decode step: scatter the new token's K and V, then fused attention (4 GiB of pool: always cold)
+    pd = wl.paged_decode(seed=0)
+    g = {k: (v.to(dev) if hasattr(v, "to") else v) for k, v in pd.items()}
+    out = torch.empty_like(g["q"])
+    L = int(pd["b_seq_len"].sum())
+    idx_b = pd["b_loc"].element_size()
+    attn_bytes = L * 16384 + L * idx_b + 2 * 64 * 32 * 128 * 2
+    scat_bytes = 2 * 64 * 8192 * 2 + 2 * 64 * idx_b
+    ck = Prepared(pkg, "diopiDestIndexCopyKV", g["k_pool"], g["k_new"], g["dest_loc"])
+    cv = Prepared(pkg, "diopiDestIndexCopyKV", g["v_pool"], g["v_new"], g["dest_loc"])
+    at = Prepared(pkg, "diopiTokenDecodeAttentionInference", out, g["q"], g["k_pool"], g["v_pool"], g["b_loc"],
+                  g["b_start_loc"], g["b_seq_len"], int(g["max_input_len"]))
+
+    def scatter():
+        ck()
+        cv()
+
+    def step():
+        ck()
+        cv()
+        at()
+    t_sc, t_at, t_step = time_ops(rt, stream, [scatter, at, step], 30, 6)
+    res.append({"op": "diopiDestIndexCopyKV(K)+(V)", "workload": "64 tokens into a 262144-slot pool", "bytes": scat_bytes,
+                "us_cold": round(t_sc, 2), "GBs_cold": round(scat_bytes / t_sc / 1e3, 1), "frac_cold": round(scat_bytes / t_sc / 1e3 / HBM_PEAK_GBS, 4)})
+    res.append({"op": "diopiTokenDecodeAttentionInference", "workload": f"batch 64, 32x128, sum(len)={L}", "bytes": attn_bytes,
+                "us_cold": round(t_at, 2), "GBs_cold": round(attn_bytes / t_at / 1e3, 1), "frac_cold": round(attn_bytes / t_at / 1e3 / HBM_PEAK_GBS, 3)})
+    res.append({"op": "decode step (scatter + attention)", "workload": "batch 64", "us_cold": round(t_step, 2),
+                "tokens_per_s": round(64 / (t_step * 1e-6), 1)})
+    del g, pd
+    # int8 weight-only linear: weights rotate through 8 copies (360 MB) for the cold figure
+    for m in (1, 4, 16):
+        q8 = wl.int8_linear(seed=0, m=m)
+        x, sc = q8["x"].to(dev), q8["scale"].to(dev)
+        W = [q8["w"].to(dev).clone() for _ in range(8)]
+        o8 = torch.empty(m, 11008, dtype=torch.bfloat16, device=dev)
+        nbytes = 4096 * 11008 + 2 * 11008 + 2 * m * 4096 + 2 * m * 11008
+        calls8 = [Prepared(pkg, "diopiWeightOnlyInt8Linear", o8, x, W[i], sc, None) for i in range(8)]
+        st8 = {"i": 0}
+
+        def rot8():
+            calls8[st8["i"] % 8]()
+            st8["i"] += 1
+        hot, cold = time_ops(rt, stream, [calls8[0], rot8], 200, 16)
+        res.append({"op": "diopiWeightOnlyInt8Linear", "workload": f"M={m}, K=4096, N=11008", "bytes": nbytes, "us_hot": round(hot, 2),
+                    "us_cold": round(cold, 2), "GBs_hot": round(nbytes / hot / 1e3, 1), "GBs_cold": round(nbytes / cold / 1e3, 1),
+                    "frac_hot": round(nbytes / hot / 1e3 / HBM_PEAK_GBS, 3), "frac_cold": round(nbytes / cold / 1e3 / HBM_PEAK_GBS, 3)})
+        del W
+    return res
+
+
+def cpu_baseline(pkg, torch):
+    """The oracle's decoder layer on the host cores, on the same batch of four 2048-token sequences."""
+    from oracle import cpu_fallback as oracle
+    x, p, cfg = pkg.workloads.llama7b_layer(seed=0, batch=4)
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    t0 = time.perf_counter()
+    oracle.decoder_block(x, p, cfg["heads"], cfg["eps"], cfg["theta"])   # warm-up (thread pool, allocations)
+    warm = time.perf_counter() - t0
+    reps = 1 if warm > 12 else (3 if warm > 4 else 8)
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        oracle.decoder_block(x, p, cfg["heads"], cfg["eps"], cfg["theta"])
+        times.append(time.perf_counter() - t0)
+    t = min(times)
+    return {"value": round(8192 / t, 2), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"the same layer and batch (4 x 2048 tokens) through the oracle: stock ATen CPU kernels in bf16, best of {reps} "
+                      f"passes after a warm-up, {t:.2f} s per pass"}
+
+
+def main():
+    args = parse()
+    if args.only_layer:
+        args.no_cpu = args.no_ops = True
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this build has no multi-GPU path (got --gpus {args.gpus}). "
+              "Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from __graft_entry__ import load_package
+    pkg = load_package()
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (torch.cuda.is_available() is False)", file=sys.stderr)
+        sys.exit(2)
+    pkg._native.impl()  # raises if the HIP library is missing: there is no fallback to measure
+    dev = torch.device("cuda:0")
+    rt = pkg.runtime
+    stream = torch.cuda.current_stream().cuda_stream
+
+    x, p, cfg = pkg.workloads.llama7b_layer(seed=0)
+    x = x.to(dev)
+    p = {k: v.to(dev) for k, v in p.items()}
+    plan, keep, flops, out = layer_plan(pkg, torch, dev, x, p, cfg)
+    tokens = x.shape[0] * x.shape[1]
+
+    for _ in range(args.warmup):
+        for _, call in plan:
+            call()
+    torch.cuda.synchronize()
+    # timed region: K steps, one event after every launch (recorded on the launch stream)
+    nev = args.steps * len(plan) + 1
+    events = [rt.createEvent() for _ in range(nev)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    rt.recordEvent(events[0], stream)
+    e = 1
+    for _ in range(args.steps):
+        for _, call in plan:
+            call()
+            rt.recordEvent(events[e], stream)
+            e += 1
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    elapsed = t1 - t0
+    per_op = {}
+    for si in range(args.steps):
+        for oi, (label, _) in enumerate(plan):
+            i = si * len(plan) + oi
+            per_op.setdefault(label, []).append(rt.eventElapsedTime(events[i], events[i + 1]) * 1e3)
+    for ev in events:
+        rt.destroyEvent(ev)
+    assert bool(torch.isfinite(out.float()).all()), "layer output is not finite"
+    ms_per_step = elapsed / args.steps * 1e3
+    value = tokens * args.steps / elapsed
+
+    gemm_labels = [l for l in flops]
+    gemm_time_us = sum(sum(per_op[l]) for l in gemm_labels) / args.steps          # per step, all 5 launches
+    gemm_flops = sum(flops.values())
+    achieved_tf = gemm_flops / (gemm_time_us * 1e-6) / 1e12
+    breakdown = {l: round(sum(v) / args.steps, 1) for l, v in per_op.items()}      # us per step (labels used twice are summed)
+    roofline = {"bound": "mfma", "kernel": "gemmMfmaKernel<bf16,256,256> (5 launches per step: qkv, o, gate, up, down)",
+                "achieved": round(achieved_tf, 1), "peak": MFMA_BF16_PEAK_TF, "unit": "TFLOP/s",
+                "frac": round(achieved_tf / MFMA_BF16_PEAK_TF, 4), "traffic": None,
+                "flops_per_step": gemm_flops, "avg_launch_us": round(gemm_time_us / 5, 1),
+                "per_gemm_TFLOPs": {l: round(flops[l] / (sum(per_op[l]) / args.steps * 1e-6) / 1e12, 1) for l in gemm_labels}}
+
+    result = {
+        "metric": "7B decoder-layer tokens/s bf16; % HBM roofline on DIOPI norm/attn ops",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "Llama-2-7B-shaped decoder layer prefill via the DIOPI C ABI: batch 4, seq 2048, hidden 4096, "
+                               "32 heads x 128, FFN 11008 SiLU-gated, RMSNorm eps 1e-5, rotary base 10000, causal attention, "
+                               "bf16 weights N(0,0.02) random init, activations N(0,1)",
+                   "tokens_per_step": tokens, "ops_per_step": len(plan)},
+        "roofline": roofline,
+        "layer_breakdown_us": breakdown,
+    }
+    if not args.no_ops:
+        result["ops"] = op_microbench(pkg, torch, dev, rt, stream)
+    if not args.no_cpu:
+        del plan, keep
+        torch.cuda.empty_cache()
+        result["cpu_baseline"] = cpu_baseline(pkg, torch)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

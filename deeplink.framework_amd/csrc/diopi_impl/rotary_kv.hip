@@ -19,7 +19,8 @@ template <typename T, typename CT, bool INTERLEAVED>
 __global__ __launch_bounds__(256) void rotaryVecKernel(T* __restrict__ out, const T* __restrict__ x,
                                                         const CT* __restrict__ cosT, const CT* __restrict__ sinT,
                                                         int64_t tokens, int heads, int d, int64_t tableRows,
-                                                        int tableCols, float sinSign) {
+                                                        int tableCols, float sinSign, int64_t xTok, int64_t xHead,
+                                                        int64_t oTok, int64_t oHead) {
   using V = typename Vec16<T>::type;
   constexpr int N = Vec16<T>::N;
   const int half = d / 2;
@@ -31,9 +32,10 @@ __global__ __launch_bounds__(256) void rotaryVecKernel(T* __restrict__ out, cons
     const int j = (int)(w % perHead);
     const int64_t th = w / perHead;
     const int64_t t = th / heads;
+    const int64_t hh = th - t * heads;
     const int64_t trow = t % tableRows;
-    const T* xr = x + th * d;
-    T* outr = out + th * d;
+    const T* xr = x + t * xTok + hh * xHead;
+    T* outr = out + t * oTok + hh * oHead;
     if constexpr (!INTERLEAVED) {
       V a = *reinterpret_cast<const V*>(xr + j * N);
       V b = *reinterpret_cast<const V*>(xr + half + j * N);
@@ -71,31 +73,37 @@ __global__ __launch_bounds__(256) void rotaryVecKernel(T* __restrict__ out, cons
 template <typename T, typename CT>
 __global__ __launch_bounds__(256) void rotaryScalarKernel(T* out, const T* x, const CT* cosT, const CT* sinT,
                                                            int64_t tokens, int heads, int d, int64_t tableRows,
-                                                           int tableCols, float sinSign, bool interleaved) {
+                                                           int tableCols, float sinSign, bool interleaved, int64_t xTok,
+                                                           int64_t xHead, int64_t oTok, int64_t oHead) {
   const int half = d / 2;
   const int64_t total = tokens * heads * half;
   for (int64_t w = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; w < total; w += (int64_t)gridDim.x * blockDim.x) {
     const int p = (int)(w % half);
     const int64_t th = w / half;
-    const int64_t trow = (th / heads) % tableRows;
+    const int64_t t = th / heads, hh = th - t * heads;
+    const int64_t trow = t % tableRows;
+    const T* xr = x + t * xTok + hh * xHead;
+    T* outr = out + t * oTok + hh * oHead;
     const int i0 = interleaved ? 2 * p : p, i1 = interleaved ? 2 * p + 1 : p + half;
     const int tc = (interleaved && tableCols == d) ? 2 * p : p;
     float c = static_cast<float>(cosT[trow * tableCols + tc]);
     float s = static_cast<float>(sinT[trow * tableCols + tc]) * sinSign;
-    float x0 = static_cast<float>(x[th * d + i0]), x1 = static_cast<float>(x[th * d + i1]);
-    out[th * d + i0] = static_cast<T>(x0 * c - x1 * s);
-    out[th * d + i1] = static_cast<T>(x0 * s + x1 * c);
+    float x0 = static_cast<float>(xr[i0]), x1 = static_cast<float>(xr[i1]);
+    outr[i0] = static_cast<T>(x0 * c - x1 * s);
+    outr[i1] = static_cast<T>(x0 * s + x1 * c);
   }
 }
 
 template <typename T, typename CT>
 static diopiError_t launchRotary(hipStream_t stream, const TensorView& out, const TensorView& x, const TensorView& c,
                                  const TensorView& s, int64_t tokens, int heads, int d, int64_t tableRows,
-                                 int tableCols, bool conj, bool interleaved) {
+                                 int tableCols, bool conj, bool interleaved, int64_t xTok, int64_t xHead, int64_t oTok,
+                                 int64_t oHead) {
   constexpr int N = Vec16<T>::N;
   const float sign = conj ? -1.f : 1.f;
   const int half = d / 2;
-  bool vec = x.aligned16() && out.aligned16() && (interleaved ? d % N == 0 : half % N == 0);
+  bool vec = x.aligned16() && out.aligned16() && (interleaved ? d % N == 0 : half % N == 0) && xTok % N == 0 &&
+             xHead % N == 0 && oTok % N == 0 && oHead % N == 0;
   if (vec) {
     int perHead = interleaved ? d / N : half / N;
     int64_t total = tokens * heads * perHead;
@@ -103,10 +111,10 @@ static diopiError_t launchRotary(hipStream_t stream, const TensorView& out, cons
     if (blocks > (1 << 20)) blocks = 1 << 20;
     if (interleaved) {
       hipLaunchKernelGGL((rotaryVecKernel<T, CT, true>), dim3((unsigned)blocks), dim3(256), 0, stream, out.ptr<T>(),
-                         x.ptr<T>(), c.ptr<CT>(), s.ptr<CT>(), tokens, heads, d, tableRows, tableCols, sign);
+                         x.ptr<T>(), c.ptr<CT>(), s.ptr<CT>(), tokens, heads, d, tableRows, tableCols, sign, xTok, xHead, oTok, oHead);
     } else {
       hipLaunchKernelGGL((rotaryVecKernel<T, CT, false>), dim3((unsigned)blocks), dim3(256), 0, stream, out.ptr<T>(),
-                         x.ptr<T>(), c.ptr<CT>(), s.ptr<CT>(), tokens, heads, d, tableRows, tableCols, sign);
+                         x.ptr<T>(), c.ptr<CT>(), s.ptr<CT>(), tokens, heads, d, tableRows, tableCols, sign, xTok, xHead, oTok, oHead);
     }
   } else {
     int64_t total = tokens * heads * half;
@@ -114,7 +122,7 @@ static diopiError_t launchRotary(hipStream_t stream, const TensorView& out, cons
     if (blocks > (1 << 20)) blocks = 1 << 20;
     hipLaunchKernelGGL((rotaryScalarKernel<T, CT>), dim3((unsigned)blocks), dim3(256), 0, stream, out.ptr<T>(),
                        x.ptr<T>(), c.ptr<CT>(), s.ptr<CT>(), tokens, heads, d, tableRows, tableCols, sign,
-                       interleaved);
+                       interleaved, xTok, xHead, oTok, oHead);
   }
   AMD_LAUNCH_CHECK();
   return diopiSuccess;
@@ -231,18 +239,40 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiRotaryEmbedd
   const int64_t tableRows = c.numel / tableCols;
   AMD_CHECK(tableRows > 0 && tokens % tableRows == 0,
             "diopiRotaryEmbedding: %ld table rows do not divide %ld tokens", (long)tableRows, (long)tokens);
-  TensorView cx, cc, cs;
-  AMD_TRY(makeContiguous(ctx, stream, x, &cx));
+  // x / out are addressed as [tokens, heads, d] with a token stride and a head stride, so the
+  // q and k slices of a fused QKV projection are rotated in place without a dense copy
+  auto tokenView = [&](const TensorView& t, int64_t* tokStride, int64_t* headStride) {
+    if (!(t.stride[t.ndim - 1] == 1 || d == 1)) return false;
+    *headStride = heads == 1 ? d : t.stride[t.ndim - 2];
+    int64_t n = 1, st = 0;
+    bool have = false;
+    for (int i = t.ndim - 3; i >= 0; --i) {
+      if (t.shape[i] == 1) continue;
+      if (!have) st = t.stride[i], have = true;
+      else if (t.stride[i] != st * n) return false;
+      n *= t.shape[i];
+    }
+    *tokStride = have ? st : (int64_t)heads * d;
+    return true;
+  };
+  TensorView cx = x, cc, cs;
+  int64_t xTok, xHead, oTok, oHead;
+  if (!tokenView(x, &xTok, &xHead)) {
+    AMD_TRY(makeContiguous(ctx, stream, x, &cx));
+    xTok = (int64_t)heads * d, xHead = d;
+  }
   AMD_TRY(makeContiguous(ctx, stream, c, &cc));
   AMD_TRY(makeContiguous(ctx, stream, s, &cs));
   TensorView cout = out;
-  bool outTemp = !out.isContiguous();
+  bool outTemp = !tokenView(out, &oTok, &oHead);
   if (outTemp) {
     diopiTensorHandle_t th;
     AMD_TRY(requireTensor(ctx, out.shape, out.ndim, out.dtype, &th, &cout));
+    oTok = (int64_t)heads * d, oHead = d;
   }
   diopiError_t err;
-#define ROTARY(T, CT) err = launchRotary<T, CT>(stream, cout, cx, cc, cs, tokens, heads, d, tableRows, tableCols, conj, interleaved)
+#define ROTARY(T, CT) \
+  err = launchRotary<T, CT>(stream, cout, cx, cc, cs, tokens, heads, d, tableRows, tableCols, conj, interleaved, xTok, xHead, oTok, oHead)
   if (x.dtype == diopi_dtype_bfloat16 && c.dtype == diopi_dtype_bfloat16) ROTARY(bf16_t, bf16_t);
   else if (x.dtype == diopi_dtype_bfloat16 && c.dtype == diopi_dtype_float32) ROTARY(bf16_t, float);
   else if (x.dtype == diopi_dtype_float16 && c.dtype == diopi_dtype_float16) ROTARY(half_t, half_t);

@@ -30,7 +30,8 @@ namespace amd {
 constexpr float kLog2eTA = 1.4426950408889634f;
 constexpr int kTaWaves = 4;
 constexpr int kTaUnroll = 4;
-constexpr int kTaChunk = 512;  // tokens of one sequence handled by one workgroup
+constexpr int kTaChunk = 512;  // tokens of one sequence handled by one workgroup (grows for very long sequences)
+constexpr int kTaMaxSplit = 64; // the merge step handles one split per lane
 
 __device__ __forceinline__ int64_t ldIndex(const void* p, int64_t i, bool is64) {
   return is64 ? reinterpret_cast<const int64_t*>(p)[i] : static_cast<int64_t>(reinterpret_cast<const int32_t*>(p)[i]);
@@ -48,7 +49,7 @@ struct TaArgs {
   int64_t kSlotStride, kHeadStride, vSlotStride, vHeadStride;  // elements
   int64_t qBatchStride, qHeadStride;
   int64_t slots;
-  int heads, kvHeads, d, maxLen, nsplit;
+  int heads, kvHeads, d, maxLen, nsplit, chunk;
   float scaleLog2e;  // log2(e) / sqrt(d)
 };
 
@@ -76,9 +77,9 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int sub = lane % LPT, grp = lane / LPT;
   const int len = (int)ldIndex(a.bLen, b, a.len64);
-  const int begin = split * kTaChunk;
+  const int begin = split * a.chunk;
   if (begin >= len && !(split == 0)) return;  // nothing to do; split 0 still writes zeros for len == 0
-  const int end = min(len, begin + kTaChunk);
+  const int end = min(len, begin + a.chunk);
   const int kvh = h / (a.heads / a.kvHeads);
   const int64_t locBase = (int64_t)b * a.locRowStride + (a.maxLen - len);
 
@@ -194,33 +195,33 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   }
 }
 
-// out[b,h,:] = merge over the chunks that hold tokens. One wave per (b,h), lane = element.
+// out[b,h,:] = merge over the chunks that hold tokens. One wave per (b,h): lane s loads the
+// (max, sum) of split s, a butterfly gives the global max and normaliser, then every lane
+// combines its elements over the splits with independent loads.
 template <typename T>
 __global__ __launch_bounds__(256) void decodeMergeKernel(T* __restrict__ out, const float* __restrict__ partial,
                                                           const void* bLen, bool len64, int64_t pairs, int heads,
-                                                          int d, int nsplit) {
+                                                          int d, int nsplit, int chunk) {
   const int lane = threadIdx.x & 63;
   const int64_t pair = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (pair >= pairs) return;
   const int b = (int)(pair / heads);
   const int len = (int)ldIndex(bLen, b, len64);
-  const int used = len <= 0 ? 1 : min(nsplit, (len + kTaChunk - 1) / kTaChunk);
+  const int used = len <= 0 ? 1 : min(nsplit, (len + chunk - 1) / chunk);
   const float* src = partial + pair * nsplit * (2 + d);
-  float m = -INFINITY;
-  for (int s = 0; s < used; ++s) m = fmaxf(m, src[s * (2 + d)]);
-  float l = 0.f;
-  for (int s = 0; s < used; ++s) {
-    float ms = src[s * (2 + d)];
-    l += (ms == -INFINITY) ? 0.f : src[s * (2 + d) + 1] * exp2f(ms - m);
+  float ms = -INFINITY, ls = 0.f;
+  if (lane < used) {
+    ms = src[lane * (2 + d)];
+    ls = src[lane * (2 + d) + 1];
   }
-  const float inv = l > 0.f ? 1.f / l : 0.f;
+  const float m = waveMax(ms);
+  float wgt = (ms == -INFINITY) ? 0.f : exp2f(ms - m);
+  const float l = waveSum(ls * wgt);
+  wgt *= l > 0.f ? 1.f / l : 0.f;
   for (int e = lane; e < d; e += 64) {
     float acc = 0.f;
-    for (int s = 0; s < used; ++s) {
-      float ms = src[s * (2 + d)];
-      if (ms != -INFINITY) acc += src[s * (2 + d) + 2 + e] * exp2f(ms - m);
-    }
-    out[pair * d + e] = static_cast<T>(acc * inv);
+    for (int s = 0; s < used; ++s) acc += __shfl(wgt, s, 64) * src[s * (2 + d) + 2 + e];
+    out[pair * d + e] = static_cast<T>(acc);
   }
 }
 
@@ -236,9 +237,9 @@ __global__ __launch_bounds__(256) void tokenLogitsKernel(TaArgs a, OT* __restric
   const int sub = lane % LPT, grp = lane / LPT;
   const int len = (int)ldIndex(a.bLen, b, a.len64);
   const int64_t start = ldIndex(a.bStart, b, a.start64);
-  const int begin = blockIdx.y * kTaChunk;
+  const int begin = blockIdx.y * a.chunk;
   if (begin >= len) return;
-  const int end = min(len, begin + kTaChunk);
+  const int end = min(len, begin + a.chunk);
   const int kvh = h / (a.heads / a.kvHeads);
   const int64_t locBase = (int64_t)b * a.locRowStride + (a.maxLen - len);
   float qf[N];
@@ -427,6 +428,9 @@ static diopiError_t fillArgs(const TaViews& t, bool needK, bool needV, int maxLe
   a->d = (int)q.shape[2];
   a->maxLen = maxLen;
   a->nsplit = 1;
+  // at most kTaMaxSplit chunks per sequence; chunks stay a multiple of 64 tokens
+  a->chunk = kTaChunk;
+  if ((int64_t)maxLen > (int64_t)kTaChunk * kTaMaxSplit) a->chunk = (int)(ceilDiv(ceilDiv(maxLen, kTaMaxSplit), 64) * 64);
   a->scaleLog2e = kLog2eTA / sqrtf((float)q.shape[2]);
   return diopiSuccess;
 }
@@ -470,7 +474,7 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiTokenDecodeA
             "token attention: out must be a dense tensor shaped like q");
   const int64_t batch = t.q.shape[0];
   if (batch == 0 || t.q.numel == 0) return diopiSuccess;
-  a.nsplit = (int)std::max<int64_t>(1, ceilDiv(maxInputLen, kTaChunk));
+  a.nsplit = (int)std::max<int64_t>(1, ceilDiv(maxInputLen, a.chunk));
   AMD_CHECK(batch <= 65535 && a.nsplit <= 65535, "token attention: batch %ld / splits %d exceed the grid limits", (long)batch,
             a.nsplit);
   float* partial = nullptr;
@@ -491,7 +495,7 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiTokenDecodeA
     dim3 mgrid((unsigned)ceilDiv(pairs, 4)), mblock(256);
 #define MERGE_CALL(T, LPT)                                                                                       \
   hipLaunchKernelGGL((decodeMergeKernel<T>), mgrid, mblock, 0, stream, out.ptr<T>(), partial, a.bLen, a.len64, pairs, \
-                     a.heads, a.d, a.nsplit)
+                     a.heads, a.d, a.nsplit, a.chunk)
     TA_DISPATCH(t.q.dtype, bytes, MERGE_CALL);
 #undef MERGE_CALL
     AMD_LAUNCH_CHECK();
@@ -520,7 +524,7 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiTokenAttenti
             "token attention: attention_out dtype must be float32 or the q dtype");
   const int64_t batch = t.q.shape[0];
   if (batch == 0 || maxInputLen == 0) return diopiSuccess;
-  int nchunk = (int)ceilDiv(maxInputLen, kTaChunk);
+  int nchunk = (int)ceilDiv(maxInputLen, a.chunk);
   AMD_CHECK(batch <= 65535 && nchunk <= 65535, "token attention: grid limits exceeded");
   dim3 grid(a.heads, nchunk, (unsigned)batch), block(256);
   const int64_t bytes = t.q.shape[2] * t.q.itemsize;

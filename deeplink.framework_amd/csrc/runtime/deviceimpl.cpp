@@ -136,6 +136,7 @@ OpStatus mallocDevice(void** p, size_t nbytes, bool throwExcepion) {
     *p = nullptr;
     return OpStatus::ERR_NOMEM;
   }
+  (void)hipGetLastError();
   throw std::runtime_error("hipMalloc failed, ret = " + std::to_string(static_cast<int>(r)) +
                            " size = " + std::to_string(nbytes));
 }

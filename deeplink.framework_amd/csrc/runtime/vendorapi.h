@@ -15,6 +15,7 @@ namespace dipu {
   {                                                                                                  \
     hipError_t ret_ = (Expr);                                                                        \
     if (ret_ != hipSuccess) {                                                                        \
+      (void)hipGetLastError(); /* the exception carries the failure; leave no sticky error behind */  \
       throw std::runtime_error(std::string("call hip error, expr = " #Expr ", ret = ") +             \
                                std::to_string(static_cast<int>(ret_)) + " (" + hipGetErrorString(ret_) + ")"); \
     }                                                                                                \

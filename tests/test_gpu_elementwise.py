@@ -218,7 +218,8 @@ def test_rotary_preserves_pair_norms_at_full_size(ops, dev, pkg):
     assert float(((n_in - n_out).abs() / (n_in + 1e-3)).max()) < 5e-2
     assert_exact(y[0], x[0].cpu())      # position 0 is the identity, bit for bit
     back = ops.rotary_emb(y, cos, sin, conj=True)
-    assert_half(back, x.cpu())
+    # two bf16 roundings and bf16 tables (cos^2 + sin^2 is 1 only to 2^-8): twice the single-op bound
+    assert_half(back, x.cpu(), rel=4e-2, abs_=2e-2)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.int8])
