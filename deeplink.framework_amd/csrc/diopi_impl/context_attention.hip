@@ -16,7 +16,7 @@
 //     K-slots of a lane, for a fixed permutation of the 16 keys of the step. The A operand
 //     (V^T) is read from an LDS copy of V stored transposed [d][keys] with exactly that
 //     permutation: two 8-byte reads per operand.
-//   * K tile rows in LDS are XOR-swizzled per 16-byte chunk (conflict-free ds_read_b128);
+//   * K tile rows in LDS are XOR-swizzled per 16-byte chunk (measured conflict-free ds_read_b128);
 //     V is transposed on the way into LDS (4 keys x 8 d per lane, 8-byte stores).
 //   * two LDS stages, register prefetch of the next tile, one barrier per tile; the heaviest
 //     query blocks (end of the sequence) are scheduled first.
@@ -68,6 +68,14 @@ struct CaMfma<half_t> {
   }
 };
 
+// XOR applied to the 16-byte chunk index of K row `key` in LDS; the patterns are the ones that
+// measure conflict-free for ds_read_b128 with 32 consecutive rows per half-wave: 256-byte rows
+// (d = 128) need key & 15, 128-byte rows (d = 64) need (key >> 1) & 7.
+template <int D>
+__device__ __forceinline__ int kSwizzle(int key) {
+  return D == 128 ? (key & 15) : ((key >> 1) & 7);
+}
+
 constexpr int kCaBQ = 128, kCaBKV = 64, kCaVtStride = 68;  // V^T rows padded to 68 keys (136 bytes)
 
 template <typename T, int D>
@@ -115,7 +123,7 @@ __global__ __launch_bounds__(256) void contextAttnMfmaKernel(CaArgs a) {
     int chunk = tid + 256 * i;
     int key = chunk / CPR, c = chunk % CPR;
     kKey[i] = key;
-    kOff[i] = key * D + ((c ^ (key & 7)) << 3);
+    kOff[i] = key * D + ((c ^ kSwizzle<D>(key)) << 3);
   }
   const int cK = (tid % CPR) * 8;
   const bool vActive = tid < 16 * (D / 8);
@@ -180,7 +188,7 @@ __global__ __launch_bounds__(256) void contextAttnMfmaKernel(CaArgs a) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           const int chunk = ks * 2 + half;
-          Frag kf = *reinterpret_cast<const Frag*>(k + key * D + ((chunk ^ (key & 7)) << 3));
+          Frag kf = *reinterpret_cast<const Frag*>(k + key * D + ((chunk ^ kSwizzle<D>(key)) << 3));
           s[kt2] = CaMfma<T>::run(kf, qf[ks], s[kt2]);
         }
       }

@@ -12,7 +12,7 @@
 //     stage while tile k is being multiplied, tile k+2 is already in flight from HBM; one
 //     barrier per K tile;
 //   * LDS rows are 128 bytes (64 elements) with the 16-byte chunk index XOR-swizzled by
-//     (row & 7): both the 16-byte stores of the staging step and the ds_read_b128 operand
+//     ((row >> 1) & 7): both the 16-byte stores of the staging step and the ds_read_b128 operand
 //     fetches (32 consecutive rows, same logical chunk) are bank-conflict free;
 //   * workgroup ids are remapped so that each of the 8 XCDs (own L2 each) works on a
 //     contiguous band of tiles, walked in groups of 8 tile-rows to reuse A and B from L2;
@@ -24,6 +24,7 @@
 // FMA engine: fp32 (and any shape/stride/alignment the MFMA engine rejects): 64x64 LDS
 // tiles, 4x4 outputs per lane, fp32 accumulate.
 #include <algorithm>
+#include <type_traits>
 
 #include "gemm.hpp"
 
@@ -105,14 +106,14 @@ __global__ __launch_bounds__(256) void gemmMfmaKernel(MfmaArgs g) {
     int row = (tid >> 3) + 32 * i;
     int grow = min(tm * BM + row, g.M - 1);
     aPtr[i] = A + (int64_t)grow * g.lda + c8;
-    aOff[i] = row * kBK + (((tid & 7) ^ (row & 7)) << 3);
+    aOff[i] = row * kBK + (((tid & 7) ^ ((row >> 1) & 7)) << 3);
   }
 #pragma unroll
   for (int i = 0; i < B_CH; ++i) {
     int row = (tid >> 3) + 32 * i;
     int grow = min(tn * BN + row, g.N - 1);
     bPtr[i] = B + (int64_t)grow * g.ldb + c8;
-    bOff[i] = row * kBK + (((tid & 7) ^ (row & 7)) << 3);
+    bOff[i] = row * kBK + (((tid & 7) ^ ((row >> 1) & 7)) << 3);
   }
   Frag ra[A_CH], rb[B_CH];
   const int nK = (g.K + kBK - 1) / kBK;
@@ -163,12 +164,12 @@ __global__ __launch_bounds__(256) void gemmMfmaKernel(MfmaArgs g) {
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
         int row = i * 32 + frow;
-        fa[i] = *reinterpret_cast<const Frag*>(a + row * kBK + ((chunk ^ (row & 7)) << 3));
+        fa[i] = *reinterpret_cast<const Frag*>(a + row * kBK + ((chunk ^ ((row >> 1) & 7)) << 3));
       }
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         int row = j * 32 + frow;
-        fb[j] = *reinterpret_cast<const Frag*>(b + row * kBK + ((chunk ^ (row & 7)) << 3));
+        fb[j] = *reinterpret_cast<const Frag*>(b + row * kBK + ((chunk ^ ((row >> 1) & 7)) << 3));
       }
 #pragma unroll
       for (int i = 0; i < TM; ++i)
@@ -183,6 +184,206 @@ __global__ __launch_bounds__(256) void gemmMfmaKernel(MfmaArgs g) {
   }
 
   // ---- epilogue
+  T* out = reinterpret_cast<T*>(g.out) + (int64_t)batch * g.sOb;
+  const T* cin = g.Cin ? reinterpret_cast<const T*>(g.Cin) + (int64_t)batch * g.sCb : nullptr;
+  const T* bias = reinterpret_cast<const T*>(g.bias);
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int col = tn * BN + wn * WN + j * 32 + frow;
+    if (col >= g.N) continue;
+    const float bv = bias ? static_cast<float>(bias[col]) : 0.f;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int rbase = tm * BM + wm * WM + i * 32 + fhalf * 4;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = rbase + (r >> 2) * 8 + (r & 3);
+        if (row < g.M) {
+          float v = acc[i][j][r] * g.alpha + bv;
+          if (cin) v += g.beta * static_cast<float>(cin[(int64_t)row * g.sCm + (int64_t)col * g.sCn]);
+          out[(int64_t)row * g.ldo + col] = static_cast<T>(v);
+        }
+      }
+    }
+  }
+}
+
+// ------------------------------------------------- software-pipelined 256x256 ---
+// Same tiling and LDS layout as gemmMfmaKernel<T,256,256>, for K a multiple of 64 with at
+// least two K tiles, with the instruction stream arranged by hand so the single wave per
+// SIMD never waits on LDS or HBM inside the K loop:
+//   k-step 0: MFMAs of step 0 | operand fetches of step 1 | LDS stores of the next A tile
+//   k-step 1: MFMAs of step 1 | operand fetches of step 2 | LDS stores of the next B tile
+//   k-step 2: MFMAs of step 2 | operand fetches of step 3 | HBM loads of the tile after next
+//   barrier (LDS only: the HBM loads stay in flight across it)
+//   k-step 3: MFMAs of step 3 | operand fetches of step 0 of the next tile
+// Operand fragments are double-buffered in registers; sched_group_barrier pins the
+// MFMA / LDS / VMEM interleave inside each k-step.
+__device__ __forceinline__ void ldsBarrier() {
+  // wait for this wave's LDS traffic only (lgkmcnt(0)); outstanding global loads keep flying
+  __builtin_amdgcn_s_waitcnt(0xc07f);
+  __builtin_amdgcn_s_barrier();
+}
+
+#define SGB_MFMA(n) __builtin_amdgcn_sched_group_barrier(0x008, n, 0)
+#define SGB_DSRD(n) __builtin_amdgcn_sched_group_barrier(0x100, n, 0)
+#define SGB_DSWR(n) __builtin_amdgcn_sched_group_barrier(0x200, n, 0)
+#define SGB_VMRD(n) __builtin_amdgcn_sched_group_barrier(0x020, n, 0)
+
+template <typename T>
+__global__ __launch_bounds__(256) void gemmMfmaPipelinedKernel(MfmaArgs g) {
+  using Frag = typename MfmaOp<T>::Frag;
+  constexpr int BM = 256, BN = 256, WM = 128, WN = 128, TM = 4, TN = 4, CH = 8;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  T* sA = reinterpret_cast<T*>(smem);  // [2][BM][64]
+  T* sB = sA + 2 * BM * kBK;           // [2][BN][64]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  int tm, tn;
+  {
+    const int total = g.tilesM * g.tilesN;
+    const int pid = blockIdx.x;
+    const int xcd = pid & 7, idx = pid >> 3;
+    const int q = total >> 3, r = total & 7;
+    const int logical = xcd * q + min(xcd, r) + idx;
+    constexpr int GROUP = 8;
+    const int width = GROUP * g.tilesN;
+    const int group = logical / width;
+    const int first = group * GROUP;
+    const int gsize = min(g.tilesM - first, GROUP);
+    const int in = logical - group * width;
+    tm = first + in % gsize;
+    tn = in / gsize;
+  }
+  const int batch = blockIdx.z;
+  const T* A = reinterpret_cast<const T*>(g.A) + (int64_t)batch * g.sAb;
+  const T* B = reinterpret_cast<const T*>(g.B) + (int64_t)batch * g.sBb;
+  const T* aPtr[CH];
+  const T* bPtr[CH];
+  const int c8 = (tid & 7) * 8;
+  const int srow = tid >> 3;  // staging row of chunk 0; chunk i is 32 rows further
+  const int sOff = srow * kBK + (((tid & 7) ^ ((srow >> 1) & 7)) << 3);  // rows 32 apart share the swizzle
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    aPtr[i] = A + (int64_t)min(tm * BM + srow + 32 * i, g.M - 1) * g.lda + c8;
+    bPtr[i] = B + (int64_t)min(tn * BN + srow + 32 * i, g.N - 1) * g.ldb + c8;
+  }
+  Frag ra[CH], rb[CH];
+  const int nK = g.K / kBK;
+
+  const int frow = lane & 31, fhalf = lane >> 5;
+  const int swz = (frow >> 1) & 7;
+  int kx[4];  // swizzled element offset of this lane's chunk for each k-step
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) kx[ks] = ((2 * ks + fhalf) ^ swz) << 3;
+  const int aBase = (wm * WM + frow) * kBK, bBase = (wn * WN + frow) * kBK;
+
+  Frag fa[2][TM], fb[2][TN];
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  auto gload = [&](int kt) {
+    const int k0 = kt * kBK;
+#pragma unroll
+    for (int i = 0; i < CH; ++i) ra[i] = *reinterpret_cast<const Frag*>(aPtr[i] + k0);
+#pragma unroll
+    for (int i = 0; i < CH; ++i) rb[i] = *reinterpret_cast<const Frag*>(bPtr[i] + k0);
+  };
+  auto swriteA = [&](int stage) {
+    T* a = sA + stage * BM * kBK + sOff;
+#pragma unroll
+    for (int i = 0; i < CH; ++i) *reinterpret_cast<Frag*>(a + i * 32 * kBK) = ra[i];
+  };
+  auto swriteB = [&](int stage) {
+    T* b = sB + stage * BN * kBK + sOff;
+#pragma unroll
+    for (int i = 0; i < CH; ++i) *reinterpret_cast<Frag*>(b + i * 32 * kBK) = rb[i];
+  };
+  auto lfrag = [&](int stage, int ks, int buf) {
+    const T* a = sA + stage * BM * kBK + aBase + kx[ks];
+    const T* b = sB + stage * BN * kBK + bBase + kx[ks];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fa[buf][i] = *reinterpret_cast<const Frag*>(a + i * 32 * kBK);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fb[buf][j] = *reinterpret_cast<const Frag*>(b + j * 32 * kBK);
+  };
+  auto mma = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[i][j] = MfmaOp<T>::run(fa[buf][i], fb[buf][j], acc[i][j]);
+  };
+
+  gload(0);
+  swriteA(0);
+  swriteB(0);
+  gload(1);
+  ldsBarrier();
+  lfrag(0, 0, 0);
+
+  auto iter = [&](auto hasNext, auto hasNext2, int kt) {
+    constexpr bool kNext = decltype(hasNext)::value, kNext2 = decltype(hasNext2)::value;
+    const int cur = kt & 1;
+    // ---- k-step 0
+    __builtin_amdgcn_sched_barrier(0);
+    lfrag(cur, 1, 1);
+    if constexpr (kNext) swriteA(cur ^ 1);
+    mma(0);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      SGB_MFMA(1);
+      SGB_DSRD(1);
+      SGB_MFMA(1);
+      if constexpr (kNext) SGB_DSWR(1);
+    }
+    // ---- k-step 1
+    __builtin_amdgcn_sched_barrier(0);
+    lfrag(cur, 2, 0);
+    if constexpr (kNext) swriteB(cur ^ 1);
+    mma(1);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      SGB_MFMA(1);
+      SGB_DSRD(1);
+      SGB_MFMA(1);
+      if constexpr (kNext) SGB_DSWR(1);
+    }
+    // ---- k-step 2
+    __builtin_amdgcn_sched_barrier(0);
+    lfrag(cur, 3, 1);
+    if constexpr (kNext2) gload(kt + 2);
+    mma(0);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      SGB_MFMA(1);
+      SGB_DSRD(1);
+      SGB_MFMA(1);
+      if constexpr (kNext2) SGB_VMRD(2);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    ldsBarrier();
+    // ---- k-step 3
+    if constexpr (kNext) lfrag(cur ^ 1, 0, 0);
+    mma(1);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      SGB_MFMA(2);
+      if constexpr (kNext) SGB_DSRD(1);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  using std::false_type;
+  using std::true_type;
+  for (int kt = 0; kt < nK - 2; ++kt) iter(true_type{}, true_type{}, kt);
+  iter(true_type{}, false_type{}, nK - 2);
+  iter(false_type{}, false_type{}, nK - 1);
+
+  // ---- epilogue (same as the generic kernel)
   T* out = reinterpret_cast<T*>(g.out) + (int64_t)batch * g.sOb;
   const T* cin = g.Cin ? reinterpret_cast<const T*>(g.Cin) + (int64_t)batch * g.sCb : nullptr;
   const T* bias = reinterpret_cast<const T*>(g.bias);
@@ -332,6 +533,28 @@ static diopiError_t launchMfma(hipStream_t stream, const GemmProblem& p) {
   return diopiSuccess;
 }
 
+template <typename T>
+static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p) {
+  MfmaArgs g;
+  g.A = p.A, g.B = p.B, g.out = p.out, g.Cin = p.Cin, g.bias = p.bias;
+  g.sAb = p.sAb, g.lda = p.sAm, g.sBb = p.sBb, g.ldb = p.sBn, g.sOb = p.sOb, g.ldo = p.sOm;
+  g.sCb = p.sCb, g.sCm = p.sCm, g.sCn = p.sCn;
+  g.M = (int)p.M, g.N = (int)p.N, g.K = (int)p.K;
+  g.tilesM = (int)ceilDiv(p.M, 256), g.tilesN = (int)ceilDiv(p.N, 256);
+  g.alpha = p.alpha, g.beta = p.beta;
+  constexpr size_t lds = 2 * (size_t)(256 + 256) * kBK * sizeof(T);
+  static bool attrSet = false;
+  if (!attrSet) {
+    AMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemmMfmaPipelinedKernel<T>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attrSet = true;
+  }
+  dim3 grid((unsigned)(g.tilesM * g.tilesN), 1, (unsigned)p.batch);
+  hipLaunchKernelGGL((gemmMfmaPipelinedKernel<T>), grid, dim3(256), lds, stream, g);
+  AMD_LAUNCH_CHECK();
+  return diopiSuccess;
+}
+
 static bool mult8(int64_t v) { return (v & 7) == 0; }
 static bool ptr16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
@@ -369,6 +592,9 @@ diopiError_t runGemm(diopiContextHandle_t ctx, hipStream_t stream, GemmProblem p
       p.B = ws, p.sBk = 1, p.sBn = p.K, p.sBb = (sbb == 0) ? 0 : p.N * p.K;
     }
     const bool big = ceilDiv(p.M, 256) * ceilDiv(p.N, 256) * p.batch >= 200;
+    if (big && p.K % kBK == 0 && p.K >= 2 * kBK) {
+      return p.dtype == diopi_dtype_bfloat16 ? launchMfmaPipelined<bf16_t>(stream, p) : launchMfmaPipelined<half_t>(stream, p);
+    }
     if (p.dtype == diopi_dtype_bfloat16) {
       return big ? launchMfma<bf16_t, 256, 256>(stream, p) : launchMfma<bf16_t, 128, 128>(stream, p);
     }
