@@ -18,7 +18,10 @@
 //     permutation: two 8-byte reads per operand.
 //   * K tile rows in LDS are XOR-swizzled per 16-byte chunk (measured conflict-free ds_read_b128);
 //     V is transposed on the way into LDS (4 keys x 8 d per lane, 8-byte stores).
-//   * two LDS stages, register prefetch of the next tile, one barrier per tile; the heaviest
+//   * two workgroups per CU (<= 256 registers per lane) so one wave's softmax VALU work overlaps
+//     another's MFMAs; exp2 is the bare hardware instruction fed by one FMA; the O^T rescale is
+//     skipped while the running max does not move;
+//   * two LDS stages, register prefetch of the next tile, one LDS-only barrier per tile; the heaviest
 //     query blocks (end of the sequence) are scheduled first.
 //   * the epilogue transposes O^T through LDS so global stores are 16-byte and coalesced.
 //
@@ -79,7 +82,7 @@ __device__ __forceinline__ int kSwizzle(int key) {
 constexpr int kCaBQ = 128, kCaBKV = 64, kCaVtStride = 68;  // V^T rows padded to 68 keys (136 bytes)
 
 template <typename T, int D>
-__global__ __launch_bounds__(256) void contextAttnMfmaKernel(CaArgs a) {
+__global__ __launch_bounds__(256, 2) void contextAttnMfmaKernel(CaArgs a) {
   using Frag = typename CaMfma<T>::Frag;
   using Half = typename CaMfma<T>::Half;
   constexpr int KS = D / 16;        // MFMA k-steps over the head dim
@@ -168,10 +171,15 @@ __global__ __launch_bounds__(256) void contextAttnMfmaKernel(CaArgs a) {
   float m = -INFINITY, l = 0.f;
   const float scale2 = a.scale * kLog2eCA;
 
+  // barrier on LDS traffic only: the global loads of the tile after next stay in flight across it
+  auto ldsBarrier = []() {
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_s_barrier();
+  };
   gload(0);
   swrite(0);
   if (ntiles > 1) gload(1);
-  __syncthreads();
+  ldsBarrier();
 
   for (int t = 0; t < ntiles; ++t) {
     const int cur = t & 1;
@@ -193,39 +201,46 @@ __global__ __launch_bounds__(256) void contextAttnMfmaKernel(CaArgs a) {
         }
       }
       // ---- online softmax for this lane's query over the 64 keys of the tile
+      // (m and mn are kept in the scaled log2 domain: score * scale * log2 e)
       const bool needMask = (k0 + kCaBKV - 1 > q0 + wave * 32) || (k0 + kCaBKV > len);
+      if (needMask) {  // wave-uniform: only the diagonal and the last tile pay for masking
+#pragma unroll
+        for (int kt2 = 0; kt2 < 2; ++kt2)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            int kj = k0 + kt2 * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+            if (kj > qiC || kj >= len) s[kt2][r] = -INFINITY;
+          }
+      }
       float mt = -INFINITY;
 #pragma unroll
       for (int kt2 = 0; kt2 < 2; ++kt2)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          float v = s[kt2][r] * scale2;
-          if (needMask) {
-            int kj = k0 + kt2 * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-            if (kj > qiC || kj >= len) v = -INFINITY;
-          }
-          s[kt2][r] = v;
-          mt = fmaxf(mt, v);
-        }
-      mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+        for (int r = 0; r < 16; ++r) mt = fmaxf(mt, s[kt2][r]);
+      mt = fmaxf(mt, __shfl_xor(mt, 32, 64)) * scale2;  // scale2 > 0, so the max commutes with the scaling
       const float mn = fmaxf(m, mt);  // key 0 is visible to every query, so mn is finite from tile 0 on
-      const float corr = exp2f(m - mn);
       float ps = 0.f;
 #pragma unroll
       for (int kt2 = 0; kt2 < 2; ++kt2)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          float p = exp2f(s[kt2][r] - mn);
+          // one fused multiply-add and one hardware exp2 per score; masked scores give exp2(-inf) = 0
+          float p = __builtin_amdgcn_exp2f(fmaf(s[kt2][r], scale2, -mn));
           s[kt2][r] = p;
           ps += p;
         }
       ps += __shfl_xor(ps, 32, 64);
-      l = l * corr + ps;
-      m = mn;
+      // the running max rarely moves after the first tiles: rescale only when some lane needs it
+      if (__builtin_amdgcn_ballot_w64(mn > m) != 0) {
+        const float corr = __builtin_amdgcn_exp2f(m - mn);
+        l *= corr;
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
+        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o[dt][r] *= corr;
+          for (int r = 0; r < 16; ++r) o[dt][r] *= corr;
+        m = mn;
+      }
+      l += ps;
       // ---- O^T += V^T . P^T
 #pragma unroll
       for (int kt2 = 0; kt2 < 2; ++kt2)
@@ -251,7 +266,7 @@ __global__ __launch_bounds__(256) void contextAttnMfmaKernel(CaArgs a) {
       swrite(cur ^ 1);
       if (t + 2 < ntiles) gload(t + 2);
     }
-    __syncthreads();
+    ldsBarrier();
   }
 
   // ---- epilogue: O^T (lane = query) -> LDS [query][d] -> coalesced 16-byte stores

@@ -209,9 +209,9 @@ __global__ __launch_bounds__(256) void gemmMfmaKernel(MfmaArgs g) {
 }
 
 // ------------------------------------------------- software-pipelined 256x256 ---
-// Same tiling and LDS layout as gemmMfmaKernel<T,256,256>, for K a multiple of 64 with at
-// least two K tiles, with the instruction stream arranged by hand so the single wave per
-// SIMD never waits on LDS or HBM inside the K loop:
+// Same macro tile and LDS layout as gemmMfmaKernel<T,256,256>, for K a multiple of 64 with at
+// least two K tiles, with the instruction stream of every wave arranged by hand so it does
+// not wait on LDS or HBM inside the K loop:
 //   k-step 0: MFMAs of step 0 | operand fetches of step 1 | LDS stores of the next A tile
 //   k-step 1: MFMAs of step 1 | operand fetches of step 2 | LDS stores of the next B tile
 //   k-step 2: MFMAs of step 2 | operand fetches of step 3 | HBM loads of the tile after next
@@ -230,15 +230,21 @@ __device__ __forceinline__ void ldsBarrier() {
 #define SGB_DSWR(n) __builtin_amdgcn_sched_group_barrier(0x200, n, 0)
 #define SGB_VMRD(n) __builtin_amdgcn_sched_group_barrier(0x020, n, 0)
 
+// 8 waves (2 x 4, wave tile 128 x 64): two waves per SIMD, so one wave's LDS / VMEM issue
+// overlaps the other's MFMAs; measured faster than 4 waves of 128 x 128 and 16 of 64 x 64.
+constexpr int kPipeWavesM = 2, kPipeWavesN = 4, kPipeThreads = kPipeWavesM * kPipeWavesN * 64;
+
 template <typename T>
-__global__ __launch_bounds__(256) void gemmMfmaPipelinedKernel(MfmaArgs g) {
+__global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs g) {
   using Frag = typename MfmaOp<T>::Frag;
-  constexpr int BM = 256, BN = 256, WM = 128, WN = 128, TM = 4, TN = 4, CH = 8;
+  constexpr int BM = 256, BN = 256, WM = BM / kPipeWavesM, WN = BN / kPipeWavesN, TM = WM / 32, TN = WN / 32;
+  constexpr int CH = 2048 / kPipeThreads;  // 16-byte chunks per thread per operand tile
+  constexpr int RS = kPipeThreads / 8;     // rows covered by one pass of the workgroup
   extern __shared__ __attribute__((aligned(16))) char smem[];
   T* sA = reinterpret_cast<T*>(smem);  // [2][BM][64]
   T* sB = sA + 2 * BM * kBK;           // [2][BN][64]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / kPipeWavesN, wn = wave % kPipeWavesN;
   int tm, tn;
   {
     const int total = g.tilesM * g.tilesN;
@@ -265,8 +271,8 @@ __global__ __launch_bounds__(256) void gemmMfmaPipelinedKernel(MfmaArgs g) {
   const int sOff = srow * kBK + (((tid & 7) ^ ((srow >> 1) & 7)) << 3);  // rows 32 apart share the swizzle
 #pragma unroll
   for (int i = 0; i < CH; ++i) {
-    aPtr[i] = A + (int64_t)min(tm * BM + srow + 32 * i, g.M - 1) * g.lda + c8;
-    bPtr[i] = B + (int64_t)min(tn * BN + srow + 32 * i, g.N - 1) * g.ldb + c8;
+    aPtr[i] = A + (int64_t)min(tm * BM + srow + RS * i, g.M - 1) * g.lda + c8;
+    bPtr[i] = B + (int64_t)min(tn * BN + srow + RS * i, g.N - 1) * g.ldb + c8;
   }
   Frag ra[CH], rb[CH];
   const int nK = g.K / kBK;
@@ -297,12 +303,12 @@ __global__ __launch_bounds__(256) void gemmMfmaPipelinedKernel(MfmaArgs g) {
   auto swriteA = [&](int stage) {
     T* a = sA + stage * BM * kBK + sOff;
 #pragma unroll
-    for (int i = 0; i < CH; ++i) *reinterpret_cast<Frag*>(a + i * 32 * kBK) = ra[i];
+    for (int i = 0; i < CH; ++i) *reinterpret_cast<Frag*>(a + i * RS * kBK) = ra[i];
   };
   auto swriteB = [&](int stage) {
     T* b = sB + stage * BN * kBK + sOff;
 #pragma unroll
-    for (int i = 0; i < CH; ++i) *reinterpret_cast<Frag*>(b + i * 32 * kBK) = rb[i];
+    for (int i = 0; i < CH; ++i) *reinterpret_cast<Frag*>(b + i * RS * kBK) = rb[i];
   };
   auto lfrag = [&](int stage, int ks, int buf) {
     const T* a = sA + stage * BM * kBK + aBase + kx[ks];
@@ -326,6 +332,9 @@ __global__ __launch_bounds__(256) void gemmMfmaPipelinedKernel(MfmaArgs g) {
   ldsBarrier();
   lfrag(0, 0, 0);
 
+  // LDS fetches / LDS stores / HBM loads to place after every second MFMA of a k-step
+  constexpr int kRd = (2 * (TM + TN) + TM * TN - 1) / (TM * TN), kWr = (2 * CH + TM * TN - 1) / (TM * TN),
+                kVm = (4 * CH + TM * TN - 1) / (TM * TN);
   auto iter = [&](auto hasNext, auto hasNext2, int kt) {
     constexpr bool kNext = decltype(hasNext)::value, kNext2 = decltype(hasNext2)::value;
     const int cur = kt & 1;
@@ -335,11 +344,11 @@ __global__ __launch_bounds__(256) void gemmMfmaPipelinedKernel(MfmaArgs g) {
     if constexpr (kNext) swriteA(cur ^ 1);
     mma(0);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < TM * TN / 2; ++i) {
       SGB_MFMA(1);
-      SGB_DSRD(1);
+      SGB_DSRD(kRd);
       SGB_MFMA(1);
-      if constexpr (kNext) SGB_DSWR(1);
+      if constexpr (kNext) SGB_DSWR(kWr);
     }
     // ---- k-step 1
     __builtin_amdgcn_sched_barrier(0);
@@ -347,11 +356,11 @@ __global__ __launch_bounds__(256) void gemmMfmaPipelinedKernel(MfmaArgs g) {
     if constexpr (kNext) swriteB(cur ^ 1);
     mma(1);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < TM * TN / 2; ++i) {
       SGB_MFMA(1);
-      SGB_DSRD(1);
+      SGB_DSRD(kRd);
       SGB_MFMA(1);
-      if constexpr (kNext) SGB_DSWR(1);
+      if constexpr (kNext) SGB_DSWR(kWr);
     }
     // ---- k-step 2
     __builtin_amdgcn_sched_barrier(0);
@@ -359,11 +368,11 @@ __global__ __launch_bounds__(256) void gemmMfmaPipelinedKernel(MfmaArgs g) {
     if constexpr (kNext2) gload(kt + 2);
     mma(0);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < TM * TN / 2; ++i) {
       SGB_MFMA(1);
-      SGB_DSRD(1);
+      SGB_DSRD(kRd);
       SGB_MFMA(1);
-      if constexpr (kNext2) SGB_VMRD(2);
+      if constexpr (kNext2) SGB_VMRD(kVm);
     }
     __builtin_amdgcn_sched_barrier(0);
     ldsBarrier();
@@ -371,9 +380,9 @@ __global__ __launch_bounds__(256) void gemmMfmaPipelinedKernel(MfmaArgs g) {
     if constexpr (kNext) lfrag(cur ^ 1, 0, 0);
     mma(1);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < TM * TN / 2; ++i) {
       SGB_MFMA(2);
-      if constexpr (kNext) SGB_DSRD(1);
+      if constexpr (kNext) SGB_DSRD(kRd);
     }
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -550,7 +559,7 @@ static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p
     attrSet = true;
   }
   dim3 grid((unsigned)(g.tilesM * g.tilesN), 1, (unsigned)p.batch);
-  hipLaunchKernelGGL((gemmMfmaPipelinedKernel<T>), grid, dim3(256), lds, stream, g);
+  hipLaunchKernelGGL((gemmMfmaPipelinedKernel<T>), grid, dim3(kPipeThreads), lds, stream, g);
   AMD_LAUNCH_CHECK();
   return diopiSuccess;
 }
