@@ -6,8 +6,8 @@
 One "step" is one pass of a Llama-2-7B-shaped decoder layer (prefill, batch 4 x seq 2048,
 hidden 4096, 32 heads x 128, FFN 11008, bf16, random weights, synthetic activations) through
 the DIOPI C ABI of libdiopi_impl.so: RMSNorm -> QKV linear -> rotary(q,k) -> causal context
-attention -> out linear -> residual add -> RMSNorm -> gate/up linears -> SiLU*mul -> down linear
--> residual add. Inputs and weights are resident in HBM before the timed region.
+attention -> out linear + residual (addmm) -> RMSNorm -> gate/up linears -> SiLU*mul -> down linear +
+residual (addmm). Inputs and weights are resident in HBM before the timed region.
 
 Prints ONE JSON line: tokens/s for the layer (whole job = the one GPU), the roofline of the
 dominant kernel (the bf16 MFMA GEMM) measured with device events on the launch stream inside the
@@ -100,14 +100,13 @@ def layer_plan(pkg, torch, dev, x, p, cfg):
         ("rotary_q", P("diopiRotaryEmbedding", qr.view(b, s, heads, hd), q4, cos, sin, False, False)),
         ("rotary_k", P("diopiRotaryEmbedding", kr.view(b, s, heads, hd), k4, cos, sin, False, False)),
         ("context_attention", P("diopiContextAttentionInference", attn, qr, kr, v3, starts, lens, int(s))),
-        ("gemm_o", P("diopiLinear", o, attn.view(T, hidden), p["wo"], None)),
-        ("add", P("diopiAdd", x1, x2, o, one)),
+        # out projection with the residual folded into the GEMM epilogue: x1 = x + attn @ Wo^T (aten::addmm)
+        ("gemm_o", P("diopiAddmm", x1, x2, attn.view(T, hidden), p["wo"].t(), one, one)),
         ("rms_norm", P("diopiRMSNorm", h2, None, x1, d.size([hidden]), p["norm2"], None, float(cfg["eps"]))),
         ("gemm_gate", P("diopiLinear", gate, h2, p["wgate"], None)),
         ("gemm_up", P("diopiLinear", up, h2, p["wup"], None)),
         ("silu_mul", P("diopiSiluMul", act, gate, up)),
-        ("gemm_down", P("diopiLinear", down, act, p["wdown"], None)),
-        ("add", P("diopiAdd", out, x1, down, one)),
+        ("gemm_down", P("diopiAddmm", out, x1, act, p["wdown"].t(), one, one)),
     ]
     keep = [h1, qkv, attn, o, x1, h2, qr, kr, gate, up, act, down, out, cos, sin, starts, lens, x2]
     flops = {"gemm_qkv": 2 * T * 3 * hidden * hidden, "gemm_o": 2 * T * hidden * hidden, "gemm_gate": 2 * T * ffn * hidden,

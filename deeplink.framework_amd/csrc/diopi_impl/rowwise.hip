@@ -5,7 +5,9 @@
 // the row in registers (up to 16 x 16-byte vectors), the max / sum / sum-of-squares are
 // wave64 butterfly reductions, and the row makes exactly one trip from and one trip to
 // HBM: algorithmic traffic = 2 * rows * cols * itemsize (+ the weight vector once).
-// No LDS, no barrier: four independent rows per 256-thread workgroup.
+// No LDS, no barrier. Waves are persistent (16 per CU): each walks its rows with the
+// next row's loads in flight while the current one is reduced, and keeps its slice of the
+// RMSNorm weight in registers.
 //
 // Generic path: one workgroup per row, LDS-staged block reduction, rows of any length;
 // softmax over a non-last dim walks the reduced dim with a stride (one lane per column).
@@ -13,6 +15,8 @@
 // Semantics: softmax as at::softmax on CPU (dipu/torch_dipu/csrc_dipu/aten/ops/CustomFallbackFunctions.hpp:466-474);
 // RMSNorm as dicp/dicp/vendor/AscendGraph/ext_ops.py:47-49 with fp32 accumulation
 // (dicp/test/model/llama/model.py:34-39).
+#include <algorithm>
+
 #include "common.hpp"
 
 namespace amd {
@@ -32,31 +36,60 @@ __global__ __launch_bounds__(256) void rowWaveKernel(T* __restrict__ out, const 
   constexpr int N = Vec16<T>::N;
   constexpr int WN = Vec16<WT>::N;
   const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= rows) return;
-  const V* src = reinterpret_cast<const V*>(in + row * inRowStride);
-  V* dst = reinterpret_cast<V*>(out + row * outRowStride);
   const int nvec = cols / N;
-
-  float f[NV][N];
+  // Persistent waves: wave w handles rows w, w + W, w + 2W, ... and fetches the next row
+  // while it reduces the current one, so every resident wave keeps loads in flight until
+  // the last row (no tail of half-empty CUs).
+  const int64_t nWaves = (int64_t)gridDim.x * 4;
+  int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  // RMSNorm: the weight vector is staged once per workgroup in LDS (NV KiB) and read from there
+  // for every row, which keeps it out of both the register file and the L1/L2 request stream.
+  constexpr int WPER = (N + WN - 1) / WN;
+  __shared__ WV wlds[OP == kRowRmsNorm ? 64 * NV * WPER : 1];
+  if (OP == kRowRmsNorm && weight != nullptr) {
+    for (int i = threadIdx.x; i < nvec * WPER; i += 256) wlds[i] = reinterpret_cast<const WV*>(weight)[i];
+  }
+  if (OP == kRowRmsNorm) __syncthreads();  // before the early exit below: every wave of the block arrives
+  if (row >= rows) return;
+  V pre[NV];
+  {
+    const V* src = reinterpret_cast<const V*>(in + row * inRowStride);
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    int idx = lane + 64 * i;
-    if (idx < nvec) {
-      V v = __builtin_nontemporal_load(src + idx);
+    for (int i = 0; i < NV; ++i)
+      if (lane + 64 * i < nvec) pre[i] = __builtin_nontemporal_load(src + lane + 64 * i);
+  }
+  for (; row < rows; row += nWaves) {
+  V* dst = reinterpret_cast<V*>(out + row * outRowStride);
+  V cur[NV];
+  if (OP == kRowRmsNorm) {
 #pragma unroll
-      for (int j = 0; j < N; ++j) f[i][j] = static_cast<float>(v[j]);
+    for (int i = 0; i < NV; ++i) cur[i] = pre[i];
+    if (row + nWaves < rows) {  // next row in flight while this one is reduced
+      const V* src = reinterpret_cast<const V*>(in + (row + nWaves) * inRowStride);
+#pragma unroll
+      for (int i = 0; i < NV; ++i)
+        if (lane + 64 * i < nvec) pre[i] = __builtin_nontemporal_load(src + lane + 64 * i);
     }
   }
 
   if constexpr (OP == kRowSoftmax) {
+    float f[NV][N];
     float m = -INFINITY;
 #pragma unroll
     for (int i = 0; i < NV; ++i)
       if (lane + 64 * i < nvec) {
 #pragma unroll
-        for (int j = 0; j < N; ++j) m = fmaxf(m, f[i][j]);
+        for (int j = 0; j < N; ++j) {
+          f[i][j] = static_cast<float>(pre[i][j]);
+          m = fmaxf(m, f[i][j]);
+        }
       }
+    if (row + nWaves < rows) {  // next row in flight while this one is reduced
+      const V* src = reinterpret_cast<const V*>(in + (row + nWaves) * inRowStride);
+#pragma unroll
+      for (int i = 0; i < NV; ++i)
+        if (lane + 64 * i < nvec) pre[i] = __builtin_nontemporal_load(src + lane + 64 * i);
+    }
     m = waveMax(m);
     const float mScaled = (m == -INFINITY) ? 0.f : m * kLog2e;  // all -inf row -> nan like the CPU kernel
     float s = 0.f;
@@ -65,7 +98,7 @@ __global__ __launch_bounds__(256) void rowWaveKernel(T* __restrict__ out, const 
       if (lane + 64 * i < nvec) {
 #pragma unroll
         for (int j = 0; j < N; ++j) {
-          f[i][j] = exp2f(f[i][j] * kLog2e - mScaled);
+          f[i][j] = __builtin_amdgcn_exp2f(fmaf(f[i][j], kLog2e, -mScaled));
           s += f[i][j];
         }
       }
@@ -87,7 +120,10 @@ __global__ __launch_bounds__(256) void rowWaveKernel(T* __restrict__ out, const 
     for (int i = 0; i < NV; ++i)
       if (lane + 64 * i < nvec) {
 #pragma unroll
-        for (int j = 0; j < N; ++j) ss += f[i][j] * f[i][j];
+        for (int j = 0; j < N; ++j) {
+          float x = static_cast<float>(cur[i][j]);
+          ss += x * x;
+        }
       }
     ss = waveSum(ss);
     const float inv = 1.0f / sqrtf(ss / (float)cols + eps);
@@ -97,13 +133,14 @@ __global__ __launch_bounds__(256) void rowWaveKernel(T* __restrict__ out, const 
       int idx = lane + 64 * i;
       if (idx < nvec) {
         V v;
+        V xv = cur[i];
+        asm volatile("" : "+v"(xv));  // re-convert from the packed row instead of keeping an fp32 copy alive
         // weight/bias vectors hold WN elements per 16 bytes; N elements of T need N/WN of them
         float w[N], b[N];
         if (weight != nullptr) {
-          constexpr int PER = (N + WN - 1) / WN;
 #pragma unroll
-          for (int p = 0; p < PER; ++p) {
-            WV wv = reinterpret_cast<const WV*>(weight)[idx * PER + p];
+          for (int p = 0; p < WPER; ++p) {
+            WV wv = wlds[idx * WPER + p];
 #pragma unroll
             for (int j = 0; j < WN && p * WN + j < N; ++j) w[p * WN + j] = static_cast<float>(wv[j]);
           }
@@ -119,7 +156,7 @@ __global__ __launch_bounds__(256) void rowWaveKernel(T* __restrict__ out, const 
         }
 #pragma unroll
         for (int j = 0; j < N; ++j) {
-          float r = f[i][j] * inv;
+          float r = static_cast<float>(xv[j]) * inv;
           if (weight != nullptr) r *= w[j];
           if (bias != nullptr) r += b[j];
           v[j] = static_cast<T>(r);
@@ -128,6 +165,7 @@ __global__ __launch_bounds__(256) void rowWaveKernel(T* __restrict__ out, const 
       }
     }
   }
+  }  // persistent row loop
 }
 
 // --------------------------------------------------------- block-per-row ----
@@ -230,6 +268,15 @@ __global__ __launch_bounds__(256) void rowMeanKernel(T* out, const T* in, int64_
   if (lane == 0) out[row] = static_cast<T>(s / (float)cols);
 }
 
+static int computeUnits() {
+  static int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    return n;
+  }();
+  return cus;
+}
+
 // ------------------------------------------------------------- dispatch ------
 template <typename T, int OP, typename WT>
 static diopiError_t launchRows(hipStream_t stream, T* out, const T* in, const WT* weight, const WT* bias,
@@ -240,7 +287,11 @@ static diopiError_t launchRows(hipStream_t stream, T* out, const T* in, const WT
   if (vectorOk && cols % N == 0 && cols / N <= 64 * 16) {
     int nvec = (int)(cols / N);
     int nv = (nvec + 63) / 64;
-    dim3 grid((unsigned)ceilDiv(rows, 4)), block(256);
+    // persistent waves: the kernels hold 16 waves per CU (4 per SIMD, <= 128 registers); give every
+    // wave the same number of rows so that no CU idles in a last partial round
+    const int64_t capacity = (int64_t)computeUnits() * 16;
+    const int64_t rowsPerWave = ceilDiv(rows, capacity);
+    dim3 grid((unsigned)ceilDiv(ceilDiv(rows, rowsPerWave), 4)), block(256);
 #define ROW_LAUNCH(NV)                                                                                            \
   hipLaunchKernelGGL((rowWaveKernel<T, NV, OP, WT>), grid, block, 0, stream, out, in, weight, bias, invRms, rows, \
                      (int)cols, inStride, outStride, eps)

@@ -97,33 +97,34 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   for (int e = 0; e < N; ++e) acc[e] = 0.f;
 
   constexpr int STEP = kTaWaves * kTaUnroll * TPW;  // tokens per workgroup iteration
+  // Two-deep software pipeline: while the rows of iteration i are being reduced, the K/V rows
+  // of iteration i+1 and the slot indices of iteration i+2 are already in flight.
   int64_t slot[kTaUnroll];
-  {
-    int t0 = begin + wave * kTaUnroll * TPW + grp;
+  V kr[kTaUnroll], vr[kTaUnroll], kn[kTaUnroll], vn[kTaUnroll];
+  bool ok[kTaUnroll], okn[kTaUnroll];
+  auto loadSlots = [&](int it) {
+    int t0 = it + wave * kTaUnroll * TPW + grp;
 #pragma unroll
     for (int u = 0; u < kTaUnroll; ++u) {
       int t = t0 + u * TPW;
       slot[u] = t < end ? ldIndex(a.bLoc, locBase + t, a.loc64) : -1;
     }
-  }
-  for (int it = begin; it < end; it += STEP) {
-    V kr[kTaUnroll], vr[kTaUnroll];
-    bool ok[kTaUnroll];
+  };
+  auto loadRows = [&](V (&kk)[kTaUnroll], V (&vv)[kTaUnroll], bool (&okk)[kTaUnroll]) {
 #pragma unroll
     for (int u = 0; u < kTaUnroll; ++u) {
-      ok[u] = slot[u] >= 0 && slot[u] < a.slots;  // slots outside the pool are skipped, never dereferenced
-      int64_t s = ok[u] ? slot[u] : 0;
-      kr[u] = *reinterpret_cast<const V*>(kBase + s * a.kSlotStride);
-      vr[u] = *reinterpret_cast<const V*>(vBase + s * a.vSlotStride);
+      okk[u] = slot[u] >= 0 && slot[u] < a.slots;  // slots outside the pool are skipped, never dereferenced
+      int64_t s = okk[u] ? slot[u] : 0;
+      kk[u] = __builtin_nontemporal_load(reinterpret_cast<const V*>(kBase + s * a.kSlotStride));
+      vv[u] = __builtin_nontemporal_load(reinterpret_cast<const V*>(vBase + s * a.vSlotStride));
     }
-    {  // indices of the next iteration, in flight during the math below
-      int t0 = it + STEP + wave * kTaUnroll * TPW + grp;
-#pragma unroll
-      for (int u = 0; u < kTaUnroll; ++u) {
-        int t = t0 + u * TPW;
-        slot[u] = t < end ? ldIndex(a.bLoc, locBase + t, a.loc64) : -1;
-      }
-    }
+  };
+  loadSlots(begin);
+  loadRows(kr, vr, ok);
+  loadSlots(begin + STEP);
+  for (int it = begin; it < end; it += STEP) {
+    loadRows(kn, vn, okn);        // rows of the next iteration (all masked past the end)
+    loadSlots(it + 2 * STEP);     // indices of the one after
     float sc[kTaUnroll];
     float mn = m;
 #pragma unroll
@@ -137,11 +138,11 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
       mn = fmaxf(mn, sc[u]);
     }
     if (mn != -INFINITY) {
-      float corr = exp2f(m - mn);  // m == -inf gives 0, acc and l are 0 then anyway
+      float corr = __builtin_amdgcn_exp2f(m - mn);  // m == -inf gives 0, acc and l are 0 then anyway
       float p[kTaUnroll], ps = 0.f;
 #pragma unroll
       for (int u = 0; u < kTaUnroll; ++u) {
-        p[u] = exp2f(sc[u] - mn);
+        p[u] = __builtin_amdgcn_exp2f(sc[u] - mn);
         ps += p[u];
       }
       l = l * corr + ps;
@@ -154,6 +155,8 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
       }
       m = mn;
     }
+#pragma unroll
+    for (int u = 0; u < kTaUnroll; ++u) kr[u] = kn[u], vr[u] = vn[u], ok[u] = okn[u];
   }
 
   // merge the TPW lane groups of the wave

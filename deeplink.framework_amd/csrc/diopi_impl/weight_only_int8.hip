@@ -3,7 +3,8 @@
 // Skinny-M (decode) shape: the int8 weight matrix is streamed from HBM exactly once and is
 // the only traffic of size (K*N bytes); everything else (x, scale, out) is tiny and stays
 // in L2. The kernel is a GEMV-shaped MFMA kernel:
-//   * a workgroup owns 16 output channels; its 4 waves split K four ways;
+//   * a workgroup owns 16 output channels; its 4 waves split K four ways; each
+//     wave keeps 8 weight + 16 activation vectors per lane in flight;
 //   * v_mfma_f32_16x16x32_{bf16,f16}: the B operand is the weight tile -- lane (n = lane%16,
 //     kgrp = lane/16) loads 32 consecutive int8 of row n (two 16-byte loads; the 4 kgrps of a
 //     row cover 128 contiguous bytes) and converts them to bf16/fp16 in registers while
@@ -61,9 +62,10 @@ __device__ __forceinline__ typename W8Mfma<T>::Frag cvt8(uint32_t lo, uint32_t h
 
 constexpr int kW8Block = 128;  // K elements one wave consumes per step (4 kgrps x 32)
 constexpr int kW8Unroll = 4;   // steps in flight
+constexpr int kW8Waves = 4;    // waves per workgroup = K splits (8 measured slower for M > 1)
 
 template <typename T>
-__global__ __launch_bounds__(256) void w8LinearKernel(W8Args a) {
+__global__ __launch_bounds__(kW8Waves * 64) void w8LinearKernel(W8Args a) {
   using Frag = typename W8Mfma<T>::Frag;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, kgrp = lane >> 4;
@@ -72,9 +74,10 @@ __global__ __launch_bounds__(256) void w8LinearKernel(W8Args a) {
   const int m = min(m0 + r16, a.M - 1);
   const int8_t* wrow = a.w + (int64_t)n * a.ldw + kgrp * 32;
   const T* xrow = reinterpret_cast<const T*>(a.x) + (int64_t)m * a.ldx + kgrp * 32;
-  // K is split in 4 contiguous quarters (rounded to the 128-element step), one per wave
+  // K is split in kW8Waves contiguous parts (rounded to the 128-element step), one per wave; at
+  // K = 4096 a wave owns 4 steps, i.e. every load of the wave is issued in one go
   const int steps = (a.K + kW8Block - 1) / kW8Block;
-  const int per = (steps + 3) / 4;
+  const int per = (steps + kW8Waves - 1) / kW8Waves;
   const int sBegin = wave * per, sEnd = min(steps, sBegin + per);
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   for (int s = sBegin; s < sEnd; s += kW8Unroll) {
@@ -101,7 +104,7 @@ __global__ __launch_bounds__(256) void w8LinearKernel(W8Args a) {
       }
     }
   }
-  __shared__ float red[4][64][4];
+  __shared__ float red[kW8Waves][64][4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) red[wave][lane][r] = acc[r];
   __syncthreads();
@@ -115,7 +118,9 @@ __global__ __launch_bounds__(256) void w8LinearKernel(W8Args a) {
       for (int r = 0; r < 4; ++r) {
         const int row = m0 + kgrp * 4 + r;
         if (row < a.M) {
-          float v = red[0][lane][r] + red[1][lane][r] + red[2][lane][r] + red[3][lane][r];
+          float v = 0.f;
+#pragma unroll
+          for (int w = 0; w < kW8Waves; ++w) v += red[w][lane][r];
           out[(int64_t)row * a.ldo + col] = static_cast<T>(v * sc + bv);
         }
       }
@@ -192,8 +197,8 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiWeightOnlyIn
   const bool fast = K % kW8Block == 0 && cin.aligned16() && cw.aligned16() && a.ldw % 16 == 0 && ceilDiv(M, 16) <= 65535;
   if (fast) {
     dim3 grid((unsigned)ceilDiv(N, 16), (unsigned)ceilDiv(M, 16));
-    if (in.dtype == diopi_dtype_bfloat16) hipLaunchKernelGGL(w8LinearKernel<bf16_t>, grid, dim3(256), 0, stream, a);
-    else hipLaunchKernelGGL(w8LinearKernel<half_t>, grid, dim3(256), 0, stream, a);
+    if (in.dtype == diopi_dtype_bfloat16) hipLaunchKernelGGL(w8LinearKernel<bf16_t>, grid, dim3(kW8Waves * 64), 0, stream, a);
+    else hipLaunchKernelGGL(w8LinearKernel<half_t>, grid, dim3(kW8Waves * 64), 0, stream, a);
   } else {
     dim3 grid((unsigned)ceilDiv(M * N, 256));
     if (in.dtype == diopi_dtype_bfloat16) hipLaunchKernelGGL(w8LinearScalarKernel<bf16_t>, grid, dim3(256), 0, stream, a);
