@@ -58,6 +58,7 @@ struct MfmaArgs {
   int M, N, K;
   int tilesM, tilesN;
   float alpha, beta;
+  bool vecEpilogue;  // out / addend / bias allow 16-byte row segments
 };
 
 constexpr int kBK = 64;  // K elements per LDS tile (128-byte rows)
@@ -392,10 +393,55 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
   iter(true_type{}, false_type{}, nK - 2);
   iter(false_type{}, false_type{}, nK - 1);
 
-  // ---- epilogue (same as the generic kernel)
+  // ---- epilogue
   T* out = reinterpret_cast<T*>(g.out) + (int64_t)batch * g.sOb;
   const T* cin = g.Cin ? reinterpret_cast<const T*>(g.Cin) + (int64_t)batch * g.sCb : nullptr;
   const T* bias = reinterpret_cast<const T*>(g.bias);
+  if (g.vecEpilogue) {
+    // Accumulators go through a wave-private LDS strip (32 rows x WN fp32, rows padded by 16 B) so
+    // that the addend is read and the result written as 16-byte row segments: full 128-byte lines
+    // instead of 2-byte column accesses. alpha/beta/bias are applied in fp32 after the transpose.
+    constexpr int RS4 = WN + 4;  // padded row, floats
+    ldsBarrier();                // every wave is done with the operand tiles the strips overlay
+    float* strip = reinterpret_cast<float*>(smem) + wave * (32 * RS4);
+    constexpr int GROUPS = WN / 8;                 // 8-column groups per strip row
+    constexpr int ITEMS = 32 * GROUPS / 64;        // (row, group) items per lane
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          strip[((r >> 2) * 8 + fhalf * 4 + (r & 3)) * RS4 + j * 32 + frow] = acc[i][j][r];
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // the strip is private to this wave: no barrier, only its own LDS ops
+#pragma unroll
+      for (int it = 0; it < ITEMS; ++it) {
+        const int item = lane + 64 * it;
+        const int srow = item / GROUPS, sg = item % GROUPS;
+        const int row = tm * BM + wm * WM + i * 32 + srow;
+        const int col = tn * BN + wn * WN + sg * 8;
+        const f32x4 lo = *reinterpret_cast<const f32x4*>(strip + srow * RS4 + sg * 8);
+        const f32x4 hi = *reinterpret_cast<const f32x4*>(strip + srow * RS4 + sg * 8 + 4);
+        if (row < g.M && col < g.N) {  // N % 8 == 0 here: a group is entirely inside or outside
+          float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          Frag o;
+          Frag cv, bvv;
+          if (cin) cv = *reinterpret_cast<const Frag*>(cin + (int64_t)row * g.sCm + col);
+          if (bias) bvv = *reinterpret_cast<const Frag*>(bias + col);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            float x = v[e] * g.alpha;
+            if (bias) x += static_cast<float>(bvv[e]);
+            if (cin) x += g.beta * static_cast<float>(cv[e]);
+            o[e] = static_cast<T>(x);
+          }
+          *reinterpret_cast<Frag*>(out + (int64_t)row * g.ldo + col) = o;
+        }
+      }
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // reads of this strip are done before the next chunk overwrites it
+    }
+    return;
+  }
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int col = tn * BN + wn * WN + j * 32 + frow;
@@ -529,6 +575,7 @@ static diopiError_t launchMfma(hipStream_t stream, const GemmProblem& p) {
   g.M = (int)p.M, g.N = (int)p.N, g.K = (int)p.K;
   g.tilesM = (int)ceilDiv(p.M, BM), g.tilesN = (int)ceilDiv(p.N, BN);
   g.alpha = p.alpha, g.beta = p.beta;
+  g.vecEpilogue = false;
   constexpr size_t lds = 2 * (size_t)(BM + BN) * kBK * sizeof(T);
   static bool attrSet = false;  // per template instance
   if (!attrSet) {
@@ -551,6 +598,9 @@ static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p
   g.M = (int)p.M, g.N = (int)p.N, g.K = (int)p.K;
   g.tilesM = (int)ceilDiv(p.M, 256), g.tilesN = (int)ceilDiv(p.N, 256);
   g.alpha = p.alpha, g.beta = p.beta;
+  auto al16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+  g.vecEpilogue = p.N % 8 == 0 && p.sOm % 8 == 0 && p.sOb % 8 == 0 && al16(p.out) &&
+                  (!p.Cin || (p.sCn == 1 && p.sCm % 8 == 0 && p.sCb % 8 == 0 && al16(p.Cin))) && (!p.bias || al16(p.bias));
   constexpr size_t lds = 2 * (size_t)(256 + 256) * kBK * sizeof(T);
   static bool attrSet = false;
   if (!attrSet) {
