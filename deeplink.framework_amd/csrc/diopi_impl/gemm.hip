@@ -265,15 +265,21 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
   const int batch = blockIdx.z;
   const T* A = reinterpret_cast<const T*>(g.A) + (int64_t)batch * g.sAb;
   const T* B = reinterpret_cast<const T*>(g.B) + (int64_t)batch * g.sBb;
-  const T* aPtr[CH];
-  const T* bPtr[CH];
+  // Operands are read through buffer descriptors: a 32-bit per-lane byte offset fixed for the whole
+  // K loop plus a scalar K offset per tile, so the loop carries no 64-bit address arithmetic.
+  // (The host guarantees both operands span less than 2 GiB.)
+  __amdgpu_buffer_rsrc_t rsA =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(A), 0, (int)(((int64_t)(g.M - 1) * g.lda + g.K) * 2), 0x00020000);
+  __amdgpu_buffer_rsrc_t rsB =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(B), 0, (int)(((int64_t)(g.N - 1) * g.ldb + g.K) * 2), 0x00020000);
+  int aOffG[CH], bOffG[CH];
   const int c8 = (tid & 7) * 8;
-  const int srow = tid >> 3;  // staging row of chunk 0; chunk i is 32 rows further
-  const int sOff = srow * kBK + (((tid & 7) ^ ((srow >> 1) & 7)) << 3);  // rows 32 apart share the swizzle
+  const int srow = tid >> 3;  // staging row of chunk 0; chunk i is RS rows further
+  const int sOff = srow * kBK + (((tid & 7) ^ ((srow >> 1) & 7)) << 3);  // rows RS apart share the swizzle
 #pragma unroll
   for (int i = 0; i < CH; ++i) {
-    aPtr[i] = A + (int64_t)min(tm * BM + srow + RS * i, g.M - 1) * g.lda + c8;
-    bPtr[i] = B + (int64_t)min(tn * BN + srow + RS * i, g.N - 1) * g.ldb + c8;
+    aOffG[i] = (int)(((int64_t)min(tm * BM + srow + RS * i, g.M - 1) * g.lda + c8) * 2);
+    bOffG[i] = (int)(((int64_t)min(tn * BN + srow + RS * i, g.N - 1) * g.ldb + c8) * 2);
   }
   Frag ra[CH], rb[CH];
   const int nK = g.K / kBK;
@@ -295,11 +301,11 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   auto gload = [&](int kt) {
-    const int k0 = kt * kBK;
+    const int k0 = kt * kBK * (int)sizeof(T);
 #pragma unroll
-    for (int i = 0; i < CH; ++i) ra[i] = *reinterpret_cast<const Frag*>(aPtr[i] + k0);
+    for (int i = 0; i < CH; ++i) ra[i] = __builtin_bit_cast(Frag, __builtin_amdgcn_raw_buffer_load_b128(rsA, aOffG[i], k0, 0));
 #pragma unroll
-    for (int i = 0; i < CH; ++i) rb[i] = *reinterpret_cast<const Frag*>(bPtr[i] + k0);
+    for (int i = 0; i < CH; ++i) rb[i] = __builtin_bit_cast(Frag, __builtin_amdgcn_raw_buffer_load_b128(rsB, bOffG[i], k0, 0));
   };
   auto swriteA = [&](int stage) {
     T* a = sA + stage * BM * kBK + sOff;
@@ -651,7 +657,8 @@ diopiError_t runGemm(diopiContextHandle_t ctx, hipStream_t stream, GemmProblem p
       p.B = ws, p.sBk = 1, p.sBn = p.K, p.sBb = (sbb == 0) ? 0 : p.N * p.K;
     }
     const bool big = ceilDiv(p.M, 256) * ceilDiv(p.N, 256) * p.batch >= 200;
-    if (big && p.K % kBK == 0 && p.K >= 2 * kBK) {
+    const bool fits2g = ((p.M - 1) * p.sAm + p.K) * 2 < (int64_t(1) << 31) && ((p.N - 1) * p.sBn + p.K) * 2 < (int64_t(1) << 31);
+    if (big && p.K % kBK == 0 && p.K >= 2 * kBK && fits2g) {
       return p.dtype == diopi_dtype_bfloat16 ? launchMfmaPipelined<bf16_t>(stream, p) : launchMfmaPipelined<half_t>(stream, p);
     }
     if (p.dtype == diopi_dtype_bfloat16) {
