@@ -200,6 +200,29 @@ SIGNATURES = {
     "diopiCopyInp": [_T, _T],
     "diopiCat": [_T, POINTER(c_void_p), c_int64, c_int64],
     "diopiIndexPutInp": [_T, _T, POINTER(c_void_p), c_int64, c_bool],
+    "diopiWhere": [_T, _T, _T, _T],
+    "diopiMaskedFill": [_T, _T, _T, _T],
+    "diopiMaskedFillInp": [_T, _T, _T],
+    "diopiMaskedFillScalar": [_T, _T, _T, _S],
+    "diopiMaskedFillInpScalar": [_T, _T, _S],
+    "diopiTril": [_T, _T, c_int64],
+    "diopiTriu": [_T, _T, c_int64],
+    "diopiTriuInp": [_T, c_int64],
+    "diopiArange": [_T, _S, _S, _S],
+    "diopiIndexSelect": [_T, _T, c_int64, _T],
+    "diopiGather": [_T, _T, c_int64, _T],
+    "diopiEq": [_T, _T, _T],
+    "diopiEqScalar": [_T, _T, _S],
+    "diopiNe": [_T, _T, _T],
+    "diopiNeScalar": [_T, _T, _S],
+    "diopiLt": [_T, _T, _T],
+    "diopiLtScalar": [_T, _T, _S],
+    "diopiLe": [_T, _T, _T],
+    "diopiLeScalar": [_T, _T, _S],
+    "diopiGt": [_T, _T, _T],
+    "diopiGtScalar": [_T, _T, _S],
+    "diopiGe": [_T, _T, _T],
+    "diopiGeScalar": [_T, _T, _S],
     "diopiMm": [_T, _T, _T],
     "diopiBmm": [_T, _T, _T],
     "diopiMatmul": [_T, _T, _T],

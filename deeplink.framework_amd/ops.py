@@ -273,6 +273,163 @@ def index_put_(self, indices, values, accumulate=False):
     return self
 
 
+# ------------------------------------------------- selection / masks / gathers
+def where(condition, self, other, *, out=None):
+    """aten::where.self -> diopiWhere (diopi_functions.yaml:1566-1571). Python numbers become
+    0-d device tensors, which is what ATen hands the wrapper after its own scalar wrapping."""
+    dev = condition.device
+    if _is_number(self) and _is_number(other):
+        dtype = torch.result_type(torch.tensor(self), torch.tensor(other))
+        self, other = torch.tensor(self, dtype=dtype, device=dev), torch.tensor(other, dtype=dtype, device=dev)
+    elif _is_number(self):
+        self = torch.tensor(self, dtype=other.dtype, device=dev)
+    elif _is_number(other):
+        other = torch.tensor(other, dtype=self.dtype, device=dev)
+    if out is None:
+        shape = torch.broadcast_shapes(condition.shape, self.shape, other.shape)
+        out = torch.empty(shape, dtype=torch.result_type(self, other), device=dev)
+    hc, pc = handle(condition)
+    ha, pa = handle(self)
+    hb, pb = handle(other)
+    ho, po = handle(out)
+    _call("diopiWhere", po, pc, pa, pb)
+    return out
+
+
+def masked_fill(self, mask, value, *, out=None):
+    """aten::masked_fill.Scalar / .Tensor -> diopiMaskedFillScalar / diopiMaskedFill
+    (diopi_functions.yaml:1432-1453); a CPU value tensor is moved to the device first (:1436)."""
+    if out is None:
+        out = torch.empty(torch.broadcast_shapes(self.shape, mask.shape), dtype=self.dtype, device=self.device)
+    ho, po = handle(out)
+    hs, ps = handle(self)
+    hm, pm = handle(mask)
+    if _is_number(value):
+        sc = scalar(value)
+        _call("diopiMaskedFillScalar", po, ps, pm, byref(sc))
+    else:
+        hv, pv = handle(value.to(self.device))
+        _call("diopiMaskedFill", po, ps, pm, pv)
+    return out
+
+
+def masked_fill_(self, mask, value):
+    hs, ps = handle(self)
+    hm, pm = handle(mask)
+    if _is_number(value):
+        sc = scalar(value)
+        _call("diopiMaskedFillInpScalar", ps, pm, byref(sc))
+    else:
+        hv, pv = handle(value.to(self.device))
+        _call("diopiMaskedFillInp", ps, pm, pv)
+    return self
+
+
+def tril(self, diagonal=0, *, out=None):
+    """aten::tril -> diopiTril (diopi_functions.yaml:1191-1197)."""
+    out = torch.empty_like(self) if out is None else out
+    ho, po = handle(out)
+    hs, ps = handle(self)
+    _call("diopiTril", po, ps, int(diagonal))
+    return out
+
+
+def triu(self, diagonal=0, *, out=None):
+    """aten::triu -> diopiTriu (diopi_functions.yaml:2505-2516)."""
+    out = torch.empty_like(self) if out is None else out
+    ho, po = handle(out)
+    hs, ps = handle(self)
+    _call("diopiTriu", po, ps, int(diagonal))
+    return out
+
+
+def triu_(self, diagonal=0):
+    hs, ps = handle(self)
+    _call("diopiTriuInp", ps, int(diagonal))
+    return self
+
+
+def arange(start, end=None, step=1, *, dtype=None, device=None, out=None):
+    """aten::arange.start_out -> diopiArange (diopi_functions.yaml:2341-2347). The element count is
+    ATen's ceil((end - start) / step); the wrapper only sizes `out` itself when it arrives empty."""
+    import math
+    if end is None:
+        start, end = 0, start
+    if out is None:
+        if dtype is None:
+            dtype = torch.get_default_dtype() if any(isinstance(v, float) for v in (start, end, step)) else torch.int64
+        out = torch.empty(int(math.ceil((end - start) / step)), dtype=dtype, device=device)
+    ho, po = handle(out)
+    s0, s1, s2 = scalar(start), scalar(end), scalar(step)
+    _call("diopiArange", po, byref(s0), byref(s1), byref(s2))
+    return out
+
+
+def index_select(self, dim, index, *, out=None):
+    """aten::index_select -> diopiIndexSelect (diopi_functions.yaml:1926-1933)."""
+    if out is None:
+        shape = list(self.shape)
+        shape[dim % self.dim()] = index.numel()
+        out = torch.empty(shape, dtype=self.dtype, device=self.device)
+    ho, po = handle(out)
+    hs, ps = handle(self)
+    hi, pi = handle(index)
+    _call("diopiIndexSelect", po, ps, int(dim), pi)
+    return out
+
+
+def gather(self, dim, index, *, out=None):
+    """aten::gather.out -> diopiGather (diopi_functions.yaml:1923-1924)."""
+    if out is None:
+        out = torch.empty(index.shape, dtype=self.dtype, device=self.device)
+    ho, po = handle(out)
+    hs, ps = handle(self)
+    hi, pi = handle(index)
+    _call("diopiGather", po, ps, int(dim), pi)
+    return out
+
+
+def _compare(name, self, other, out):
+    other = _peel_cpu_scalar(other)
+    if out is None:
+        shape = torch.broadcast_shapes(self.shape, other.shape) if isinstance(other, torch.Tensor) else self.shape
+        out = torch.empty(shape, dtype=torch.bool, device=self.device)
+    ho, po = handle(out)
+    hs, ps = handle(self)
+    if _is_number(other):
+        sc = scalar(other)
+        _call(f"diopi{name}Scalar", po, ps, byref(sc))
+    else:
+        hb, pb = handle(other)
+        _call(f"diopi{name}", po, ps, pb)
+    return out
+
+
+def eq(self, other, *, out=None):
+    """aten::eq.Tensor_out / eq.Scalar_out -> diopiEq / diopiEqScalar (diopi_functions.yaml:409-420)."""
+    return _compare("Eq", self, other, out)
+
+
+def ne(self, other, *, out=None):
+    return _compare("Ne", self, other, out)
+
+
+def lt(self, other, *, out=None):
+    return _compare("Lt", self, other, out)
+
+
+def le(self, other, *, out=None):
+    return _compare("Le", self, other, out)
+
+
+def gt(self, other, *, out=None):
+    return _compare("Gt", self, other, out)
+
+
+def ge(self, other, *, out=None):
+    return _compare("Ge", self, other, out)
+
+
 # ------------------------------------------------------------------ contractions
 def mm(self, mat2, *, out=None):
     """aten::mm -> diopiMm (diopi_functions.yaml:1829-1837)."""

@@ -99,6 +99,64 @@ DIOPI_API diopiError_t diopiIndexPutInp(diopiContextHandle_t ctx, diopiTensorHan
                                         diopiConstTensorHandle_t values, diopiConstTensorHandle_t* indices,
                                         int64_t indices_counts, bool accumulate);
 
+/* ---- selection, masks, comparisons, gathers (what a decoder layer written in primitive aten ops needs) ---- */
+/* out = condition ? input : other, all three broadcast to out. yaml:1566-1571 */
+DIOPI_API diopiError_t diopiWhere(diopiContextHandle_t ctx, diopiTensorHandle_t out,
+                                  diopiConstTensorHandle_t condition, diopiConstTensorHandle_t input,
+                                  diopiConstTensorHandle_t other);
+/* out = mask ? value : input; value is a 0-d device tensor or a Scalar. yaml:1432-1453 */
+DIOPI_API diopiError_t diopiMaskedFill(diopiContextHandle_t ctx, diopiTensorHandle_t out,
+                                       diopiConstTensorHandle_t input, diopiConstTensorHandle_t mask,
+                                       diopiConstTensorHandle_t value);
+DIOPI_API diopiError_t diopiMaskedFillInp(diopiContextHandle_t ctx, diopiTensorHandle_t input,
+                                          diopiConstTensorHandle_t mask, diopiConstTensorHandle_t value);
+DIOPI_API diopiError_t diopiMaskedFillScalar(diopiContextHandle_t ctx, diopiTensorHandle_t out,
+                                             diopiConstTensorHandle_t input, diopiConstTensorHandle_t mask,
+                                             const diopiScalar_t* value);
+DIOPI_API diopiError_t diopiMaskedFillInpScalar(diopiContextHandle_t ctx, diopiTensorHandle_t input,
+                                                diopiConstTensorHandle_t mask, const diopiScalar_t* value);
+/* lower / upper triangle of the last two dims, zero elsewhere. yaml:1191-1197, 2505-2516 */
+DIOPI_API diopiError_t diopiTril(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiConstTensorHandle_t input,
+                                 int64_t diagonal);
+DIOPI_API diopiError_t diopiTriu(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiConstTensorHandle_t input,
+                                 int64_t diagonal);
+DIOPI_API diopiError_t diopiTriuInp(diopiContextHandle_t ctx, diopiTensorHandle_t input, int64_t diagonal);
+/* out[i] = start + i*step for the elements the caller sized out to. yaml:2341-2347 */
+DIOPI_API diopiError_t diopiArange(diopiContextHandle_t ctx, diopiTensorHandle_t out, const diopiScalar_t* start,
+                                   const diopiScalar_t* end, const diopiScalar_t* step);
+/* out = input.index_select(dim, index), index 1-d int32/int64. yaml:1926-1933 */
+DIOPI_API diopiError_t diopiIndexSelect(diopiContextHandle_t ctx, diopiTensorHandle_t out,
+                                        diopiConstTensorHandle_t input, int64_t dim, diopiConstTensorHandle_t index);
+/* out[i][j][k] = input[index[i][j][k]][j][k] (for dim 0), out shaped like index. yaml:1923-1924 */
+DIOPI_API diopiError_t diopiGather(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiConstTensorHandle_t input,
+                                   int64_t dim, diopiConstTensorHandle_t index);
+/* out (normally bool) = input <cmp> other, broadcasting; Scalar forms take the right operand as a Scalar.
+ * yaml:409-420 eq, :443-454 lt, :466-477 ne, :489-500 ge, :512-523 gt, :535-546 le */
+DIOPI_API diopiError_t diopiEq(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiConstTensorHandle_t input,
+                               diopiConstTensorHandle_t other);
+DIOPI_API diopiError_t diopiEqScalar(diopiContextHandle_t ctx, diopiTensorHandle_t out,
+                                     diopiConstTensorHandle_t input, const diopiScalar_t* other);
+DIOPI_API diopiError_t diopiNe(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiConstTensorHandle_t input,
+                               diopiConstTensorHandle_t other);
+DIOPI_API diopiError_t diopiNeScalar(diopiContextHandle_t ctx, diopiTensorHandle_t out,
+                                     diopiConstTensorHandle_t input, const diopiScalar_t* other);
+DIOPI_API diopiError_t diopiLt(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiConstTensorHandle_t input,
+                               diopiConstTensorHandle_t other);
+DIOPI_API diopiError_t diopiLtScalar(diopiContextHandle_t ctx, diopiTensorHandle_t out,
+                                     diopiConstTensorHandle_t input, const diopiScalar_t* other);
+DIOPI_API diopiError_t diopiLe(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiConstTensorHandle_t input,
+                               diopiConstTensorHandle_t other);
+DIOPI_API diopiError_t diopiLeScalar(diopiContextHandle_t ctx, diopiTensorHandle_t out,
+                                     diopiConstTensorHandle_t input, const diopiScalar_t* other);
+DIOPI_API diopiError_t diopiGt(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiConstTensorHandle_t input,
+                               diopiConstTensorHandle_t other);
+DIOPI_API diopiError_t diopiGtScalar(diopiContextHandle_t ctx, diopiTensorHandle_t out,
+                                     diopiConstTensorHandle_t input, const diopiScalar_t* other);
+DIOPI_API diopiError_t diopiGe(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiConstTensorHandle_t input,
+                               diopiConstTensorHandle_t other);
+DIOPI_API diopiError_t diopiGeScalar(diopiContextHandle_t ctx, diopiTensorHandle_t out,
+                                     diopiConstTensorHandle_t input, const diopiScalar_t* other);
+
 /* ---- dense contractions (MFMA for bf16/fp16, fp32 FMA tiles otherwise) ---- */
 /* out[M,N] = input[M,K] @ mat2[K,N]. yaml:1829-1837 */
 DIOPI_API diopiError_t diopiMm(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiConstTensorHandle_t input,

@@ -99,6 +99,42 @@ def index_put_(x, indices, values, accumulate=False):
     return x.index_put_(tuple(indices), values, accumulate=accumulate)
 
 
+# ---- selection / mask / gather helpers: the generic boxed CPU fallback, i.e. stock ATen ----
+# (dipu/torch_dipu/csrc_dipu/aten/RegisterDIPU.cpp:131-158). Known answers the reference's
+# tests hold: dipu/tests/python/unittests/test_gather.py:10-16, test_arange.py:8-24,
+# test_tri.py:9-20, test_where.py:11-31, test_masked_fill.py:8-76, test_ge.py:14-24.
+def where(cond, a, b):
+    return torch.where(cond, a, b)
+
+
+def masked_fill(x, mask, value):
+    return torch.masked_fill(x, mask, value)
+
+
+def tril(x, diagonal=0):
+    return torch.tril(x, diagonal)
+
+
+def triu(x, diagonal=0):
+    return torch.triu(x, diagonal)
+
+
+def arange(start, end, step, dtype=None):
+    return torch.arange(start, end, step, dtype=dtype)
+
+
+def index_select(x, dim, index):
+    return torch.index_select(x, dim, index.long())
+
+
+def gather(x, dim, index):
+    return torch.gather(x, dim, index.long())
+
+
+def compare(name, a, b):
+    return getattr(torch, name)(a, b)
+
+
 # ---- fused ops restated from the reference's PyTorch definitions -----------
 def rms_norm(x, weight, eps):
     """lightllm_rms_norm_impl, ext_ops.py:47-49 (arithmetic in x's own dtype)."""

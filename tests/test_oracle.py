@@ -255,3 +255,25 @@ def test_decoder_block_matches_independent_composition():
     h2 = F.rms_norm(x1, (64,), p["norm2"], cfg["eps"])
     want = x1 + (F.silu(h2 @ p["wgate"].t()) * (h2 @ p["wup"].t())) @ p["wdown"].t()
     assert torch.allclose(out, want, atol=1e-5)
+
+
+# ---- selection / mask / gather helpers: known answers and brute force ---------------------------
+def test_select_helpers_known_answers():
+    # dipu/tests/python/unittests/test_gather.py:10-16
+    t = torch.tensor([[1, 2], [3, 4]])
+    assert oracle.gather(t, 1, torch.tensor([[0, 0], [1, 0]])).tolist() == [[1, 1], [4, 3]]
+    # dipu/tests/python/unittests/test_arange.py:8-24
+    assert oracle.arange(5, 20, 1).tolist() == list(range(5, 20))
+    assert oracle.arange(10, -7, -3).tolist() == [10, 7, 4, 1, -2, -5]
+    x = torch.arange(24.0).view(4, 6)
+    for d in (-2, 0, 1):
+        lo, up = oracle.tril(x, d), oracle.triu(x, d)
+        for r in range(4):
+            for c in range(6):
+                assert lo[r, c] == (x[r, c] if c - r <= d else 0)
+                assert up[r, c] == (x[r, c] if c - r >= d else 0)
+    m = torch.tensor([[True, False], [False, True]])
+    assert oracle.masked_fill(torch.ones(2, 2), m, 7).tolist() == [[7, 1], [1, 7]]
+    assert oracle.where(m, torch.zeros(2, 2), torch.ones(2, 2)).tolist() == [[0, 1], [1, 0]]
+    assert oracle.index_select(x, 1, torch.tensor([5, 0])).tolist() == [[5, 0], [11, 6], [17, 12], [23, 18]]
+    assert oracle.compare("ge", torch.tensor([1, 2, 3]), 2).tolist() == [False, True, True]
