@@ -327,4 +327,12 @@ int dipuAmdContextWorkspace(void* ctx, uint64_t* tensors, uint64_t* bytes) {
   return guarded([&] { contextWorkspace(ctx, tensors, bytes); });
 }
 
+int dipuAmdProfilerEnable(const char* dump_path) {
+  return guarded([&] { dipu::devapis::enableProfiler(dump_path ? dump_path : "", false, false, false); });
+}
+int dipuAmdProfilerDisable() { return guarded([&] { dipu::devapis::disableProfiler(); }); }
+int dipuAmdProfilerCounts(uint64_t* started, uint64_t* stopped, int* roctx_bound) {
+  return guarded([&] { dipu::profile::counts(started, stopped, roctx_bound); });
+}
+
 }  // extern "C"

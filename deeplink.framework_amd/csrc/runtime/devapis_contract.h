@@ -85,5 +85,17 @@ void memCopyD2DAsync(deviceStream_t stream, size_t nbytes, deviceId_t dstDevId, 
 void memCopyH2DAsync(deviceStream_t stream, size_t nbytes, void* dst, const void* src);
 void memCopyD2HAsync(deviceStream_t stream, size_t nbytes, void* dst, const void* src);
 
+
+// ---- profiler hooks (runtime/device/profilerapis.h:12-14) ----
+void enableProfiler(const std::string& dump_path, bool call_stack, bool record_shapes, bool profile_memory);
+void disableProfiler();
+
 }  // namespace devapis
+
+namespace profile {
+bool enabled();
+void* rangeStart(const char* name);  // nullptr while the profiler is disabled
+void rangeStop(void* record);
+void counts(uint64_t* started, uint64_t* stopped, int* roctxBound);
+}  // namespace profile
 }  // namespace dipu

@@ -199,13 +199,17 @@ DIOPI_RT_API diopiError_t diopiGeneratorSetSeedAndOffset(diopiGeneratorHandle_t,
   return diopiNoImplement;
 }
 
-// Ranges are accepted and dropped: measurement on this backend is done with rocprofv3.
-DIOPI_RT_API diopiError_t diopiRecordStart(const char*, void** record) {
-  *record = nullptr;
+// Named host ranges: ROCTX ranges while devapis::enableProfiler is in effect, nothing otherwise
+// (diopirt_impl.cpp:224-237 wraps the same pair around a RecordBlockCreator).
+DIOPI_RT_API diopiError_t diopiRecordStart(const char* record_name, void** record) {
+  if (!record) return diopiErrorOccurred;
+  *record = dipu::profile::rangeStart(record_name);
   return diopiSuccess;
 }
 DIOPI_RT_API diopiError_t diopiRecordEnd(void** record) {
-  if (record) *record = nullptr;
+  if (!record) return diopiErrorOccurred;
+  dipu::profile::rangeStop(*record);
+  *record = nullptr;
   return diopiSuccess;
 }
 

@@ -310,3 +310,36 @@ class SimAllocator:
         b, n = c_uint64(), c_uint64()
         _check(_rt().dipuAmdSimAllocatorBackendUsage(self.h, byref(b), byref(n)))
         return b.value, n.value
+
+
+# ---- profiler hooks (runtime/device/profilerapis.h:12-14; diopirt_impl.cpp:224-237) ----
+def enableProfiler(dump_path=""):
+    _check(_rt().dipuAmdProfilerEnable(dump_path.encode()))
+
+
+def disableProfiler():
+    _check(_rt().dipuAmdProfilerDisable())
+
+
+def profilerCounts():
+    """(ranges started, ranges ended, whether a ROCTX library is bound)."""
+    a, b, r = c_uint64(), c_uint64(), c_int()
+    _check(_rt().dipuAmdProfilerCounts(byref(a), byref(b), byref(r)))
+    return a.value, b.value, bool(r.value)
+
+
+def recordStart(name):
+    """diopiRecordStart as an operator library would call it; returns the opaque record."""
+    rec = c_void_p()
+    f = _rt().diopiRecordStart
+    f.argtypes = [c_char_p, ctypes.POINTER(c_void_p)]
+    if f(name.encode(), byref(rec)) != 0:
+        raise RuntimeError_("diopiRecordStart failed")
+    return rec
+
+
+def recordEnd(rec):
+    f = _rt().diopiRecordEnd
+    f.argtypes = [ctypes.POINTER(c_void_p)]
+    if f(byref(rec)) != 0:
+        raise RuntimeError_("diopiRecordEnd failed")

@@ -138,6 +138,14 @@ DIPU_AMD_API int dipuAmdContextDestroy(void* ctx);
 DIPU_AMD_API int dipuAmdContextReset(void* ctx);  /* release workspace, keep the context */
 DIPU_AMD_API int dipuAmdContextWorkspace(void* ctx, uint64_t* tensors, uint64_t* bytes);
 
+/* ---- profiler hooks: dipu/torch_dipu/csrc_dipu/runtime/device/profilerapis.h:12-14 (enableProfiler /
+ * disableProfiler) and the diopiRecordStart / diopiRecordEnd pair, diopirt/diopirt_impl.cpp:224-237.
+ * While enabled, every diopiRecordStart/End pair becomes a ROCTX range (when a ROCTX library can be loaded)
+ * and is counted; dipuAmdProfilerCounts reports ranges started, ranges ended, and whether ROCTX is bound. */
+DIPU_AMD_API int dipuAmdProfilerEnable(const char* dump_path);
+DIPU_AMD_API int dipuAmdProfilerDisable(void);
+DIPU_AMD_API int dipuAmdProfilerCounts(uint64_t* started, uint64_t* stopped, int* roctx_bound);
+
 #if defined(__cplusplus)
 }
 #endif

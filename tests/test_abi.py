@@ -80,3 +80,29 @@ def test_version_and_error_string(pkg):
     rt.diopiGetVersion.restype = ctypes.c_char_p
     assert rt.diopiGetVersion().startswith(b"DIOPI Version: ")
     assert isinstance(pkg.diopi.last_error(), str)
+
+
+def test_profiler_hooks_count_ranges_only_while_enabled(pkg):
+    """devapis::enableProfiler / disableProfiler and the diopiRecordStart/End pair
+    (dipu/torch_dipu/csrc_dipu/runtime/device/profilerapis.h:12-14, diopirt/diopirt_impl.cpp:224-237):
+    disabled -> null record, nothing counted; enabled -> one range started and ended per pair."""
+    rt = pkg.runtime
+    rt.disableProfiler()
+    s0, e0, _ = rt.profilerCounts()
+    rec = rt.recordStart("idle")
+    assert not rec.value
+    rt.recordEnd(rec)
+    assert rt.profilerCounts()[:2] == (s0, e0)
+    rt.enableProfiler("/tmp/unused")
+    try:
+        recs = [rt.recordStart(f"diopiOp{i}") for i in range(3)]
+        assert all(r.value for r in recs)
+        s1, e1, _ = rt.profilerCounts()
+        assert (s1 - s0, e1 - e0) == (3, 0)
+        for r in reversed(recs):
+            rt.recordEnd(r)
+            assert not r.value
+        s2, e2, _ = rt.profilerCounts()
+        assert (s2 - s0, e2 - e0) == (3, 3)
+    finally:
+        rt.disableProfiler()
