@@ -36,6 +36,10 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-ops", action="store_true", help="skip the per-op HBM microbenchmarks")
     ap.add_argument("--only-layer", action="store_true", help="alias for --no-cpu --no-ops")
+    ap.add_argument("--gemm", metavar="M,N,K", help="profiling aid: time only diopiLinear on bf16 [M,K] x [N,K]^T "
+                    "(activations N(0,1), weights N(0,0.02)) for --steps launches and print one JSON line")
+    ap.add_argument("--attention", action="store_true", help="profiling aid: time only the prefill attention of the "
+                    "layer workload (batch 4 x seq 2048, 32 heads x 128, bf16) for --steps launches")
     return ap.parse_args()
 
 
@@ -231,6 +235,30 @@ def op_microbench(pkg, torch, dev, rt, stream):
     return res
 
 
+def single_kernel(pkg, torch, dev, rt, stream, args):
+    """One kernel of the layer on its own, for counter runs that should see nothing else."""
+    if args.gemm:
+        m, n, k = (int(v) for v in args.gemm.split(","))
+        g = torch.Generator().manual_seed(0)
+        a = torch.randn(m, k, generator=g).bfloat16().to(dev)
+        w = (torch.randn(n, k, generator=g) * 0.02).bfloat16().to(dev)
+        out = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+        call = Prepared(pkg, "diopiLinear", out, a, w, None)
+        work, unit, label = 2.0 * m * n * k / 1e12, "TFLOP/s", f"diopiLinear bf16 {m}x{n}x{k}"
+    else:
+        b, s, h, hd = 4, 2048, 32, 128
+        g = torch.Generator().manual_seed(0)
+        q, k_, v = (torch.randn(b * s, h, hd, generator=g).bfloat16().to(dev) for _ in range(3))
+        out = torch.empty_like(q)
+        starts = (torch.arange(b, dtype=torch.int32) * s).to(dev)
+        lens = torch.full((b,), s, dtype=torch.int32).to(dev)
+        call = Prepared(pkg, "diopiContextAttentionInference", out, q, k_, v, starts, lens, s)
+        work, unit, label = 4.0 * s * s * hd * b * h / 2 / 1e12, "TFLOP/s (causal-useful)", "context attention bf16 4x2048x32x128"
+    us = time_ops(rt, stream, [call], args.steps, args.warmup)[0]
+    print(json.dumps({"kernel": label, "launches": args.steps, "avg_launch_us": round(us, 2),
+                      "achieved": round(work / (us * 1e-6), 1), "unit": unit}), flush=True)
+
+
 def cpu_baseline(pkg, torch):
     """The oracle's decoder layer on the host cores, on the same batch of four 2048-token sequences."""
     from oracle import cpu_fallback as oracle
@@ -270,6 +298,9 @@ def main():
     dev = torch.device("cuda:0")
     rt = pkg.runtime
     stream = torch.cuda.current_stream().cuda_stream
+    if args.gemm or args.attention:
+        single_kernel(pkg, torch, dev, rt, stream, args)
+        return
 
     x, p, cfg = pkg.workloads.llama7b_layer(seed=0)
     x = x.to(dev)

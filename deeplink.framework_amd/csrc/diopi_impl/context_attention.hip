@@ -118,34 +118,39 @@ __global__ __launch_bounds__(256, 2) void contextAttnMfmaKernel(CaArgs a) {
   const int ntiles = (min(len, q0 + kCaBQ) + kCaBKV - 1) / kCaBKV;
   const int waveMaxQ = min(q0 + wave * 32 + 31, len - 1);
 
-  // ---- staging roles
+  // ---- staging roles. K and V rows come through buffer descriptors that end at the sequence's last
+  // row: a lane's offset is computed once (32 bits), the tile advances a scalar offset, and rows past
+  // the sequence read as zeros without any clamping arithmetic.
   Frag kr[K_CH];
-  int kKey[K_CH], kOff[K_CH];
+  int kOff[K_CH], kVoff[K_CH];
+  const int cK = (tid % CPR) * 8;
 #pragma unroll
   for (int i = 0; i < K_CH; ++i) {
     int chunk = tid + 256 * i;
     int key = chunk / CPR, c = chunk % CPR;
-    kKey[i] = key;
     kOff[i] = key * D + ((c ^ kSwizzle<D>(key)) << 3);
+    kVoff[i] = (key * (int)a.kTok + cK) * (int)sizeof(T);
   }
-  const int cK = (tid % CPR) * 8;
   const bool vActive = tid < 16 * (D / 8);
   const int vKg = tid & 15, vDc = tid >> 4;
   Frag vr[4];
+  int vVoff[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) vVoff[j] = ((vKg * 4 + j) * (int)a.vTok + vDc * 8) * (int)sizeof(T);
+  const __amdgpu_buffer_rsrc_t rsK = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T*>(kg), 0, (int)(((int64_t)(len - 1) * a.kTok + D) * sizeof(T)), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsV = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T*>(vg), 0, (int)(((int64_t)(len - 1) * a.vTok + D) * sizeof(T)), 0x00020000);
 
   auto gload = [&](int t) {
-    const int k0 = t * kCaBKV;
+    const int kS = t * kCaBKV * (int)a.kTok * (int)sizeof(T), vS = t * kCaBKV * (int)a.vTok * (int)sizeof(T);
 #pragma unroll
-    for (int i = 0; i < K_CH; ++i) {
-      int key = min(k0 + kKey[i], len - 1);
-      kr[i] = *reinterpret_cast<const Frag*>(kg + (int64_t)key * a.kTok + cK);
-    }
+    for (int i = 0; i < K_CH; ++i)
+      kr[i] = __builtin_bit_cast(Frag, __builtin_amdgcn_raw_buffer_load_b128(rsK, kVoff[i], kS, 0));
     if (vActive) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        int key = min(k0 + vKg * 4 + j, len - 1);
-        vr[j] = *reinterpret_cast<const Frag*>(vg + (int64_t)key * a.vTok + vDc * 8);
-      }
+      for (int j = 0; j < 4; ++j)
+        vr[j] = __builtin_bit_cast(Frag, __builtin_amdgcn_raw_buffer_load_b128(rsV, vVoff[j], vS, 0));
     }
   };
   auto swrite = [&](int stage) {
@@ -189,13 +194,17 @@ __global__ __launch_bounds__(256, 2) void contextAttnMfmaKernel(CaArgs a) {
       const T* vt = sVt + cur * V_STAGE;
       f32x16 s[2];
 #pragma unroll
-      for (int kt2 = 0; kt2 < 2; ++kt2) {
+      for (int kt2 = 0; kt2 < 2; ++kt2)
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[kt2][r] = 0.f;
-        const int key = kt2 * 32 + l31;
+      // the two 32-key halves are independent accumulation chains: alternate them so that no MFMA
+      // waits for the one issued just before it
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const int chunk = ks * 2 + half;
+      for (int ks = 0; ks < KS; ++ks) {
+        const int chunk = ks * 2 + half;
+#pragma unroll
+        for (int kt2 = 0; kt2 < 2; ++kt2) {
+          const int key = kt2 * 32 + l31;
           Frag kf = *reinterpret_cast<const Frag*>(k + key * D + ((chunk ^ kSwizzle<D>(key)) << 3));
           s[kt2] = CaMfma<T>::run(kf, qf[ks], s[kt2]);
         }
@@ -413,7 +422,9 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiContextAtten
     return t.aligned16() && (t.stride[0] * t.itemsize) % 16 == 0 && (t.stride[1] * t.itemsize) % 16 == 0;
   };
   diopiError_t err;
-  if (half && (a.d == 64 || a.d == 128) && al(cq) && al(ck) && al(cv) && al(co)) {
+  // the MFMA kernel addresses K and V rows of one sequence with 32-bit byte offsets
+  const bool fits32 = ((int64_t)maxInputLen + kCaBKV) * std::max(a.kTok, a.vTok) * (int64_t)q.itemsize < (int64_t)1 << 31;
+  if (half && (a.d == 64 || a.d == 128) && al(cq) && al(ck) && al(cv) && al(co) && fits32) {
     if (q.dtype == diopi_dtype_bfloat16)
       err = a.d == 128 ? launchCaMfma<bf16_t, 128>(stream, a, maxInputLen, batch) : launchCaMfma<bf16_t, 64>(stream, a, maxInputLen, batch);
     else
