@@ -81,8 +81,9 @@ __device__ __forceinline__ int kSwizzle(int key) {
 
 constexpr int kCaBQ = 128, kCaBKV = 64, kCaVtStride = 68;  // V^T rows padded to 68 keys (136 bytes)
 
+// One 128-query block of one (sequence, head): the whole flash-attention pass over its key tiles.
 template <typename T, int D>
-__global__ __launch_bounds__(256, 2) void contextAttnMfmaKernel(CaArgs a) {
+__device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb) {
   using Frag = typename CaMfma<T>::Frag;
   using Half = typename CaMfma<T>::Half;
   constexpr int KS = D / 16;        // MFMA k-steps over the head dim
@@ -98,7 +99,6 @@ __global__ __launch_bounds__(256, 2) void contextAttnMfmaKernel(CaArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l31 = lane & 31, half = lane >> 5;
   const int h = blockIdx.y, b = blockIdx.z;
-  const int qb = gridDim.x - 1 - blockIdx.x;  // heavy blocks first
   const int64_t start = ldIdxCA(a.bStart, b, a.start64);
   const int len = (int)ldIdxCA(a.bLen, b, a.len64);
   const int q0 = qb * kCaBQ;
@@ -250,26 +250,37 @@ __global__ __launch_bounds__(256, 2) void contextAttnMfmaKernel(CaArgs a) {
         m = mn;
       }
       l += ps;
-      // ---- O^T += V^T . P^T
+      // ---- O^T += V^T . P^T: 4 key groups of 16 x DT row tiles. The V^T fragment of MFMA i + kVAhead is
+      // read while MFMA i issues, and a scheduling fence after every MFMA keeps that order, so the LDS
+      // latency of a fragment is covered by the MFMAs in front of it.
+      {
+        constexpr int NPV = 4 * DT, kVAhead = 3;
+        auto vfrag = [&](int i) {
+          const int g = i / DT, dt = i % DT;  // key group (kt2 * 2 + t2), d tile
+          const T* row = vt + (dt * 32 + l31) * kCaVtStride + g * 16 + half * 4;
+          Half lo = *reinterpret_cast<const Half*>(row);
+          Half hi = *reinterpret_cast<const Half*>(row + 8);
+          Frag vf;
+          vf[0] = lo[0], vf[1] = lo[1], vf[2] = lo[2], vf[3] = lo[3];
+          vf[4] = hi[0], vf[5] = hi[1], vf[6] = hi[2], vf[7] = hi[3];
+          return vf;
+        };
+        Frag vfr[kVAhead + 1];
 #pragma unroll
-      for (int kt2 = 0; kt2 < 2; ++kt2)
+        for (int i = 0; i < kVAhead; ++i) vfr[i] = vfrag(i);
+        Frag pf;
 #pragma unroll
-        for (int t2 = 0; t2 < 2; ++t2) {
-          Frag pf;
+        for (int i = 0; i < NPV; ++i) {
+          const int g = i / DT, dt = i % DT;
+          if (dt == 0) {
 #pragma unroll
-          for (int j = 0; j < 8; ++j) pf[j] = static_cast<T>(s[kt2][8 * t2 + j]);
-          const int base = kt2 * 32 + t2 * 16 + half * 4;
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt) {
-            const T* row = vt + (dt * 32 + l31) * kCaVtStride + base;
-            Half lo = *reinterpret_cast<const Half*>(row);
-            Half hi = *reinterpret_cast<const Half*>(row + 8);
-            Frag vf;
-            vf[0] = lo[0], vf[1] = lo[1], vf[2] = lo[2], vf[3] = lo[3];
-            vf[4] = hi[0], vf[5] = hi[1], vf[6] = hi[2], vf[7] = hi[3];
-            o[dt] = CaMfma<T>::run(vf, pf, o[dt]);
+            for (int j = 0; j < 8; ++j) pf[j] = static_cast<T>(s[g >> 1][8 * (g & 1) + j]);
           }
+          if (i + kVAhead < NPV) vfr[(i + kVAhead) % (kVAhead + 1)] = vfrag(i + kVAhead);
+          o[dt] = CaMfma<T>::run(vfr[i % (kVAhead + 1)], pf, o[dt]);
+          __builtin_amdgcn_sched_barrier(0);
         }
+      }
     }
     if (t + 1 < ntiles) {
       swrite(cur ^ 1);
@@ -299,6 +310,22 @@ __global__ __launch_bounds__(256, 2) void contextAttnMfmaKernel(CaArgs a) {
     int row = chunk / CPR, c = chunk % CPR;
     int qrow = q0 + wave * 32 + row;
     if (qrow < len) *reinterpret_cast<Frag*>(og + (int64_t)qrow * a.oTok + c * 8) = *reinterpret_cast<const Frag*>(sO + row * OS + c * 8);
+  }
+}
+
+// Causal work grows linearly with the query block index, so a workgroup takes the heaviest remaining
+// block and then the lightest one: every workgroup streams the same number of key tiles, the grid is
+// an exact multiple of what the chip holds at typical shapes, and the blocks of one head still run
+// side by side and share their K/V tiles in L2.
+template <typename T, int D>
+__global__ __launch_bounds__(256, 2) void contextAttnMfmaKernel(CaArgs a, int numQBlocks) {
+  const int heavy = numQBlocks - 1 - (int)blockIdx.x, light = (int)blockIdx.x;
+  for (int pass = 0; pass < 2; ++pass) {
+    if (pass == 1) {
+      if (light == heavy) break;
+      __syncthreads();  // the first block's output staging aliases the K/V stages the second one fills
+    }
+    contextAttnBlock<T, D>(a, pass == 0 ? heavy : light);
   }
 }
 
@@ -359,8 +386,9 @@ static diopiError_t launchCaMfma(hipStream_t stream, const CaArgs& a, int maxLen
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     attrSet = true;
   }
-  dim3 grid((unsigned)ceilDiv(maxLen, kCaBQ), a.heads, (unsigned)batch);
-  hipLaunchKernelGGL((contextAttnMfmaKernel<T, D>), grid, dim3(256), lds, stream, a);
+  const int numQBlocks = (int)ceilDiv(maxLen, kCaBQ);
+  dim3 grid((unsigned)((numQBlocks + 1) / 2), a.heads, (unsigned)batch);
+  hipLaunchKernelGGL((contextAttnMfmaKernel<T, D>), grid, dim3(256), lds, stream, a, numQBlocks);
   AMD_LAUNCH_CHECK();
   return diopiSuccess;
 }
