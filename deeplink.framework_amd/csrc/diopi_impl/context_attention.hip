@@ -83,7 +83,7 @@ constexpr int kCaBQ = 128, kCaBKV = 64, kCaVtStride = 68;  // V^T rows padded to
 
 // One 128-query block of one (sequence, head): the whole flash-attention pass over its key tiles.
 template <typename T, int D>
-__device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb) {
+__device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, const int h, const int b) {
   using Frag = typename CaMfma<T>::Frag;
   using Half = typename CaMfma<T>::Half;
   constexpr int KS = D / 16;        // MFMA k-steps over the head dim
@@ -98,7 +98,6 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb) 
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l31 = lane & 31, half = lane >> 5;
-  const int h = blockIdx.y, b = blockIdx.z;
   const int64_t start = ldIdxCA(a.bStart, b, a.start64);
   const int len = (int)ldIdxCA(a.bLen, b, a.len64);
   const int q0 = qb * kCaBQ;
@@ -317,15 +316,32 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb) 
 // block and then the lightest one: every workgroup streams the same number of key tiles, the grid is
 // an exact multiple of what the chip holds at typical shapes, and the blocks of one head still run
 // side by side and share their K/V tiles in L2.
+//
+// Workgroups are dealt to the 8 XCDs round-robin by their linear id, and each XCD has its own L2. The
+// grid is therefore one-dimensional and decoded so that all workgroups of one (sequence, head), and
+// of neighbouring heads (which share K/V under grouped-query attention), land on the same XCD next to
+// each other in time: a K/V tile is fetched from HBM once and then served from that L2.
 template <typename T, int D>
-__global__ __launch_bounds__(256, 2) void contextAttnMfmaKernel(CaArgs a, int numQBlocks) {
-  const int heavy = numQBlocks - 1 - (int)blockIdx.x, light = (int)blockIdx.x;
+__global__ __launch_bounds__(256, 2) void contextAttnMfmaKernel(CaArgs a, int numQBlocks, int numSeq) {
+  const int pairs = (numQBlocks + 1) / 2, hb = a.heads * numSeq;
+  const int flat = (int)blockIdx.x;
+  int headSeq, pair;
+  if ((hb & 7) == 0) {
+    const int xcd = flat & 7, idx = flat >> 3;
+    headSeq = xcd * (hb >> 3) + idx / pairs;
+    pair = idx % pairs;
+  } else {
+    headSeq = flat / pairs;
+    pair = flat % pairs;
+  }
+  const int h = headSeq % a.heads, b = headSeq / a.heads;
+  const int heavy = numQBlocks - 1 - pair, light = pair;
   for (int pass = 0; pass < 2; ++pass) {
     if (pass == 1) {
       if (light == heavy) break;
       __syncthreads();  // the first block's output staging aliases the K/V stages the second one fills
     }
-    contextAttnBlock<T, D>(a, pass == 0 ? heavy : light);
+    contextAttnBlock<T, D>(a, pass == 0 ? heavy : light, h, b);
   }
 }
 
@@ -387,8 +403,9 @@ static diopiError_t launchCaMfma(hipStream_t stream, const CaArgs& a, int maxLen
     attrSet = true;
   }
   const int numQBlocks = (int)ceilDiv(maxLen, kCaBQ);
-  dim3 grid((unsigned)((numQBlocks + 1) / 2), a.heads, (unsigned)batch);
-  hipLaunchKernelGGL((contextAttnMfmaKernel<T, D>), grid, dim3(256), lds, stream, a, numQBlocks);
+  const int64_t blocks = (int64_t)((numQBlocks + 1) / 2) * a.heads * batch;
+  AMD_CHECK(blocks < ((int64_t)1 << 31), "context attention: grid limits exceeded");
+  hipLaunchKernelGGL((contextAttnMfmaKernel<T, D>), dim3((unsigned)blocks), dim3(256), lds, stream, a, numQBlocks, (int)batch);
   AMD_LAUNCH_CHECK();
   return diopiSuccess;
 }
