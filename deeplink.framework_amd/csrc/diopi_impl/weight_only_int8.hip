@@ -1,21 +1,26 @@
 // diopiWeightOnlyInt8Linear for gfx950: out[M,N] = x[M,K] . (W_int8[N,K] * scale[N])^T + bias.
 //
 // Skinny-M (decode) shape: the int8 weight matrix is streamed from HBM exactly once and is
-// the only traffic of size (K*N bytes); everything else (x, scale, out) is tiny and stays
-// in L2. The kernel is a GEMV-shaped MFMA kernel:
-//   * a workgroup owns 16 output channels; its 4 waves split K four ways; each
-//     wave keeps 8 weight + 16 activation vectors per lane in flight;
+// the only traffic of size (K*N bytes). The kernel is a GEMV-shaped MFMA kernel:
+//   * a workgroup owns NTW tiles of 16 output channels; each tile has 4 waves that split K
+//     four ways, so a workgroup is NTW*4 waves. NTW grows with N until the grid is about
+//     one workgroup per CU: the activations are then fetched once per CU instead of once
+//     per 16 channels (at M = 16 they are 3x the bytes of a 16-channel weight tile);
+//   * the (up to 16) activation rows the workgroup needs are staged once in LDS (rows padded
+//     by 16 bytes so the 16 rows of a fragment read fall in different banks) and read from
+//     there as MFMA A operands; K larger than the LDS budget is processed in chunks;
 //   * v_mfma_f32_16x16x32_{bf16,f16}: the B operand is the weight tile -- lane (n = lane%16,
 //     kgrp = lane/16) loads 32 consecutive int8 of row n (two 16-byte loads; the 4 kgrps of a
 //     row cover 128 contiguous bytes) and converts them to bf16/fp16 in registers while
-//     the next loads are in flight: the dequantisation is fused into the operand load;
-//   * the A operand is x (rows beyond M are clamped and discarded), read with the same
-//     K permutation as the weights, so no shuffle is needed;
-//   * fp32 accumulators of the 4 waves are summed through LDS; the per-channel scale is
-//     applied to the fp32 sum (identical to scaling the weights first, one rounding fewer),
+//     the next loads are in flight: the dequantisation is fused into the operand load.
+//     The first weight loads of a chunk are issued before the activations are staged;
+//   * fp32 accumulators of the 4 K-split waves are summed through LDS; the per-channel scale
+//     is applied to the fp32 sum (identical to scaling the weights first, one rounding fewer),
 //     then bias, then one conversion to the output dtype.
 // Rows of x beyond 16 are handled by more workgroups along grid.y (weights are then re-read
 // per group of 16 rows; large-M prefill should dequantise once and use the dense GEMM).
+#include <algorithm>
+
 #include "common.hpp"
 
 namespace amd {
@@ -36,6 +41,17 @@ struct W8Mfma<half_t> {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
 };
+
+static int computeUnitsW8() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
+}
 
 struct W8Args {
   const void* x;
@@ -60,55 +76,79 @@ __device__ __forceinline__ typename W8Mfma<T>::Frag cvt8(uint32_t lo, uint32_t h
   return f;
 }
 
-constexpr int kW8Block = 128;  // K elements one wave consumes per step (4 kgrps x 32)
-constexpr int kW8Unroll = 4;   // steps in flight
-constexpr int kW8Waves = 4;    // waves per workgroup = K splits (8 measured slower for M > 1)
+constexpr int kW8Block = 128;   // K elements one wave consumes per step (4 kgrps x 32)
+constexpr int kW8Unroll = 2;    // steps (4 weight loads per lane) in flight ahead of the MFMAs
+constexpr int kW8KSplit = 4;    // waves per 16-channel tile = K splits
+constexpr int kW8MaxTiles = 4;  // 16-channel tiles per workgroup (16 waves at most)
+constexpr int kW8Pad = 8;       // elements appended to every staged activation row (16 bytes)
+constexpr int kW8ChunkK = 4096; // activation columns staged per pass: 16 x (4096 + 8) x 2 B = 128.25 KiB
 
-template <typename T>
-__global__ __launch_bounds__(kW8Waves * 64) void w8LinearKernel(W8Args a) {
+template <typename T, int NTW>
+__global__ __launch_bounds__(NTW * kW8KSplit * 64) void w8LinearKernel(W8Args a) {
   using Frag = typename W8Mfma<T>::Frag;
+  constexpr int THREADS = NTW * kW8KSplit * 64;
+  extern __shared__ __attribute__((aligned(16))) char w8smem[];
+  T* sx = reinterpret_cast<T*>(w8smem);
+  __shared__ float red[NTW * kW8KSplit][64][4];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = wave / kW8KSplit, ks = wave % kW8KSplit;
   const int r16 = lane & 15, kgrp = lane >> 4;
-  const int n0 = blockIdx.x * 16, m0 = blockIdx.y * 16;
-  const int n = min(n0 + r16, a.N - 1);
-  const int m = min(m0 + r16, a.M - 1);
-  const int8_t* wrow = a.w + (int64_t)n * a.ldw + kgrp * 32;
-  const T* xrow = reinterpret_cast<const T*>(a.x) + (int64_t)m * a.ldx + kgrp * 32;
-  // K is split in kW8Waves contiguous parts (rounded to the 128-element step), one per wave; at
-  // K = 4096 a wave owns 4 steps, i.e. every load of the wave is issued in one go
-  const int steps = (a.K + kW8Block - 1) / kW8Block;
-  const int per = (steps + kW8Waves - 1) / kW8Waves;
-  const int sBegin = wave * per, sEnd = min(steps, sBegin + per);
+  const int n0 = (blockIdx.x * NTW + tile) * 16, m0 = blockIdx.y * 16;
+  const int rows = min(16, a.M - m0);
+  const int mrow = min(r16, rows - 1);  // fragment rows past M repeat the last row and are discarded
+  const int8_t* wrow = a.w + (int64_t)min(n0 + r16, a.N - 1) * a.ldw + kgrp * 32;
+  const T* xg = reinterpret_cast<const T*>(a.x) + (int64_t)m0 * a.ldx;
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int s = sBegin; s < sEnd; s += kW8Unroll) {
+  for (int kc = 0; kc < a.K; kc += kW8ChunkK) {
+    const int kcLen = min(kW8ChunkK, a.K - kc);  // a multiple of 128, as K is
+    const int ldx = kcLen + kW8Pad;
+    // this wave's share of the chunk: a contiguous run of 128-element steps
+    const int steps = kcLen / kW8Block;
+    const int per = (steps + kW8KSplit - 1) / kW8KSplit;
+    const int sBegin = ks * per, sEnd = min(steps, sBegin + per);
+    const int8_t* wk = wrow + kc;
+    // the first weight loads go out before the activations are staged
     u32x4 wv[kW8Unroll][2];
-    Frag xv[kW8Unroll][4];
 #pragma unroll
     for (int u = 0; u < kW8Unroll; ++u) {
-      const int k = (s + u) * kW8Block;
-      // K % 128 == 0 is guaranteed by the host, so a step is entirely inside or outside
-      const bool in = s + u < sEnd;
-      const int kk = in ? k : 0;
-      wv[u][0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow + kk));
-      wv[u][1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow + kk + 16));
-#pragma unroll
-      for (int j = 0; j < 4; ++j) xv[u][j] = *reinterpret_cast<const Frag*>(xrow + kk + j * 8);
+      const int kk = (sBegin + u < sEnd) ? (sBegin + u) * kW8Block : 0;
+      wv[u][0] = *reinterpret_cast<const u32x4*>(wk + kk);
+      wv[u][1] = *reinterpret_cast<const u32x4*>(wk + kk + 16);
     }
+    if (kc > 0) __syncthreads();  // everyone is done with the previous chunk's activations
+    const int cpr = kcLen / 8;
+    for (int i = threadIdx.x; i < rows * cpr; i += THREADS) {
+      const int r = i / cpr, c = i - r * cpr;
+      *reinterpret_cast<Frag*>(sx + r * ldx + c * 8) = *reinterpret_cast<const Frag*>(xg + (int64_t)r * a.ldx + kc + c * 8);
+    }
+    __syncthreads();
+    const T* xrow = sx + mrow * ldx + kgrp * 32;
+    for (int s = sBegin; s < sEnd; s += kW8Unroll) {
+      u32x4 wn[kW8Unroll][2];
 #pragma unroll
-    for (int u = 0; u < kW8Unroll; ++u) {
-      if (s + u < sEnd) {
-        acc = W8Mfma<T>::run(xv[u][0], cvt8<T>(wv[u][0][0], wv[u][0][1]), acc);
-        acc = W8Mfma<T>::run(xv[u][1], cvt8<T>(wv[u][0][2], wv[u][0][3]), acc);
-        acc = W8Mfma<T>::run(xv[u][2], cvt8<T>(wv[u][1][0], wv[u][1][1]), acc);
-        acc = W8Mfma<T>::run(xv[u][3], cvt8<T>(wv[u][1][2], wv[u][1][3]), acc);
+      for (int u = 0; u < kW8Unroll; ++u) {
+        const int kk = (s + kW8Unroll + u < sEnd) ? (s + kW8Unroll + u) * kW8Block : 0;
+        wn[u][0] = *reinterpret_cast<const u32x4*>(wk + kk);
+        wn[u][1] = *reinterpret_cast<const u32x4*>(wk + kk + 16);
       }
+#pragma unroll
+      for (int u = 0; u < kW8Unroll; ++u) {
+        if (s + u < sEnd) {
+          const T* xp = xrow + (s + u) * kW8Block;
+          acc = W8Mfma<T>::run(*reinterpret_cast<const Frag*>(xp), cvt8<T>(wv[u][0][0], wv[u][0][1]), acc);
+          acc = W8Mfma<T>::run(*reinterpret_cast<const Frag*>(xp + 8), cvt8<T>(wv[u][0][2], wv[u][0][3]), acc);
+          acc = W8Mfma<T>::run(*reinterpret_cast<const Frag*>(xp + 16), cvt8<T>(wv[u][1][0], wv[u][1][1]), acc);
+          acc = W8Mfma<T>::run(*reinterpret_cast<const Frag*>(xp + 24), cvt8<T>(wv[u][1][2], wv[u][1][3]), acc);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kW8Unroll; ++u) wv[u][0] = wn[u][0], wv[u][1] = wn[u][1];
     }
   }
-  __shared__ float red[kW8Waves][64][4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) red[wave][lane][r] = acc[r];
   __syncthreads();
-  if (wave == 0) {
+  if (ks == 0) {
     const int col = n0 + r16;
     if (col < a.N) {
       const float sc = loadAs<float>(a.scale, col, a.scaleDtype);
@@ -120,11 +160,41 @@ __global__ __launch_bounds__(kW8Waves * 64) void w8LinearKernel(W8Args a) {
         if (row < a.M) {
           float v = 0.f;
 #pragma unroll
-          for (int w = 0; w < kW8Waves; ++w) v += red[w][lane][r];
+          for (int w = 0; w < kW8KSplit; ++w) v += red[tile * kW8KSplit + w][lane][r];
           out[(int64_t)row * a.ldo + col] = static_cast<T>(v * sc + bv);
         }
       }
     }
+  }
+}
+
+template <typename T, int NTW>
+static diopiError_t launchW8(hipStream_t stream, const W8Args& a, size_t lds) {
+  static bool attrSet = false;  // the largest request (16 rows x one chunk) covers every later one
+  if (!attrSet) {
+    const int maxLds = 16 * (kW8ChunkK + kW8Pad) * (int)sizeof(T);
+    AMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&w8LinearKernel<T, NTW>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, maxLds));
+    attrSet = true;
+  }
+  const int tiles = (a.N + 15) / 16;
+  dim3 grid((unsigned)((tiles + NTW - 1) / NTW), (unsigned)((a.M + 15) / 16));
+  hipLaunchKernelGGL((w8LinearKernel<T, NTW>), grid, dim3(NTW * kW8KSplit * 64), lds, stream, a);
+  AMD_LAUNCH_CHECK();
+  return diopiSuccess;
+}
+
+template <typename T>
+static diopiError_t launchW8ForShape(hipStream_t stream, const W8Args& a) {
+  // 16-channel tiles per workgroup: enough to bring the grid down to about one workgroup per CU
+  const int tiles = (a.N + 15) / 16;
+  const int ntw = std::min(kW8MaxTiles, std::max(1, (tiles + computeUnitsW8() - 1) / computeUnitsW8()));
+  const size_t lds = (size_t)std::min(16, a.M) * (std::min(a.K, kW8ChunkK) + kW8Pad) * sizeof(T);
+  switch (ntw) {
+    case 1: return launchW8<T, 1>(stream, a, lds);
+    case 2: return launchW8<T, 2>(stream, a, lds);
+    case 3: return launchW8<T, 3>(stream, a, lds);
+    default: return launchW8<T, 4>(stream, a, lds);
   }
 }
 
@@ -196,9 +266,8 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiWeightOnlyIn
   a.scaleDtype = csc.dtype, a.biasDtype = bias.defined() ? cb.dtype : diopi_dtype_float32;
   const bool fast = K % kW8Block == 0 && cin.aligned16() && cw.aligned16() && a.ldw % 16 == 0 && ceilDiv(M, 16) <= 65535;
   if (fast) {
-    dim3 grid((unsigned)ceilDiv(N, 16), (unsigned)ceilDiv(M, 16));
-    if (in.dtype == diopi_dtype_bfloat16) hipLaunchKernelGGL(w8LinearKernel<bf16_t>, grid, dim3(kW8Waves * 64), 0, stream, a);
-    else hipLaunchKernelGGL(w8LinearKernel<half_t>, grid, dim3(kW8Waves * 64), 0, stream, a);
+    if (in.dtype == diopi_dtype_bfloat16) AMD_TRY(launchW8ForShape<bf16_t>(stream, a));
+    else AMD_TRY(launchW8ForShape<half_t>(stream, a));
   } else {
     dim3 grid((unsigned)ceilDiv(M * N, 256));
     if (in.dtype == diopi_dtype_bfloat16) hipLaunchKernelGGL(w8LinearScalarKernel<bf16_t>, grid, dim3(256), 0, stream, a);
