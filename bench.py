@@ -26,6 +26,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TF = 2500.0   # MI355X dense bf16, published
+# Bytes that leave L2 per GEMM launch (mean of the layer's 5 GEMMs), from two rocprofv3 --pmc runs of
+# `bench.py --only-layer` (FETCH_SIZE, then WRITE_SIZE), scaled by what the same counters read for a
+# 64 MiB device copy: (2 x 528 737 + 135 987) KiB. The summary is profiles/decoder_layer_hbm_traffic_counters.md;
+# a counter cannot be read from inside this process, so the figure is carried here as measured.
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 1_222_000_000
 
 
 def parse():
@@ -343,9 +348,9 @@ def main():
     gemm_flops = sum(flops.values())
     achieved_tf = gemm_flops / (gemm_time_us * 1e-6) / 1e12
     breakdown = {l: round(sum(v) / args.steps, 1) for l, v in per_op.items()}      # us per step (labels used twice are summed)
-    roofline = {"bound": "mfma", "kernel": "gemmMfmaKernel<bf16,256,256> (5 launches per step: qkv, o, gate, up, down)",
+    roofline = {"bound": "mfma", "kernel": "gemmMfmaPipelinedKernel<bf16> 256x256x64 (5 launches per step: qkv, o, gate, up, down)",
                 "achieved": round(achieved_tf, 1), "peak": MFMA_BF16_PEAK_TF, "unit": "TFLOP/s",
-                "frac": round(achieved_tf / MFMA_BF16_PEAK_TF, 4), "traffic": None,
+                "frac": round(achieved_tf / MFMA_BF16_PEAK_TF, 4), "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH,
                 "flops_per_step": gemm_flops, "avg_launch_us": round(gemm_time_us / 5, 1),
                 "per_gemm_TFLOPs": {l: round(flops[l] / (sum(per_op[l]) / args.steps * 1e-6) / 1e12, 1) for l in gemm_labels}}
 

@@ -21,8 +21,11 @@
 //   * two workgroups per CU (<= 256 registers per lane) so one wave's softmax VALU work overlaps
 //     another's MFMAs; exp2 is the bare hardware instruction fed by one FMA; the O^T rescale is
 //     skipped while the running max does not move;
-//   * two LDS stages, register prefetch of the next tile, one LDS-only barrier per tile; the heaviest
-//     query blocks (end of the sequence) are scheduled first.
+//   * two LDS stages, register prefetch of the next tile through buffer descriptors (no per-row
+//     address arithmetic, rows past the sequence read as zero), one LDS-only barrier per tile;
+//   * causal work grows with the query block index: a workgroup processes the heaviest remaining
+//     block and then the lightest, so all workgroups stream the same number of key tiles; the
+//     one-dimensional grid is decoded so the workgroups of a head share one XCD (one L2).
 //   * the epilogue transposes O^T through LDS so global stores are 16-byte and coalesced.
 //
 // Scalar kernel: any dtype / head_dim, one workgroup per (query, head); correctness path

@@ -5,19 +5,24 @@
 // MFMA engine (bf16 / fp16 inputs, fp32 accumulate) -- C[M,N] = A[M,K] . B[N,K]^T with both
 // operands K-contiguous, which is exactly what v_mfma_f32_32x32x16_{bf16,f16} wants: every
 // lane feeds 8 consecutive K elements (one 16-byte LDS read) of one row.
-//   * workgroup = 256 threads = 4 waves in a 2x2 arrangement; macro tile BM x BN x 64
-//     (256x256 for large problems: each wave owns 128x128 = 4x4 MFMA tiles, 256 fp32
-//     accumulators per lane; 128x128 otherwise);
+//   * large problems: 256x256x64 macro tile, workgroup = 512 threads = 8 waves in a 2x4
+//     arrangement (wave tile 128x64 = 4x2 MFMA tiles, 128 fp32 accumulators per lane, two waves
+//     per SIMD so one wave's LDS traffic hides behind the other's MFMAs); small or ragged
+//     problems: 128x128 tiles with 4 waves;
 //   * global -> registers -> LDS with a two-stage LDS ring: tile k+1 is written to the other
 //     stage while tile k is being multiplied, tile k+2 is already in flight from HBM; one
-//     barrier per K tile;
+//     barrier per K tile that waits on LDS traffic only. Operand rows are addressed through
+//     buffer descriptors (32-bit lane offset + scalar K offset, rows past M / N read as zero);
+//   * fragments are double-buffered in registers and the MFMA / LDS-read / LDS-write / global-load
+//     interleave of a K tile is pinned with sched_group_barrier;
 //   * LDS rows are 128 bytes (64 elements) with the 16-byte chunk index XOR-swizzled by
 //     ((row >> 1) & 7): both the 16-byte stores of the staging step and the ds_read_b128 operand
 //     fetches (32 consecutive rows, same logical chunk) are bank-conflict free;
 //   * workgroup ids are remapped so that each of the 8 XCDs (own L2 each) works on a
 //     contiguous band of tiles, walked in groups of 8 tile-rows to reuse A and B from L2;
-//   * epilogue: alpha * acc + beta * C + bias, converted and stored straight from the
-//     accumulator layout.
+//   * epilogue: alpha * acc + beta * C + bias; in the 256x256 kernel the accumulators go through
+//     LDS strips so that C and the addend move in 16-byte row pieces (the 128x128 kernel stores
+//     straight from the accumulator layout).
 // Operands that are not K-contiguous (mm with a row-major mat2, bmm's second operand) are
 // transposed once into workspace by a tiled LDS transpose, then use the same engine.
 //

@@ -16,11 +16,12 @@
 //   * every lane group keeps its OWN running (max, sum, acc[8]) online-softmax state, so the
 //     inner loop needs no cross-group traffic: per token only the log2(LPT) butterfly steps
 //     of the dot product;
-//   * K and V loads of an iteration are issued together, before any math, 4 + 4 wave-loads
-//     (8 KiB) in flight per wave; the slot indices of the NEXT iteration are fetched before
-//     the math of the current one, hiding the index -> address dependency;
-//   * a workgroup = 4 waves owns a chunk of the sequence (split-KV); states are merged by
-//     wave butterflies, then through LDS, then across chunks by a small second kernel.
+//   * two-deep pipeline: while iteration i does its math, the K and V rows of iteration i + 1
+//     (4 + 4 wave-loads, 8 KiB per wave) and the slot indices of iteration i + 2 are in flight,
+//     so neither the row latency nor the index -> address dependency is exposed;
+//   * a workgroup = 4 waves owns a chunk of the sequence (split-KV, chunks of at least 512
+//     tokens and at most 64 per sequence); states are merged by wave butterflies, then through
+//     LDS, then across chunks by a small lane-parallel second kernel.
 #include <algorithm>
 
 #include "common.hpp"
