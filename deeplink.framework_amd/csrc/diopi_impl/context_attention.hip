@@ -230,17 +230,13 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
         for (int r = 0; r < 16; ++r) mt = fmaxf(mt, s[kt2][r]);
       mt = fmaxf(mt, __shfl_xor(mt, 32, 64)) * scale2;  // scale2 > 0, so the max commutes with the scaling
       const float mn = fmaxf(m, mt);  // key 0 is visible to every query, so mn is finite from tile 0 on
-      float ps = 0.f;
 #pragma unroll
       for (int kt2 = 0; kt2 < 2; ++kt2)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           // one fused multiply-add and one hardware exp2 per score; masked scores give exp2(-inf) = 0
-          float p = __builtin_amdgcn_exp2f(fmaf(s[kt2][r], scale2, -mn));
-          s[kt2][r] = p;
-          ps += p;
+          s[kt2][r] = __builtin_amdgcn_exp2f(fmaf(s[kt2][r], scale2, -mn));
         }
-      ps += __shfl_xor(ps, 32, 64);
       // the running max rarely moves after the first tiles: rescale only when some lane needs it
       if (__builtin_amdgcn_ballot_w64(mn > m) != 0) {
         const float corr = __builtin_amdgcn_exp2f(m - mn);
@@ -251,7 +247,6 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
           for (int r = 0; r < 16; ++r) o[dt][r] *= corr;
         m = mn;
       }
-      l += ps;
       // ---- O^T += V^T . P^T: 4 key groups of 16 x DT row tiles. The V^T fragment of MFMA i + kVAhead is
       // read while MFMA i issues, and a scheduling fence after every MFMA keeps that order, so the LDS
       // latency of a fragment is covered by the MFMAs in front of it.
@@ -270,18 +265,28 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
         Frag vfr[kVAhead + 1];
 #pragma unroll
         for (int i = 0; i < kVAhead; ++i) vfr[i] = vfrag(i);
-        Frag pf;
+        // The softmax denominator comes off the matrix pipe too: a V^T row of ones makes every
+        // accumulator of lsum the sum of this query's (rounded) probabilities over the 16 keys of a
+        // group, which takes 32 additions per tile off the VALU, the unit this kernel is bound by.
+        Frag pf, ones;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ones[j] = static_cast<T>(1.0f);
+        f32x16 lsum;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) lsum[r] = 0.f;
 #pragma unroll
         for (int i = 0; i < NPV; ++i) {
           const int g = i / DT, dt = i % DT;
           if (dt == 0) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) pf[j] = static_cast<T>(s[g >> 1][8 * (g & 1) + j]);
+            lsum = CaMfma<T>::run(ones, pf, lsum);
           }
           if (i + kVAhead < NPV) vfr[(i + kVAhead) % (kVAhead + 1)] = vfrag(i + kVAhead);
           o[dt] = CaMfma<T>::run(vfr[i % (kVAhead + 1)], pf, o[dt]);
           __builtin_amdgcn_sched_barrier(0);
         }
+        l += lsum[0];
       }
     }
     if (t + 1 < ntiles) {
