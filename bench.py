@@ -5,7 +5,7 @@
 
 One "step" is one pass of a Llama-2-7B-shaped decoder layer (prefill, batch 4 x seq 2048,
 hidden 4096, 32 heads x 128, FFN 11008, bf16, random weights, synthetic activations) through
-the DIOPI C ABI of libdiopi_impl.so: RMSNorm -> QKV linear -> rotary(q,k) -> causal context
+the DIOPI C ABI of libdiopi_impl.so: RMSNorm -> QKV linear -> rotary (q and k heads in one launch) -> causal context
 attention -> out linear + residual (addmm) -> RMSNorm -> gate/up linears -> SiLU*mul -> down linear +
 residual (addmm). Inputs and weights are resident in HBM before the timed region.
 
@@ -91,7 +91,8 @@ def layer_plan(pkg, torch, dev, x, p, cfg):
     bf = x.dtype
     new = lambda *shape: torch.empty(*shape, dtype=bf, device=dev)
     h1, qkv, attn, o, x1, h2 = new(T, hidden), new(T, 3 * hidden), new(T, heads, hd), new(T, hidden), new(T, hidden), new(T, hidden)
-    qr, kr = new(T, heads, hd), new(T, heads, hd)
+    qk_rot = new(T, 2 * heads, hd)  # rotated q heads then rotated k heads of a token, one rotary launch for both
+    qr, kr = qk_rot[:, :heads], qk_rot[:, heads:]
     gate, up, act, down, out = new(T, ffn), new(T, ffn), new(T, ffn), new(T, hidden), new(T, hidden)
     cos, sin = pkg.workloads.rotary_tables(hd, s, cfg["theta"], dtype=bf)
     cos, sin = cos.to(dev), sin.to(dev)
@@ -99,15 +100,14 @@ def layer_plan(pkg, torch, dev, x, p, cfg):
     lens = torch.full((b,), s, dtype=torch.int32).to(dev)
     x2 = x.reshape(T, hidden)
     q, k, v = qkv.split(hidden, dim=-1)
-    q4, k4 = q.reshape(b, s, heads, hd), k.reshape(b, s, heads, hd)
+    qk4 = qkv[:, :2 * hidden].view(b, s, 2 * heads, hd)  # q and k are neighbours in the fused projection's output
     v3 = v.reshape(T, heads, hd)
     one = d.scalar(1)
     P = lambda name, *a: Prepared(pkg, name, *a)
     plan = [
         ("rms_norm", P("diopiRMSNorm", h1, None, x2, d.size([hidden]), p["norm1"], None, float(cfg["eps"]))),
         ("gemm_qkv", P("diopiLinear", qkv, h1, p["wqkv"], None)),
-        ("rotary_q", P("diopiRotaryEmbedding", qr.view(b, s, heads, hd), q4, cos, sin, False, False)),
-        ("rotary_k", P("diopiRotaryEmbedding", kr.view(b, s, heads, hd), k4, cos, sin, False, False)),
+        ("rotary_qk", P("diopiRotaryEmbedding", qk_rot.view(b, s, 2 * heads, hd), qk4, cos, sin, False, False)),
         ("context_attention", P("diopiContextAttentionInference", attn, qr, kr, v3, starts, lens, int(s))),
         # out projection with the residual folded into the GEMM epilogue: x1 = x + attn @ Wo^T (aten::addmm)
         ("gemm_o", P("diopiAddmm", x1, x2, attn.view(T, hidden), p["wo"].t(), one, one)),
@@ -117,7 +117,7 @@ def layer_plan(pkg, torch, dev, x, p, cfg):
         ("silu_mul", P("diopiSiluMul", act, gate, up)),
         ("gemm_down", P("diopiAddmm", out, x1, act, p["wdown"].t(), one, one)),
     ]
-    keep = [h1, qkv, attn, o, x1, h2, qr, kr, gate, up, act, down, out, cos, sin, starts, lens, x2]
+    keep = [h1, qkv, attn, o, x1, h2, qk_rot, qr, kr, gate, up, act, down, out, cos, sin, starts, lens, x2]
     flops = {"gemm_qkv": 2 * T * 3 * hidden * hidden, "gemm_o": 2 * T * hidden * hidden, "gemm_gate": 2 * T * ffn * hidden,
              "gemm_up": 2 * T * ffn * hidden, "gemm_down": 2 * T * hidden * ffn}
     return plan, keep, flops, out
