@@ -136,6 +136,22 @@ def test_context_attention_uniform_keys_give_running_mean_at_length_2048(ops, de
     run_mean = torch.cumsum(v.float(), 0) / torch.arange(1, n + 1).view(-1, 1, 1)
     assert_half(got, run_mean)
 
+def test_context_attention_long_ragged_batch_paired_blocks(ops, dev):
+    """Ragged sequences up to 2048 tokens with grouped-query heads: exercises the heavy + light query-block pairing
+    (odd and even block counts, sequences shorter than the longest one) and the workgroup decoding used when
+    heads x sequences is a multiple of 8."""
+    lens = [1000, 2048, 517]
+    heads, kvh, d = 8, 2, 128
+    starts = [0, 1000, 3048]
+    total = sum(lens)
+    q = torch.randn(total, heads, d, generator=g(27)).bfloat16()
+    k = torch.randn(total, kvh, d, generator=g(28)).bfloat16()
+    v = torch.randn(total, kvh, d, generator=g(29)).bfloat16()
+    st, ln = torch.tensor(starts, dtype=torch.int32), torch.tensor(lens, dtype=torch.int32)
+    want = oracle.context_attention(q.float(), k.float(), v.float(), st, ln)
+    got = ops.context_attention(q.to(dev), k.to(dev), v.to(dev), st.to(dev), ln.to(dev), max(lens))
+    assert_half(got, want)
+
 
 # ------------------------------------------------------------------ decode attention
 @pytest.mark.parametrize("dtype,d,idt", [(torch.bfloat16, 128, torch.int32), (torch.float16, 64, torch.int64),
