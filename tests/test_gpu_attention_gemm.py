@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from oracle import cpu_fallback as oracle
-from tests.decoder import run_decoder_block
+from tests.decoder import run_decoder_block, run_decomposed_decoder_block
 from tests.parity import assert_close, assert_exact, assert_fp32, assert_half
 
 pytestmark = pytest.mark.gpu
@@ -257,4 +257,18 @@ def test_small_decoder_block_bf16(ops, dev, pkg):
     want, _ = oracle.decoder_block(x.float(), {k: v.float() for k, v in p.items()}, cfg["heads"], cfg["eps"], cfg["theta"])
     got, _ = run_decoder_block(ops, x.to(dev), {k: v.to(dev) for k, v in p.items()}, cfg, fused_ffn=True)
     # eleven chained bf16 roundings: 3e-2 relative / 3e-2 absolute on an O(1) output
+    assert_half(got, want, rel=3e-2, abs_=3e-2)
+
+
+def test_decoder_block_from_primitive_ops_only(ops, dev, pkg):
+    """No fused ext op: RMSNorm, rotary tables and rotation, causal mask and attention all come from primitive
+    diopi ops (pow, mean, rsqrt, arange, exp, cos, sin, cat, comparisons, masked_fill, softmax, bmm, strided copies)."""
+    x, p, cfg = pkg.workloads.tiny_block(seed=1)
+    want, _ = oracle.decoder_block(x, p, cfg["heads"], cfg["eps"], cfg["theta"])
+    got = run_decomposed_decoder_block(ops, x.to(dev), {k: v.to(dev) for k, v in p.items()}, cfg)
+    # the decomposed rotary tables come from exp() on the device instead of pow() on the host: 2e-5 on the tensor scale
+    assert_fp32(got, want, rel=2e-5)
+    x, p, cfg = pkg.workloads.llama7b_layer(seed=2, batch=2, seq=128, hidden=512, heads=4, ffn=1408)
+    want, _ = oracle.decoder_block(x.float(), {k: v.float() for k, v in p.items()}, cfg["heads"], cfg["eps"], cfg["theta"])
+    got = run_decomposed_decoder_block(ops, x.to(dev), {k: v.to(dev) for k, v in p.items()}, cfg)
     assert_half(got, want, rel=3e-2, abs_=3e-2)
