@@ -31,7 +31,6 @@
 // Scalar kernel: any dtype / head_dim, one workgroup per (query, head); correctness path
 // for fp32 and odd head sizes.
 #include <algorithm>
-#include <type_traits>
 
 #include "common.hpp"
 
@@ -62,7 +61,6 @@ template <>
 struct CaMfma<bf16_t> {
   typedef bf16x8 Frag;
   typedef bf16x4 Half;
-  typedef __bf16 Pair __attribute__((ext_vector_type(2)));
   static __device__ __forceinline__ f32x16 run(Frag a, Frag b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
@@ -71,7 +69,6 @@ template <>
 struct CaMfma<half_t> {
   typedef f16x8 Frag;
   typedef f16x4 Half;
-  typedef _Float16 Pair __attribute__((ext_vector_type(2)));
   static __device__ __forceinline__ f32x16 run(Frag a, Frag b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
@@ -356,341 +353,6 @@ __global__ __launch_bounds__(256, 2) void contextAttnMfmaKernel(CaArgs a, int nu
   }
 }
 
-// ---------------------------------------------------------------- ping-pong kernel
-// Two waves share a SIMD. Left to themselves they drift into the same phase (both in their MFMAs, then
-// both in their softmax), and the matrix pipe and the VALU take turns instead of overlapping. Here the
-// two waves of a SIMD belong to one workgroup of 8 waves = 2 groups of 4, and the groups run half a tile
-// apart, separated by barriers: while one group issues the MFMAs of a tile (P.V of tile t, then the raw
-// scores of tile t + 1, 36 MFMAs back to back at raised priority), the other runs its softmax on the
-// VALU (max, exp2, conversion of P to the MFMA operand format, rescale of O). The workgroup owns 256
-// queries, so a staged K/V tile serves twice the queries of the kernel above and the staging work per
-// thread halves. The eight 32-query slices are dealt to the groups alternately, which keeps their causal
-// extents equal.
-//
-//   half-period hp:      0      1      2      3      4   ...
-//   group 0:           V(0)   M(0)   V(1)   M(1)   V(2)        V(t) = softmax of tile t
-//   group 1:           S(0)   V(0)   M(0)   V(1)   M(1)        M(t) = P.V of tile t, scores of tile t + 1
-//   all threads:              stage         stage              stage at hp = 2t + 1: K(t+2), V(t+1) -> LDS,
-//                                                                 loads of K(t+3), V(t+2) issued
-// K stage j & 1 holds K(j), V stage j & 1 holds V(j); a stage is rewritten one barrier after its last reader.
-constexpr int kPpBQ = 256, kPpThreads = 512;
-// V^T rows in this kernel: 72 keys (144 bytes, a multiple of 16) and, inside every group of 16 keys, the order
-// 0-3, 8-11, 4-7, 12-15: the 8 keys a lane feeds to one P.V MFMA (two runs of 4, 8 apart, because P^T comes
-// straight from the score accumulators) are then contiguous and arrive with one 16-byte LDS read.
-constexpr int kPpVtStride = 72;
-__device__ __forceinline__ int ppKeySlot(int key) { return (key & ~12) | ((key & 4) << 1) | ((key & 8) >> 1); }
-
-template <typename T, int D>
-__device__ __forceinline__ void contextAttnPingPongBlock(const CaArgs& a, const int qb, const int h, const int b) {
-  using Frag = typename CaMfma<T>::Frag;
-  using Half = typename CaMfma<T>::Half;
-  using Pair = typename CaMfma<T>::Pair;
-  constexpr int KS = D / 16;        // MFMA k-steps over the head dim
-  constexpr int DT = D / 32;        // 32-row tiles of O^T
-  constexpr int CPR = D / 8;        // 16-byte chunks per K row
-  constexpr int K_CH = kCaBKV * CPR / kPpThreads;  // K chunks per thread
-  constexpr int K_STAGE = kCaBKV * D;               // elements
-  constexpr int V_STAGE = D * kPpVtStride;
-  static_assert(K_CH >= 1, "every thread stages at least one K chunk");
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-  T* sK = reinterpret_cast<T*>(smem);   // [2][64][D] swizzled
-  T* sVt = sK + 2 * K_STAGE;            // [2][D][72]
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int l31 = lane & 31, half = lane >> 5;
-  const int group = wave >> 2;             // ping-pong group
-  const int sb = 2 * (wave & 3) + group;   // this wave's 32-query slice of the block
-  const int64_t start = ldIdxCA(a.bStart, b, a.start64);
-  const int len = (int)ldIdxCA(a.bLen, b, a.len64);
-  const int q0 = qb * kPpBQ;
-  if (q0 >= len) return;
-  const int kvh = h / (a.heads / a.kvHeads);
-  const T* qg = reinterpret_cast<const T*>(a.q) + start * a.qTok + (int64_t)h * a.qHead;
-  const T* kg = reinterpret_cast<const T*>(a.k) + start * a.kTok + (int64_t)kvh * a.kHead;
-  const T* vg = reinterpret_cast<const T*>(a.v) + start * a.vTok + (int64_t)kvh * a.vHead;
-
-  const int qw0 = q0 + sb * 32;              // first query of the wave
-  const int qi = qw0 + l31;                  // this lane's query (column of S^T)
-  const int qiC = min(qi, len - 1);          // rows past the sequence compute on the last row, never stored
-  Frag qf[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks)
-    qf[ks] = *reinterpret_cast<const Frag*>(qg + (int64_t)qiC * a.qTok + ks * 16 + half * 8);
-
-  const int ntiles = (min(len, q0 + kPpBQ) + kCaBKV - 1) / kCaBKV;
-  const int waveMaxQ = min(qw0 + 31, len - 1);
-  // K fragment of (k-step ks, key half kt2) sits at byte  kt2 * 32 rows + (kFragLane ^ (ks << 5))  of a K stage:
-  // the chunk index 2 ks + half, XORed with the row's swizzle, equals (2 ks) ^ (half ^ swizzle) because 2 ks has
-  // bit 0 clear, so one XOR with a per-lane constant replaces a table of sixteen addresses.
-  const int kFragLane = l31 * D * (int)sizeof(T) + ((half ^ kSwizzle<D>(l31)) << 4);
-  static_assert(D == 128 || D == 64, "swizzle algebra below assumes these row sizes");
-
-  // ---- staging roles (all 512 threads): buffer descriptors ending at the sequence's last row
-  Frag kr[K_CH];
-  int kOff[K_CH], kVoff[K_CH];
-  const int cK = (tid % CPR) * 8;
-#pragma unroll
-  for (int i = 0; i < K_CH; ++i) {
-    int chunk = tid + kPpThreads * i;
-    int key = chunk / CPR, c = chunk % CPR;
-    kOff[i] = key * D + ((c ^ kSwizzle<D>(key)) << 3);
-    kVoff[i] = (key * (int)a.kTok + cK) * (int)sizeof(T);
-  }
-  // V: a thread moves 2 keys x 8 d and writes them transposed (8 stores of one key pair)
-  const int vKp = tid & 31, vDc = tid >> 5;
-  const bool vActive = vDc < CPR;
-  Frag vr[2];
-  int vVoff[2];
-#pragma unroll
-  for (int j = 0; j < 2; ++j) vVoff[j] = ((vKp * 2 + j) * (int)a.vTok + vDc * 8) * (int)sizeof(T);
-  const __amdgpu_buffer_rsrc_t rsK = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<T*>(kg), 0, (int)(((int64_t)(len - 1) * a.kTok + D) * sizeof(T)), 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsV = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<T*>(vg), 0, (int)(((int64_t)(len - 1) * a.vTok + D) * sizeof(T)), 0x00020000);
-  auto gloadK = [&](int t) {
-    const int kS = t * kCaBKV * (int)a.kTok * (int)sizeof(T);
-#pragma unroll
-    for (int i = 0; i < K_CH; ++i)
-      kr[i] = __builtin_bit_cast(Frag, __builtin_amdgcn_raw_buffer_load_b128(rsK, kVoff[i], kS, 0));
-  };
-  auto gloadV = [&](int t) {
-    const int vS = t * kCaBKV * (int)a.vTok * (int)sizeof(T);
-    if (vActive) {
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-        vr[j] = __builtin_bit_cast(Frag, __builtin_amdgcn_raw_buffer_load_b128(rsV, vVoff[j], vS, 0));
-    }
-  };
-  auto swriteK = [&](int stage) {
-    T* k = sK + stage * K_STAGE;
-#pragma unroll
-    for (int i = 0; i < K_CH; ++i) *reinterpret_cast<Frag*>(k + kOff[i]) = kr[i];
-  };
-  auto swriteV = [&](int stage) {
-    T* vt = sVt + stage * V_STAGE;
-    if (vActive) {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        Pair p;
-        p[0] = vr[0][e], p[1] = vr[1][e];
-        *reinterpret_cast<Pair*>(vt + (vDc * 8 + e) * kPpVtStride + ppKeySlot(vKp * 2)) = p;
-      }
-    }
-  };
-  auto ldsBarrier = []() {
-    __builtin_amdgcn_s_waitcnt(0xc07f);
-    __builtin_amdgcn_s_barrier();
-  };
-
-  f32x16 o[DT], s[2];
-  Frag pf[4];
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) o[dt][r] = 0.f;
-  float m = -INFINITY, l = 0.f;
-  const float scale2 = a.scale * kLog2eCA;
-
-  // raw scores S^T = K . Q^T of the tile in K stage `stage`: two alternating accumulation chains
-  auto scoreTile = [&](int stage) {
-    const char* k = reinterpret_cast<const char*>(sK + stage * K_STAGE);
-#pragma unroll
-    for (int kt2 = 0; kt2 < 2; ++kt2)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) s[kt2][r] = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-#pragma unroll
-      for (int kt2 = 0; kt2 < 2; ++kt2) {
-        Frag kf = *reinterpret_cast<const Frag*>(k + kt2 * 32 * D * (int)sizeof(T) + (kFragLane ^ (ks << 5)));
-        s[kt2] = CaMfma<T>::run(kf, qf[ks], s[kt2]);
-      }
-    }
-  };
-  // V(t): online softmax of this lane's query over the 64 keys of tile t; leaves P in pf
-  auto softmaxPhase = [&](int t) {
-    const int k0 = t * kCaBKV;
-    if (k0 > waveMaxQ) return;  // wave-uniform
-    const bool needMask = (k0 + kCaBKV - 1 > qw0) || (k0 + kCaBKV > len);
-    if (needMask) {
-#pragma unroll
-      for (int kt2 = 0; kt2 < 2; ++kt2)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          int kj = k0 + kt2 * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-          if (kj > qiC || kj >= len) s[kt2][r] = -INFINITY;
-        }
-    }
-    float mt = -INFINITY;
-#pragma unroll
-    for (int kt2 = 0; kt2 < 2; ++kt2)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) mt = fmaxf(mt, s[kt2][r]);
-    mt = fmaxf(mt, __shfl_xor(mt, 32, 64)) * scale2;  // scale2 > 0, so the max commutes with the scaling
-    const float mn = fmaxf(m, mt);  // key 0 is visible to every query, so mn is finite from tile 0 on
-    float ps = 0.f;
-#pragma unroll
-    for (int g = 0; g < 4; ++g)
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float p = __builtin_amdgcn_exp2f(fmaf(s[g >> 1][8 * (g & 1) + j], scale2, -mn));
-        pf[g][j] = static_cast<T>(p);
-        ps += p;
-      }
-    ps += __shfl_xor(ps, 32, 64);
-    if (__builtin_amdgcn_ballot_w64(mn > m) != 0) {
-      const float corr = __builtin_amdgcn_exp2f(m - mn);
-      l *= corr;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) o[dt][r] *= corr;
-      m = mn;
-    }
-    l += ps;
-  };
-  // M(t): O^T += V^T . P^T for tile t (DT accumulation chains) interleaved with the raw scores of tile t + 1
-  // (2 chains), so that no MFMA waits for the result of a recent one.
-  // Operand fragments are read kAhead MFMAs of their own stream ahead; a scheduling fence after every MFMA
-  // keeps the order.
-  auto mfmaPhase = [&](auto hasNext, int t) {
-    constexpr bool kNext = decltype(hasNext)::value;
-    constexpr int NS = 2 * KS, kAhead = 3;
-    __builtin_amdgcn_s_setprio(2);
-    const T* vt = sVt + (t & 1) * V_STAGE;
-    const T* kn = sK + ((t + 1) & 1) * K_STAGE;
-    auto vfrag = [&](int iv) {  // iv = key group * DT + d tile
-      const int g = iv / DT, dt = iv % DT;
-      return *reinterpret_cast<const Frag*>(vt + (dt * 32 + l31) * kPpVtStride + g * 16 + half * 8);
-    };
-    auto kfrag = [&](int i) {   // i = k-step * 2 + key half
-      const char* base = reinterpret_cast<const char*>(kn) + (i & 1) * 32 * D * (int)sizeof(T);
-      return *reinterpret_cast<const Frag*>(base + (kFragLane ^ ((i >> 1) << 5)));
-    };
-    Frag vfr[kAhead + 1], kfr[kAhead + 1];
-#pragma unroll
-    for (int i = 0; i < kAhead; ++i) vfr[i] = vfrag(i);
-    if constexpr (kNext) {
-#pragma unroll
-      for (int i = 0; i < kAhead; ++i) kfr[i] = kfrag(i);
-#pragma unroll
-      for (int kt2 = 0; kt2 < 2; ++kt2)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) s[kt2][r] = 0.f;
-    }
-    auto pSlot = [&](int iv) {  // P.V stream: key group iv / DT, row tile iv % DT
-      if (iv + kAhead < 4 * DT) vfr[(iv + kAhead) % (kAhead + 1)] = vfrag(iv + kAhead);
-      o[iv % DT] = CaMfma<T>::run(vfr[iv % (kAhead + 1)], pf[iv / DT], o[iv % DT]);
-      __builtin_amdgcn_sched_barrier(0);
-    };
-    auto sSlot = [&](int i) {  // score stream of the next tile
-      if (i + kAhead < NS) kfr[(i + kAhead) % (kAhead + 1)] = kfrag(i + kAhead);
-      s[i & 1] = CaMfma<T>::run(kfr[i % (kAhead + 1)], qf[i >> 1], s[i & 1]);
-      __builtin_amdgcn_sched_barrier(0);
-    };
-    constexpr int NPV = 4 * DT;
-    if constexpr (kNext) {
-      // merge the two streams proportionally: after every MFMA issue the one whose stream is furthest behind
-      int ip = 0, is = 0;
-#pragma unroll
-      for (int n = 0; n < NPV + NS; ++n) {
-        if (is * NPV < ip * NS || ip >= NPV) {
-          if (is < NS) sSlot(is++);
-        } else {
-          pSlot(ip++);
-        }
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < NPV; ++i) pSlot(i);
-    }
-    __builtin_amdgcn_s_setprio(0);
-  };
-
-  gloadK(0);
-  gloadV(0);
-  swriteK(0);
-  swriteV(0);
-  gloadK(1);
-  swriteK(1);
-  gloadK(2);
-  gloadV(1);
-  ldsBarrier();
-  if (group == 0) scoreTile(0);  // key 0 is visible to every query: tile 0 is active for every wave
-  const int halfPeriods = 2 * ntiles + 1;
-  for (int hp = 0; hp < halfPeriods; ++hp) {
-    if (hp & 1) {
-      const int t = hp >> 1;
-      swriteK(t & 1);         // K(t + 2)
-      swriteV((t + 1) & 1);   // V(t + 1)
-      gloadK(t + 3);          // rows past the sequence read as zeros
-      gloadV(t + 2);
-    }
-    const int x = hp - group;  // position in this group's own V(0) M(0) V(1) M(1) ... sequence
-    if (x < 0) {
-      scoreTile(0);
-    } else if (x < 2 * ntiles) {
-      const int t = x >> 1;
-      if (x & 1) {
-        if (t * kCaBKV <= waveMaxQ) {  // wave-uniform, as is the choice of variant
-          if (t + 1 < ntiles && (t + 1) * kCaBKV <= waveMaxQ) mfmaPhase(std::true_type{}, t);
-          else mfmaPhase(std::false_type{}, t);
-        }
-      } else {
-        softmaxPhase(t);
-      }
-    }
-    ldsBarrier();
-  }
-
-  // ---- epilogue: O^T (lane = query) -> LDS [query][d] -> coalesced 16-byte stores
-  constexpr int OS = D + 8;  // padded row, elements
-  T* sO = reinterpret_cast<T*>(smem) + wave * 32 * OS;
-  const float inv = l > 0.f ? 1.f / l : 0.f;
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      Half p;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) p[e] = static_cast<T>(o[dt][g * 4 + e] * inv);
-      *reinterpret_cast<Half*>(sO + l31 * OS + dt * 32 + g * 8 + half * 4) = p;
-    }
-  __syncthreads();
-  T* og = reinterpret_cast<T*>(a.out) + start * a.oTok + (int64_t)h * a.oHead;
-#pragma unroll
-  for (int i = 0; i < 32 * CPR / 64; ++i) {
-    int chunk = lane + 64 * i;
-    int row = chunk / CPR, c = chunk % CPR;
-    int qrow = qw0 + row;
-    if (qrow < len) *reinterpret_cast<Frag*>(og + (int64_t)qrow * a.oTok + c * 8) = *reinterpret_cast<const Frag*>(sO + row * OS + c * 8);
-  }
-}
-
-template <typename T, int D>
-__global__ __launch_bounds__(kPpThreads) void contextAttnPingPongKernel(CaArgs a, int numQBlocks, int numSeq) {
-  const int pairs = (numQBlocks + 1) / 2, hb = a.heads * numSeq;
-  const int flat = (int)blockIdx.x;
-  int headSeq, pair;
-  if ((hb & 7) == 0) {  // same XCD-aware decoding as contextAttnMfmaKernel
-    const int xcd = flat & 7, idx = flat >> 3;
-    headSeq = xcd * (hb >> 3) + idx / pairs;
-    pair = idx % pairs;
-  } else {
-    headSeq = flat / pairs;
-    pair = flat % pairs;
-  }
-  const int h = headSeq % a.heads, b = headSeq / a.heads;
-  const int heavy = numQBlocks - 1 - pair, light = pair;
-  for (int pass = 0; pass < 2; ++pass) {
-    if (pass == 1) {
-      if (light == heavy) break;
-      __syncthreads();  // the first block's output staging aliases the K/V stages the second one fills
-    }
-    contextAttnPingPongBlock<T, D>(a, pass == 0 ? heavy : light, h, b);
-  }
-}
-
 // One workgroup per (query token, head): scores to LDS, softmax, then P.V with lanes over d.
 template <typename T>
 __global__ __launch_bounds__(256) void contextAttnScalarKernel(CaArgs a, int maxLen) {
@@ -756,26 +418,6 @@ static diopiError_t launchCaMfma(hipStream_t stream, const CaArgs& a, int maxLen
   return diopiSuccess;
 }
 
-template <typename T, int D>
-static diopiError_t launchCaPingPong(hipStream_t stream, const CaArgs& a, int maxLen, int64_t batch) {
-  constexpr size_t stages = 2 * (size_t)(kCaBKV * D + D * kPpVtStride) * sizeof(T);
-  constexpr size_t staging = (size_t)(kPpThreads / 64) * 32 * (D + 8) * sizeof(T);  // output rows of the 8 waves
-  constexpr size_t lds = stages > staging ? stages : staging;
-  static bool attrSet = false;
-  if (!attrSet) {
-    AMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&contextAttnPingPongKernel<T, D>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attrSet = true;
-  }
-  const int numQBlocks = (int)ceilDiv(maxLen, kPpBQ);
-  const int64_t blocks = (int64_t)((numQBlocks + 1) / 2) * a.heads * batch;
-  AMD_CHECK(blocks < ((int64_t)1 << 31), "context attention: grid limits exceeded");
-  hipLaunchKernelGGL((contextAttnPingPongKernel<T, D>), dim3((unsigned)blocks), dim3(kPpThreads), lds, stream, a, numQBlocks,
-                     (int)batch);
-  AMD_LAUNCH_CHECK();
-  return diopiSuccess;
-}
-
 }  // namespace amd
 
 using namespace amd;
@@ -836,15 +478,10 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiContextAtten
   // the MFMA kernel addresses K and V rows of one sequence with 32-bit byte offsets
   const bool fits32 = ((int64_t)maxInputLen + kCaBKV) * std::max(a.kTok, a.vTok) * (int64_t)q.itemsize < (int64_t)1 << 31;
   if (half && (a.d == 64 || a.d == 128) && al(cq) && al(ck) && al(cv) && al(co) && fits32) {
-    // sequences longer than one 128-query block: 256-query blocks with the two wave groups in ping-pong
-    const bool pp = maxInputLen > kCaBQ;
-    if (q.dtype == diopi_dtype_bfloat16) {
-      if (a.d == 128) err = pp ? launchCaPingPong<bf16_t, 128>(stream, a, maxInputLen, batch) : launchCaMfma<bf16_t, 128>(stream, a, maxInputLen, batch);
-      else err = pp ? launchCaPingPong<bf16_t, 64>(stream, a, maxInputLen, batch) : launchCaMfma<bf16_t, 64>(stream, a, maxInputLen, batch);
-    } else {
-      if (a.d == 128) err = pp ? launchCaPingPong<half_t, 128>(stream, a, maxInputLen, batch) : launchCaMfma<half_t, 128>(stream, a, maxInputLen, batch);
-      else err = pp ? launchCaPingPong<half_t, 64>(stream, a, maxInputLen, batch) : launchCaMfma<half_t, 64>(stream, a, maxInputLen, batch);
-    }
+    if (q.dtype == diopi_dtype_bfloat16)
+      err = a.d == 128 ? launchCaMfma<bf16_t, 128>(stream, a, maxInputLen, batch) : launchCaMfma<bf16_t, 64>(stream, a, maxInputLen, batch);
+    else
+      err = a.d == 128 ? launchCaMfma<half_t, 128>(stream, a, maxInputLen, batch) : launchCaMfma<half_t, 64>(stream, a, maxInputLen, batch);
   } else {
     AMD_CHECK(maxInputLen <= 12000, "context attention: the scalar path supports sequences up to 12000 tokens, got %d", maxInputLen);
     AMD_CHECK(maxInputLen <= 65535, "context attention: grid limits exceeded");
