@@ -280,9 +280,25 @@ def cpu_baseline(pkg, torch):
         oracle.decoder_block(x, p, cfg["heads"], cfg["eps"], cfg["theta"])
         times.append(time.perf_counter() - t0)
     t = min(times)
+    # What DIPU's CPU fallback adds per op on top of the CPU kernel: operands to the host and the result back
+    # (dipu/torch_dipu/csrc_dipu/aten/ops/DIPUCopy.hpp:282-325, pageable memory, stream-synchronous). One
+    # [4, 2048, 4096] bf16 activation each way is timed here; a layer run op by op through the fallback pays about
+    # this much for every one of its operands.
+    dev = torch.device("cuda:0")
+    xd = x.to(dev)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    xh = xd.cpu()
+    d2h = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    xh.to(dev)
+    torch.cuda.synchronize()
+    h2d = time.perf_counter() - t0
     return {"value": round(8192 / t, 2), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
             "sample": f"the same layer and batch (4 x 2048 tokens) through the oracle: stock ATen CPU kernels in bf16, best of {reps} "
-                      f"passes after a warm-up, {t:.2f} s per pass"}
+                      f"passes after a warm-up, {t:.2f} s per pass",
+            "fallback_copy_ms": {"tensor": "bf16 [4, 2048, 4096] (64 MiB), pageable host memory", "d2h": round(d2h * 1e3, 2),
+                                 "h2d": round(h2d * 1e3, 2)}}
 
 
 def main():
