@@ -3,26 +3,30 @@
 // 1534-1548,1755-1765,1829-1837,1852-1893).
 //
 // MFMA engine (bf16 / fp16 inputs, fp32 accumulate) -- C[M,N] = A[M,K] . B[N,K]^T with both
-// operands K-contiguous, which is exactly what v_mfma_f32_32x32x16_{bf16,f16} wants: every
-// lane feeds 8 consecutive K elements (one 16-byte LDS read) of one row.
-//   * large problems: 256x256x64 macro tile, workgroup = 512 threads = 8 waves in a 2x4
-//     arrangement (wave tile 128x64 = 4x2 MFMA tiles, 128 fp32 accumulators per lane, two waves
-//     per SIMD so one wave's LDS traffic hides behind the other's MFMAs); small or ragged
-//     problems: 128x128 tiles with 4 waves;
-//   * global -> registers -> LDS with a two-stage LDS ring: tile k+1 is written to the other
-//     stage while tile k is being multiplied, tile k+2 is already in flight from HBM; one
-//     barrier per K tile that waits on LDS traffic only. Operand rows are addressed through
-//     buffer descriptors (32-bit lane offset + scalar K offset, rows past M / N read as zero);
-//   * fragments are double-buffered in registers and the MFMA / LDS-read / LDS-write / global-load
-//     interleave of a K tile is pinned with sched_group_barrier;
+// operands K-contiguous, which is exactly what the MFMA instructions want: every lane feeds 8
+// consecutive K elements (one 16-byte LDS read) of one row.
+//   * large problems (K a multiple of 64): 256x256x64 macro tile, workgroup = 512 threads = 8 waves
+//     in a 2x4 arrangement (wave tile 128x64 = 8x4 tiles of v_mfma_f32_16x16x32, 128 fp32
+//     accumulators per lane, two waves per SIMD so one wave's LDS traffic hides behind the other's
+//     MFMAs). The 16x16x32 shape draws less power per flop than 32x32x16 (an MFMA-only loop holds
+//     ~2.02 GHz against ~1.86 GHz on random operands), and this kernel runs at the power limit;
+//   * its operand tiles go from memory straight into a two-stage LDS ring (buffer_load ... lds, no
+//     registers and no ds_write in between): tile k+1 lands in the other stage while tile k is
+//     being multiplied, and the loads of tile k+2 start as soon as every wave is past the one
+//     barrier per K tile. Operand rows are addressed through buffer descriptors (32-bit lane offset
+//     + scalar K offset);
+//   * fragments are double-buffered (A) or refilled in place (B) in registers and the order of
+//     MFMAs, fragment reads and tile loads is pinned in groups of four MFMAs;
 //   * LDS rows are 128 bytes (64 elements) with the 16-byte chunk index XOR-swizzled by
-//     ((row >> 1) & 7): both the 16-byte stores of the staging step and the ds_read_b128 operand
-//     fetches (32 consecutive rows, same logical chunk) are bank-conflict free;
+//     ((row >> 1) & 7): the 1 KiB blocks written by the tile loads and the ds_read_b128 operand
+//     fetches (16 consecutive rows, 4 consecutive logical chunks) are bank-conflict free;
 //   * workgroup ids are remapped so that each of the 8 XCDs (own L2 each) works on a
 //     contiguous band of tiles, walked in groups of 8 tile-rows to reuse A and B from L2;
-//   * epilogue: alpha * acc + beta * C + bias; in the 256x256 kernel the accumulators go through
-//     LDS strips so that C and the addend move in 16-byte row pieces (the 128x128 kernel stores
-//     straight from the accumulator layout).
+//   * epilogue: alpha * acc + beta * C + bias; the accumulators go through LDS strips so that C
+//     and the addend move in 16-byte row pieces;
+//   * small or ragged problems: 128x128 (or 256x256) tiles with 4 waves of v_mfma_f32_32x32x16,
+//     staged through registers, any K that is a multiple of 8, stores straight from the
+//     accumulator layout.
 // Operands that are not K-contiguous (mm with a row-major mat2, bmm's second operand) are
 // transposed once into workspace by a tiled LDS transpose, then use the same engine.
 //
@@ -215,37 +219,65 @@ __global__ __launch_bounds__(256) void gemmMfmaKernel(MfmaArgs g) {
 }
 
 // ------------------------------------------------- software-pipelined 256x256 ---
-// Same macro tile and LDS layout as gemmMfmaKernel<T,256,256>, for K a multiple of 64 with at
-// least two K tiles, with the instruction stream of every wave arranged by hand so it does
-// not wait on LDS or HBM inside the K loop:
-//   k-step 0: MFMAs of step 0 | operand fetches of step 1 | LDS stores of the next A tile
-//   k-step 1: MFMAs of step 1 | operand fetches of step 2 | LDS stores of the next B tile
-//   k-step 2: MFMAs of step 2 | operand fetches of step 3 | HBM loads of the tile after next
-//   barrier (LDS only: the HBM loads stay in flight across it)
-//   k-step 3: MFMAs of step 3 | operand fetches of step 0 of the next tile
-// Operand fragments are double-buffered in registers; sched_group_barrier pins the
-// MFMA / LDS / VMEM interleave inside each k-step.
+// For K a multiple of 64 with at least two K tiles. Same LDS layout as gemmMfmaKernel<T,256,256>;
+// the instruction stream of every wave is arranged by hand in four phases of 16 MFMAs per K tile
+// so that it does not wait on LDS or HBM inside the K loop:
+//   phase 0: k-step 0, rows 0-63   | A fragments of phase 1
+//   phase 1: k-step 0, rows 64-127 | A fragments of phase 2, B fragments of k-step 1
+//   phase 2: k-step 1, rows 0-63   | A fragments of phase 3
+//   wait for this wave's tile loads, barrier: the next tile is published, this stage is free
+//   phase 3: k-step 1, rows 64-127 | A and B fragments of phase 0 of the next tile |
+//            direct-to-LDS loads of the tile after next into the stage just freed
 __device__ __forceinline__ void ldsBarrier() {
   // wait for this wave's LDS traffic only (lgkmcnt(0)); outstanding global loads keep flying
   __builtin_amdgcn_s_waitcnt(0xc07f);
   __builtin_amdgcn_s_barrier();
 }
 
-#define SGB_MFMA(n) __builtin_amdgcn_sched_group_barrier(0x008, n, 0)
-#define SGB_DSRD(n) __builtin_amdgcn_sched_group_barrier(0x100, n, 0)
-#define SGB_DSWR(n) __builtin_amdgcn_sched_group_barrier(0x200, n, 0)
-#define SGB_VMRD(n) __builtin_amdgcn_sched_group_barrier(0x020, n, 0)
 
 // 8 waves (2 x 4, wave tile 128 x 64): two waves per SIMD, so one wave's LDS / VMEM issue
 // overlaps the other's MFMAs; measured faster than 4 waves of 128 x 128 and 16 of 64 x 64.
 constexpr int kPipeWavesM = 2, kPipeWavesN = 4, kPipeThreads = kPipeWavesM * kPipeWavesN * 64;
 
+// v_mfma_f32_16x16x32: lane l feeds row (l & 15), K elements [8 * (l >> 4), +8) of both operands and
+// receives C[4 * (l >> 4) + r][l & 15], r = 0..3.
+template <typename T>
+struct MfmaOp16;
+template <>
+struct MfmaOp16<bf16_t> {
+  static __device__ __forceinline__ f32x4 run(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct MfmaOp16<half_t> {
+  static __device__ __forceinline__ f32x4 run(f16x8 a, f16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+// buffer_load_dwordx4 ... lds: lane l of the wave fetches 16 bytes at rsrc + voffset + soffset and the
+// data lands in LDS at ldsAddr + 16 * l without passing through registers. Issued as inline assembly so
+// that the compiler does not order it against fragment reads of the other stage; the kernel waits for
+// these loads itself (vmcnt) before the barrier that publishes a stage.
+__device__ __forceinline__ void loadToLds16(u32x4 rsrc, int voffset, int soffset, unsigned ldsAddr) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "buffer_load_dwordx4 %1, %2, %3 offen lds"
+      :
+      : "s"(ldsAddr), "v"(voffset), "s"(rsrc), "s"(soffset)
+      : "memory", "m0");
+}
+
 template <typename T>
 __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs g) {
   using Frag = typename MfmaOp<T>::Frag;
-  constexpr int BM = 256, BN = 256, WM = BM / kPipeWavesM, WN = BN / kPipeWavesN, TM = WM / 32, TN = WN / 32;
+  constexpr int BM = 256, BN = 256, WM = BM / kPipeWavesM, WN = BN / kPipeWavesN, TM = WM / 16, TN = WN / 16;
+  constexpr int HM = TM / 2;               // A fragments of one phase (half of the wave's rows)
   constexpr int CH = 2048 / kPipeThreads;  // 16-byte chunks per thread per operand tile
   constexpr int RS = kPipeThreads / 8;     // rows covered by one pass of the workgroup
+  static_assert(HM == 4 && TN == 4 && CH == 4, "the phase schedule below is written for 4 x 4 fragments");
   extern __shared__ __attribute__((aligned(16))) char smem[];
   T* sA = reinterpret_cast<T*>(smem);  // [2][BM][64]
   T* sB = sA + 2 * BM * kBK;           // [2][BN][64]
@@ -270,133 +302,150 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
   const int batch = blockIdx.z;
   const T* A = reinterpret_cast<const T*>(g.A) + (int64_t)batch * g.sAb;
   const T* B = reinterpret_cast<const T*>(g.B) + (int64_t)batch * g.sBb;
-  // Operands are read through buffer descriptors: a 32-bit per-lane byte offset fixed for the whole
-  // K loop plus a scalar K offset per tile, so the loop carries no 64-bit address arithmetic.
+  // Operand tiles go from memory straight into LDS: lane l of a wave fills the l-th 16-byte slot of a
+  // 1 KiB block (8 rows of 128 bytes), so the chunk swizzle is applied on the global side: the lane
+  // that owns physical slot (row, c) fetches logical chunk c ^ ((row >> 1) & 7). A 32-bit per-lane
+  // byte offset is fixed for the whole K loop and a scalar K offset moves per tile; rows past M / N
+  // are clamped to the last row (their products are never stored).
   // (The host guarantees both operands span less than 2 GiB.)
-  __amdgpu_buffer_rsrc_t rsA =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(A), 0, (int)(((int64_t)(g.M - 1) * g.lda + g.K) * 2), 0x00020000);
-  __amdgpu_buffer_rsrc_t rsB =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(B), 0, (int)(((int64_t)(g.N - 1) * g.ldb + g.K) * 2), 0x00020000);
+  auto descriptor = [](const T* base, int64_t bytes) {
+    const uint64_t p = reinterpret_cast<uint64_t>(base);
+    u32x4 d = {(uint32_t)p, (uint32_t)(p >> 32) & 0xffffu, (uint32_t)bytes, 0x00020000u};
+    return d;
+  };
+  const u32x4 rsA = descriptor(A, ((int64_t)(g.M - 1) * g.lda + g.K) * 2);
+  const u32x4 rsB = descriptor(B, ((int64_t)(g.N - 1) * g.ldb + g.K) * 2);
   int aOffG[CH], bOffG[CH];
-  const int c8 = (tid & 7) * 8;
-  const int srow = tid >> 3;  // staging row of chunk 0; chunk i is RS rows further
-  const int sOff = srow * kBK + (((tid & 7) ^ ((srow >> 1) & 7)) << 3);  // rows RS apart share the swizzle
+  const int srow = tid >> 3;  // staging row of chunk 0; chunk i is RS rows further (same swizzle)
+  const int c8 = ((tid & 7) ^ ((srow >> 1) & 7)) * 8;
 #pragma unroll
   for (int i = 0; i < CH; ++i) {
     aOffG[i] = (int)(((int64_t)min(tm * BM + srow + RS * i, g.M - 1) * g.lda + c8) * 2);
     bOffG[i] = (int)(((int64_t)min(tn * BN + srow + RS * i, g.N - 1) * g.ldb + c8) * 2);
   }
-  Frag ra[CH], rb[CH];
+  // LDS byte address of this wave's 1 KiB block in stage 0 of A; stage 1 is kStageBytes further, B 2 * kStageBytes
+  constexpr unsigned kStageBytes = BM * kBK * sizeof(T), kPassBytes = RS * kBK * sizeof(T);
+  const unsigned ldsWave = (unsigned)(size_t)(__attribute__((address_space(3))) char*)smem +
+                           __builtin_amdgcn_readfirstlane(wave) * 1024u;
   const int nK = g.K / kBK;
 
-  const int frow = lane & 31, fhalf = lane >> 5;
-  const int swz = (frow >> 1) & 7;
-  int kx[4];  // swizzled element offset of this lane's chunk for each k-step
+  const int frow = lane & 15, kq = lane >> 4;
+  const int swz = (frow >> 1) & 7;  // fragment rows are 16 apart: they all share this lane's swizzle
+  int kx[2];                        // swizzled element offset of this lane's chunk for each 32-wide k-step
 #pragma unroll
-  for (int ks = 0; ks < 4; ++ks) kx[ks] = ((2 * ks + fhalf) ^ swz) << 3;
+  for (int ks = 0; ks < 2; ++ks) kx[ks] = ((4 * ks + kq) ^ swz) << 3;
   const int aBase = (wm * WM + frow) * kBK, bBase = (wn * WN + frow) * kBK;
 
-  Frag fa[2][TM], fb[2][TN];
-  f32x16 acc[TM][TN];
+  Frag fa[2][HM], fb[TN];
+  f32x4 acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 
-  auto gload = [&](int kt) {
-    const int k0 = kt * kBK * (int)sizeof(T);
-#pragma unroll
-    for (int i = 0; i < CH; ++i) ra[i] = __builtin_bit_cast(Frag, __builtin_amdgcn_raw_buffer_load_b128(rsA, aOffG[i], k0, 0));
-#pragma unroll
-    for (int i = 0; i < CH; ++i) rb[i] = __builtin_bit_cast(Frag, __builtin_amdgcn_raw_buffer_load_b128(rsB, bOffG[i], k0, 0));
+  auto dmaA = [&](int stage, int kt, int i) {
+    loadToLds16(rsA, aOffG[i], kt * kBK * (int)sizeof(T), ldsWave + stage * kStageBytes + i * kPassBytes);
   };
-  auto swriteA = [&](int stage) {
-    T* a = sA + stage * BM * kBK + sOff;
-#pragma unroll
-    for (int i = 0; i < CH; ++i) *reinterpret_cast<Frag*>(a + i * RS * kBK) = ra[i];
+  auto dmaB = [&](int stage, int kt, int i) {
+    loadToLds16(rsB, bOffG[i], kt * kBK * (int)sizeof(T), ldsWave + (2 + stage) * kStageBytes + i * kPassBytes);
   };
-  auto swriteB = [&](int stage) {
-    T* b = sB + stage * BN * kBK + sOff;
-#pragma unroll
-    for (int i = 0; i < CH; ++i) *reinterpret_cast<Frag*>(b + i * RS * kBK) = rb[i];
+  auto loadA = [&](int stage, int ks, int half, int buf, int i) {
+    fa[buf][i] = *reinterpret_cast<const Frag*>(sA + stage * BM * kBK + aBase + kx[ks] + (half * HM + i) * 16 * kBK);
   };
-  auto lfrag = [&](int stage, int ks, int buf) {
-    const T* a = sA + stage * BM * kBK + aBase + kx[ks];
-    const T* b = sB + stage * BN * kBK + bBase + kx[ks];
-#pragma unroll
-    for (int i = 0; i < TM; ++i) fa[buf][i] = *reinterpret_cast<const Frag*>(a + i * 32 * kBK);
-#pragma unroll
-    for (int j = 0; j < TN; ++j) fb[buf][j] = *reinterpret_cast<const Frag*>(b + j * 32 * kBK);
+  auto loadB = [&](int stage, int ks, int j) {
+    fb[j] = *reinterpret_cast<const Frag*>(sB + stage * BN * kBK + bBase + kx[ks] + j * 16 * kBK);
   };
-  auto mma = [&](int buf) {
+  // One phase = 16 MFMAs: half of the wave's rows (4 A fragments) against its 4 B fragments for
+  // one 32-wide k-step, B-major in four groups of four. B fragment j is dead after group j and is
+  // refilled in place for the next k-step; the A fragments of the next phase arrive in the other
+  // register buffer during the first two groups. Every group is fenced so the order holds.
+  auto phase = [&](int half, int buf, auto&& before, auto&& after) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int j = 0; j < TN; ++j) {
+      before(j);
 #pragma unroll
-      for (int j = 0; j < TN; ++j) acc[i][j] = MfmaOp<T>::run(fa[buf][i], fb[buf][j], acc[i][j]);
+      for (int i = 0; i < HM; ++i)
+        acc[half * HM + i][j] = MfmaOp16<T>::run(fa[buf][i], fb[j], acc[half * HM + i][j]);
+      after(j);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // Publishes a stage: this wave's loads into it have landed (vmcnt) and its fragment reads of the
+  // stage about to be refilled are done (lgkmcnt), then all waves meet.
+  auto publish = [&]() {
+    __builtin_amdgcn_s_waitcnt(0x0070);
+    __builtin_amdgcn_s_barrier();
   };
 
-  gload(0);
-  swriteA(0);
-  swriteB(0);
-  gload(1);
-  ldsBarrier();
-  lfrag(0, 0, 0);
+#pragma unroll
+  for (int i = 0; i < CH; ++i) dmaA(0, 0, i);
+#pragma unroll
+  for (int i = 0; i < CH; ++i) dmaB(0, 0, i);
+  publish();
+#pragma unroll
+  for (int i = 0; i < CH; ++i) dmaA(1, 1, i);
+#pragma unroll
+  for (int i = 0; i < CH; ++i) dmaB(1, 1, i);
+#pragma unroll
+  for (int j = 0; j < TN; ++j) loadB(0, 0, j);
+#pragma unroll
+  for (int i = 0; i < HM; ++i) loadA(0, 0, 0, 0, i);
 
-  // LDS fetches / LDS stores / HBM loads to place after every second MFMA of a k-step
-  constexpr int kRd = (2 * (TM + TN) + TM * TN - 1) / (TM * TN), kWr = (2 * CH + TM * TN - 1) / (TM * TN),
-                kVm = (4 * CH + TM * TN - 1) / (TM * TN);
+  // Iteration kt multiplies tile kt out of stage kt & 1. The tile after it is already landing in the
+  // other stage; once every wave has passed the barrier before phase 3 nobody reads this stage any
+  // more, so the loads of tile kt + 2 into it start right there: three phases in flight.
   auto iter = [&](auto hasNext, auto hasNext2, int kt) {
     constexpr bool kNext = decltype(hasNext)::value, kNext2 = decltype(hasNext2)::value;
     const int cur = kt & 1;
-    // ---- k-step 0
     __builtin_amdgcn_sched_barrier(0);
-    lfrag(cur, 1, 1);
-    if constexpr (kNext) swriteA(cur ^ 1);
-    mma(0);
-#pragma unroll
-    for (int i = 0; i < TM * TN / 2; ++i) {
-      SGB_MFMA(1);
-      SGB_DSRD(kRd);
-      SGB_MFMA(1);
-      if constexpr (kNext) SGB_DSWR(kWr);
-    }
-    // ---- k-step 1
+    // ---- phase 0: k-step 0, rows 0-63 | A fragments of phase 1
+    phase(0, 0,
+          [&](int j) {
+            if (j < 2) {
+              loadA(cur, 0, 1, 1, 2 * j);
+              loadA(cur, 0, 1, 1, 2 * j + 1);
+            }
+          },
+          [&](int) {});
+    // ---- phase 1: k-step 0, rows 64-127 | A of phase 2, B of k-step 1
+    phase(1, 1,
+          [&](int j) {
+            if (j < 2) {
+              loadA(cur, 1, 0, 0, 2 * j);
+              loadA(cur, 1, 0, 0, 2 * j + 1);
+            }
+          },
+          [&](int j) { loadB(cur, 1, j); });
+    // ---- phase 2: k-step 1, rows 0-63 | A of phase 3
+    phase(0, 0,
+          [&](int j) {
+            if (j < 2) {
+              loadA(cur, 1, 1, 1, 2 * j);
+              loadA(cur, 1, 1, 1, 2 * j + 1);
+            }
+          },
+          [&](int) {});
+    if constexpr (kNext) publish();
     __builtin_amdgcn_sched_barrier(0);
-    lfrag(cur, 2, 0);
-    if constexpr (kNext) swriteB(cur ^ 1);
-    mma(1);
-#pragma unroll
-    for (int i = 0; i < TM * TN / 2; ++i) {
-      SGB_MFMA(1);
-      SGB_DSRD(kRd);
-      SGB_MFMA(1);
-      if constexpr (kNext) SGB_DSWR(kWr);
-    }
-    // ---- k-step 2
-    __builtin_amdgcn_sched_barrier(0);
-    lfrag(cur, 3, 1);
-    if constexpr (kNext2) gload(kt + 2);
-    mma(0);
-#pragma unroll
-    for (int i = 0; i < TM * TN / 2; ++i) {
-      SGB_MFMA(1);
-      SGB_DSRD(kRd);
-      SGB_MFMA(1);
-      if constexpr (kNext2) SGB_VMRD(kVm);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    ldsBarrier();
-    // ---- k-step 3
-    if constexpr (kNext) lfrag(cur ^ 1, 0, 0);
-    mma(1);
-#pragma unroll
-    for (int i = 0; i < TM * TN / 2; ++i) {
-      SGB_MFMA(2);
-      if constexpr (kNext) SGB_DSRD(kRd);
-    }
-    __builtin_amdgcn_sched_barrier(0);
+    // ---- phase 3: k-step 1, rows 64-127 | A and B of phase 0 of the next tile | loads of tile kt + 2
+    phase(1, 1,
+          [&](int j) {
+            if constexpr (kNext2) {
+              dmaA(cur, kt + 2, j);
+              dmaB(cur, kt + 2, j);
+            }
+            if constexpr (kNext) {
+              if (j < 2) {
+                loadA(cur ^ 1, 0, 0, 0, 2 * j);
+                loadA(cur ^ 1, 0, 0, 0, 2 * j + 1);
+              }
+            }
+          },
+          [&](int j) {
+            if constexpr (kNext) loadB(cur ^ 1, 0, j);
+          });
   };
   using std::false_type;
   using std::true_type;
@@ -418,18 +467,19 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
     constexpr int GROUPS = WN / 8;                 // 8-column groups per strip row
     constexpr int ITEMS = 32 * GROUPS / 64;        // (row, group) items per lane
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
+    for (int ip = 0; ip < TM / 2; ++ip) {  // two 16-row fragment rows per strip
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
+      for (int ii = 0; ii < 2; ++ii)
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          strip[((r >> 2) * 8 + fhalf * 4 + (r & 3)) * RS4 + j * 32 + frow] = acc[i][j][r];
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) strip[(ii * 16 + kq * 4 + r) * RS4 + j * 16 + frow] = acc[2 * ip + ii][j][r];
       __builtin_amdgcn_s_waitcnt(0xc07f);  // the strip is private to this wave: no barrier, only its own LDS ops
 #pragma unroll
       for (int it = 0; it < ITEMS; ++it) {
         const int item = lane + 64 * it;
         const int srow = item / GROUPS, sg = item % GROUPS;
-        const int row = tm * BM + wm * WM + i * 32 + srow;
+        const int row = tm * BM + wm * WM + ip * 32 + srow;
         const int col = tn * BN + wn * WN + sg * 8;
         const f32x4 lo = *reinterpret_cast<const f32x4*>(strip + srow * RS4 + sg * 8);
         const f32x4 hi = *reinterpret_cast<const f32x4*>(strip + srow * RS4 + sg * 8 + 4);
@@ -455,15 +505,15 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
   }
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
-    const int col = tn * BN + wn * WN + j * 32 + frow;
+    const int col = tn * BN + wn * WN + j * 16 + frow;
     if (col >= g.N) continue;
     const float bv = bias ? static_cast<float>(bias[col]) : 0.f;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      const int rbase = tm * BM + wm * WM + i * 32 + fhalf * 4;
+      const int rbase = tm * BM + wm * WM + i * 16 + kq * 4;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = rbase + (r >> 2) * 8 + (r & 3);
+      for (int r = 0; r < 4; ++r) {
+        const int row = rbase + r;
         if (row < g.M) {
           float v = acc[i][j][r] * g.alpha + bv;
           if (cin) v += g.beta * static_cast<float>(cin[(int64_t)row * g.sCm + (int64_t)col * g.sCn]);

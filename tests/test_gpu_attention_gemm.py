@@ -88,6 +88,35 @@ def test_gemm_linearity_at_7b_shapes(ops, dev):
     assert_exact(ops.linear(onehot, w), w[:, cols].t().contiguous().cpu())
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,n,k", [(3500, 3700, 128), (3500, 3700, 192), (3841, 3585, 320), (4096, 4096, 1088)])
+def test_large_tile_gemm_edges_and_k_tile_counts(ops, dev, dtype, m, n, k):
+    """At least 200 tiles of 256 x 256 and K a multiple of 64 select the 8-wave kernel whose tiles are loaded
+    straight into LDS: two, three, five and seventeen K tiles (even and odd ring positions at the end),
+    ragged last tile rows / columns, bias, and the alpha / beta epilogue."""
+    x = torch.randn(m, k, generator=g(40)).to(dtype)
+    w = (torch.randn(n, k, generator=g(41)) * 0.05).to(dtype)
+    b = torch.randn(n, generator=g(42)).to(dtype)
+    want = x.float() @ w.float().t()
+    dx, dw = x.to(dev), w.to(dev)
+    assert_half(ops.linear(dx, dw), want)
+    assert_half(ops.linear(dx, dw, b.to(dev)), want + b.float())
+    c = torch.randn(m, n, generator=g(43)).to(dtype)
+    assert_half(ops.addmm(c.to(dev), dx, dw.t(), beta=0.5, alpha=2), 0.5 * c.float() + 2 * want)
+
+
+def test_large_tile_gemm_batched_and_row_strided_operands(ops, dev):
+    # 4 batches of 8 x 8 tiles; A rows taken out of a wider buffer (row stride > K), B shared by all batches
+    wide = torch.randn(4, 2000, 512, generator=g(44)).bfloat16().to(dev)
+    a = wide[:, :, 128:128 + 320]
+    assert not a.is_contiguous()
+    w = (torch.randn(1900, 320, generator=g(45)) * 0.05).bfloat16()
+    want = a.float().cpu() @ w.float().t()
+    assert_half(ops.matmul(a, w.to(dev).t()), want)
+    bb = (torch.randn(4, 1900, 320, generator=g(46)) * 0.05).bfloat16()
+    assert_half(ops.bmm(a, bb.to(dev).transpose(1, 2)), torch.bmm(a.float().cpu(), bb.float().transpose(1, 2)))
+
+
 # ------------------------------------------------------------------ prefill attention
 @pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 128), (torch.float16, 128), (torch.bfloat16, 64),
                                      (torch.float32, 64), (torch.float32, 40)])
