@@ -52,6 +52,11 @@ void setLastError(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 // Checked after every launch; clears nothing on success.
 #define AMD_LAUNCH_CHECK() AMD_HIP(hipGetLastError())
 
+// Raises a kernel's dynamic-LDS limit (kernels here use up to 128 KiB of the CU's 160 KiB; the
+// default limit is 64 KiB). Done once per (kernel, device); callable from any thread before
+// every launch.
+hipError_t allowDynamicLds(const void* kernel, int bytes);
+
 // ------------------------------------------------------------ tensor view ---
 struct TensorView {
   void* data = nullptr;

@@ -404,12 +404,7 @@ template <typename T, int D>
 static diopiError_t launchCaMfma(hipStream_t stream, const CaArgs& a, int maxLen, int64_t batch) {
   constexpr size_t lds = 2 * (size_t)(kCaBKV * D + D * kCaVtStride) * sizeof(T);
   static_assert(lds >= 4 * 32 * (D + 8) * sizeof(T), "epilogue staging must fit in the tile buffers");
-  static bool attrSet = false;
-  if (!attrSet) {
-    AMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&contextAttnMfmaKernel<T, D>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attrSet = true;
-  }
+  AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&contextAttnMfmaKernel<T, D>), (int)lds));
   const int numQBlocks = (int)ceilDiv(maxLen, kCaBQ);
   const int64_t blocks = (int64_t)((numQBlocks + 1) / 2) * a.heads * batch;
   AMD_CHECK(blocks < ((int64_t)1 << 31), "context attention: grid limits exceeded");

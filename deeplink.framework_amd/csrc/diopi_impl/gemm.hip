@@ -259,15 +259,20 @@ struct MfmaOp16<half_t> {
 // buffer_load_dwordx4 ... lds: lane l of the wave fetches 16 bytes at rsrc + voffset + soffset and the
 // data lands in LDS at ldsAddr + 16 * l without passing through registers. Issued as inline assembly so
 // that the compiler does not order it against fragment reads of the other stage; the kernel waits for
-// these loads itself (vmcnt) before the barrier that publishes a stage.
+// these loads itself (vmcnt) before the barrier that publishes a stage. The LDS address travels in M0,
+// which is read when the load issues; the previous M0 is put back so the statement has no side effect
+// on registers the compiler owns.
 __device__ __forceinline__ void loadToLds16(u32x4 rsrc, int voffset, int soffset, unsigned ldsAddr) {
+  unsigned savedM0;
   asm volatile(
-      "s_mov_b32 m0, %0\n\t"
+      "s_mov_b32 %0, m0\n\t"
+      "s_mov_b32 m0, %1\n\t"
       "s_nop 0\n\t"
-      "buffer_load_dwordx4 %1, %2, %3 offen lds"
-      :
+      "buffer_load_dwordx4 %2, %3, %4 offen lds\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(savedM0)
       : "s"(ldsAddr), "v"(voffset), "s"(rsrc), "s"(soffset)
-      : "memory", "m0");
+      : "memory");
 }
 
 template <typename T>
@@ -638,12 +643,7 @@ static diopiError_t launchMfma(hipStream_t stream, const GemmProblem& p) {
   g.alpha = p.alpha, g.beta = p.beta;
   g.vecEpilogue = false;
   constexpr size_t lds = 2 * (size_t)(BM + BN) * kBK * sizeof(T);
-  static bool attrSet = false;  // per template instance
-  if (!attrSet) {
-    AMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemmMfmaKernel<T, BM, BN>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attrSet = true;
-  }
+  AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmMfmaKernel<T, BM, BN>), (int)lds));
   dim3 grid((unsigned)(g.tilesM * g.tilesN), 1, (unsigned)p.batch);
   hipLaunchKernelGGL((gemmMfmaKernel<T, BM, BN>), grid, dim3(256), lds, stream, g);
   AMD_LAUNCH_CHECK();
@@ -663,12 +663,7 @@ static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p
   g.vecEpilogue = p.N % 8 == 0 && p.sOm % 8 == 0 && p.sOb % 8 == 0 && al16(p.out) &&
                   (!p.Cin || (p.sCn == 1 && p.sCm % 8 == 0 && p.sCb % 8 == 0 && al16(p.Cin))) && (!p.bias || al16(p.bias));
   constexpr size_t lds = 2 * (size_t)(256 + 256) * kBK * sizeof(T);
-  static bool attrSet = false;
-  if (!attrSet) {
-    AMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemmMfmaPipelinedKernel<T>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attrSet = true;
-  }
+  AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmMfmaPipelinedKernel<T>), (int)lds));
   dim3 grid((unsigned)(g.tilesM * g.tilesN), 1, (unsigned)p.batch);
   hipLaunchKernelGGL((gemmMfmaPipelinedKernel<T>), grid, dim3(kPipeThreads), lds, stream, g);
   AMD_LAUNCH_CHECK();

@@ -2,6 +2,9 @@
 // The impl library only ever learns about a tensor through these callbacks
 // (dipu/torch_dipu/csrc_dipu/diopirt/diopirt_impl.cpp:24-173 is the provider in DIPU).
 #include <cstring>
+#include <mutex>
+#include <set>
+#include <utility>
 
 #include "common.hpp"
 
@@ -19,6 +22,19 @@ void setLastError(const char* fmt, ...) {
 }
 
 const char* lastError() { return g_last_error; }
+
+hipError_t allowDynamicLds(const void* kernel, int bytes) {
+  static std::mutex mu;
+  static std::set<std::pair<const void*, int>> done;  // (kernel, device)
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return e;
+  std::lock_guard<std::mutex> lock(mu);
+  if (done.count({kernel, device})) return hipSuccess;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess) done.insert({kernel, device});
+  return e;
+}
 
 int64_t dtypeSize(diopiDtype_t dt) {
   switch (dt) {

@@ -170,13 +170,8 @@ __global__ __launch_bounds__(NTW * kW8KSplit * 64) void w8LinearKernel(W8Args a)
 
 template <typename T, int NTW>
 static diopiError_t launchW8(hipStream_t stream, const W8Args& a, size_t lds) {
-  static bool attrSet = false;  // the largest request (16 rows x one chunk) covers every later one
-  if (!attrSet) {
-    const int maxLds = 16 * (kW8ChunkK + kW8Pad) * (int)sizeof(T);
-    AMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&w8LinearKernel<T, NTW>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, maxLds));
-    attrSet = true;
-  }
+  // the largest request (16 rows x one chunk) covers every later one
+  AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&w8LinearKernel<T, NTW>), 16 * (kW8ChunkK + kW8Pad) * (int)sizeof(T)));
   const int tiles = (a.N + 15) / 16;
   dim3 grid((unsigned)((tiles + NTW - 1) / NTW), (unsigned)((a.M + 15) / 16));
   hipLaunchKernelGGL((w8LinearKernel<T, NTW>), grid, dim3(NTW * kW8KSplit * 64), lds, stream, a);
