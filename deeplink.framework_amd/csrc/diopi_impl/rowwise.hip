@@ -46,18 +46,19 @@ __global__ __launch_bounds__(256) void rowWaveKernel(T* __restrict__ out, const 
   // for every row, which keeps it out of both the register file and the L1/L2 request stream.
   constexpr int WPER = (N + WN - 1) / WN;
   __shared__ WV wlds[OP == kRowRmsNorm ? 64 * NV * WPER : 1];
-  if (OP == kRowRmsNorm && weight != nullptr) {
-    for (int i = threadIdx.x; i < nvec * WPER; i += 256) wlds[i] = reinterpret_cast<const WV*>(weight)[i];
-  }
-  if (OP == kRowRmsNorm) __syncthreads();  // before the early exit below: every wave of the block arrives
-  if (row >= rows) return;
+  // The first row's loads go out before the weights are staged, so the two latencies overlap.
   V pre[NV];
-  {
+  if (row < rows) {
     const V* src = reinterpret_cast<const V*>(in + row * inRowStride);
 #pragma unroll
     for (int i = 0; i < NV; ++i)
       if (lane + 64 * i < nvec) pre[i] = __builtin_nontemporal_load(src + lane + 64 * i);
   }
+  if (OP == kRowRmsNorm && weight != nullptr) {
+    for (int i = threadIdx.x; i < nvec * WPER; i += 256) wlds[i] = reinterpret_cast<const WV*>(weight)[i];
+  }
+  if (OP == kRowRmsNorm) __syncthreads();  // before the early exit below: every wave of the block arrives
+  if (row >= rows) return;
   for (; row < rows; row += nWaves) {
   V* dst = reinterpret_cast<V*>(out + row * outRowStride);
   V cur[NV];
