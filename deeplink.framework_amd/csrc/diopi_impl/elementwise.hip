@@ -132,6 +132,48 @@ __global__ __launch_bounds__(kEwThreads) void ewVecKernel(T* out, const T* a,
   }
 }
 
+// Same as ewVecKernel for 2-D operands whose rows are dense but sit further apart than their length
+// (column slices of a wider matrix, e.g. the gate and up halves of a fused projection): the flat
+// vector index is split into (row, vector in row) and every operand brings its own row stride.
+template <int OP, typename T>
+__global__ __launch_bounds__(kEwThreads) void ewVecRowsKernel(T* out, const T* a, const T* b, int64_t nvec,
+                                                               int rowVecs, int64_t so, int64_t sa, int64_t sb,
+                                                               float p0) {
+  using V = typename Vec16<T>::type;
+  constexpr int N = Vec16<T>::N;
+  const V* av = reinterpret_cast<const V*>(a);
+  const V* bv = reinterpret_cast<const V*>(b);
+  V* ov = reinterpret_cast<V*>(out);
+  int64_t base = (int64_t)blockIdx.x * (kEwThreads * kEwUnroll) + threadIdx.x;
+  V ra[kEwUnroll], rb[kEwUnroll];
+  int64_t oo[kEwUnroll];
+#pragma unroll
+  for (int u = 0; u < kEwUnroll; ++u) {
+    int64_t i = base + (int64_t)u * kEwThreads;
+    if (i < nvec) {
+      const int64_t r = i / rowVecs;
+      const int64_t c = i - r * rowVecs;
+      oo[u] = r * so + c;
+      if constexpr (opHasA(OP)) ra[u] = __builtin_nontemporal_load(av + r * sa + c);
+      if constexpr (opHasB(OP)) rb[u] = __builtin_nontemporal_load(bv + r * sb + c);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < kEwUnroll; ++u) {
+    int64_t i = base + (int64_t)u * kEwThreads;
+    if (i < nvec) {
+      V r;
+#pragma unroll
+      for (int j = 0; j < N; ++j) {
+        float fa = opHasA(OP) ? static_cast<float>(ra[u][j]) : 0.f;
+        float fb = opHasB(OP) ? static_cast<float>(rb[u][j]) : 0.f;
+        r[j] = static_cast<T>(ewApply<OP, float>(fa, fb, p0));
+      }
+      __builtin_nontemporal_store(r, ov + oo[u]);
+    }
+  }
+}
+
 template <int OP, typename T>
 __global__ void ewTailKernel(T* out, const T* a, const T* b, int64_t start, int64_t n, float p0) {
   int64_t i = start + (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -156,6 +198,18 @@ diopiError_t launchVec(hipStream_t stream, void* out, const void* a, const void*
     hipLaunchKernelGGL((ewTailKernel<OP, T>), dim3(1), dim3(64), 0, stream, (T*)out, (const T*)a, (const T*)b,
                        nvec * N, n, (float)p0);
   }
+  AMD_LAUNCH_CHECK();
+  return diopiSuccess;
+}
+
+template <int OP, typename T>
+diopiError_t launchVecRows(hipStream_t stream, void* out, const void* a, const void* b, int64_t rows, int64_t cols,
+                           int64_t so, int64_t sa, int64_t sb, double p0) {
+  constexpr int N = Vec16<T>::N;  // cols and the row strides are multiples of N (checked by the caller)
+  const int64_t nvec = rows * (cols / N);
+  int64_t blocks = ceilDiv(nvec, (int64_t)kEwThreads * kEwUnroll);
+  hipLaunchKernelGGL((ewVecRowsKernel<OP, T>), dim3((unsigned)blocks), dim3(kEwThreads), 0, stream, (T*)out, (const T*)a,
+                     (const T*)b, nvec, (int)(cols / N), so / N, sa / N, sb / N, (float)p0);
   AMD_LAUNCH_CHECK();
   return diopiSuccess;
 }
@@ -290,6 +344,40 @@ static bool vecEligible(const TensorView& out, const TensorView* a, const Tensor
   return true;
 }
 
+// A tensor that is [rows, cols] in memory: unit stride on the last dim, all leading dims jointly strided by one
+// row stride (a column slice of a dense matrix with any number of batch dims), 16-byte vectors never straddling a
+// row. *rowStride in elements.
+static bool denseRows(const TensorView& t, int n, int64_t* rowStride) {
+  if (t.ndim < 2 || !t.aligned16()) return false;
+  const int64_t cols = t.shape[t.ndim - 1];
+  if (cols % n != 0 || cols >= ((int64_t)1 << 31) * n) return false;
+  if (cols != 1 && t.stride[t.ndim - 1] != 1) return false;
+  int64_t st = cols;  // used when there is a single row
+  bool have = false;
+  int64_t inner = 1;  // rows spanned by the dims already walked
+  for (int d = t.ndim - 2; d >= 0; --d) {
+    if (t.shape[d] == 1) continue;
+    if (!have) st = t.stride[d], have = true;
+    else if (t.stride[d] != st * inner) return false;
+    inner *= t.shape[d];
+  }
+  *rowStride = st;
+  return st >= cols && st % n == 0;
+}
+
+// Same dtype and shape everywhere, rows dense, row strides free: the column-slice case.
+static bool vecRowsEligible(const TensorView& out, const TensorView* a, const TensorView* b, int64_t* so, int64_t* sa,
+                            int64_t* sb) {
+  if (!(out.dtype == diopi_dtype_bfloat16 || out.dtype == diopi_dtype_float16 || out.dtype == diopi_dtype_float32))
+    return false;
+  const int n = 16 / (int)out.itemsize;
+  *sa = *sb = 0;
+  if (!denseRows(out, n, so)) return false;
+  if (a && !(a->dtype == out.dtype && sameShape(*a, out) && denseRows(*a, n, sa))) return false;
+  if (b && !(b->dtype == out.dtype && sameShape(*b, out) && denseRows(*b, n, sb))) return false;
+  return true;
+}
+
 template <int OP>
 diopiError_t runEw(diopiContextHandle_t ctx, diopiTensorHandle_t outH, diopiConstTensorHandle_t aH,
                    diopiConstTensorHandle_t bH, const diopiScalar_t* p0s, double p0Default) {
@@ -322,6 +410,18 @@ diopiError_t runEw(diopiContextHandle_t ctx, diopiTensorHandle_t outH, diopiCons
       default: return launchVec<OP, float>(stream, out.data, da, db, out.numel, p);
     }
   }
+  int64_t so, sa, sb;
+  if (vecRowsEligible(out, pa, pb, &so, &sa, &sb)) {
+    double p = p0IsFloat ? p0f : (double)p0i;
+    const void* da = pa ? a.data : nullptr;
+    const void* db = pb ? b.data : nullptr;
+    const int64_t cols = out.shape[out.ndim - 1], rows = out.numel / cols;
+    switch (out.dtype) {
+      case diopi_dtype_bfloat16: return launchVecRows<OP, bf16_t>(stream, out.data, da, db, rows, cols, so, sa, sb, p);
+      case diopi_dtype_float16: return launchVecRows<OP, half_t>(stream, out.data, da, db, rows, cols, so, sa, sb, p);
+      default: return launchVecRows<OP, float>(stream, out.data, da, db, rows, cols, so, sa, sb, p);
+    }
+  }
   return launchGeneric<OP>(stream, out, pa, pb, p0f, p0i, p0IsFloat);
 }
 
@@ -331,6 +431,15 @@ diopiError_t stridedCopy(hipStream_t stream, const TensorView& src, const Tensor
   if (src.dtype == dst.dtype && sameShape(src, dst) && src.isContiguous() && dst.isContiguous()) {
     AMD_HIP(hipMemcpyAsync(dst.data, src.data, (size_t)dst.numel * dst.itemsize, hipMemcpyDeviceToDevice, stream));
     return diopiSuccess;
+  }
+  int64_t so, sa, sb;
+  if (vecRowsEligible(dst, &src, nullptr, &so, &sa, &sb)) {
+    const int64_t cols = dst.shape[dst.ndim - 1], rows = dst.numel / cols;
+    switch (dst.dtype) {
+      case diopi_dtype_bfloat16: return launchVecRows<kCopy, bf16_t>(stream, dst.data, src.data, nullptr, rows, cols, so, sa, sb, 0.0);
+      case diopi_dtype_float16: return launchVecRows<kCopy, half_t>(stream, dst.data, src.data, nullptr, rows, cols, so, sa, sb, 0.0);
+      default: return launchVecRows<kCopy, float>(stream, dst.data, src.data, nullptr, rows, cols, so, sa, sb, 0.0);
+    }
   }
   return launchGeneric<kCopy>(stream, dst, &src, nullptr, 0.0, 0, true);
 }
@@ -467,7 +576,7 @@ EW_EXPORT diopiError_t diopiCopyInp(diopiContextHandle_t ctx, diopiConstTensorHa
     if (same) return stridedCopy(stream, s, d);
   }
   if (d.numel == 0) return diopiSuccess;
-  return launchGeneric<kCopy>(stream, d, &s, nullptr, 0.0, 0, true);
+  return stridedCopy(stream, s, d);
 }
 
 // out = cat(tensors, dim): one strided copy per input into the matching slice of out.

@@ -3,7 +3,7 @@ Mirrors oracle.cpu_fallback.decoder_block step for step so every intermediate ca
 import torch
 
 
-def run_decoder_block(ops, x, p, cfg, fused_ffn=False):
+def run_decoder_block(ops, x, p, cfg, fused_ffn=False, stacked_gate_up=False):
     heads, eps, theta = cfg["heads"], cfg["eps"], cfg["theta"]
     b, s, hidden = x.shape
     d = hidden // heads
@@ -30,8 +30,13 @@ def run_decoder_block(ops, x, p, cfg, fused_ffn=False):
     inter["res1"] = x1
     h2 = ops.rms_norm(x1, p["norm2"], eps)
     inter["norm2"] = h2
-    gate = ops.linear(h2, p["wgate"])
-    up = ops.linear(h2, p["wup"])
+    if stacked_gate_up:  # one projection with the two weights stacked; gate and up are its column halves (strided views)
+        ffn = p["wgate"].shape[0]
+        gu = ops.linear(h2, torch.cat([p["wgate"], p["wup"]], dim=0))
+        gate, up = gu[..., :ffn], gu[..., ffn:]
+    else:
+        gate = ops.linear(h2, p["wgate"])
+        up = ops.linear(h2, p["wup"])
     act = ops.silu_mul(gate, up) if fused_ffn else ops.mul(ops.silu(gate), up)
     inter["act"] = act
     down = ops.linear(act, p["wdown"])

@@ -279,6 +279,10 @@ def test_tiny_decoder_block_fp32_every_intermediate(ops, dev, pkg):
         assert_fp32(a.reshape(b.shape), b, rel=1e-5)
     got2, _ = run_decoder_block(ops, x.to(dev), {k: v.to(dev) for k, v in p.items()}, cfg, fused_ffn=True)
     assert_fp32(got2, want)
+    # gate and up as the column halves of one stacked projection: the same numbers, op for op
+    got3, gi3 = run_decoder_block(ops, x.to(dev), {k: v.to(dev) for k, v in p.items()}, cfg, fused_ffn=True, stacked_gate_up=True)
+    assert_fp32(gi3["act"].cpu().reshape(wi["act"].shape), wi["act"], rel=1e-5)
+    assert_fp32(got3, want)
 
 
 def test_small_decoder_block_bf16(ops, dev, pkg):
@@ -286,6 +290,8 @@ def test_small_decoder_block_bf16(ops, dev, pkg):
     want, _ = oracle.decoder_block(x.float(), {k: v.float() for k, v in p.items()}, cfg["heads"], cfg["eps"], cfg["theta"])
     got, _ = run_decoder_block(ops, x.to(dev), {k: v.to(dev) for k, v in p.items()}, cfg, fused_ffn=True)
     # eleven chained bf16 roundings: 3e-2 relative / 3e-2 absolute on an O(1) output
+    assert_half(got, want, rel=3e-2, abs_=3e-2)
+    got, _ = run_decoder_block(ops, x.to(dev), {k: v.to(dev) for k, v in p.items()}, cfg, fused_ffn=True, stacked_gate_up=True)
     assert_half(got, want, rel=3e-2, abs_=3e-2)
 
 

@@ -55,6 +55,41 @@ def test_broadcast_strided_mixed_and_inplace(ops, dev):
     assert_exact(ops.div((i1 * 7).to(dev), 5, rounding_mode="floor"), torch.div(i1 * 7, 5, rounding_mode="floor"))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_column_slices_of_a_wider_matrix(ops, dev, dtype):
+    """The halves of a fused gate/up projection: rows dense, row stride twice the row length, with and
+    without batch dims, as inputs, as the output, in place, and as the source of a copy."""
+    ffn = 1376
+    gu = torch.randn(6, 40, 2 * ffn, generator=g(50)).to(dtype)
+    dgu = gu.to(dev)
+    for view, dview in [(gu, dgu), (gu.reshape(240, 2 * ffn), dgu.reshape(240, 2 * ffn))]:
+        gate, up = view[..., :ffn], view[..., ffn:]
+        dgate, dup = dview[..., :ffn], dview[..., ffn:]
+        assert not dgate.is_contiguous()
+        assert_close(ops.silu_mul(dgate, dup), (oracle.silu(gate).float() * up.float()).to(dtype))
+        assert_close(ops.add(dgate, dup, alpha=0.5), oracle.add(gate, up, alpha=0.5))
+        assert_close(ops.mul(dgate, dup), oracle.mul(gate, up))
+        assert_close(ops.silu(dup), oracle.silu(up))
+    # strided output (and untouched neighbours), in-place on a slice, copy out of / into a slice
+    dst = torch.zeros(240, 2 * ffn, dtype=dtype, device=dev)
+    a2, b2 = gu.reshape(240, 2 * ffn)[:, :ffn], gu.reshape(240, 2 * ffn)[:, ffn:]
+    ops.mul(dgu.reshape(240, 2 * ffn)[:, :ffn], dgu.reshape(240, 2 * ffn)[:, ffn:], out=dst[:, ffn:])
+    assert_close(dst[:, ffn:], oracle.mul(a2, b2))
+    assert_exact(dst[:, :ffn], torch.zeros(240, ffn, dtype=dtype))
+    work = dgu.reshape(240, 2 * ffn).clone()
+    ops.add_(work[:, :ffn], work[:, ffn:])
+    assert_close(work[:, :ffn], oracle.add(a2, b2))
+    assert_exact(work[:, ffn:], b2)
+    dense = torch.empty(240, ffn, dtype=dtype, device=dev)
+    ops.copy_(dense, dgu.reshape(240, 2 * ffn)[:, ffn:])
+    assert_exact(dense, b2)
+    ops.copy_(dst[:, :ffn], dense)
+    assert_exact(dst[:, :ffn], b2)
+    # a slice whose start is not 16-byte aligned, or whose length is not a whole number of vectors, takes the generic path
+    odd = dgu.reshape(240, 2 * ffn)[:, 3:3 + 1001]
+    assert_close(ops.mul(odd, odd), oracle.mul(gu.reshape(240, 2 * ffn)[:, 3:3 + 1001], gu.reshape(240, 2 * ffn)[:, 3:3 + 1001]))
+
+
 def test_scalar_forms(ops, dev):
     x = torch.randn(100, 3, generator=g(10))
     assert_close(ops.add(x.to(dev), 1.5), x + 1.5)
