@@ -57,6 +57,9 @@ void setLastError(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 // every launch.
 hipError_t allowDynamicLds(const void* kernel, int bytes);
 
+// Compute units of the current device (256 on MI355X), queried once; launch sizing only.
+int computeUnits();
+
 // ------------------------------------------------------------ tensor view ---
 struct TensorView {
   void* data = nullptr;

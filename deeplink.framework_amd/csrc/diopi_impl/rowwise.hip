@@ -269,15 +269,6 @@ __global__ __launch_bounds__(256) void rowMeanKernel(T* out, const T* in, int64_
   if (lane == 0) out[row] = static_cast<T>(s / (float)cols);
 }
 
-static int computeUnits() {
-  static int cus = [] {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    return n;
-  }();
-  return cus;
-}
-
 // ------------------------------------------------------------- dispatch ------
 template <typename T, int OP, typename WT>
 static diopiError_t launchRows(hipStream_t stream, T* out, const T* in, const WT* weight, const WT* bias,

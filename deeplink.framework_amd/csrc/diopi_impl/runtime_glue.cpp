@@ -23,6 +23,17 @@ void setLastError(const char* fmt, ...) {
 
 const char* lastError() { return g_last_error; }
 
+int computeUnits() {
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    return n;
+  }();
+  return cus;
+}
+
 hipError_t allowDynamicLds(const void* kernel, int bytes) {
   static std::mutex mu;
   static std::set<std::pair<const void*, int>> done;  // (kernel, device)

@@ -42,17 +42,6 @@ struct W8Mfma<half_t> {
   }
 };
 
-static int computeUnitsW8() {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
-    if (cus <= 0) cus = 256;
-  }
-  return cus;
-}
-
 struct W8Args {
   const void* x;
   const int8_t* w;
@@ -183,7 +172,7 @@ template <typename T>
 static diopiError_t launchW8ForShape(hipStream_t stream, const W8Args& a) {
   // 16-channel tiles per workgroup: enough to bring the grid down to about one workgroup per CU
   const int tiles = (a.N + 15) / 16;
-  const int ntw = std::min(kW8MaxTiles, std::max(1, (tiles + computeUnitsW8() - 1) / computeUnitsW8()));
+  const int ntw = std::min(kW8MaxTiles, std::max(1, (tiles + computeUnits() - 1) / computeUnits()));
   const size_t lds = (size_t)std::min(16, a.M) * (std::min(a.K, kW8ChunkK) + kW8Pad) * sizeof(T);
   switch (ntw) {
     case 1: return launchW8<T, 1>(stream, a, lds);
