@@ -199,33 +199,62 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   }
 }
 
-// out[b,h,:] = merge over the chunks that hold tokens. One wave per (b,h): lane s loads the
-// (max, sum) of split s, a butterfly gives the global max and normaliser, then every lane
-// combines its elements over the splits with independent loads.
+// out[b,h,:] = merge over the chunks that hold tokens. One wave per (b,h): lane s takes the (max, sum) of
+// split s, a butterfly gives the global max and normaliser, then every lane combines its elements over the
+// splits. Nothing here waits for anything else before it is requested: the sequence length, the (max, sum)
+// pairs and the first eight splits' elements are all loaded up front (splits that hold no tokens were never
+// written; what is read from them is discarded by a select, never multiplied).
 template <typename T>
 __global__ __launch_bounds__(256) void decodeMergeKernel(T* __restrict__ out, const float* __restrict__ partial,
                                                           const void* bLen, bool len64, int64_t pairs, int heads,
                                                           int d, int nsplit, int chunk) {
+  constexpr int kBatch = 8, kMaxPerLane = 4;  // d <= 256
   const int lane = threadIdx.x & 63;
   const int64_t pair = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (pair >= pairs) return;
   const int b = (int)(pair / heads);
-  const int len = (int)ldIndex(bLen, b, len64);
-  const int used = len <= 0 ? 1 : min(nsplit, (len + chunk - 1) / chunk);
-  const float* src = partial + pair * nsplit * (2 + d);
+  const int row = 2 + d;
+  const float* src = partial + pair * nsplit * row;
   float ms = -INFINITY, ls = 0.f;
-  if (lane < used) {
-    ms = src[lane * (2 + d)];
-    ls = src[lane * (2 + d) + 1];
+  if (lane < nsplit) {
+    ms = src[lane * row];
+    ls = src[lane * row + 1];
   }
-  const float m = waveMax(ms);
-  float wgt = (ms == -INFINITY) ? 0.f : exp2f(ms - m);
-  const float l = waveSum(ls * wgt);
-  wgt *= l > 0.f ? 1.f / l : 0.f;
-  for (int e = lane; e < d; e += 64) {
-    float acc = 0.f;
-    for (int s = 0; s < used; ++s) acc += __shfl(wgt, s, 64) * src[s * (2 + d) + 2 + e];
-    out[pair * d + e] = static_cast<T>(acc);
+  const int len = (int)ldIndex(bLen, b, len64);
+  float acc[kMaxPerLane] = {0.f, 0.f, 0.f, 0.f};
+  float m = 0.f, wgt = 0.f;
+  int used = 0;
+  for (int sb = 0; sb < nsplit; sb += kBatch) {
+    float v[kBatch][kMaxPerLane];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const float* r = src + (int64_t)min(sb + u, nsplit - 1) * row + 2;
+#pragma unroll
+      for (int k = 0; k < kMaxPerLane; ++k) {
+        const int e = lane + 64 * k;
+        v[u][k] = e < d ? r[e] : 0.f;
+      }
+    }
+    if (sb == 0) {  // the weights of all splits, once, while the loads above are in flight
+      used = len <= 0 ? 1 : min(nsplit, (len + chunk - 1) / chunk);
+      if (lane >= used) ms = -INFINITY, ls = 0.f;
+      m = waveMax(ms);
+      wgt = (ms == -INFINITY) ? 0.f : exp2f(ms - m);
+      const float l = waveSum(ls * wgt);
+      wgt *= l > 0.f ? 1.f / l : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int sp = sb + u;
+      const float w = __shfl(wgt, sp & 63, 64);
+#pragma unroll
+      for (int k = 0; k < kMaxPerLane; ++k) acc[k] += sp < used ? w * v[u][k] : 0.f;
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < kMaxPerLane; ++k) {
+    const int e = lane + 64 * k;
+    if (e < d) out[pair * d + e] = static_cast<T>(acc[k]);
   }
 }
 
