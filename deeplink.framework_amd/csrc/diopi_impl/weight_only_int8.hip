@@ -87,6 +87,13 @@ __global__ __launch_bounds__(NTW * kW8KSplit * 64) void w8LinearKernel(W8Args a)
   const int mrow = min(r16, rows - 1);  // fragment rows past M repeat the last row and are discarded
   const int8_t* wrow = a.w + (int64_t)min(n0 + r16, a.N - 1) * a.ldw + kgrp * 32;
   const T* xg = reinterpret_cast<const T*>(a.x) + (int64_t)m0 * a.ldx;
+  // scale and bias of this lane's output channel: requested now, used after the last weight has been consumed
+  const int col = n0 + r16;
+  float sc = 0.f, bv = 0.f;
+  if (ks == 0 && col < a.N) {
+    sc = loadAs<float>(a.scale, col, a.scaleDtype);
+    if (a.bias) bv = loadAs<float>(a.bias, col, a.biasDtype);
+  }
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   for (int kc = 0; kc < a.K; kc += kW8ChunkK) {
     const int kcLen = min(kW8ChunkK, a.K - kc);  // a multiple of 128, as K is
@@ -138,10 +145,7 @@ __global__ __launch_bounds__(NTW * kW8KSplit * 64) void w8LinearKernel(W8Args a)
   for (int r = 0; r < 4; ++r) red[wave][lane][r] = acc[r];
   __syncthreads();
   if (ks == 0) {
-    const int col = n0 + r16;
     if (col < a.N) {
-      const float sc = loadAs<float>(a.scale, col, a.scaleDtype);
-      const float bv = a.bias ? loadAs<float>(a.bias, col, a.biasDtype) : 0.f;
       T* out = reinterpret_cast<T*>(a.out);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
