@@ -17,8 +17,9 @@
 //     inner loop needs no cross-group traffic: per token only the log2(LPT) butterfly steps
 //     of the dot product;
 //   * two-deep pipeline: while iteration i does its math, the K and V rows of iteration i + 1
-//     (4 + 4 wave-loads, 8 KiB per wave) and the slot indices of iteration i + 2 are in flight,
-//     so neither the row latency nor the index -> address dependency is exposed;
+//     (2 + 2 wave-loads, 4 KiB per wave) and the slot indices of iteration i + 2 are in flight,
+//     so neither the row latency nor the index -> address dependency is exposed. A deeper queue is
+//     slower, not faster: 4 + 4 loads per wave measured 458 us where 2 + 2 take 432 (8 + 8: 509);
 //   * a workgroup = 4 waves owns a chunk of the sequence (split-KV, chunks of at least 512
 //     tokens and at most 64 per sequence); states are merged by wave butterflies, then through
 //     LDS, then across chunks by a small lane-parallel second kernel.
@@ -30,7 +31,7 @@ namespace amd {
 
 constexpr float kLog2eTA = 1.4426950408889634f;
 constexpr int kTaWaves = 4;
-constexpr int kTaUnroll = 4;
+constexpr int kTaUnroll = 2;
 constexpr int kTaChunk = 512;  // tokens of one sequence handled by one workgroup (grows for very long sequences)
 constexpr int kTaMaxSplit = 64; // the merge step handles one split per lane
 
