@@ -93,11 +93,11 @@ def layer_plan(pkg, torch, dev, x, p, cfg):
     h1, qkv, attn, o, x1, h2 = new(T, hidden), new(T, 3 * hidden), new(T, heads, hd), new(T, hidden), new(T, hidden), new(T, hidden)
     qk_rot = new(T, 2 * heads, hd)  # rotated q heads then rotated k heads of a token, one rotary launch for both
     qr, kr = qk_rot[:, :heads], qk_rot[:, heads:]
-    # gate and up come out of one projection (their weights stacked, as the q, k and v weights are): 86 tile
-    # columns of 256 fill the 256 CUs to 98 % in the last round where two launches of 43 reach 90 % each
-    gate_up, act, down, out = new(T, 2 * ffn), new(T, ffn), new(T, hidden), new(T, hidden)
-    gate, up = gate_up[:, :ffn], gate_up[:, ffn:]
-    w_gate_up = torch.cat([p["wgate"], p["wup"]], dim=0).contiguous()
+    # gate and up come out of one projection (their weights interleaved in one matrix at load time, as the q, k and
+    # v weights are stacked): 86 tile columns of 256 fill the 256 CUs to 98 % in the last round where two launches
+    # of 43 reach 90 % each, and silu(gate) * up is applied to the accumulators, so gate and up never reach HBM
+    act, down, out = new(T, ffn), new(T, hidden), new(T, hidden)
+    w_gate_up = pkg.ops.interleave_gate_up(p["wgate"], p["wup"])
     cos, sin = pkg.workloads.rotary_tables(hd, s, cfg["theta"], dtype=bf)
     cos, sin = cos.to(dev), sin.to(dev)
     starts = (torch.arange(b, dtype=torch.int32) * s).to(dev)
@@ -116,13 +116,12 @@ def layer_plan(pkg, torch, dev, x, p, cfg):
         # out projection with the residual folded into the GEMM epilogue: x1 = x + attn @ Wo^T (aten::addmm)
         ("gemm_o", P("diopiAddmm", x1, x2, attn.view(T, hidden), p["wo"].t(), one, one)),
         ("rms_norm", P("diopiRMSNorm", h2, None, x1, d.size([hidden]), p["norm2"], None, float(cfg["eps"]))),
-        ("gemm_gate_up", P("diopiLinear", gate_up, h2, w_gate_up, None)),
-        ("silu_mul", P("diopiSiluMul", act, gate, up)),
+        ("gemm_gate_up_silu", P("diopiLinearSiluMul", act, h2, w_gate_up)),
         ("gemm_down", P("diopiAddmm", out, x1, act, p["wdown"].t(), one, one)),
     ]
-    keep = [h1, qkv, attn, o, x1, h2, qk_rot, qr, kr, gate_up, gate, up, w_gate_up, act, down, out, cos, sin, starts, lens, x2]
+    keep = [h1, qkv, attn, o, x1, h2, qk_rot, qr, kr, w_gate_up, act, down, out, cos, sin, starts, lens, x2]
     flops = {"gemm_qkv": 2 * T * 3 * hidden * hidden, "gemm_o": 2 * T * hidden * hidden,
-             "gemm_gate_up": 2 * T * 2 * ffn * hidden, "gemm_down": 2 * T * hidden * ffn}
+             "gemm_gate_up_silu": 2 * T * 2 * ffn * hidden, "gemm_down": 2 * T * hidden * ffn}
     return plan, keep, flops, out
 
 
@@ -367,7 +366,7 @@ def main():
     gemm_flops = sum(flops.values())
     achieved_tf = gemm_flops / (gemm_time_us * 1e-6) / 1e12
     breakdown = {l: round(sum(v) / args.steps, 1) for l, v in per_op.items()}      # us per step (labels used twice are summed)
-    roofline = {"bound": "mfma", "kernel": "gemmMfmaPipelinedKernel<bf16> 256x256x64 (4 launches per step: qkv, o, gate+up, down)",
+    roofline = {"bound": "mfma", "kernel": "gemmMfmaPipelinedKernel<bf16> 256x256x64 (4 launches per step: qkv, o + residual, gate+up with silu*mul, down + residual)",
                 "achieved": round(achieved_tf, 1), "peak": MFMA_BF16_PEAK_TF, "unit": "TFLOP/s",
                 "frac": round(achieved_tf / MFMA_BF16_PEAK_TF, 4), "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH,
                 "flops_per_step": gemm_flops, "avg_launch_us": round(gemm_time_us / len(gemm_labels), 1),

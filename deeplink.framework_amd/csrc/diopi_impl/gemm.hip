@@ -275,7 +275,12 @@ __device__ __forceinline__ void loadToLds16(u32x4 rsrc, int voffset, int soffset
       : "memory");
 }
 
-template <typename T>
+// EPI selects the epilogue: kEpiLinear is alpha * acc + beta * C + bias; kEpiSiluMul treats every 64 consecutive
+// output columns as 32 gate columns followed by the 32 up columns of the same channels and stores
+// silu(gate) * up, half as wide (out has N / 2 columns).
+enum PipeEpilogue { kEpiLinear = 0, kEpiSiluMul = 1 };
+
+template <typename T, int EPI>
 __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs g) {
   using Frag = typename MfmaOp<T>::Frag;
   constexpr int BM = 256, BN = 256, WM = BM / kPipeWavesM, WN = BN / kPipeWavesN, TM = WM / 16, TN = WN / 16;
@@ -467,8 +472,9 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
     constexpr int RS4 = WN + 4;  // padded row, floats
     ldsBarrier();                // every wave is done with the operand tiles the strips overlay
     float* strip = reinterpret_cast<float*>(smem) + wave * (32 * RS4);
-    constexpr int GROUPS = WN / 8;                 // 8-column groups per strip row
-    constexpr int ITEMS = 32 * GROUPS / 64;        // (row, group) items per lane
+    constexpr int GROUPS = (EPI == kEpiSiluMul ? WN / 2 : WN) / 8;  // 8-column output groups per strip row
+    constexpr int ITEMS = 32 * GROUPS / 64;                         // (row, group) items per lane
+    static_assert(EPI == kEpiLinear || WN == 64, "a wave's strip is one 32 + 32 gate / up block");
 #pragma unroll
     for (int ip = 0; ip < TM / 2; ++ip) {  // two 16-row fragment rows per strip
 #pragma unroll
@@ -486,6 +492,21 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
         const int col = tn * BN + wn * WN + sg * 8;
         const f32x4 lo = *reinterpret_cast<const f32x4*>(strip + srow * RS4 + sg * 8);
         const f32x4 hi = *reinterpret_cast<const f32x4*>(strip + srow * RS4 + sg * 8 + 4);
+        if constexpr (EPI == kEpiSiluMul) {
+          // columns [0, 32) of the strip are gate, [32, 64) the up values of the same 32 channels
+          const f32x4 ulo = *reinterpret_cast<const f32x4*>(strip + srow * RS4 + 32 + sg * 8);
+          const f32x4 uhi = *reinterpret_cast<const f32x4*>(strip + srow * RS4 + 32 + sg * 8 + 4);
+          if (row < g.M && col + 32 < g.N) {  // N % 64 == 0 here: a gate / up block is entirely inside or outside
+            const float gv[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            const float uv[8] = {ulo[0], ulo[1], ulo[2], ulo[3], uhi[0], uhi[1], uhi[2], uhi[3]};
+            Frag o;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = static_cast<T>(gv[e] / (1.f + __expf(-gv[e])) * uv[e]);
+            const int ocol = (tn * BN + wn * WN) / 2 + sg * 8;
+            *reinterpret_cast<Frag*>(out + (int64_t)row * g.ldo + ocol) = o;
+          }
+          continue;
+        }
         if (row < g.M && col < g.N) {  // N % 8 == 0 here: a group is entirely inside or outside
           float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
           Frag o;
@@ -648,7 +669,7 @@ static diopiError_t launchMfma(hipStream_t stream, const GemmProblem& p) {
   return diopiSuccess;
 }
 
-template <typename T>
+template <typename T, int EPI = kEpiLinear>
 static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p) {
   MfmaArgs g;
   g.A = p.A, g.B = p.B, g.out = p.out, g.Cin = p.Cin, g.bias = p.bias;
@@ -661,9 +682,10 @@ static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p
   g.vecEpilogue = p.N % 8 == 0 && p.sOm % 8 == 0 && p.sOb % 8 == 0 && al16(p.out) &&
                   (!p.Cin || (p.sCn == 1 && p.sCm % 8 == 0 && p.sCb % 8 == 0 && al16(p.Cin))) && (!p.bias || al16(p.bias));
   constexpr size_t lds = 2 * (size_t)(256 + 256) * kBK * sizeof(T);
-  AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmMfmaPipelinedKernel<T>), (int)lds));
+  AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmMfmaPipelinedKernel<T, EPI>), (int)lds));
   dim3 grid((unsigned)(g.tilesM * g.tilesN), 1, (unsigned)p.batch);
-  hipLaunchKernelGGL((gemmMfmaPipelinedKernel<T>), grid, dim3(kPipeThreads), lds, stream, g);
+  if (EPI == kEpiSiluMul) AMD_CHECK(g.vecEpilogue, "gated linear: output rows must allow 16-byte stores");
+  hipLaunchKernelGGL((gemmMfmaPipelinedKernel<T, EPI>), grid, dim3(kPipeThreads), lds, stream, g);
   AMD_LAUNCH_CHECK();
   return diopiSuccess;
 }
@@ -735,6 +757,59 @@ diopiError_t runGemm(diopiContextHandle_t ctx, hipStream_t stream, GemmProblem p
 
 // ------------------------------------------------------------- entry helpers --
 // Folds leading dims of a dense-enough view into one batch dim; returns false if impossible.
+// ------------------------------------------------------- gated SiLU linear ----
+// Second pass of the two-pass form: out[m, 32 b + j] = silu(gu[m, 64 b + j]) * gu[m, 64 b + 32 + j].
+template <typename T>
+__global__ __launch_bounds__(256) void gatedSiluKernel(T* __restrict__ out, const T* __restrict__ gu, int64_t rows,
+                                                        int64_t f, int64_t ldo) {
+  const int64_t total = rows * f;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t m = i / f, c = i - m * f;
+    const T* row = gu + m * 2 * f + (c >> 5) * 64 + (c & 31);
+    const float g = static_cast<float>(row[0]), u = static_cast<float>(row[32]);
+    out[m * ldo + c] = static_cast<T>(g / (1.f + __expf(-g)) * u);
+  }
+}
+
+// out[M, F] = silu(A W_gate^T) * (A W_up^T) with the two weights interleaved in one [2F, K] matrix (see
+// diopiLinearSiluMul). One launch of the large-tile kernel when the problem qualifies, else GEMM + pass.
+static diopiError_t runGatedSiluGemm(diopiContextHandle_t ctx, hipStream_t stream, GemmProblem p) {
+  const int64_t f = p.N / 2;
+  const bool half = p.dtype == diopi_dtype_bfloat16 || p.dtype == diopi_dtype_float16;
+  const bool direct = half && p.batch == 1 && p.sAk == 1 && mult8(p.sAm) && ptr16(p.A) && p.sBk == 1 && mult8(p.sBn) && ptr16(p.B) &&
+                      ceilDiv(p.M, 256) * ceilDiv(p.N, 256) >= 200 && p.K % kBK == 0 && p.K >= 2 * kBK &&
+                      ((p.M - 1) * p.sAm + p.K) * 2 < (int64_t(1) << 31) && ((p.N - 1) * p.sBn + p.K) * 2 < (int64_t(1) << 31) &&
+                      mult8(p.sOm) && ptr16(p.out) && p.M < (int64_t(1) << 31) && p.N < (int64_t(1) << 31);
+  if (direct) {
+    return p.dtype == diopi_dtype_bfloat16 ? launchMfmaPipelined<bf16_t, kEpiSiluMul>(stream, p)
+                                           : launchMfmaPipelined<half_t, kEpiSiluMul>(stream, p);
+  }
+  // two passes: the full-width projection into workspace, then the gate
+  void* ws = nullptr;
+  const int64_t item = dtypeSize(p.dtype);
+  AMD_TRY(requireWorkspace(ctx, p.M * p.N * item, &ws));
+  GemmProblem q = p;
+  void* finalOut = p.out;
+  const int64_t ldo = p.sOm;
+  q.out = ws, q.sOm = p.N, q.sOb = p.M * p.N;
+  AMD_TRY(runGemm(ctx, stream, q));
+  int64_t blocks = std::min<int64_t>(ceilDiv(p.M * f, 256), 65536);
+  switch (p.dtype) {
+    case diopi_dtype_bfloat16:
+      hipLaunchKernelGGL(gatedSiluKernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, (bf16_t*)finalOut, (const bf16_t*)ws, p.M, f, ldo);
+      break;
+    case diopi_dtype_float16:
+      hipLaunchKernelGGL(gatedSiluKernel<half_t>, dim3((unsigned)blocks), dim3(256), 0, stream, (half_t*)finalOut, (const half_t*)ws, p.M, f, ldo);
+      break;
+    case diopi_dtype_float32:
+      hipLaunchKernelGGL(gatedSiluKernel<float>, dim3((unsigned)blocks), dim3(256), 0, stream, (float*)finalOut, (const float*)ws, p.M, f, ldo);
+      break;
+    default: setLastError("gated linear: unsupported dtype %s", dtypeName(p.dtype)); return diopiErrorOccurred;
+  }
+  AMD_LAUNCH_CHECK();
+  return diopiSuccess;
+}
+
 static bool foldBatch(const TensorView& t, int lead, int64_t* count, int64_t* stride) {
   int64_t n = 1, s = 0;
   bool have = false;
@@ -988,4 +1063,45 @@ GEMM_EXPORT diopiError_t diopiLinear(diopiContextHandle_t ctx, diopiTensorHandle
   TensorView in2 = in, out2 = out;
   if (in.ndim == 1) in2 = unsqueeze(in, 0), out2 = unsqueeze(out, 0);
   return batchedMatmul(ctx, stream, out2, in2, w, nullptr, bias.defined() ? &cb : nullptr, 1.f, 0.f, true);
+}
+
+// out[..., F] = silu(input W_gate^T) * (input W_up^T), weight = the two [F, K] matrices interleaved in blocks
+// of 32 rows (see functions_ext.h). The reference model runs two linears, silu and mul
+// (dicp/test/model/llama/model.py:196-200; diopi_functions.yaml:902-909,1767-1775,181-196).
+GEMM_EXPORT diopiError_t diopiLinearSiluMul(diopiContextHandle_t ctx, diopiTensorHandle_t outH,
+                                            diopiConstTensorHandle_t inH, diopiConstTensorHandle_t wH) {
+  hipStream_t stream;
+  AMD_TRY(getStream(ctx, &stream));
+  TensorView out, in, w;
+  AMD_TRY(getView(outH, &out, "out"));
+  AMD_TRY(getView(inH, &in, "input"));
+  AMD_TRY(getView(wH, &w, "weight"));
+  AMD_CHECK(out.defined() && in.defined() && w.defined(), "diopiLinearSiluMul: null tensor");
+  AMD_CHECK(w.ndim == 2 && in.ndim >= 1 && out.ndim == in.ndim, "diopiLinearSiluMul: weight must be [2F, K], out shaped like input");
+  AMD_CHECK(in.dtype == out.dtype && w.dtype == out.dtype, "diopiLinearSiluMul: input, weight and out must share a dtype");
+  const int64_t k = in.shape[in.ndim - 1], f = out.shape[out.ndim - 1];
+  AMD_CHECK(w.shape[1] == k && w.shape[0] == 2 * f, "diopiLinearSiluMul: weight is [%ld, %ld], expected [%ld, %ld]",
+            (long)w.shape[0], (long)w.shape[1], (long)(2 * f), (long)k);
+  AMD_CHECK(f % 32 == 0, "diopiLinearSiluMul: %ld output channels are not a multiple of the 32-row interleave", (long)f);
+  for (int d = 0; d + 1 < in.ndim; ++d)
+    AMD_CHECK(in.shape[d] == out.shape[d], "diopiLinearSiluMul: leading extent mismatch at dim %d", d);
+  if (out.numel == 0) return diopiSuccess;
+  TensorView cin, cw;
+  AMD_TRY(makeContiguous(ctx, stream, in, &cin));
+  AMD_TRY(makeContiguous(ctx, stream, w, &cw));
+  TensorView cout = out;
+  const bool outTemp = !out.isContiguous();
+  if (outTemp) {
+    diopiTensorHandle_t th;
+    AMD_TRY(requireTensor(ctx, out.shape, out.ndim, out.dtype, &th, &cout));
+  }
+  GemmProblem p;
+  p.dtype = out.dtype;
+  p.M = in.numel / k, p.N = 2 * f, p.K = k;
+  p.A = cin.data, p.sAm = k, p.sAk = 1;
+  p.B = cw.data, p.sBn = k, p.sBk = 1;
+  p.out = cout.data, p.sOm = f;
+  AMD_TRY(runGatedSiluGemm(ctx, stream, p));
+  if (outTemp) AMD_TRY(stridedCopy(stream, cout, out));
+  return diopiSuccess;
 }

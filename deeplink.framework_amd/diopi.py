@@ -238,6 +238,7 @@ SIGNATURES = {
     "diopiTokenDecodeAttentionInference": [_T, _T, _T, _T, _T, _T, _T, c_int],
     "diopiWeightOnlyInt8Linear": [_T, _T, _T, _T, _T],
     "diopiSiluMul": [_T, _T, _T],
+    "diopiLinearSiluMul": [_T, _T, _T],
 }
 
 _bound = {}

@@ -211,6 +211,27 @@ def silu_mul(gate, up, *, out=None):
     return out
 
 
+def interleave_gate_up(w_gate, w_up):
+    """The [2F, K] weight diopiLinearSiluMul expects: w_gate and w_up [F, K] interleaved in blocks of 32 rows
+    (a load-time permutation of the checkpoint)."""
+    f, k = w_gate.shape
+    assert w_up.shape == (f, k) and f % 32 == 0
+    return torch.stack([w_gate.reshape(f // 32, 32, k), w_up.reshape(f // 32, 32, k)], dim=1).reshape(2 * f, k).contiguous()
+
+
+def linear_silu_mul(input, weight_gate_up, *, out=None):
+    """silu(input @ w_gate^T) * (input @ w_up^T) in one launch (backend extension; see functions_ext.h).
+    weight_gate_up = interleave_gate_up(w_gate, w_up)."""
+    f = weight_gate_up.shape[0] // 2
+    if out is None:
+        out = torch.empty(*input.shape[:-1], f, dtype=input.dtype, device=input.device)
+    ho, po = handle(out)
+    hi, pi = handle(input)
+    hw, pw = handle(weight_gate_up)
+    _call("diopiLinearSiluMul", po, pi, pw)
+    return out
+
+
 # ------------------------------------------------------------------ reductions
 def softmax(self, dim, *, out=None):
     """aten::_softmax.out -> diopiSoftmax (diopi_functions.yaml:1290-1292)."""

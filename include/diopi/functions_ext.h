@@ -97,4 +97,13 @@ DIOPI_API diopiError_t diopiWeightOnlyInt8Linear(diopiContextHandle_t ctx, diopi
 DIOPI_API diopiError_t diopiSiluMul(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiConstTensorHandle_t gate,
                                     diopiConstTensorHandle_t up);
 
+/* out[..., F] = silu(input @ w_gate^T) * (input @ w_up^T): the SiLU-gated FFN's two projections and its
+ * elementwise stage in one pass; gate and up never reach memory. weight is [2F, K] and holds w_gate [F, K] and
+ * w_up [F, K] interleaved in blocks of 32 rows: rows [64 b, 64 b + 32) = w_gate[32 b : 32 b + 32],
+ * rows [64 b + 32, 64 b + 64) = w_up[32 b : 32 b + 32] (a load-time permutation of the checkpoint, like stacking
+ * q, k and v). F must be a multiple of 32. The reference model runs two linears, silu and mul
+ * (dicp/test/model/llama/model.py:196-200). */
+DIOPI_API diopiError_t diopiLinearSiluMul(diopiContextHandle_t ctx, diopiTensorHandle_t out,
+                                          diopiConstTensorHandle_t input, diopiConstTensorHandle_t weight);
+
 #endif /* DIOPI_FUNCTIONS_EXT_H_ */

@@ -30,14 +30,18 @@ def run_decoder_block(ops, x, p, cfg, fused_ffn=False, stacked_gate_up=False):
     inter["res1"] = x1
     h2 = ops.rms_norm(x1, p["norm2"], eps)
     inter["norm2"] = h2
-    if stacked_gate_up:  # one projection with the two weights stacked; gate and up are its column halves (strided views)
+    if stacked_gate_up == "interleaved":  # both projections and the gate in one launch
+        act = ops.linear_silu_mul(h2, ops.interleave_gate_up(p["wgate"], p["wup"]))
+        gate = up = None
+    elif stacked_gate_up:  # one projection with the two weights stacked; gate and up are its column halves (strided views)
         ffn = p["wgate"].shape[0]
         gu = ops.linear(h2, torch.cat([p["wgate"], p["wup"]], dim=0))
         gate, up = gu[..., :ffn], gu[..., ffn:]
     else:
         gate = ops.linear(h2, p["wgate"])
         up = ops.linear(h2, p["wup"])
-    act = ops.silu_mul(gate, up) if fused_ffn else ops.mul(ops.silu(gate), up)
+    if gate is not None:
+        act = ops.silu_mul(gate, up) if fused_ffn else ops.mul(ops.silu(gate), up)
     inter["act"] = act
     down = ops.linear(act, p["wdown"])
     inter["down"] = down

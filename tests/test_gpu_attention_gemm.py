@@ -117,6 +117,28 @@ def test_large_tile_gemm_batched_and_row_strided_operands(ops, dev):
     assert_half(ops.bmm(a, bb.to(dev).transpose(1, 2)), torch.bmm(a.float().cpu(), bb.float().transpose(1, 2)))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("m,f,k", [(4096, 3584, 256), (3700, 4000 - 32, 192), (96, 64, 80), (1, 32, 8)])
+def test_linear_silu_mul(ops, dev, dtype, m, f, k):
+    """silu(x Wg^T) * (x Wu^T) from the interleaved weight: the single-launch path (at least 200 tiles, K a
+    multiple of 64, 16-bit dtypes) and the two-pass path, against the reference's four-op form in fp32."""
+    x = torch.randn(m, k, generator=g(60)).to(dtype)
+    wg = (torch.randn(f, k, generator=g(61)) * 0.08).to(dtype)
+    wu = (torch.randn(f, k, generator=g(62)) * 0.08).to(dtype)
+    gate, up = x.float() @ wg.float().t(), x.float() @ wu.float().t()
+    want = torch.nn.functional.silu(gate) * up
+    w = ops.interleave_gate_up(wg.to(dev), wu.to(dev))
+    assert_exact(w[32:64], wu[:32])  # block 0: 32 gate rows, then 32 up rows
+    got = ops.linear_silu_mul(x.to(dev), w)
+    (assert_fp32 if dtype == torch.float32 else assert_half)(got, want)
+    if m >= 96:  # batch dims and a strided destination
+        x3 = x[:96].reshape(2, 48, k)
+        dst = torch.zeros(2, 48, 2 * f, dtype=dtype, device=dev)
+        ops.linear_silu_mul(x3.to(dev), w, out=dst[..., :f])
+        (assert_fp32 if dtype == torch.float32 else assert_half)(dst[..., :f], want[:96].reshape(2, 48, f))
+        assert_exact(dst[..., f:], torch.zeros(2, 48, f, dtype=dtype))
+
+
 # ------------------------------------------------------------------ prefill attention
 @pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 128), (torch.float16, 128), (torch.bfloat16, 64),
                                      (torch.float32, 64), (torch.float32, 40)])
@@ -283,6 +305,9 @@ def test_tiny_decoder_block_fp32_every_intermediate(ops, dev, pkg):
     got3, gi3 = run_decoder_block(ops, x.to(dev), {k: v.to(dev) for k, v in p.items()}, cfg, fused_ffn=True, stacked_gate_up=True)
     assert_fp32(gi3["act"].cpu().reshape(wi["act"].shape), wi["act"], rel=1e-5)
     assert_fp32(got3, want)
+    got4, gi4 = run_decoder_block(ops, x.to(dev), {k: v.to(dev) for k, v in p.items()}, cfg, stacked_gate_up="interleaved")
+    assert_fp32(gi4["act"].cpu().reshape(wi["act"].shape), wi["act"], rel=1e-5)
+    assert_fp32(got4, want)
 
 
 def test_small_decoder_block_bf16(ops, dev, pkg):
@@ -292,6 +317,8 @@ def test_small_decoder_block_bf16(ops, dev, pkg):
     # eleven chained bf16 roundings: 3e-2 relative / 3e-2 absolute on an O(1) output
     assert_half(got, want, rel=3e-2, abs_=3e-2)
     got, _ = run_decoder_block(ops, x.to(dev), {k: v.to(dev) for k, v in p.items()}, cfg, fused_ffn=True, stacked_gate_up=True)
+    assert_half(got, want, rel=3e-2, abs_=3e-2)
+    got, _ = run_decoder_block(ops, x.to(dev), {k: v.to(dev) for k, v in p.items()}, cfg, stacked_gate_up="interleaved")
     assert_half(got, want, rel=3e-2, abs_=3e-2)
 
 
