@@ -240,6 +240,24 @@ def op_microbench(pkg, torch, dev, rt, stream):
                     "us_cold": round(cold, 2), "GBs_hot": round(nbytes / hot / 1e3, 1), "GBs_cold": round(nbytes / cold / 1e3, 1),
                     "frac_hot": round(nbytes / hot / 1e3 / HBM_PEAK_GBS, 3), "frac_cold": round(nbytes / cold / 1e3 / HBM_PEAK_GBS, 3)})
         del W
+    # bf16 linear at decode shapes (a handful of rows against a [11008, 4096] weight): the weight stream is the traffic
+    for m in (1, 16):
+        gq = torch.Generator().manual_seed(7)
+        x = torch.randn(m, 4096, generator=gq).bfloat16().to(dev)
+        W = [(torch.randn(11008, 4096, generator=gq) * 0.02).bfloat16().to(dev) for _ in range(4)]
+        ob = torch.empty(m, 11008, dtype=torch.bfloat16, device=dev)
+        nbytes = 2 * (4096 * 11008 + m * 4096 + m * 11008)
+        callsb = [Prepared(pkg, "diopiLinear", ob, x, W[i], None) for i in range(4)]
+        stb = {"i": 0}
+
+        def rotb():
+            callsb[stb["i"] % 4]()
+            stb["i"] += 1
+        hot, cold = time_ops(rt, stream, [callsb[0], rotb], 200, 16)
+        res.append({"op": "diopiLinear (decode)", "workload": f"bf16 M={m}, K=4096, N=11008", "bytes": nbytes, "us_hot": round(hot, 2),
+                    "us_cold": round(cold, 2), "GBs_hot": round(nbytes / hot / 1e3, 1), "GBs_cold": round(nbytes / cold / 1e3, 1),
+                    "frac_hot": round(nbytes / hot / 1e3 / HBM_PEAK_GBS, 3), "frac_cold": round(nbytes / cold / 1e3 / HBM_PEAK_GBS, 3)})
+        del W
     return res
 
 

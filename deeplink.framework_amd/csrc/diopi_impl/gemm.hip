@@ -22,11 +22,15 @@
 //     fetches (16 consecutive rows, 4 consecutive logical chunks) are bank-conflict free;
 //   * workgroup ids are remapped so that each of the 8 XCDs (own L2 each) works on a
 //     contiguous band of tiles, walked in groups of 8 tile-rows to reuse A and B from L2;
-//   * epilogue: alpha * acc + beta * C + bias; the accumulators go through LDS strips so that C
-//     and the addend move in 16-byte row pieces;
+//   * epilogue: alpha * acc + beta * C + bias straight from the accumulators: the weight fragment is
+//     the first MFMA operand, so a lane holds consecutive columns of one output row, and one lane
+//     swap per register turns that into 16-byte pieces of C and of the addend; the stream never
+//     waits for a store (code that may load an addend otherwise waits for the store before it);
 //   * small or ragged problems: 128x128 (or 256x256) tiles with 4 waves of v_mfma_f32_32x32x16,
 //     staged through registers, any K that is a multiple of 8, stores straight from the
-//     accumulator layout.
+//     accumulator layout;
+//   * at most 32 rows (64 while N is small), the decode shape: a weight-streaming kernel with 16-column tiles
+//     whose waves split K and stage the activation rows in LDS.
 // Operands that are not K-contiguous (mm with a row-major mat2, bmm's second operand) are
 // transposed once into workspace by a tiled LDS transpose, then use the same engine.
 //
@@ -197,25 +201,43 @@ __global__ __launch_bounds__(256) void gemmMfmaKernel(MfmaArgs g) {
   T* out = reinterpret_cast<T*>(g.out) + (int64_t)batch * g.sOb;
   const T* cin = g.Cin ? reinterpret_cast<const T*>(g.Cin) + (int64_t)batch * g.sCb : nullptr;
   const T* bias = reinterpret_cast<const T*>(g.bias);
+  // Two instruction streams: loads and stores share one in-order counter, so the addend of a whole
+  // 32 x 32 block is requested before its first store (one wait per block instead of one per element,
+  // each of which would also wait for the store before it), and without an addend nothing is loaded.
+  auto store = [&](auto withAddend) {
+    constexpr bool kAddend = decltype(withAddend)::value;
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int col = tn * BN + wn * WN + j * 32 + frow;
-    if (col >= g.N) continue;
-    const float bv = bias ? static_cast<float>(bias[col]) : 0.f;
+    for (int j = 0; j < TN; ++j) {
+      const int col = tn * BN + wn * WN + j * 32 + frow;
+      if (col >= g.N) continue;
+      const float bv = bias ? static_cast<float>(bias[col]) : 0.f;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int rbase = tm * BM + wm * WM + i * 32 + fhalf * 4;
+      for (int i = 0; i < TM; ++i) {
+        const int rbase = tm * BM + wm * WM + i * 32 + fhalf * 4;
+        float c[16];
+        if constexpr (kAddend) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = rbase + (r >> 2) * 8 + (r & 3);
-        if (row < g.M) {
-          float v = acc[i][j][r] * g.alpha + bv;
-          if (cin) v += g.beta * static_cast<float>(cin[(int64_t)row * g.sCm + (int64_t)col * g.sCn]);
-          out[(int64_t)row * g.ldo + col] = static_cast<T>(v);
+          for (int r = 0; r < 16; ++r) {
+            const int row = min(rbase + (r >> 2) * 8 + (r & 3), g.M - 1);
+            c[r] = static_cast<float>(cin[(int64_t)row * g.sCm + (int64_t)col * g.sCn]);
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = rbase + (r >> 2) * 8 + (r & 3);
+          if (row < g.M) {
+            float v = acc[i][j][r] * g.alpha + bv;
+            if constexpr (kAddend) v += g.beta * c[r];
+            out[(int64_t)row * g.ldo + col] = static_cast<T>(v);
+          }
         }
       }
     }
-  }
+  };
+  if (cin)
+    store(std::true_type{});
+  else
+    store(std::false_type{});
 }
 
 // ------------------------------------------------- software-pipelined 256x256 ---
@@ -240,7 +262,8 @@ __device__ __forceinline__ void ldsBarrier() {
 constexpr int kPipeWavesM = 2, kPipeWavesN = 4, kPipeThreads = kPipeWavesM * kPipeWavesN * 64;
 
 // v_mfma_f32_16x16x32: lane l feeds row (l & 15), K elements [8 * (l >> 4), +8) of both operands and
-// receives C[4 * (l >> 4) + r][l & 15], r = 0..3.
+// receives D[4 * (l >> 4) + r][l & 15], r = 0..3. The large-tile kernel passes the weight fragment
+// first, so D is the transposed block and a lane holds four consecutive columns of output row (l & 15).
 template <typename T>
 struct MfmaOp16;
 template <>
@@ -377,7 +400,7 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
       before(j);
 #pragma unroll
       for (int i = 0; i < HM; ++i)
-        acc[half * HM + i][j] = MfmaOp16<T>::run(fa[buf][i], fb[j], acc[half * HM + i][j]);
+        acc[half * HM + i][j] = MfmaOp16<T>::run(fb[j], fa[buf][i], acc[half * HM + i][j]);
       after(j);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -466,85 +489,263 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
   const T* cin = g.Cin ? reinterpret_cast<const T*>(g.Cin) + (int64_t)batch * g.sCb : nullptr;
   const T* bias = reinterpret_cast<const T*>(g.bias);
   if (g.vecEpilogue) {
-    // Accumulators go through a wave-private LDS strip (32 rows x WN fp32, rows padded by 16 B) so
-    // that the addend is read and the result written as 16-byte row segments: full 128-byte lines
-    // instead of 2-byte column accesses. alpha/beta/bias are applied in fp32 after the transpose.
-    constexpr int RS4 = WN + 4;  // padded row, floats
-    ldsBarrier();                // every wave is done with the operand tiles the strips overlay
-    float* strip = reinterpret_cast<float*>(smem) + wave * (32 * RS4);
-    constexpr int GROUPS = (EPI == kEpiSiluMul ? WN / 2 : WN) / 8;  // 8-column output groups per strip row
-    constexpr int ITEMS = 32 * GROUPS / 64;                         // (row, group) items per lane
-    static_assert(EPI == kEpiLinear || WN == 64, "a wave's strip is one 32 + 32 gate / up block");
+    // Straight from the accumulators. A lane holds 4 consecutive columns of one row in each 16-column
+    // fragment; v_permlane16_swap between the two fragments of a 32-column pair leaves it with 8
+    // consecutive columns instead (lane group q gets the columns starting at 16 * (q & 1) + 8 * (q >> 1)),
+    // so the addend is read and the result written as 16-byte pieces, 64 contiguous bytes per row and
+    // instruction, without a trip through LDS. alpha / beta / bias are applied in fp32 after the swap.
+    // Output and addend go through buffer descriptors (the host guarantees both span less than 2 GiB):
+    // a piece outside the matrix gets an offset past the end, which the hardware drops (stores) or
+    // answers with zeros (loads), so the instruction stream has no branches and the compiler can count
+    // outstanding accesses exactly. Loads and stores share one in-order counter: a wait for an addend
+    // piece also waits for every store before it, so the pieces of fragment row i + 1 are requested
+    // before the stores of row i, and without an addend there is no load (and no wait) in the stream.
+    const int cperm = (kq & 1) * 16 + (kq >> 1) * 8;
+    auto swapPair = [](f32x4& x0, f32x4& x1) {
 #pragma unroll
-    for (int ip = 0; ip < TM / 2; ++ip) {  // two 16-row fragment rows per strip
-#pragma unroll
-      for (int ii = 0; ii < 2; ++ii)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) strip[(ii * 16 + kq * 4 + r) * RS4 + j * 16 + frow] = acc[2 * ip + ii][j][r];
-      __builtin_amdgcn_s_waitcnt(0xc07f);  // the strip is private to this wave: no barrier, only its own LDS ops
-#pragma unroll
-      for (int it = 0; it < ITEMS; ++it) {
-        const int item = lane + 64 * it;
-        const int srow = item / GROUPS, sg = item % GROUPS;
-        const int row = tm * BM + wm * WM + ip * 32 + srow;
-        const int col = tn * BN + wn * WN + sg * 8;
-        const f32x4 lo = *reinterpret_cast<const f32x4*>(strip + srow * RS4 + sg * 8);
-        const f32x4 hi = *reinterpret_cast<const f32x4*>(strip + srow * RS4 + sg * 8 + 4);
-        if constexpr (EPI == kEpiSiluMul) {
-          // columns [0, 32) of the strip are gate, [32, 64) the up values of the same 32 channels
-          const f32x4 ulo = *reinterpret_cast<const f32x4*>(strip + srow * RS4 + 32 + sg * 8);
-          const f32x4 uhi = *reinterpret_cast<const f32x4*>(strip + srow * RS4 + 32 + sg * 8 + 4);
-          if (row < g.M && col + 32 < g.N) {  // N % 64 == 0 here: a gate / up block is entirely inside or outside
-            const float gv[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-            const float uv[8] = {ulo[0], ulo[1], ulo[2], ulo[3], uhi[0], uhi[1], uhi[2], uhi[3]};
-            Frag o;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) o[e] = static_cast<T>(gv[e] / (1.f + __expf(-gv[e])) * uv[e]);
-            const int ocol = (tn * BN + wn * WN) / 2 + sg * 8;
-            *reinterpret_cast<Frag*>(out + (int64_t)row * g.ldo + ocol) = o;
-          }
-          continue;
-        }
-        if (row < g.M && col < g.N) {  // N % 8 == 0 here: a group is entirely inside or outside
-          float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-          Frag o;
-          Frag cv, bvv;
-          if (cin) cv = *reinterpret_cast<const Frag*>(cin + (int64_t)row * g.sCm + col);
-          if (bias) bvv = *reinterpret_cast<const Frag*>(bias + col);
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            float x = v[e] * g.alpha;
-            if (bias) x += static_cast<float>(bvv[e]);
-            if (cin) x += g.beta * static_cast<float>(cv[e]);
-            o[e] = static_cast<T>(x);
-          }
-          *reinterpret_cast<Frag*>(out + (int64_t)row * g.ldo + col) = o;
-        }
+      for (int r = 0; r < 4; ++r) {
+        const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(x0[r]), __float_as_uint(x1[r]), false, false);
+        x0[r] = __uint_as_float(sw[0]);
+        x1[r] = __uint_as_float(sw[1]);
       }
-      __builtin_amdgcn_s_waitcnt(0xc07f);  // reads of this strip are done before the next chunk overwrites it
+    };
+    constexpr int kOutside = (int)0x80000000u;
+    constexpr int OW = EPI == kEpiSiluMul ? 2 : 1;  // input columns per output column
+    const int outCols = g.N / OW;
+    const __amdgpu_buffer_rsrc_t rsOut =
+        __builtin_amdgcn_make_buffer_rsrc(out, 0, (int)(((int64_t)(g.M - 1) * g.ldo + outCols) * sizeof(T)), 0x00020000);
+    const int col0 = (tn * BN + wn * WN) / OW + cperm;  // this lane's first output column
+    auto offsetOf = [&](int i, int jp, int64_t pitch) {
+      const int row = tm * BM + wm * WM + i * 16 + frow, col = col0 + jp * 32;
+      return row < g.M && col < outCols ? (int)(((int64_t)row * pitch + col) * sizeof(T)) : kOutside;
+    };
+    auto put = [&](int i, int jp, const Frag& o) {
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o), rsOut, offsetOf(i, jp, g.ldo), 0, 0);
+    };
+    if constexpr (EPI == kEpiSiluMul) {
+      // fragments 0, 1 of a wave are gate, 2, 3 the up values of the same 32 channels
+      static_assert(WN == 64, "a wave's columns are one 32 + 32 gate / up block");
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        f32x4 x0, x1;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float g0 = acc[i][0][r], g1 = acc[i][1][r];
+          x0[r] = g0 / (1.f + __expf(-g0)) * acc[i][2][r];
+          x1[r] = g1 / (1.f + __expf(-g1)) * acc[i][3][r];
+        }
+        swapPair(x0, x1);
+        Frag o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = static_cast<T>(x0[e]), o[4 + e] = static_cast<T>(x1[e]);
+        put(i, 0, o);
+      }
+    } else {
+      float bv[TN / 2][8];
+#pragma unroll
+      for (int jp = 0; jp < TN / 2; ++jp) {
+        const int col = min(col0 + jp * 32, g.N - 8);  // N % 8 == 0 here; a clamped piece is never stored
+        Frag b8;
+        if (bias) b8 = *reinterpret_cast<const Frag*>(bias + col);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) bv[jp][e] = bias ? static_cast<float>(b8[e]) : 0.f;
+      }
+      auto store = [&](auto withAddend) {
+        constexpr bool kAddend = decltype(withAddend)::value;
+        const __amdgpu_buffer_rsrc_t rsC = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<T*>(kAddend ? cin : out), 0, (int)(((int64_t)(g.M - 1) * g.sCm + g.N) * sizeof(T)), 0x00020000);
+        u32x4 cv[2][TN / 2];
+        auto fetch = [&](int i) {
+#pragma unroll
+          for (int jp = 0; jp < TN / 2; ++jp)
+            cv[i & 1][jp] = __builtin_amdgcn_raw_buffer_load_b128(rsC, offsetOf(i, jp, g.sCm), 0, 0);
+        };
+        if constexpr (kAddend) fetch(0);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          if constexpr (kAddend)
+            if (i + 1 < TM) fetch(i + 1);
+#pragma unroll
+          for (int jp = 0; jp < TN / 2; ++jp) {
+            f32x4 x0 = acc[i][2 * jp], x1 = acc[i][2 * jp + 1];
+            swapPair(x0, x1);
+            const float v[8] = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+            Frag o, c8;
+            if constexpr (kAddend) c8 = __builtin_bit_cast(Frag, cv[i & 1][jp]);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              float x = v[e] * g.alpha + bv[jp][e];
+              if constexpr (kAddend) x += g.beta * static_cast<float>(c8[e]);
+              o[e] = static_cast<T>(x);
+            }
+            put(i, jp, o);
+          }
+        }
+      };
+      if (cin)
+        store(std::true_type{});
+      else
+        store(std::false_type{});
     }
     return;
   }
-#pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int col = tn * BN + wn * WN + j * 16 + frow;
-    if (col >= g.N) continue;
-    const float bv = bias ? static_cast<float>(bias[col]) : 0.f;
+  // element-wise stores for outputs that do not allow 16-byte pieces; the addend of a fragment row is
+  // requested before the row's first store, for the reason given above
+  auto storeScalar = [&](auto withAddend) {
+    constexpr bool kAddend = decltype(withAddend)::value;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      const int rbase = tm * BM + wm * WM + i * 16 + kq * 4;
+      const int row = tm * BM + wm * WM + i * 16 + frow;
+      if (row >= g.M) continue;
+      float c[TN][4];
+      if constexpr (kAddend) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int row = rbase + r;
-        if (row < g.M) {
-          float v = acc[i][j][r] * g.alpha + bv;
-          if (cin) v += g.beta * static_cast<float>(cin[(int64_t)row * g.sCm + (int64_t)col * g.sCn]);
-          out[(int64_t)row * g.ldo + col] = static_cast<T>(v);
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int col = min(tn * BN + wn * WN + j * 16 + kq * 4 + r, g.N - 1);
+            c[j][r] = static_cast<float>(cin[(int64_t)row * g.sCm + (int64_t)col * g.sCn]);
+          }
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int col = tn * BN + wn * WN + j * 16 + kq * 4 + r;
+          if (col < g.N) {
+            float v = acc[i][j][r] * g.alpha + (bias ? static_cast<float>(bias[col]) : 0.f);
+            if constexpr (kAddend) v += g.beta * c[j][r];
+            out[(int64_t)row * g.ldo + col] = static_cast<T>(v);
+          }
         }
       }
     }
+  };
+  if (cin)
+    storeScalar(std::true_type{});
+  else
+    storeScalar(std::false_type{});
+}
+
+// ------------------------------------------------------------ skinny M (decode) ---
+// At most 64 activation rows against a large K-contiguous weight: the weight matrix is the only traffic
+// that matters and is streamed exactly once. Laid out like the int8 weight-only kernel:
+//   * a workgroup owns NTW tiles of 16 output columns; the KS waves of a tile split K between them and their
+//     fp32 partial sums meet in LDS. NTW * KS is 15 or 16 waves: with few tiles (N / 16 below a few per CU) all of
+//     them go into the K split so that a CU still has 16 waves' worth of loads in flight;
+//   * the activation rows (G groups of 16) are staged once per workgroup in LDS (rows padded by 16 bytes)
+//     by direct-to-LDS loads and read from there as the first MFMA operand; K is processed in chunks of
+//     4096 / G columns so that the staged rows fit. A weight fragment is multiplied against all G groups
+//     while it is in registers;
+//   * lane (n = lane % 16, kgrp = lane / 16) loads 32 consecutive weights of row n per step of 128 (four
+//     16-byte loads; the four kgrps of a row cover 256 contiguous bytes), one step ahead of the MFMAs. Which
+//     K index sits in which MFMA slot is free as long as both operands agree, so no shuffling is needed.
+struct SkinnyArgs {
+  const void* A;
+  const void* B;
+  const void* Cin;
+  const void* bias;
+  void* out;
+  int64_t lda, ldb, ldo, sCm, sCn;
+  int M, N, K;
+  float alpha, beta;
+};
+
+constexpr int kSkinnyStep = 128;    // K elements one wave consumes per step (4 kgrps x 32)
+constexpr int kSkinnyPad = 8;       // elements appended to every staged activation row
+constexpr int kSkinnyRowsK = 16 * 4096;  // staged rows x columns per pass: 16 G x (4096 / G + 8) x 2 B <= 129 KiB
+constexpr int kSkinnyMaxM = 64;     // beyond this the tiled kernels take over
+
+template <typename T, int NTW, int KS, int G>
+__global__ __launch_bounds__(NTW * KS * 64) void gemmSkinnyKernel(SkinnyArgs a) {
+  using Frag = typename MfmaOp<T>::Frag;
+  constexpr int THREADS = NTW * KS * 64, CHUNK = kSkinnyRowsK / (16 * G);
+  static_assert(CHUNK / kSkinnyStep >= KS, "every wave of the K split needs a step of the chunk");
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  T* sx = reinterpret_cast<T*>(smem);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = wave / KS, ks = wave % KS;
+  const int r16 = lane & 15, kgrp = lane >> 4;
+  const int n0 = (blockIdx.x * NTW + tile) * 16;
+  const T* wrow = reinterpret_cast<const T*>(a.B) + (int64_t)min(n0 + r16, a.N - 1) * a.ldb + kgrp * 32;
+  const uint64_t xp = reinterpret_cast<uint64_t>(a.A);
+  const u32x4 rsX = {(uint32_t)xp, (uint32_t)(xp >> 32) & 0xffffu, (uint32_t)(((int64_t)(a.M - 1) * a.lda + a.K) * sizeof(T)),
+                     0x00020000u};
+  const unsigned ldsBase = (unsigned)(size_t)(__attribute__((address_space(3))) char*)smem;
+  f32x4 acc[G];
+#pragma unroll
+  for (int gi = 0; gi < G; ++gi) acc[gi] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int kc = 0; kc < a.K; kc += CHUNK) {
+    const int kcLen = min(CHUNK, a.K - kc);  // a multiple of 128, as K is
+    const int ldx = kcLen + kSkinnyPad;
+    // this wave's share of the chunk: a contiguous run of 128-element steps
+    const int steps = kcLen / kSkinnyStep;
+    const int per = (steps + KS - 1) / KS;
+    const int sBegin = ks * per, sEnd = min(steps, sBegin + per);
+    const T* wk = wrow + kc;
+    // the first weight loads go out before the activations are staged
+    Frag w[4];
+    if (sBegin < sEnd) {  // wave-uniform
+#pragma unroll
+      for (int t = 0; t < 4; ++t) w[t] = *reinterpret_cast<const Frag*>(wk + sBegin * kSkinnyStep + 8 * t);
+    }
+    if (kc > 0) __syncthreads();  // everyone is done with the previous chunk's activations
+    // The activations go from memory straight into LDS, 512 columns of one row (1 KiB) per wave instruction:
+    // the row and column of a piece are wave-uniform and travel in the scalar offset and in M0.
+    const int segs = (kcLen + 511) / 512;
+    for (int i = __builtin_amdgcn_readfirstlane(wave); i < a.M * segs; i += THREADS / 64) {
+      const int r = i / segs, c0 = (i - r * segs) * 512;
+      const int from = __builtin_amdgcn_readfirstlane((int)(((int64_t)r * a.lda + kc + c0) * sizeof(T)));
+      const unsigned to = __builtin_amdgcn_readfirstlane(ldsBase + (unsigned)((r * ldx + c0) * sizeof(T)));
+      if (c0 + lane * 8 < kcLen) loadToLds16(rsX, lane * 16, from, to);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0070);  // this wave's pieces have landed
+    __syncthreads();
+    const T* xrow[G];  // fragment rows past M repeat the last row and are discarded
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi) xrow[gi] = sx + min(gi * 16 + r16, a.M - 1) * ldx + kgrp * 32;
+    for (int s = sBegin; s < sEnd; ++s) {
+      Frag c[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) c[t] = w[t];
+      if (s + 1 < sEnd) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) w[t] = *reinterpret_cast<const Frag*>(wk + (s + 1) * kSkinnyStep + 8 * t);
+      }
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int gi = 0; gi < G; ++gi)
+          acc[gi] = MfmaOp16<T>::run(*reinterpret_cast<const Frag*>(xrow[gi] + s * kSkinnyStep + 8 * t), c[t], acc[gi]);
+    }
+  }
+  // the partial sums of the K split meet where the activations were
+  __syncthreads();
+  float* red = reinterpret_cast<float*>(smem);  // [NTW * KS][G][4][64]
+#pragma unroll
+  for (int gi = 0; gi < G; ++gi)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[((wave * G + gi) * 4 + r) * 64 + lane] = acc[gi][r];
+  __syncthreads();
+  const int col = n0 + r16;
+  if (ks == 0 && col < a.N) {
+    T* out = reinterpret_cast<T*>(a.out);
+    const T* cin = reinterpret_cast<const T*>(a.Cin);
+    const float bv = a.bias ? static_cast<float>(reinterpret_cast<const T*>(a.bias)[col]) : 0.f;
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = gi * 16 + kgrp * 4 + r;
+        if (row < a.M) {
+          float v = 0.f;
+#pragma unroll
+          for (int w2 = 0; w2 < KS; ++w2) v += red[(((tile * KS + w2) * G + gi) * 4 + r) * 64 + lane];
+          v = v * a.alpha + bv;
+          if (cin) v += a.beta * static_cast<float>(cin[(int64_t)row * a.sCm + (int64_t)col * a.sCn]);
+          out[(int64_t)row * a.ldo + col] = static_cast<T>(v);
+        }
+      }
   }
 }
 
@@ -679,7 +880,10 @@ static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p
   g.tilesM = (int)ceilDiv(p.M, 256), g.tilesN = (int)ceilDiv(p.N, 256);
   g.alpha = p.alpha, g.beta = p.beta;
   auto al16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
-  g.vecEpilogue = p.N % 8 == 0 && p.sOm % 8 == 0 && p.sOb % 8 == 0 && al16(p.out) &&
+  // the vector epilogue addresses one batch of the output and of the addend with 32-bit byte offsets
+  const bool span32 = ((p.M - 1) * p.sOm + p.N) * (int64_t)sizeof(T) < (int64_t(1) << 31) &&
+                      (!p.Cin || ((p.M - 1) * p.sCm + p.N) * (int64_t)sizeof(T) < (int64_t(1) << 31));
+  g.vecEpilogue = p.N % 8 == 0 && p.sOm % 8 == 0 && p.sOb % 8 == 0 && al16(p.out) && span32 &&
                   (!p.Cin || (p.sCn == 1 && p.sCm % 8 == 0 && p.sCb % 8 == 0 && al16(p.Cin))) && (!p.bias || al16(p.bias));
   constexpr size_t lds = 2 * (size_t)(256 + 256) * kBK * sizeof(T);
   AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmMfmaPipelinedKernel<T, EPI>), (int)lds));
@@ -688,6 +892,48 @@ static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p
   hipLaunchKernelGGL((gemmMfmaPipelinedKernel<T, EPI>), grid, dim3(kPipeThreads), lds, stream, g);
   AMD_LAUNCH_CHECK();
   return diopiSuccess;
+}
+
+template <typename T, int NTW, int KS, int G>
+static diopiError_t launchSkinny(hipStream_t stream, const SkinnyArgs& a) {
+  constexpr int CHUNK = kSkinnyRowsK / (16 * G);
+  const size_t staged = (size_t)a.M * (std::min(a.K, CHUNK) + kSkinnyPad) * sizeof(T);
+  const size_t lds = std::max(staged, (size_t)NTW * KS * G * 4 * 64 * sizeof(float));
+  // the largest request (16 G rows x one chunk) covers every later one
+  AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmSkinnyKernel<T, NTW, KS, G>),
+                          16 * G * (CHUNK + kSkinnyPad) * (int)sizeof(T)));
+  const int tiles = (a.N + 15) / 16;
+  dim3 grid((unsigned)((tiles + NTW - 1) / NTW));
+  hipLaunchKernelGGL((gemmSkinnyKernel<T, NTW, KS, G>), grid, dim3(NTW * KS * 64), lds, stream, a);
+  AMD_LAUNCH_CHECK();
+  return diopiSuccess;
+}
+
+template <typename T>
+static diopiError_t launchSkinnyForShape(hipStream_t stream, const GemmProblem& p) {
+  SkinnyArgs a;
+  a.A = p.A, a.B = p.B, a.Cin = p.Cin, a.bias = p.bias, a.out = p.out;
+  a.lda = p.sAm, a.ldb = p.sBn, a.ldo = p.sOm, a.sCm = p.sCm, a.sCn = p.sCn;
+  a.M = (int)p.M, a.N = (int)p.N, a.K = (int)p.K;
+  a.alpha = p.alpha, a.beta = p.beta;
+  // 16-column tiles per workgroup: about one workgroup per CU, the other waves of the 16 split K (a chunk of
+  // 1024 columns, at four row groups, has only 8 steps to split)
+  const int tiles = (a.N + 15) / 16, perCu = (tiles + computeUnits() - 1) / computeUnits();
+  if (a.M <= 16) {
+    if (perCu >= 4) return launchSkinny<T, 4, 4, 1>(stream, a);
+    if (perCu == 3) return launchSkinny<T, 3, 5, 1>(stream, a);
+    if (perCu == 2) return launchSkinny<T, 2, 8, 1>(stream, a);
+    return launchSkinny<T, 1, 16, 1>(stream, a);
+  }
+  if (a.M <= 32) {
+    if (perCu >= 4) return launchSkinny<T, 4, 4, 2>(stream, a);
+    if (perCu == 3) return launchSkinny<T, 3, 5, 2>(stream, a);
+    if (perCu == 2) return launchSkinny<T, 2, 8, 2>(stream, a);
+    return launchSkinny<T, 1, 16, 2>(stream, a);
+  }
+  if (perCu >= 4) return launchSkinny<T, 4, 4, 4>(stream, a);
+  if (perCu == 3) return launchSkinny<T, 3, 5, 4>(stream, a);
+  return launchSkinny<T, 2, 8, 4>(stream, a);
 }
 
 static bool mult8(int64_t v) { return (v & 7) == 0; }
@@ -726,6 +972,11 @@ diopiError_t runGemm(diopiContextHandle_t ctx, hipStream_t stream, GemmProblem p
       AMD_TRY(launchTranspose<uint16_t>(stream, ws, p.B, nb, p.K, p.N, p.sBk, p.sBn, sbb));
       p.B = ws, p.sBk = 1, p.sBn = p.K, p.sBb = (sbb == 0) ? 0 : p.N * p.K;
     }
+    // up to 32 rows always; up to 64 only while N is too small to give the tiled kernel a tile per CU
+    // (measured at K = 4096: 64 rows take 21 us against 52 us at N = 4096, 57 us against 53 us at N = 22016)
+    if (p.batch == 1 && (p.M <= 32 || (p.M <= kSkinnyMaxM && p.N <= 8192)) && p.K % kSkinnyStep == 0 && p.N >= 16 &&
+        ((p.M - 1) * p.sAm + p.K) * item < (int64_t(1) << 31))
+      return p.dtype == diopi_dtype_bfloat16 ? launchSkinnyForShape<bf16_t>(stream, p) : launchSkinnyForShape<half_t>(stream, p);
     const bool big = ceilDiv(p.M, 256) * ceilDiv(p.N, 256) * p.batch >= 200;
     const bool fits2g = ((p.M - 1) * p.sAm + p.K) * 2 < (int64_t(1) << 31) && ((p.N - 1) * p.sBn + p.K) * 2 < (int64_t(1) << 31);
     if (big && p.K % kBK == 0 && p.K >= 2 * kBK && fits2g) {

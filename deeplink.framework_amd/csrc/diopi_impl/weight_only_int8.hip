@@ -6,9 +6,9 @@
 //     four ways, so a workgroup is NTW*4 waves. NTW grows with N until the grid is about
 //     one workgroup per CU: the activations are then fetched once per CU instead of once
 //     per 16 channels (at M = 16 they are 3x the bytes of a 16-channel weight tile);
-//   * the (up to 16) activation rows the workgroup needs are staged once in LDS (rows padded
-//     by 16 bytes so the 16 rows of a fragment read fall in different banks) and read from
-//     there as MFMA A operands; K larger than the LDS budget is processed in chunks;
+//   * the (up to 16) activation rows the workgroup needs are staged once in LDS by direct-to-LDS
+//     loads (rows padded by 16 bytes so the 16 rows of a fragment read fall in different banks)
+//     and read from there as MFMA A operands; K larger than the LDS budget is processed in chunks;
 //   * v_mfma_f32_16x16x32_{bf16,f16}: the B operand is the weight tile -- lane (n = lane%16,
 //     kgrp = lane/16) loads 32 consecutive int8 of row n (two 16-byte loads; the 4 kgrps of a
 //     row cover 128 contiguous bytes) and converts them to bf16/fp16 in registers while
@@ -74,6 +74,21 @@ __device__ __forceinline__ typename W8Mfma<T>::Frag cvt8(uint32_t lo, uint32_t h
   return r;
 }
 
+// buffer_load_dwordx4 ... lds: lane l fetches 16 bytes at rsrc + voffset + soffset and the data lands in LDS at
+// ldsAddr + 16 * l without passing through registers (the LDS address travels in M0, which is put back).
+__device__ __forceinline__ void loadToLds16(u32x4 rsrc, int voffset, int soffset, unsigned ldsAddr) {
+  unsigned savedM0;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\t"
+      "s_mov_b32 m0, %1\n\t"
+      "s_nop 0\n\t"
+      "buffer_load_dwordx4 %2, %3, %4 offen lds\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(savedM0)
+      : "s"(ldsAddr), "v"(voffset), "s"(rsrc), "s"(soffset)
+      : "memory");
+}
+
 constexpr int kW8Block = 128;   // K elements one wave consumes per step (4 kgrps x 32)
 // One step (two 16-byte loads per lane) is in flight ahead of the one being multiplied, no more: measured,
 // a deeper queue is slower (9.7 us with four steps ahead, 10.4 with eight, 8.8 with one or two at M = 1).
@@ -96,7 +111,10 @@ __global__ __launch_bounds__(NTW * kW8KSplit * 64) void w8LinearKernel(W8Args a)
   const int rows = min(16, a.M - m0);
   const int mrow = min(r16, rows - 1);  // fragment rows past M repeat the last row and are discarded
   const int8_t* wrow = a.w + (int64_t)min(n0 + r16, a.N - 1) * a.ldw + kgrp * 32;
-  const T* xg = reinterpret_cast<const T*>(a.x) + (int64_t)m0 * a.ldx;
+  const uint64_t xp = reinterpret_cast<uint64_t>(reinterpret_cast<const T*>(a.x) + (int64_t)m0 * a.ldx);
+  const u32x4 rsX = {(uint32_t)xp, (uint32_t)(xp >> 32) & 0xffffu, (uint32_t)(((int64_t)(rows - 1) * a.ldx + a.K) * sizeof(T)),
+                     0x00020000u};
+  const unsigned ldsBase = (unsigned)(size_t)(__attribute__((address_space(3))) char*)w8smem;
   // scale and bias of this lane's output channel: requested now, used after the last weight has been consumed
   const int col = n0 + r16;
   float sc = 0.f, bv = 0.f;
@@ -120,11 +138,16 @@ __global__ __launch_bounds__(NTW * kW8KSplit * 64) void w8LinearKernel(W8Args a)
       w1 = *reinterpret_cast<const u32x4*>(wk + sBegin * kW8Block + 16);
     }
     if (kc > 0) __syncthreads();  // everyone is done with the previous chunk's activations
-    const int cpr = kcLen / 8;
-    for (int i = threadIdx.x; i < rows * cpr; i += THREADS) {
-      const int r = i / cpr, c = i - r * cpr;
-      *reinterpret_cast<Frag*>(sx + r * ldx + c * 8) = *reinterpret_cast<const Frag*>(xg + (int64_t)r * a.ldx + kc + c * 8);
+    // The activations go from memory straight into LDS, 512 columns of one row (1 KiB) per wave instruction:
+    // the row and column of a piece are wave-uniform and travel in the scalar offset and in M0.
+    const int segs = (kcLen + 511) / 512;
+    for (int i = __builtin_amdgcn_readfirstlane(wave); i < rows * segs; i += THREADS / 64) {
+      const int r = i / segs, c0 = (i - r * segs) * 512;
+      const int from = __builtin_amdgcn_readfirstlane((int)(((int64_t)r * a.ldx + kc + c0) * sizeof(T)));
+      const unsigned to = __builtin_amdgcn_readfirstlane(ldsBase + (unsigned)((r * ldx + c0) * sizeof(T)));
+      if (c0 + lane * 8 < kcLen) loadToLds16(rsX, lane * 16, from, to);
     }
+    __builtin_amdgcn_s_waitcnt(0x0070);  // this wave's pieces have landed
     __syncthreads();
     const T* xrow = sx + mrow * ldx + kgrp * 32;
     for (int s = sBegin; s < sEnd; ++s) {

@@ -117,6 +117,31 @@ def test_large_tile_gemm_batched_and_row_strided_operands(ops, dev):
     assert_half(ops.bmm(a, bb.to(dev).transpose(1, 2)), torch.bmm(a.float().cpu(), bb.float().transpose(1, 2)))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (5, 100, 8192 + 128), (16, 11008, 4096), (17, 4096, 11008),
+                                   (40, 16 * 7 + 3, 384), (64, 32000, 128), (1, 16, 128)])
+def test_skinny_m_linear_and_addmm(ops, dev, dtype, m, n, k):
+    """At most 64 rows against a K-contiguous weight with K a multiple of 128 select the weight-streaming kernel:
+    one, two and four 16-column tiles per workgroup (N = 4096, 11008, 32000), K in one and in two staged chunks
+    and down to a single step per wave, row groups of 16 with a ragged last group, ragged N, bias, and the
+    alpha / beta epilogue with a full and a broadcast addend."""
+    x = torch.randn(m, k, generator=g(50)).to(dtype)
+    w = (torch.randn(n, k, generator=g(51)) * 0.05).to(dtype)
+    b = torch.randn(n, generator=g(52)).to(dtype)
+    want = x.float() @ w.float().t()
+    dx, dw = x.to(dev), w.to(dev)
+    assert_half(ops.linear(dx, dw), want)
+    assert_half(ops.linear(dx, dw, b.to(dev)), want + b.float())
+    c = torch.randn(m, n, generator=g(53)).to(dtype)
+    assert_half(ops.addmm(c.to(dev), dx, dw.t(), beta=0.5, alpha=2), 0.5 * c.float() + 2 * want)
+    assert_half(ops.addmm(b.to(dev), dx, dw.t()), b.float() + want)
+    # a one-hot row selects a weight column exactly
+    onehot = torch.zeros(m, k, dtype=dtype, device=dev)
+    cols = torch.randint(0, k, (m,), generator=g(54)).to(dev)
+    onehot[torch.arange(m, device=dev), cols] = 1
+    assert_exact(ops.linear(onehot, dw), dw[:, cols].t().contiguous().cpu())
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("m,f,k", [(4096, 3584, 256), (3700, 4000 - 32, 192), (96, 64, 80), (1, 32, 8)])
 def test_linear_silu_mul(ops, dev, dtype, m, f, k):
