@@ -72,6 +72,8 @@ struct MfmaArgs {
   int tilesM, tilesN;
   float alpha, beta;
   bool vecEpilogue;  // out / addend / bias allow 16-byte row segments
+  float* partial = nullptr;  // split-K: fp32 partial products [gridDim.y][M][N]
+  int kTilesPerSplit = 0;
 };
 
 constexpr int kBK = 64;  // K elements per LDS tile (128-byte rows)
@@ -300,8 +302,10 @@ __device__ __forceinline__ void loadToLds16(u32x4 rsrc, int voffset, int soffset
 
 // EPI selects the epilogue: kEpiLinear is alpha * acc + beta * C + bias; kEpiSiluMul treats every 64 consecutive
 // output columns as 32 gate columns followed by the 32 up columns of the same channels and stores
-// silu(gate) * up, half as wide (out has N / 2 columns).
-enum PipeEpilogue { kEpiLinear = 0, kEpiSiluMul = 1 };
+// silu(gate) * up, half as wide (out has N / 2 columns); kEpiPartial is the split-K form: workgroup (tile, s)
+// multiplies K tiles [s * kTilesPerSplit, ...) and stores its fp32 accumulators to partial[s], to be summed and
+// given the linear epilogue by splitKReduceKernel.
+enum PipeEpilogue { kEpiLinear = 0, kEpiSiluMul = 1, kEpiPartial = 2 };
 
 template <typename T, int EPI>
 __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs g) {
@@ -333,8 +337,10 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
     tn = in / gsize;
   }
   const int batch = blockIdx.z;
-  const T* A = reinterpret_cast<const T*>(g.A) + (int64_t)batch * g.sAb;
-  const T* B = reinterpret_cast<const T*>(g.B) + (int64_t)batch * g.sBb;
+  // split-K: this workgroup's K range starts kFirst tiles in (0 otherwise); the operands are simply entered there
+  const int kFirst = EPI == kEpiPartial ? (int)blockIdx.y * g.kTilesPerSplit : 0;
+  const T* A = reinterpret_cast<const T*>(g.A) + (int64_t)batch * g.sAb + kFirst * kBK;
+  const T* B = reinterpret_cast<const T*>(g.B) + (int64_t)batch * g.sBb + kFirst * kBK;
   // Operand tiles go from memory straight into LDS: lane l of a wave fills the l-th 16-byte slot of a
   // 1 KiB block (8 rows of 128 bytes), so the chunk swizzle is applied on the global side: the lane
   // that owns physical slot (row, c) fetches logical chunk c ^ ((row >> 1) & 7). A 32-bit per-lane
@@ -346,8 +352,8 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
     u32x4 d = {(uint32_t)p, (uint32_t)(p >> 32) & 0xffffu, (uint32_t)bytes, 0x00020000u};
     return d;
   };
-  const u32x4 rsA = descriptor(A, ((int64_t)(g.M - 1) * g.lda + g.K) * 2);
-  const u32x4 rsB = descriptor(B, ((int64_t)(g.N - 1) * g.ldb + g.K) * 2);
+  const u32x4 rsA = descriptor(A, ((int64_t)(g.M - 1) * g.lda + g.K - kFirst * kBK) * 2);
+  const u32x4 rsB = descriptor(B, ((int64_t)(g.N - 1) * g.ldb + g.K - kFirst * kBK) * 2);
   int aOffG[CH], bOffG[CH];
   const int srow = tid >> 3;  // staging row of chunk 0; chunk i is RS rows further (same swizzle)
   const int c8 = ((tid & 7) ^ ((srow >> 1) & 7)) * 8;
@@ -360,7 +366,7 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
   constexpr unsigned kStageBytes = BM * kBK * sizeof(T), kPassBytes = RS * kBK * sizeof(T);
   const unsigned ldsWave = (unsigned)(size_t)(__attribute__((address_space(3))) char*)smem +
                            __builtin_amdgcn_readfirstlane(wave) * 1024u;
-  const int nK = g.K / kBK;
+  const int nK = EPI == kEpiPartial ? min(g.kTilesPerSplit, g.K / kBK - kFirst) : g.K / kBK;
 
   const int frow = lane & 15, kq = lane >> 4;
   const int swz = (frow >> 1) & 7;  // fragment rows are 16 apart: they all share this lane's swizzle
@@ -485,6 +491,23 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
   iter(false_type{}, false_type{}, nK - 1);
 
   // ---- epilogue
+  if constexpr (EPI == kEpiPartial) {
+    // the accumulators as they are: a lane holds 4 consecutive fp32 columns of one row per fragment, one 16-byte
+    // store each; pieces outside the matrix get an offset past the end of the buffer and are dropped
+    float* part = g.partial + (int64_t)blockIdx.y * g.M * g.N;
+    const __amdgpu_buffer_rsrc_t rsP = __builtin_amdgcn_make_buffer_rsrc(part, 0, (int)((int64_t)g.M * g.N * 4), 0x00020000);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int row = tm * BM + wm * WM + i * 16 + frow;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int col = tn * BN + wn * WN + j * 16 + kq * 4;
+        const int off = row < g.M && col < g.N ? (int)(((int64_t)row * g.N + col) * 4) : (int)0x80000000u;
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][j]), rsP, off, 0, 0);
+      }
+    }
+    return;
+  }
   T* out = reinterpret_cast<T*>(g.out) + (int64_t)batch * g.sOb;
   const T* cin = g.Cin ? reinterpret_cast<const T*>(g.Cin) + (int64_t)batch * g.sCb : nullptr;
   const T* bias = reinterpret_cast<const T*>(g.bias);
@@ -870,8 +893,52 @@ static diopiError_t launchMfma(hipStream_t stream, const GemmProblem& p) {
   return diopiSuccess;
 }
 
+// Second pass of split-K: out = alpha * sum_s partial[s] + bias + beta * C, 8 columns per lane.
+template <typename T>
+__global__ __launch_bounds__(256) void splitKReduceKernel(MfmaArgs g, int splits) {
+  using Frag = typename MfmaOp<T>::Frag;
+  const int groups = g.N / 8;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)g.M * groups) return;
+  const int row = (int)(idx / groups), col = (int)(idx - (int64_t)row * groups) * 8;
+  const float* src = g.partial + (int64_t)row * g.N + col;
+  f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = lo;
+  for (int sp = 0; sp < splits; ++sp) {
+    lo += *reinterpret_cast<const f32x4*>(src + (int64_t)sp * g.M * g.N);
+    hi += *reinterpret_cast<const f32x4*>(src + (int64_t)sp * g.M * g.N + 4);
+  }
+  const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  const T* cin = reinterpret_cast<const T*>(g.Cin);
+  const T* bias = reinterpret_cast<const T*>(g.bias);
+  Frag o, cv, bv;
+  if (cin) cv = *reinterpret_cast<const Frag*>(cin + (int64_t)row * g.sCm + col);
+  if (bias) bv = *reinterpret_cast<const Frag*>(bias + col);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    float x = v[e] * g.alpha;
+    if (bias) x += static_cast<float>(bv[e]);
+    if (cin) x += g.beta * static_cast<float>(cv[e]);
+    o[e] = static_cast<T>(x);
+  }
+  *reinterpret_cast<Frag*>(reinterpret_cast<T*>(g.out) + (int64_t)row * g.ldo + col) = o;
+}
+
+// How many ways to split K so that a problem with few 256 x 256 tiles still fills the chip: tiles * splits close
+// to the CU count, at least four K tiles per split, at most 16 splits. 1 = do not split.
+// *perSplit receives the K tiles per split; the last split has the remainder, never fewer than two (the kernel's
+// pipeline needs two).
+static int splitKWays(int64_t tiles, int64_t kTiles, int* perSplit) {
+  const int64_t byChip = computeUnits() / std::max<int64_t>(tiles, 1), byK = kTiles / 4;
+  int64_t splits = std::max<int64_t>(1, std::min<int64_t>(16, std::min(byChip, byK)));
+  int64_t per = ceilDiv(kTiles, splits);
+  while (per < kTiles && kTiles % per == 1) ++per;
+  *perSplit = (int)per;
+  return (int)ceilDiv(kTiles, per);
+}
+
 template <typename T, int EPI = kEpiLinear>
-static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p) {
+static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p, float* partial = nullptr, int splits = 1,
+                                        int kTilesPerSplit = 0) {
   MfmaArgs g;
   g.A = p.A, g.B = p.B, g.out = p.out, g.Cin = p.Cin, g.bias = p.bias;
   g.sAb = p.sAb, g.lda = p.sAm, g.sBb = p.sBb, g.ldb = p.sBn, g.sOb = p.sOb, g.ldo = p.sOm;
@@ -887,10 +954,18 @@ static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p
                   (!p.Cin || (p.sCn == 1 && p.sCm % 8 == 0 && p.sCb % 8 == 0 && al16(p.Cin))) && (!p.bias || al16(p.bias));
   constexpr size_t lds = 2 * (size_t)(256 + 256) * kBK * sizeof(T);
   AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmMfmaPipelinedKernel<T, EPI>), (int)lds));
-  dim3 grid((unsigned)(g.tilesM * g.tilesN), 1, (unsigned)p.batch);
+  g.partial = partial;
+  g.kTilesPerSplit = kTilesPerSplit;
+  dim3 grid((unsigned)(g.tilesM * g.tilesN), (unsigned)splits, (unsigned)p.batch);
   if (EPI == kEpiSiluMul) AMD_CHECK(g.vecEpilogue, "gated linear: output rows must allow 16-byte stores");
+  if (EPI == kEpiPartial) AMD_CHECK(g.vecEpilogue && p.batch == 1 && partial, "split-K: needs the vector epilogue and one batch");
   hipLaunchKernelGGL((gemmMfmaPipelinedKernel<T, EPI>), grid, dim3(kPipeThreads), lds, stream, g);
   AMD_LAUNCH_CHECK();
+  if (EPI == kEpiPartial) {
+    const int64_t items = p.M * (p.N / 8);
+    hipLaunchKernelGGL(splitKReduceKernel<T>, dim3((unsigned)ceilDiv(items, 256)), dim3(256), 0, stream, g, splits);
+    AMD_LAUNCH_CHECK();
+  }
   return diopiSuccess;
 }
 
@@ -977,10 +1052,26 @@ diopiError_t runGemm(diopiContextHandle_t ctx, hipStream_t stream, GemmProblem p
     if (p.batch == 1 && (p.M <= 32 || (p.M <= kSkinnyMaxM && p.N <= 8192)) && p.K % kSkinnyStep == 0 && p.N >= 16 &&
         ((p.M - 1) * p.sAm + p.K) * item < (int64_t(1) << 31))
       return p.dtype == diopi_dtype_bfloat16 ? launchSkinnyForShape<bf16_t>(stream, p) : launchSkinnyForShape<half_t>(stream, p);
-    const bool big = ceilDiv(p.M, 256) * ceilDiv(p.N, 256) * p.batch >= 200;
+    // from 144 tiles (56 % of the CUs in one round) the large-tile kernel beats the 128 x 128 one even unsplit
+    const bool big = ceilDiv(p.M, 256) * ceilDiv(p.N, 256) * p.batch >= 144;
     const bool fits2g = ((p.M - 1) * p.sAm + p.K) * 2 < (int64_t(1) << 31) && ((p.N - 1) * p.sBn + p.K) * 2 < (int64_t(1) << 31);
     if (big && p.K % kBK == 0 && p.K >= 2 * kBK && fits2g) {
       return p.dtype == diopi_dtype_bfloat16 ? launchMfmaPipelined<bf16_t>(stream, p) : launchMfmaPipelined<half_t>(stream, p);
+    }
+    // In between (too few 256 x 256 tiles for the chip, too many rows for the weight-streaming kernel): the same
+    // large-tile kernel with K split over grid.y, fp32 partial products in workspace and a reduction pass.
+    if (!big && p.batch == 1 && p.K % kBK == 0 && fits2g && p.N % 8 == 0 && p.sOm % 8 == 0 && ptr16(p.out) &&
+        (!p.Cin || (p.sCn == 1 && p.sCm % 8 == 0 && ptr16(p.Cin))) && (!p.bias || ptr16(p.bias)) &&
+        p.M * p.N * 4 < (int64_t(1) << 31)) {
+      int per = 0;
+      const int splits = splitKWays(ceilDiv(p.M, 256) * ceilDiv(p.N, 256), p.K / kBK, &per);
+      if (splits >= 2) {
+        void* ws = nullptr;
+        AMD_TRY(requireWorkspace(ctx, (int64_t)splits * p.M * p.N * 4, &ws));
+        return p.dtype == diopi_dtype_bfloat16
+                   ? launchMfmaPipelined<bf16_t, kEpiPartial>(stream, p, static_cast<float*>(ws), splits, per)
+                   : launchMfmaPipelined<half_t, kEpiPartial>(stream, p, static_cast<float*>(ws), splits, per);
+      }
     }
     if (p.dtype == diopi_dtype_bfloat16) {
       return big ? launchMfma<bf16_t, 256, 256>(stream, p) : launchMfma<bf16_t, 128, 128>(stream, p);
@@ -1028,7 +1119,7 @@ static diopiError_t runGatedSiluGemm(diopiContextHandle_t ctx, hipStream_t strea
   const int64_t f = p.N / 2;
   const bool half = p.dtype == diopi_dtype_bfloat16 || p.dtype == diopi_dtype_float16;
   const bool direct = half && p.batch == 1 && p.sAk == 1 && mult8(p.sAm) && ptr16(p.A) && p.sBk == 1 && mult8(p.sBn) && ptr16(p.B) &&
-                      ceilDiv(p.M, 256) * ceilDiv(p.N, 256) >= 200 && p.K % kBK == 0 && p.K >= 2 * kBK &&
+                      ceilDiv(p.M, 256) * ceilDiv(p.N, 256) >= 144 && p.K % kBK == 0 && p.K >= 2 * kBK &&
                       ((p.M - 1) * p.sAm + p.K) * 2 < (int64_t(1) << 31) && ((p.N - 1) * p.sBn + p.K) * 2 < (int64_t(1) << 31) &&
                       mult8(p.sOm) && ptr16(p.out) && p.M < (int64_t(1) << 31) && p.N < (int64_t(1) << 31);
   if (direct) {

@@ -91,7 +91,7 @@ def test_gemm_linearity_at_7b_shapes(ops, dev):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("m,n,k", [(3500, 3700, 128), (3500, 3700, 192), (3841, 3585, 320), (4096, 4096, 1088)])
 def test_large_tile_gemm_edges_and_k_tile_counts(ops, dev, dtype, m, n, k):
-    """At least 200 tiles of 256 x 256 and K a multiple of 64 select the 8-wave kernel whose tiles are loaded
+    """At least 144 tiles of 256 x 256 and K a multiple of 64 select the 8-wave kernel whose tiles are loaded
     straight into LDS: two, three, five and seventeen K tiles (even and odd ring positions at the end),
     ragged last tile rows / columns, bias, and the alpha / beta epilogue."""
     x = torch.randn(m, k, generator=g(40)).to(dtype)
@@ -115,6 +115,29 @@ def test_large_tile_gemm_batched_and_row_strided_operands(ops, dev):
     assert_half(ops.matmul(a, w.to(dev).t()), want)
     bb = (torch.randn(4, 1900, 320, generator=g(46)) * 0.05).bfloat16()
     assert_half(ops.bmm(a, bb.to(dev).transpose(1, 2)), torch.bmm(a.float().cpu(), bb.float().transpose(1, 2)))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,n,k", [(1024, 4096, 4096), (300, 520, 1024), (65, 4096, 4096 + 64), (2047, 2048, 576),
+                                   (512, 768, 4096)])
+def test_split_k_gemm(ops, dev, dtype, m, n, k):
+    """More than 64 rows but fewer than 144 tiles of 256 x 256, K a multiple of 64 with at least eight K tiles: the
+    large-tile kernel with K split over the grid (4, 4, 13, 2 and 16 ways here; 65 K tiles in splits of 5, 9 in splits
+    of 5 + 4), fp32 partial products and a reduction pass that applies bias and the alpha / beta epilogue; ragged
+    last tile rows and columns."""
+    x = torch.randn(m, k, generator=g(60)).to(dtype)
+    w = (torch.randn(n, k, generator=g(61)) * 0.05).to(dtype)
+    b = torch.randn(n, generator=g(62)).to(dtype)
+    want = x.float() @ w.float().t()
+    dx, dw = x.to(dev), w.to(dev)
+    assert_half(ops.linear(dx, dw), want)
+    assert_half(ops.linear(dx, dw, b.to(dev)), want + b.float())
+    c = torch.randn(m, n, generator=g(63)).to(dtype)
+    assert_half(ops.addmm(c.to(dev), dx, dw.t(), beta=0.5, alpha=2), 0.5 * c.float() + 2 * want)
+    onehot = torch.zeros(m, k, dtype=dtype, device=dev)
+    cols = torch.randint(0, k, (m,), generator=g(64)).to(dev)
+    onehot[torch.arange(m, device=dev), cols] = 1
+    assert_exact(ops.linear(onehot, dw), dw[:, cols].t().contiguous().cpu())
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
@@ -145,7 +168,7 @@ def test_skinny_m_linear_and_addmm(ops, dev, dtype, m, n, k):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("m,f,k", [(4096, 3584, 256), (3700, 4000 - 32, 192), (96, 64, 80), (1, 32, 8)])
 def test_linear_silu_mul(ops, dev, dtype, m, f, k):
-    """silu(x Wg^T) * (x Wu^T) from the interleaved weight: the single-launch path (at least 200 tiles, K a
+    """silu(x Wg^T) * (x Wu^T) from the interleaved weight: the single-launch path (at least 144 tiles, K a
     multiple of 64, 16-bit dtypes) and the two-pass path, against the reference's four-op form in fp32."""
     x = torch.randn(m, k, generator=g(60)).to(dtype)
     wg = (torch.randn(f, k, generator=g(61)) * 0.08).to(dtype)
