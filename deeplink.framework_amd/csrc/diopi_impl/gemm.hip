@@ -29,6 +29,8 @@
 //   * small or ragged problems: 128x128 (or 256x256) tiles with 4 waves of v_mfma_f32_32x32x16,
 //     staged through registers, any K that is a multiple of 8, stores straight from the
 //     accumulator layout;
+//   * more than 64 rows but too few 256x256 tiles to fill the chip: the large-tile kernel with K split over
+//     grid.y, fp32 partial products in workspace, and a reduction pass that applies the epilogue;
 //   * at most 32 rows (64 while N is small), the decode shape: a weight-streaming kernel with 16-column tiles
 //     whose waves split K and stage the activation rows in LDS.
 // Operands that are not K-contiguous (mm with a row-major mat2, bmm's second operand) are
