@@ -658,6 +658,9 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
 //   * a workgroup owns NTW tiles of 16 output columns; the KS waves of a tile split K between them and their
 //     fp32 partial sums meet in LDS. NTW * KS is 15 or 16 waves: with few tiles (N / 16 below a few per CU) all of
 //     them go into the K split so that a CU still has 16 waves' worth of loads in flight;
+//   * with four row groups K is also split over grid.y, one staged chunk per workgroup, and workgroups are up to
+//     four tiles wide: every workgroup stages all the rows, and at one tile per workgroup the activations would
+//     be four times the weight bytes on the L2 -> CU path. The slices meet in fp32 workspace (splitKReduceKernel);
 //   * the activation rows (G groups of 16) are staged once per workgroup in LDS (rows padded by 16 bytes)
 //     by direct-to-LDS loads and read from there as the first MFMA operand; K is processed in chunks of
 //     4096 / G columns so that the staged rows fit. A weight fragment is multiplied against all G groups
@@ -674,6 +677,8 @@ struct SkinnyArgs {
   int64_t lda, ldb, ldo, sCm, sCn;
   int M, N, K;
   float alpha, beta;
+  float* partial;  // K split over grid.y: fp32 partial products [gridDim.y][M][N] for splitKReduceKernel, else null
+  int kPerWg;      // K columns per grid.y slice (K when not split)
 };
 
 constexpr int kSkinnyStep = 128;    // K elements one wave consumes per step (4 kgrps x 32)
@@ -700,8 +705,9 @@ __global__ __launch_bounds__(NTW * KS * 64) void gemmSkinnyKernel(SkinnyArgs a) 
   f32x4 acc[G];
 #pragma unroll
   for (int gi = 0; gi < G; ++gi) acc[gi] = f32x4{0.f, 0.f, 0.f, 0.f};
-  for (int kc = 0; kc < a.K; kc += CHUNK) {
-    const int kcLen = min(CHUNK, a.K - kc);  // a multiple of 128, as K is
+  const int kBegin = blockIdx.y * a.kPerWg, kEnd = min(a.K, kBegin + a.kPerWg);
+  for (int kc = kBegin; kc < kEnd; kc += CHUNK) {
+    const int kcLen = min(CHUNK, kEnd - kc);  // a multiple of 128, as K and the slices are
     const int ldx = kcLen + kSkinnyPad;
     // this wave's share of the chunk: a contiguous run of 128-element steps
     const int steps = kcLen / kSkinnyStep;
@@ -714,7 +720,7 @@ __global__ __launch_bounds__(NTW * KS * 64) void gemmSkinnyKernel(SkinnyArgs a) 
 #pragma unroll
       for (int t = 0; t < 4; ++t) w[t] = *reinterpret_cast<const Frag*>(wk + sBegin * kSkinnyStep + 8 * t);
     }
-    if (kc > 0) __syncthreads();  // everyone is done with the previous chunk's activations
+    if (kc > kBegin) __syncthreads();  // everyone is done with the previous chunk's activations
     // The activations go from memory straight into LDS, 512 columns of one row (1 KiB) per wave instruction:
     // the row and column of a piece are wave-uniform and travel in the scalar offset and in M0.
     const int segs = (kcLen + 511) / 512;
@@ -766,6 +772,10 @@ __global__ __launch_bounds__(NTW * KS * 64) void gemmSkinnyKernel(SkinnyArgs a) 
           float v = 0.f;
 #pragma unroll
           for (int w2 = 0; w2 < KS; ++w2) v += red[(((tile * KS + w2) * G + gi) * 4 + r) * 64 + lane];
+          if (a.partial) {  // this slice's sum; the reduction pass applies the epilogue
+            a.partial[((int64_t)blockIdx.y * a.M + row) * a.N + col] = v;
+            continue;
+          }
           v = v * a.alpha + bv;
           if (cin) v += a.beta * static_cast<float>(cin[(int64_t)row * a.sCm + (int64_t)col * a.sCn]);
           out[(int64_t)row * a.ldo + col] = static_cast<T>(v);
@@ -979,42 +989,67 @@ static diopiError_t launchSkinny(hipStream_t stream, const SkinnyArgs& a) {
   // the largest request (16 G rows x one chunk) covers every later one
   AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmSkinnyKernel<T, NTW, KS, G>),
                           16 * G * (CHUNK + kSkinnyPad) * (int)sizeof(T)));
-  const int tiles = (a.N + 15) / 16;
-  dim3 grid((unsigned)((tiles + NTW - 1) / NTW));
+  const int tiles = (a.N + 15) / 16, splits = (a.K + a.kPerWg - 1) / a.kPerWg;
+  dim3 grid((unsigned)((tiles + NTW - 1) / NTW), (unsigned)splits);
   hipLaunchKernelGGL((gemmSkinnyKernel<T, NTW, KS, G>), grid, dim3(NTW * KS * 64), lds, stream, a);
   AMD_LAUNCH_CHECK();
+  if (a.partial) {
+    MfmaArgs g;
+    g.out = a.out, g.Cin = a.Cin, g.bias = a.bias, g.partial = a.partial;
+    g.ldo = a.ldo, g.sCm = a.sCm, g.sCn = a.sCn;
+    g.M = a.M, g.N = a.N, g.K = a.K, g.alpha = a.alpha, g.beta = a.beta;
+    hipLaunchKernelGGL(splitKReduceKernel<T>, dim3((unsigned)ceilDiv((int64_t)a.M * (a.N / 8), 256)), dim3(256), 0, stream, g,
+                       splits);
+    AMD_LAUNCH_CHECK();
+  }
   return diopiSuccess;
 }
 
+static bool mult8(int64_t v) { return (v & 7) == 0; }
+static bool ptr16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
 template <typename T>
-static diopiError_t launchSkinnyForShape(hipStream_t stream, const GemmProblem& p) {
+static diopiError_t launchSkinnyForShape(diopiContextHandle_t ctx, hipStream_t stream, const GemmProblem& p) {
   SkinnyArgs a;
   a.A = p.A, a.B = p.B, a.Cin = p.Cin, a.bias = p.bias, a.out = p.out;
   a.lda = p.sAm, a.ldb = p.sBn, a.ldo = p.sOm, a.sCm = p.sCm, a.sCn = p.sCn;
   a.M = (int)p.M, a.N = (int)p.N, a.K = (int)p.K;
   a.alpha = p.alpha, a.beta = p.beta;
-  // 16-column tiles per workgroup: about one workgroup per CU, the other waves of the 16 split K (a chunk of
-  // 1024 columns, at four row groups, has only 8 steps to split)
-  const int tiles = (a.N + 15) / 16, perCu = (tiles + computeUnits() - 1) / computeUnits();
+  a.partial = nullptr, a.kPerWg = a.K;
+  const int tiles = (a.N + 15) / 16, cus = computeUnits(), perCu = (tiles + cus - 1) / cus;
   if (a.M <= 16) {
+    // 16-column tiles per workgroup: about one workgroup per CU, the other waves of the 15 or 16 split K
     if (perCu >= 4) return launchSkinny<T, 4, 4, 1>(stream, a);
     if (perCu == 3) return launchSkinny<T, 3, 5, 1>(stream, a);
     if (perCu == 2) return launchSkinny<T, 2, 8, 1>(stream, a);
     return launchSkinny<T, 1, 16, 1>(stream, a);
   }
-  if (a.M <= 32) {
-    if (perCu >= 4) return launchSkinny<T, 4, 4, 2>(stream, a);
-    if (perCu == 3) return launchSkinny<T, 3, 5, 2>(stream, a);
-    if (perCu == 2) return launchSkinny<T, 2, 8, 2>(stream, a);
+  // More than one group of rows: every workgroup stages all the rows, so with one 16-column tile per workgroup the
+  // activations would be 2-4 times the weight bytes on the L2 -> CU path. Wider workgroups (up to 4 tiles) bring
+  // that to 1:1, and K is split over grid.y as well, one staged chunk per workgroup, to keep the chip full; the
+  // slices meet in fp32 workspace and the split-K reduction pass applies the epilogue.
+  const int groups = a.M <= 32 ? 2 : 4, chunk = kSkinnyRowsK / (16 * groups);
+  const bool canSplit = a.N % 8 == 0 && mult8(p.sOm) && ptr16(p.out) && (!p.bias || ptr16(p.bias)) &&
+                        (!p.Cin || (p.sCn == 1 && mult8(p.sCm) && ptr16(p.Cin)));
+  const int splits = canSplit && groups == 4 ? (a.K + chunk - 1) / chunk : 1;  // two groups: measured no gain
+  if (splits > 1) {
+    void* ws = nullptr;
+    AMD_TRY(requireWorkspace(ctx, (int64_t)splits * a.M * a.N * 4, &ws));
+    a.partial = static_cast<float*>(ws), a.kPerWg = chunk;
+  }
+  const int want = std::max(1, std::min(4, tiles * splits / cus));  // tiles per workgroup that still fill the chip
+  if (groups == 2) {
+    if (want >= 4) return launchSkinny<T, 4, 4, 2>(stream, a);
+    if (want == 3) return launchSkinny<T, 3, 5, 2>(stream, a);
+    if (want == 2) return launchSkinny<T, 2, 8, 2>(stream, a);
     return launchSkinny<T, 1, 16, 2>(stream, a);
   }
-  if (perCu >= 4) return launchSkinny<T, 4, 4, 4>(stream, a);
-  if (perCu == 3) return launchSkinny<T, 3, 5, 4>(stream, a);
-  return launchSkinny<T, 2, 8, 4>(stream, a);
+  if (want >= 4) return launchSkinny<T, 4, 4, 4>(stream, a);
+  if (want == 3) return launchSkinny<T, 3, 5, 4>(stream, a);
+  if (want == 2) return launchSkinny<T, 2, 8, 4>(stream, a);
+  return launchSkinny<T, 1, 8, 4>(stream, a);
 }
 
-static bool mult8(int64_t v) { return (v & 7) == 0; }
-static bool ptr16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 template <typename U>
 static diopiError_t launchTranspose(hipStream_t stream, void* dst, const void* src, int64_t batch, int64_t rows,
@@ -1049,11 +1084,13 @@ diopiError_t runGemm(diopiContextHandle_t ctx, hipStream_t stream, GemmProblem p
       AMD_TRY(launchTranspose<uint16_t>(stream, ws, p.B, nb, p.K, p.N, p.sBk, p.sBn, sbb));
       p.B = ws, p.sBk = 1, p.sBn = p.K, p.sBb = (sbb == 0) ? 0 : p.N * p.K;
     }
-    // up to 32 rows always; up to 64 only while N is too small to give the tiled kernel a tile per CU
-    // (measured at K = 4096: 64 rows take 21 us against 52 us at N = 4096, 57 us against 53 us at N = 22016)
-    if (p.batch == 1 && (p.M <= 32 || (p.M <= kSkinnyMaxM && p.N <= 8192)) && p.K % kSkinnyStep == 0 && p.N >= 16 &&
+    // up to 32 rows always; up to 64 while N is moderate (measured at 64 rows, K = 4096, kernel + reduction
+    // pass: 16 us against 50 us for the split-K tiled kernel at N = 4096, 36 against 52 at N = 12288, 63 against 51
+    // at N = 22016)
+    if (p.batch == 1 && (p.M <= 32 || (p.M <= kSkinnyMaxM && p.N <= 16384)) && p.K % kSkinnyStep == 0 && p.N >= 16 &&
         ((p.M - 1) * p.sAm + p.K) * item < (int64_t(1) << 31))
-      return p.dtype == diopi_dtype_bfloat16 ? launchSkinnyForShape<bf16_t>(stream, p) : launchSkinnyForShape<half_t>(stream, p);
+      return p.dtype == diopi_dtype_bfloat16 ? launchSkinnyForShape<bf16_t>(ctx, stream, p)
+                                             : launchSkinnyForShape<half_t>(ctx, stream, p);
     // from 144 tiles (56 % of the CUs in one round) the large-tile kernel beats the 128 x 128 one even unsplit
     const bool big = ceilDiv(p.M, 256) * ceilDiv(p.N, 256) * p.batch >= 144;
     const bool fits2g = ((p.M - 1) * p.sAm + p.K) * 2 < (int64_t(1) << 31) && ((p.N - 1) * p.sBn + p.K) * 2 < (int64_t(1) << 31);
