@@ -6,7 +6,7 @@
 //     four ways, so a workgroup is NTW*4 waves. NTW grows with N until the grid is about
 //     one workgroup per CU: the activations are then fetched once per CU instead of once
 //     per 16 channels (at M = 16 they are 3x the bytes of a 16-channel weight tile);
-//   * the (up to 16) activation rows the workgroup needs are staged once in LDS by direct-to-LDS
+//   * the (up to 64) activation rows the workgroup needs are staged once in LDS by direct-to-LDS
 //     loads (rows padded by 16 bytes so the 16 rows of a fragment read fall in different banks)
 //     and read from there as MFMA A operands; K larger than the LDS budget is processed in chunks;
 //   * v_mfma_f32_16x16x32_{bf16,f16}: the B operand is the weight tile -- lane (n = lane%16,
@@ -17,8 +17,9 @@
 //   * fp32 accumulators of the 4 K-split waves are summed through LDS; the per-channel scale
 //     is applied to the fp32 sum (identical to scaling the weights first, one rounding fewer),
 //     then bias, then one conversion to the output dtype.
-// Rows of x beyond 16 are handled by more workgroups along grid.y (weights are then re-read
-// per group of 16 rows; large-M prefill should dequantise once and use the dense GEMM).
+// Up to 64 rows of x (4 groups of 16) share every weight fragment while it is in registers; rows
+// beyond 64 are handled by more workgroups along grid.y (weights are then re-read per 64 rows;
+// large-M prefill should dequantise once and use the dense GEMM).
 #include <algorithm>
 
 #include "common.hpp"
@@ -95,21 +96,21 @@ constexpr int kW8Block = 128;   // K elements one wave consumes per step (4 kgrp
 constexpr int kW8KSplit = 4;    // waves per 16-channel tile = K splits
 constexpr int kW8MaxTiles = 4;  // 16-channel tiles per workgroup (16 waves at most)
 constexpr int kW8Pad = 8;       // elements appended to every staged activation row (16 bytes)
-constexpr int kW8ChunkK = 4096; // activation columns staged per pass: 16 x (4096 + 8) x 2 B = 128.25 KiB
+constexpr int kW8RowsK = 16 * 4096; // staged rows x columns per pass: 16 G x (4096 / G + 8) x 2 B <= 129 KiB
 
-template <typename T, int NTW>
+// G groups of 16 activation rows share every weight fragment while it is in registers (K is then staged in chunks
+// of 4096 / G columns so that the rows fit in LDS); more than 16 G rows go to further workgroups along grid.y.
+template <typename T, int NTW, int G>
 __global__ __launch_bounds__(NTW * kW8KSplit * 64) void w8LinearKernel(W8Args a) {
   using Frag = typename W8Mfma<T>::Frag;
-  constexpr int THREADS = NTW * kW8KSplit * 64;
+  constexpr int THREADS = NTW * kW8KSplit * 64, kW8ChunkK = kW8RowsK / (16 * G);
   extern __shared__ __attribute__((aligned(16))) char w8smem[];
   T* sx = reinterpret_cast<T*>(w8smem);
-  __shared__ float red[NTW * kW8KSplit][64][4];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int tile = wave / kW8KSplit, ks = wave % kW8KSplit;
   const int r16 = lane & 15, kgrp = lane >> 4;
-  const int n0 = (blockIdx.x * NTW + tile) * 16, m0 = blockIdx.y * 16;
-  const int rows = min(16, a.M - m0);
-  const int mrow = min(r16, rows - 1);  // fragment rows past M repeat the last row and are discarded
+  const int n0 = (blockIdx.x * NTW + tile) * 16, m0 = blockIdx.y * 16 * G;
+  const int rows = min(16 * G, a.M - m0);
   const int8_t* wrow = a.w + (int64_t)min(n0 + r16, a.N - 1) * a.ldw + kgrp * 32;
   const uint64_t xp = reinterpret_cast<uint64_t>(reinterpret_cast<const T*>(a.x) + (int64_t)m0 * a.ldx);
   const u32x4 rsX = {(uint32_t)xp, (uint32_t)(xp >> 32) & 0xffffu, (uint32_t)(((int64_t)(rows - 1) * a.ldx + a.K) * sizeof(T)),
@@ -122,7 +123,9 @@ __global__ __launch_bounds__(NTW * kW8KSplit * 64) void w8LinearKernel(W8Args a)
     sc = loadAs<float>(a.scale, col, a.scaleDtype);
     if (a.bias) bv = loadAs<float>(a.bias, col, a.biasDtype);
   }
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  f32x4 acc[G];
+#pragma unroll
+  for (int gi = 0; gi < G; ++gi) acc[gi] = f32x4{0.f, 0.f, 0.f, 0.f};
   for (int kc = 0; kc < a.K; kc += kW8ChunkK) {
     const int kcLen = min(kW8ChunkK, a.K - kc);  // a multiple of 128, as K is
     const int ldx = kcLen + kW8Pad;
@@ -149,63 +152,83 @@ __global__ __launch_bounds__(NTW * kW8KSplit * 64) void w8LinearKernel(W8Args a)
     }
     __builtin_amdgcn_s_waitcnt(0x0070);  // this wave's pieces have landed
     __syncthreads();
-    const T* xrow = sx + mrow * ldx + kgrp * 32;
+    const T* xrow[G];  // fragment rows past M repeat the last row and are discarded
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi) xrow[gi] = sx + min(gi * 16 + r16, rows - 1) * ldx + kgrp * 32;
     for (int s = sBegin; s < sEnd; ++s) {
       const u32x4 c0 = w0, c1 = w1;
       if (s + 1 < sEnd) {
         w0 = *reinterpret_cast<const u32x4*>(wk + (s + 1) * kW8Block);
         w1 = *reinterpret_cast<const u32x4*>(wk + (s + 1) * kW8Block + 16);
       }
-      const T* xp = xrow + s * kW8Block;
-      acc = W8Mfma<T>::run(*reinterpret_cast<const Frag*>(xp), cvt8<T>(c0[0], c0[1]), acc);
-      acc = W8Mfma<T>::run(*reinterpret_cast<const Frag*>(xp + 8), cvt8<T>(c0[2], c0[3]), acc);
-      acc = W8Mfma<T>::run(*reinterpret_cast<const Frag*>(xp + 16), cvt8<T>(c1[0], c1[1]), acc);
-      acc = W8Mfma<T>::run(*reinterpret_cast<const Frag*>(xp + 24), cvt8<T>(c1[2], c1[3]), acc);
-    }
-  }
+      const Frag f0 = cvt8<T>(c0[0], c0[1]), f1 = cvt8<T>(c0[2], c0[3]), f2 = cvt8<T>(c1[0], c1[1]), f3 = cvt8<T>(c1[2], c1[3]);
 #pragma unroll
-  for (int r = 0; r < 4; ++r) red[wave][lane][r] = acc[r];
-  __syncthreads();
-  if (ks == 0) {
-    if (col < a.N) {
-      T* out = reinterpret_cast<T*>(a.out);
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int row = m0 + kgrp * 4 + r;
-        if (row < a.M) {
-          float v = 0.f;
-#pragma unroll
-          for (int w = 0; w < kW8KSplit; ++w) v += red[tile * kW8KSplit + w][lane][r];
-          out[(int64_t)row * a.ldo + col] = static_cast<T>(v * sc + bv);
-        }
+      for (int gi = 0; gi < G; ++gi) {
+        const T* xp = xrow[gi] + s * kW8Block;
+        acc[gi] = W8Mfma<T>::run(*reinterpret_cast<const Frag*>(xp), f0, acc[gi]);
+        acc[gi] = W8Mfma<T>::run(*reinterpret_cast<const Frag*>(xp + 8), f1, acc[gi]);
+        acc[gi] = W8Mfma<T>::run(*reinterpret_cast<const Frag*>(xp + 16), f2, acc[gi]);
+        acc[gi] = W8Mfma<T>::run(*reinterpret_cast<const Frag*>(xp + 24), f3, acc[gi]);
       }
     }
   }
+  // the partial sums of the K split meet where the activations were
+  __syncthreads();
+  float* red = reinterpret_cast<float*>(w8smem);  // [NTW * kW8KSplit][G][4][64]
+#pragma unroll
+  for (int gi = 0; gi < G; ++gi)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[((wave * G + gi) * 4 + r) * 64 + lane] = acc[gi][r];
+  __syncthreads();
+  if (ks == 0 && col < a.N) {
+    T* out = reinterpret_cast<T*>(a.out);
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = m0 + gi * 16 + kgrp * 4 + r;
+        if (row < a.M) {
+          float v = 0.f;
+#pragma unroll
+          for (int w = 0; w < kW8KSplit; ++w) v += red[(((tile * kW8KSplit + w) * G + gi) * 4 + r) * 64 + lane];
+          out[(int64_t)row * a.ldo + col] = static_cast<T>(v * sc + bv);
+        }
+      }
+  }
 }
 
-template <typename T, int NTW>
-static diopiError_t launchW8(hipStream_t stream, const W8Args& a, size_t lds) {
-  // the largest request (16 rows x one chunk) covers every later one
-  AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&w8LinearKernel<T, NTW>), 16 * (kW8ChunkK + kW8Pad) * (int)sizeof(T)));
+template <typename T, int NTW, int G>
+static diopiError_t launchW8(hipStream_t stream, const W8Args& a) {
+  constexpr int CHUNK = kW8RowsK / (16 * G);
+  const size_t staged = (size_t)std::min(16 * G, a.M) * (std::min(a.K, CHUNK) + kW8Pad) * sizeof(T);
+  const size_t lds = std::max(staged, (size_t)NTW * kW8KSplit * G * 4 * 64 * sizeof(float));
+  // the largest request (16 G rows x one chunk) covers every later one
+  AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&w8LinearKernel<T, NTW, G>), 16 * G * (CHUNK + kW8Pad) * (int)sizeof(T)));
   const int tiles = (a.N + 15) / 16;
-  dim3 grid((unsigned)((tiles + NTW - 1) / NTW), (unsigned)((a.M + 15) / 16));
-  hipLaunchKernelGGL((w8LinearKernel<T, NTW>), grid, dim3(NTW * kW8KSplit * 64), lds, stream, a);
+  dim3 grid((unsigned)((tiles + NTW - 1) / NTW), (unsigned)((a.M + 16 * G - 1) / (16 * G)));
+  hipLaunchKernelGGL((w8LinearKernel<T, NTW, G>), grid, dim3(NTW * kW8KSplit * 64), lds, stream, a);
   AMD_LAUNCH_CHECK();
   return diopiSuccess;
 }
 
-template <typename T>
-static diopiError_t launchW8ForShape(hipStream_t stream, const W8Args& a) {
+template <typename T, int G>
+static diopiError_t launchW8ForTiles(hipStream_t stream, const W8Args& a) {
   // 16-channel tiles per workgroup: enough to bring the grid down to about one workgroup per CU
   const int tiles = (a.N + 15) / 16;
   const int ntw = std::min(kW8MaxTiles, std::max(1, (tiles + computeUnits() - 1) / computeUnits()));
-  const size_t lds = (size_t)std::min(16, a.M) * (std::min(a.K, kW8ChunkK) + kW8Pad) * sizeof(T);
   switch (ntw) {
-    case 1: return launchW8<T, 1>(stream, a, lds);
-    case 2: return launchW8<T, 2>(stream, a, lds);
-    case 3: return launchW8<T, 3>(stream, a, lds);
-    default: return launchW8<T, 4>(stream, a, lds);
+    case 1: return launchW8<T, 1, G>(stream, a);
+    case 2: return launchW8<T, 2, G>(stream, a);
+    case 3: return launchW8<T, 3, G>(stream, a);
+    default: return launchW8<T, 4, G>(stream, a);
   }
+}
+
+template <typename T>
+static diopiError_t launchW8ForShape(hipStream_t stream, const W8Args& a) {
+  if (a.M <= 16) return launchW8ForTiles<T, 1>(stream, a);
+  if (a.M <= 32) return launchW8ForTiles<T, 2>(stream, a);
+  return launchW8ForTiles<T, 4>(stream, a);
 }
 
 // Any K / alignment: one lane per output element, fp32 accumulate (correctness path).
@@ -274,7 +297,8 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiWeightOnlyIn
   a.ldx = K, a.ldw = N > 1 ? cw.stride[0] : K, a.ldo = N;
   a.M = (int)M, a.N = (int)N, a.K = (int)K;
   a.scaleDtype = csc.dtype, a.biasDtype = bias.defined() ? cb.dtype : diopi_dtype_float32;
-  const bool fast = K % kW8Block == 0 && cin.aligned16() && cw.aligned16() && a.ldw % 16 == 0 && ceilDiv(M, 16) <= 65535;
+  const bool fast = K % kW8Block == 0 && cin.aligned16() && cw.aligned16() && a.ldw % 16 == 0 && ceilDiv(M, 64) <= 65535 &&
+                    (std::min<int64_t>(M, 64) * K + K) * 2 < (int64_t(1) << 31);
   if (fast) {
     if (in.dtype == diopi_dtype_bfloat16) AMD_TRY(launchW8ForShape<bf16_t>(stream, a));
     else AMD_TRY(launchW8ForShape<half_t>(stream, a));

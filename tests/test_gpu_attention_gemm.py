@@ -332,7 +332,8 @@ def test_weight_only_int8_full_shape_exact_cases(ops, dev, pkg):
     got = ops.weight_only_int8_linear(w["x"].to(dev), w["w"].to(dev), w["scale"].to(dev))
     assert_half(got, oracle.weight_only_int8_linear(w["x"], w["w"], w["scale"]))
 
-@pytest.mark.parametrize("m,k,n", [(1, 11008, 4096), (5, 8192 + 128, 100), (37, 4096, 16 * 7 + 3), (16, 4096, 22016)])
+@pytest.mark.parametrize("m,k,n", [(1, 11008, 4096), (5, 8192 + 128, 100), (37, 4096, 16 * 7 + 3), (16, 4096, 22016),
+                                   (64, 4096, 4096), (100, 1024 + 256, 520), (29, 2048 + 128, 11008)])
 def test_weight_only_int8_linear_chunked_k_row_groups_and_tile_counts(ops, dev, pkg, m, k, n):
     """K beyond one staged activation chunk (4096 columns), more than 16 rows (row groups), channel counts that leave
     partly filled workgroups, and an N large enough to use the widest workgroup."""
