@@ -5,9 +5,10 @@
 
 One "step" is one pass of a Llama-2-7B-shaped decoder layer (prefill, batch 4 x seq 2048,
 hidden 4096, 32 heads x 128, FFN 11008, bf16, random weights, synthetic activations) through
-the DIOPI C ABI of libdiopi_impl.so: RMSNorm -> QKV linear -> rotary (q and k heads in one launch) -> causal context
-attention -> out linear + residual (addmm) -> RMSNorm -> gate/up linears -> SiLU*mul -> down linear +
-residual (addmm). Inputs and weights are resident in HBM before the timed region.
+the DIOPI C ABI of libdiopi_impl.so: RMSNorm -> QKV linear with the rotary embedding of the q and k heads in its
+epilogue -> causal context attention -> out linear + residual (addmm) -> RMSNorm -> gate/up linear with SiLU*mul in
+its epilogue -> down linear + residual (addmm): 7 launches. Inputs and weights are resident in HBM before the timed
+region.
 
 Prints ONE JSON line: tokens/s for the layer (whole job = the one GPU), the roofline of the
 dominant kernel (the bf16 MFMA GEMM) measured with device events on the launch stream inside the
@@ -92,8 +93,11 @@ def layer_plan(pkg, torch, dev, x, p, cfg):
     bf = x.dtype
     new = lambda *shape: torch.empty(*shape, dtype=bf, device=dev)
     h1, qkv, attn, o, x1, h2 = new(T, hidden), new(T, 3 * hidden), new(T, heads, hd), new(T, hidden), new(T, hidden), new(T, hidden)
-    qk_rot = new(T, 2 * heads, hd)  # rotated q heads then rotated k heads of a token, one rotary launch for both
-    qr, kr = qk_rot[:, :heads], qk_rot[:, heads:]
+    # The q and k heads come out of the stacked projection already rotated (rotary embedding in the GEMM epilogue,
+    # adjacent-pair form): the q and k weight rows of every head are permuted at load time from the half-split
+    # convention to the adjacent-pair one, which leaves every q . k, and so the layer's output, unchanged.
+    w_qkv = torch.cat([pkg.ops.interleave_rotary_rows(p["wqkv"][:hidden], hd), pkg.ops.interleave_rotary_rows(p["wqkv"][hidden:2 * hidden], hd),
+                       p["wqkv"][2 * hidden:]], dim=0).contiguous()
     # gate and up come out of one projection (their weights interleaved in one matrix at load time, as the q, k and
     # v weights are stacked): 86 tile columns of 256 fill the 256 CUs to 98 % in the last round where two launches
     # of 43 reach 90 % each, and silu(gate) * up is applied to the accumulators, so gate and up never reach HBM
@@ -105,14 +109,12 @@ def layer_plan(pkg, torch, dev, x, p, cfg):
     lens = torch.full((b,), s, dtype=torch.int32).to(dev)
     x2 = x.reshape(T, hidden)
     q, k, v = qkv.split(hidden, dim=-1)
-    qk4 = qkv[:, :2 * hidden].view(b, s, 2 * heads, hd)  # q and k are neighbours in the fused projection's output
-    v3 = v.reshape(T, heads, hd)
+    qr, kr, v3 = q.view(T, heads, hd), k.view(T, heads, hd), v.view(T, heads, hd)
     one = d.scalar(1)
     P = lambda name, *a: Prepared(pkg, name, *a)
     plan = [
         ("rms_norm", P("diopiRMSNorm", h1, None, x2, d.size([hidden]), p["norm1"], None, float(cfg["eps"]))),
-        ("gemm_qkv", P("diopiLinear", qkv, h1, p["wqkv"], None)),
-        ("rotary_qk", P("diopiRotaryEmbedding", qk_rot.view(b, s, 2 * heads, hd), qk4, cos, sin, False, False)),
+        ("gemm_qkv", P("diopiLinearRotary", qkv, h1, w_qkv, None, cos, sin, 2 * hidden, hd, False, True)),
         ("context_attention", P("diopiContextAttentionInference", attn, qr, kr, v3, starts, lens, int(s))),
         # out projection with the residual folded into the GEMM epilogue: x1 = x + attn @ Wo^T (aten::addmm)
         ("gemm_o", P("diopiAddmm", x1, x2, attn.view(T, hidden), p["wo"].t(), one, one)),
@@ -120,7 +122,7 @@ def layer_plan(pkg, torch, dev, x, p, cfg):
         ("gemm_gate_up_silu", P("diopiLinearSiluMul", act, h2, w_gate_up)),
         ("gemm_down", P("diopiAddmm", out, x1, act, p["wdown"].t(), one, one)),
     ]
-    keep = [h1, qkv, attn, o, x1, h2, qk_rot, qr, kr, w_gate_up, act, down, out, cos, sin, starts, lens, x2]
+    keep = [h1, qkv, attn, o, x1, h2, w_qkv, qr, kr, v3, w_gate_up, act, down, out, cos, sin, starts, lens, x2]
     flops = {"gemm_qkv": 2 * T * 3 * hidden * hidden, "gemm_o": 2 * T * hidden * hidden,
              "gemm_gate_up_silu": 2 * T * 2 * ffn * hidden, "gemm_down": 2 * T * hidden * ffn}
     return plan, keep, flops, out
@@ -385,7 +387,7 @@ def main():
     gemm_flops = sum(flops.values())
     achieved_tf = gemm_flops / (gemm_time_us * 1e-6) / 1e12
     breakdown = {l: round(sum(v) / args.steps, 1) for l, v in per_op.items()}      # us per step (labels used twice are summed)
-    roofline = {"bound": "mfma", "kernel": "gemmMfmaPipelinedKernel<bf16> 256x256x64 (4 launches per step: qkv, o + residual, gate+up with silu*mul, down + residual)",
+    roofline = {"bound": "mfma", "kernel": "gemmMfmaPipelinedKernel<bf16> 256x256x64 (4 launches per step: qkv with rotary, o + residual, gate+up with silu*mul, down + residual)",
                 "achieved": round(achieved_tf, 1), "peak": MFMA_BF16_PEAK_TF, "unit": "TFLOP/s",
                 "frac": round(achieved_tf / MFMA_BF16_PEAK_TF, 4), "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH,
                 "flops_per_step": gemm_flops, "avg_launch_us": round(gemm_time_us / len(gemm_labels), 1),

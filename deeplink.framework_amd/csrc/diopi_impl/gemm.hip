@@ -76,6 +76,13 @@ struct MfmaArgs {
   bool vecEpilogue;  // out / addend / bias allow 16-byte row segments
   float* partial = nullptr;  // split-K: fp32 partial products [gridDim.y][M][N]
   int kTilesPerSplit = 0;
+  // rotary epilogue: adjacent column pairs (2i, 2i + 1) of every head of rotHeadDim columns below rotCols are
+  // rotated by the angle whose cosine / sine sit at table[(row % rotTableRows) * rotHeadDim / 2 + i]
+  const void* rotCos = nullptr;
+  const void* rotSin = nullptr;
+  int rotCols = 0, rotHeadDim = 0, rotTableRows = 1;
+  bool rotTableF32 = false;
+  float rotSinSign = 1.f;
 };
 
 constexpr int kBK = 64;  // K elements per LDS tile (128-byte rows)
@@ -306,8 +313,9 @@ __device__ __forceinline__ void loadToLds16(u32x4 rsrc, int voffset, int soffset
 // output columns as 32 gate columns followed by the 32 up columns of the same channels and stores
 // silu(gate) * up, half as wide (out has N / 2 columns); kEpiPartial is the split-K form: workgroup (tile, s)
 // multiplies K tiles [s * kTilesPerSplit, ...) and stores its fp32 accumulators to partial[s], to be summed and
-// given the linear epilogue by splitKReduceKernel.
-enum PipeEpilogue { kEpiLinear = 0, kEpiSiluMul = 1, kEpiPartial = 2 };
+// given the linear epilogue by splitKReduceKernel; kEpiRotary is acc + bias followed by the interleaved rotary
+// embedding on the leading rotCols columns (the q and k heads of a stacked QKV projection).
+enum PipeEpilogue { kEpiLinear = 0, kEpiSiluMul = 1, kEpiPartial = 2, kEpiRotary = 3 };
 
 template <typename T, int EPI>
 __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs g) {
@@ -564,6 +572,71 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
 #pragma unroll
         for (int e = 0; e < 4; ++e) o[e] = static_cast<T>(x0[e]), o[4 + e] = static_cast<T>(x1[e]);
         put(i, 0, o);
+      }
+    } else if constexpr (EPI == kEpiRotary) {
+      // A lane's 8 consecutive columns are 4 adjacent pairs of one head; their angles are 4 consecutive table
+      // entries of the lane's row. Pieces at or past rotCols (the v heads) pass through with cos = 1, sin = 0.
+      // The table entries of fragment row i + 1 are requested before the stores of row i (one in-order counter).
+      float bv[TN / 2][8];
+      int pair0[TN / 2];
+      bool rot[TN / 2];
+#pragma unroll
+      for (int jp = 0; jp < TN / 2; ++jp) {
+        const int col = min(col0 + jp * 32, g.N - 8);
+        Frag b8;
+        if (bias) b8 = *reinterpret_cast<const Frag*>(bias + col);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) bv[jp][e] = bias ? static_cast<float>(b8[e]) : 0.f;
+        rot[jp] = col < g.rotCols;
+        pair0[jp] = (col % g.rotHeadDim) >> 1;
+      }
+      const int half = g.rotHeadDim >> 1;
+      const int tsz = g.rotTableF32 ? 4 : (int)sizeof(T);
+      const __amdgpu_buffer_rsrc_t rsCos = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<void*>(g.rotCos), 0, (int)((int64_t)g.rotTableRows * half * tsz), 0x00020000);
+      const __amdgpu_buffer_rsrc_t rsSin = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<void*>(g.rotSin), 0, (int)((int64_t)g.rotTableRows * half * tsz), 0x00020000);
+      float cs[2][TN / 2][4], sn[2][TN / 2][4];
+      auto fetch = [&](int i) {
+        const int row = tm * BM + wm * WM + i * 16 + frow;
+#pragma unroll
+        for (int jp = 0; jp < TN / 2; ++jp) {
+          const int off = row < g.M ? ((row % g.rotTableRows) * half + pair0[jp]) * tsz : kOutside;
+          if (g.rotTableF32) {
+            const u32x4 c4 = __builtin_amdgcn_raw_buffer_load_b128(rsCos, off, 0, 0);
+            const u32x4 s4 = __builtin_amdgcn_raw_buffer_load_b128(rsSin, off, 0, 0);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) cs[i & 1][jp][e] = __uint_as_float(c4[e]), sn[i & 1][jp][e] = __uint_as_float(s4[e]);
+          } else {
+            typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+            typedef T T4 __attribute__((ext_vector_type(4)));
+            const T4 c4 = __builtin_bit_cast(T4, __builtin_amdgcn_raw_buffer_load_b64(rsCos, off, 0, 0));
+            const T4 s4 = __builtin_bit_cast(T4, __builtin_amdgcn_raw_buffer_load_b64(rsSin, off, 0, 0));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) cs[i & 1][jp][e] = static_cast<float>(c4[e]), sn[i & 1][jp][e] = static_cast<float>(s4[e]);
+          }
+        }
+      };
+      fetch(0);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        if (i + 1 < TM) fetch(i + 1);
+#pragma unroll
+        for (int jp = 0; jp < TN / 2; ++jp) {
+          f32x4 x0 = acc[i][2 * jp], x1 = acc[i][2 * jp + 1];
+          swapPair(x0, x1);
+          const float v[8] = {x0[0] + bv[jp][0], x0[1] + bv[jp][1], x0[2] + bv[jp][2], x0[3] + bv[jp][3],
+                              x1[0] + bv[jp][4], x1[1] + bv[jp][5], x1[2] + bv[jp][6], x1[3] + bv[jp][7]};
+          Frag o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float c = rot[jp] ? cs[i & 1][jp][e] : 1.f;
+            const float sv = rot[jp] ? sn[i & 1][jp][e] * g.rotSinSign : 0.f;
+            o[2 * e] = static_cast<T>(v[2 * e] * c - v[2 * e + 1] * sv);
+            o[2 * e + 1] = static_cast<T>(v[2 * e] * sv + v[2 * e + 1] * c);
+          }
+          put(i, jp, o);
+        }
       }
     } else {
       float bv[TN / 2][8];
@@ -948,9 +1021,17 @@ static int splitKWays(int64_t tiles, int64_t kTiles, int* perSplit) {
   return (int)ceilDiv(kTiles, per);
 }
 
+struct RotaryEpilogue {
+  const void* cosT;
+  const void* sinT;
+  int cols, headDim, tableRows;
+  bool tableF32;
+  float sinSign;
+};
+
 template <typename T, int EPI = kEpiLinear>
 static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p, float* partial = nullptr, int splits = 1,
-                                        int kTilesPerSplit = 0) {
+                                        int kTilesPerSplit = 0, const RotaryEpilogue* rot = nullptr) {
   MfmaArgs g;
   g.A = p.A, g.B = p.B, g.out = p.out, g.Cin = p.Cin, g.bias = p.bias;
   g.sAb = p.sAb, g.lda = p.sAm, g.sBb = p.sBb, g.ldb = p.sBn, g.sOb = p.sOb, g.ldo = p.sOm;
@@ -968,6 +1049,11 @@ static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p
   AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmMfmaPipelinedKernel<T, EPI>), (int)lds));
   g.partial = partial;
   g.kTilesPerSplit = kTilesPerSplit;
+  if (EPI == kEpiRotary) {
+    AMD_CHECK(rot && g.vecEpilogue && !p.Cin && p.alpha == 1.f, "rotary epilogue: needs tables, the vector epilogue and no addend");
+    g.rotCos = rot->cosT, g.rotSin = rot->sinT, g.rotCols = rot->cols, g.rotHeadDim = rot->headDim, g.rotTableRows = rot->tableRows;
+    g.rotTableF32 = rot->tableF32, g.rotSinSign = rot->sinSign;
+  }
   dim3 grid((unsigned)(g.tilesM * g.tilesN), (unsigned)splits, (unsigned)p.batch);
   if (EPI == kEpiSiluMul) AMD_CHECK(g.vecEpilogue, "gated linear: output rows must allow 16-byte stores");
   if (EPI == kEpiPartial) AMD_CHECK(g.vecEpilogue && p.batch == 1 && partial, "split-K: needs the vector epilogue and one batch");
@@ -1483,6 +1569,91 @@ GEMM_EXPORT diopiError_t diopiLinearSiluMul(diopiContextHandle_t ctx, diopiTenso
   p.B = cw.data, p.sBn = k, p.sBk = 1;
   p.out = cout.data, p.sOm = f;
   AMD_TRY(runGatedSiluGemm(ctx, stream, p));
+  if (outTemp) AMD_TRY(stridedCopy(stream, cout, out));
+  return diopiSuccess;
+}
+
+// out[..., N] = input W^T + bias, then the rotary embedding on the first rotary_cols columns viewed as heads of
+// head_dim columns, with one table row per row of the flattened input (cos / sin of shape [rows, head_dim / 2]):
+// the q and k heads of a stacked QKV projection come out rotated and v passes through. The reference model
+// runs the projections and the rotation as separate steps (dicp/test/model/llama/model.py:108-160 with the
+// interleaved rotation of :58-69; the half-split form is dicp/dicp/vendor/AscendGraph/ext_ops.py:24-33).
+// One launch of the large-tile kernel for the interleaved form when the problem qualifies (the pairs of a head
+// are then adjacent columns, which one lane holds), else the projection followed by the rotary kernel.
+GEMM_EXPORT diopiError_t diopiLinearRotary(diopiContextHandle_t ctx, diopiTensorHandle_t outH, diopiConstTensorHandle_t inH,
+                                           diopiConstTensorHandle_t wH, diopiConstTensorHandle_t biasH,
+                                           diopiConstTensorHandle_t cosH, diopiConstTensorHandle_t sinH,
+                                           int64_t rotaryCols, int64_t headDim, bool conj, bool interleaved) {
+  hipStream_t stream;
+  AMD_TRY(getStream(ctx, &stream));
+  TensorView out, in, w, bias, c, s;
+  AMD_TRY(getView(outH, &out, "out"));
+  AMD_TRY(getView(inH, &in, "input"));
+  AMD_TRY(getView(wH, &w, "weight"));
+  AMD_TRY(getView(biasH, &bias, "bias"));
+  AMD_TRY(getView(cosH, &c, "cos"));
+  AMD_TRY(getView(sinH, &s, "sin"));
+  AMD_CHECK(out.defined() && in.defined() && w.defined() && c.defined() && s.defined(), "diopiLinearRotary: null tensor");
+  AMD_CHECK(w.ndim == 2 && in.ndim >= 1 && out.ndim == in.ndim, "diopiLinearRotary: weight must be [N, K], out shaped like input");
+  AMD_CHECK(in.dtype == out.dtype && w.dtype == out.dtype, "diopiLinearRotary: input, weight and out must share a dtype");
+  const int64_t k = in.shape[in.ndim - 1], n = out.shape[out.ndim - 1];
+  AMD_CHECK(w.shape[1] == k && w.shape[0] == n, "diopiLinearRotary: weight is [%ld, %ld], expected [%ld, %ld]", (long)w.shape[0],
+            (long)w.shape[1], (long)n, (long)k);
+  AMD_CHECK(headDim > 0 && headDim % 2 == 0 && rotaryCols >= 0 && rotaryCols <= n && rotaryCols % headDim == 0,
+            "diopiLinearRotary: rotary_cols %ld must be a multiple of the even head_dim %ld and at most %ld", (long)rotaryCols,
+            (long)headDim, (long)n);
+  for (int d = 0; d + 1 < in.ndim; ++d) AMD_CHECK(in.shape[d] == out.shape[d], "diopiLinearRotary: leading extent mismatch at dim %d", d);
+  if (out.numel == 0) return diopiSuccess;
+  const int64_t rows = in.numel / k, half = headDim / 2;
+  const int64_t tableRows = c.numel / half;
+  AMD_CHECK(c.dtype == s.dtype && c.numel == s.numel && tableRows > 0 && c.numel == tableRows * half && rows % tableRows == 0,
+            "diopiLinearRotary: cos and sin must both hold [t, %ld] values with t dividing the %ld rows", (long)half, (long)rows);
+  TensorView cin, cw, cb, cc, cs;
+  AMD_TRY(makeContiguous(ctx, stream, in, &cin));
+  AMD_TRY(makeContiguous(ctx, stream, w, &cw));
+  AMD_TRY(makeContiguous(ctx, stream, c, &cc));
+  AMD_TRY(makeContiguous(ctx, stream, s, &cs));
+  if (bias.defined()) {
+    AMD_CHECK(bias.numel == n && bias.dtype == out.dtype, "diopiLinearRotary: bias must hold N elements of the output dtype");
+    AMD_TRY(makeContiguous(ctx, stream, bias, &cb));
+  }
+  TensorView cout = out;
+  const bool outTemp = !out.isContiguous();
+  if (outTemp) {
+    diopiTensorHandle_t th;
+    AMD_TRY(requireTensor(ctx, out.shape, out.ndim, out.dtype, &th, &cout));
+  }
+  GemmProblem p;
+  p.dtype = out.dtype;
+  p.M = rows, p.N = n, p.K = k;
+  p.A = cin.data, p.sAm = k, p.sAk = 1;
+  p.B = cw.data, p.sBn = k, p.sBk = 1;
+  p.out = cout.data, p.sOm = n;
+  if (bias.defined()) p.bias = cb.data;
+  const bool halfT = p.dtype == diopi_dtype_bfloat16 || p.dtype == diopi_dtype_float16;
+  const bool tableOk = (cc.dtype == out.dtype || cc.dtype == diopi_dtype_float32) && ptr16(cc.data) && ptr16(cs.data) && half % 4 == 0 &&
+                       tableRows * half * 4 < (int64_t(1) << 31);
+  const bool direct = interleaved && rotaryCols > 0 && halfT && headDim % 8 == 0 && tableOk && mult8(k) && ptr16(p.A) && ptr16(p.B) &&
+                      ceilDiv(p.M, 256) * ceilDiv(p.N, 256) >= 144 && k % kBK == 0 && k >= 2 * kBK && n % 8 == 0 && ptr16(p.out) &&
+                      (!p.bias || ptr16(p.bias)) && p.M * k * 2 < (int64_t(1) << 31) && n * k * 2 < (int64_t(1) << 31) &&
+                      p.M * n * 2 < (int64_t(1) << 31);
+  if (direct) {
+    RotaryEpilogue r;
+    r.cosT = cc.data, r.sinT = cs.data, r.cols = (int)rotaryCols, r.headDim = (int)headDim, r.tableRows = (int)tableRows;
+    r.tableF32 = cc.dtype == diopi_dtype_float32, r.sinSign = conj ? -1.f : 1.f;
+    AMD_TRY(p.dtype == diopi_dtype_bfloat16 ? (launchMfmaPipelined<bf16_t, kEpiRotary>(stream, p, nullptr, 1, 0, &r))
+                                            : (launchMfmaPipelined<half_t, kEpiRotary>(stream, p, nullptr, 1, 0, &r)));
+  } else {
+    AMD_TRY(runGemm(ctx, stream, p));
+    if (rotaryCols > 0) {
+      TensorView v;
+      v.data = cout.data, v.ndim = 3, v.dtype = out.dtype, v.itemsize = out.itemsize;
+      v.shape[0] = rows, v.shape[1] = rotaryCols / headDim, v.shape[2] = headDim;
+      v.stride[0] = n, v.stride[1] = headDim, v.stride[2] = 1;
+      v.numel = rows * rotaryCols;
+      AMD_TRY(runRotary(ctx, stream, v, v, cc, cs, conj, interleaved));
+    }
+  }
   if (outTemp) AMD_TRY(stridedCopy(stream, cout, out));
   return diopiSuccess;
 }

@@ -27,4 +27,8 @@ struct GemmProblem {
 
 diopiError_t runGemm(diopiContextHandle_t ctx, hipStream_t stream, GemmProblem p);
 
+// diopiRotaryEmbedding on views (rotary_kv.hip): out and x of shape [..., heads, head_dim], strided views allowed.
+diopiError_t runRotary(diopiContextHandle_t ctx, hipStream_t stream, const TensorView& out, const TensorView& x,
+                       const TensorView& cosT, const TensorView& sinT, bool conj, bool interleaved);
+
 }  // namespace amd

@@ -10,7 +10,7 @@
 //
 // DestIndexCopyKV: out[dest_loc[i], :, :] = k[i, :, :], a pure byte move done with the
 // widest vector the row size and pointers allow; one workgroup per token row.
-#include "common.hpp"
+#include "gemm.hpp"
 
 namespace amd {
 
@@ -222,6 +222,12 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiRotaryEmbedd
   AMD_TRY(getView(xH, &x, "x"));
   AMD_TRY(getView(cosH, &c, "cos"));
   AMD_TRY(getView(sinH, &s, "sin"));
+  return amd::runRotary(ctx, stream, out, x, c, s, conj, interleaved);
+}
+
+// The body of diopiRotaryEmbedding on views (also the second pass of diopiLinearRotary's two-pass form).
+diopiError_t amd::runRotary(diopiContextHandle_t ctx, hipStream_t stream, const TensorView& out, const TensorView& x,
+                            const TensorView& c, const TensorView& s, bool conj, bool interleaved) {
   AMD_CHECK(out.defined() && x.defined() && c.defined() && s.defined(), "diopiRotaryEmbedding: null tensor");
   AMD_CHECK(x.ndim >= 2, "diopiRotaryEmbedding: x must be [..., heads, head_dim]");
   AMD_CHECK(out.dtype == x.dtype && out.ndim == x.ndim, "diopiRotaryEmbedding: out must match x");

@@ -239,6 +239,7 @@ SIGNATURES = {
     "diopiWeightOnlyInt8Linear": [_T, _T, _T, _T, _T],
     "diopiSiluMul": [_T, _T, _T],
     "diopiLinearSiluMul": [_T, _T, _T],
+    "diopiLinearRotary": [_T, _T, _T, _T, _T, _T, c_int64, c_int64, c_bool, c_bool],
 }
 
 _bound = {}

@@ -232,6 +232,30 @@ def linear_silu_mul(input, weight_gate_up, *, out=None):
     return out
 
 
+def interleave_rotary_rows(w, head_dim):
+    """Rows of a q or k projection weight [heads * head_dim, K] reordered inside every head from the half-split
+    rotary convention to the interleaved one: row 2 i <- row i, row 2 i + 1 <- row i + head_dim / 2. q . k does
+    not change when both are permuted this way, so attention is unaffected (a load-time permutation)."""
+    n, k = w.shape
+    assert n % head_dim == 0 and head_dim % 2 == 0
+    return w.reshape(n // head_dim, 2, head_dim // 2, k).transpose(1, 2).reshape(n, k).contiguous()
+
+
+def linear_rotary(input, weight, cos, sin, rotary_cols, head_dim, bias=None, *, conj=False, interleaved=True, out=None):
+    """input @ weight^T (+ bias) with the rotary embedding applied to the first rotary_cols output columns
+    (backend extension; see functions_ext.h). cos / sin: [rows, head_dim / 2]."""
+    if out is None:
+        out = torch.empty(*input.shape[:-1], weight.shape[0], dtype=input.dtype, device=input.device)
+    ho, po = handle(out)
+    hi, pi = handle(input)
+    hw, pw = handle(weight)
+    hb, pb = handle(bias)
+    hc, pc = handle(cos)
+    hs, ps = handle(sin)
+    _call("diopiLinearRotary", po, pi, pw, pb, pc, ps, int(rotary_cols), int(head_dim), bool(conj), bool(interleaved))
+    return out
+
+
 # ------------------------------------------------------------------ reductions
 def softmax(self, dim, *, out=None):
     """aten::_softmax.out -> diopiSoftmax (diopi_functions.yaml:1290-1292)."""

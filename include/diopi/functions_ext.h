@@ -106,4 +106,19 @@ DIOPI_API diopiError_t diopiSiluMul(diopiContextHandle_t ctx, diopiTensorHandle_
 DIOPI_API diopiError_t diopiLinearSiluMul(diopiContextHandle_t ctx, diopiTensorHandle_t out,
                                           diopiConstTensorHandle_t input, diopiConstTensorHandle_t weight);
 
+/* out[..., N] = input @ weight^T + bias, followed by diopiRotaryEmbedding on the first rotary_cols columns of out
+ * viewed as heads of head_dim columns: the q and k heads of a stacked [q; k; v] projection come out rotated, v passes
+ * through, and the rotary pass over q and k (read + write) disappears. cos / sin are [t, head_dim / 2] with t
+ * dividing the rows of the flattened input (row r uses table row r % t, as diopiRotaryEmbedding does); conj and interleaved as in diopiRotaryEmbedding. With interleaved == true
+ * (adjacent pairs, dicp/test/model/llama/model.py:58-69) and a large problem this is one GEMM launch; otherwise the
+ * projection and the rotation run as two passes with the same result. A checkpoint in the half-split convention
+ * (dicp/dicp/vendor/AscendGraph/ext_ops.py:24-33) can use the single-launch form after a load-time permutation of
+ * the q and k weight rows of every head (row 2 i <- row i, row 2 i + 1 <- row i + head_dim / 2): q . k is
+ * invariant under a permutation of the head dim applied to both. bias may be null. The reference model runs the
+ * projections and the rotation as separate steps (model.py:108-160). */
+DIOPI_API diopiError_t diopiLinearRotary(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiConstTensorHandle_t input,
+                                         diopiConstTensorHandle_t weight, diopiConstTensorHandle_t bias,
+                                         diopiConstTensorHandle_t cos, diopiConstTensorHandle_t sin, int64_t rotary_cols,
+                                         int64_t head_dim, bool conj, bool interleaved);
+
 #endif /* DIOPI_FUNCTIONS_EXT_H_ */

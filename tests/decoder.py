@@ -3,22 +3,34 @@ Mirrors oracle.cpu_fallback.decoder_block step for step so every intermediate ca
 import torch
 
 
-def run_decoder_block(ops, x, p, cfg, fused_ffn=False, stacked_gate_up=False):
+def run_decoder_block(ops, x, p, cfg, fused_ffn=False, stacked_gate_up=False, fused_rotary=False):
     heads, eps, theta = cfg["heads"], cfg["eps"], cfg["theta"]
     b, s, hidden = x.shape
     d = hidden // heads
     inter = {}
     h1 = ops.rms_norm(x, p["norm1"], eps)
     inter["norm1"] = h1
-    qkv = ops.linear(h1, p["wqkv"])
-    inter["qkv"] = qkv
-    q, k, v = qkv.split(hidden, dim=-1)  # strided views: the rotary kernel sees non-contiguous input
     inv = 1.0 / (theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
     ang = torch.outer(torch.arange(s, dtype=torch.float32), inv)
     cos, sin = torch.cos(ang).to(x.dtype).to(x.device), torch.sin(ang).to(x.dtype).to(x.device)
-    q = ops.rotary_emb(q.reshape(b, s, heads, d), cos, sin)
-    k = ops.rotary_emb(k.reshape(b, s, heads, d), cos, sin)
-    inter["q_rot"], inter["k_rot"] = q, k
+    if fused_rotary:
+        # q and k leave the stacked projection rotated (adjacent-pair form on weight rows permuted at load time);
+        # their head dims are then a fixed permutation of the half-split results, which attention does not see
+        w = torch.cat([ops.interleave_rotary_rows(p["wqkv"][:hidden], d), ops.interleave_rotary_rows(p["wqkv"][hidden:2 * hidden], d),
+                       p["wqkv"][2 * hidden:]], dim=0)
+        qkv = ops.linear_rotary(h1, w, cos, sin, 2 * hidden, d, interleaved=True)
+        q, k, v = qkv.split(hidden, dim=-1)
+        q, k = q.reshape(b, s, heads, d), k.reshape(b, s, heads, d)
+        unperm = lambda t: t.reshape(b, s, heads, d // 2, 2).transpose(3, 4).reshape(b, s, heads, d)
+        inter["qkv"] = torch.cat([unperm(q).reshape(b, s, hidden), unperm(k).reshape(b, s, hidden), v], dim=-1)  # rotated q, k
+        inter["q_rot"], inter["k_rot"] = unperm(q), unperm(k)
+    else:
+        qkv = ops.linear(h1, p["wqkv"])
+        inter["qkv"] = qkv
+        q, k, v = qkv.split(hidden, dim=-1)  # strided views: the rotary kernel sees non-contiguous input
+        q = ops.rotary_emb(q.reshape(b, s, heads, d), cos, sin)
+        k = ops.rotary_emb(k.reshape(b, s, heads, d), cos, sin)
+        inter["q_rot"], inter["k_rot"] = q, k
     starts = (torch.arange(b, dtype=torch.int32) * s).to(x.device)
     lens = torch.full((b,), s, dtype=torch.int32).to(x.device)
     vv = v.reshape(b * s, heads, d).contiguous()

@@ -191,6 +191,55 @@ def test_linear_silu_mul(ops, dev, dtype, m, f, k):
 
 
 # ------------------------------------------------------------------ prefill attention
+@pytest.mark.parametrize("dtype,table_dtype", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float32)])
+@pytest.mark.parametrize("m,heads,hd,vcols,k,interleaved,conj,bias", [
+    (2304, 16, 128, 2048, 256, True, False, False),   # 9 x 16 tiles: one launch; q and k rotated, v through
+    (2400, 57, 64, 0, 192, True, True, True),         # ragged rows and columns, all columns rotated, negative angle, bias
+    (2304, 16, 128, 2048, 256, False, False, False),  # half-split pairs: projection + rotary kernel
+    (40, 4, 64, 128, 128, True, False, True),         # small: projection + rotary kernel
+])
+def test_linear_rotary(ops, dev, dtype, table_dtype, m, heads, hd, vcols, k, interleaved, conj, bias):
+    """The stacked projection with the rotary embedding in its epilogue against the oracle's projection followed by
+    the oracle's rotation (half-split: ext_ops.py:24-33; interleaved: model.py:58-69), and against this backend's
+    own two separate ops."""
+    rot = heads * hd
+    n = rot + vcols
+    x = torch.randn(m, k, generator=g(70)).to(dtype)
+    w = (torch.randn(n, k, generator=g(71)) * 0.05).to(dtype)
+    b = torch.randn(n, generator=g(72)).to(dtype) if bias else None
+    cos, sin = oracle.precompute_freqs(hd, m)
+    cos_t, sin_t = cos.to(table_dtype), sin.to(table_dtype)
+    y = x.float() @ w.float().t() + (b.float() if bias else 0)
+    sgn = -1.0 if conj else 1.0
+    yr = y[:, :rot].reshape(m, heads, hd)
+    want_rot = (oracle.rotary_emb_interleaved if interleaved else oracle.rotary_emb)(yr, cos_t.float(), sgn * sin_t.float())
+    want = torch.cat([want_rot.reshape(m, rot), y[:, rot:]], dim=1)
+    db = b.to(dev) if bias else None
+    got = ops.linear_rotary(x.to(dev), w.to(dev), cos_t.to(dev), sin_t.to(dev), rot, hd, db, conj=conj, interleaved=interleaved)
+    assert_half(got, want, rel=2e-2, abs_=2e-2)
+    # this backend's separate ops (one rounding more between them)
+    sep = ops.linear(x.to(dev), w.to(dev), db)
+    q = sep[:, :rot].view(m, heads, hd)
+    ops.rotary_emb(q, cos_t.to(dev), sin_t.to(dev), conj=conj, interleaved=interleaved, out=q)
+    assert_half(got, sep.float().cpu(), rel=2e-2, abs_=3e-2)
+
+
+def test_rotary_row_permutation_keeps_attention_scores(ops, dev):
+    """A half-split checkpoint through the interleaved single-launch form: with the q / k weight rows of every head
+    permuted (row 2i <- row i, row 2i + 1 <- row i + d / 2) the rotated q and k are the same permutation of the
+    half-split results, so every q . k is unchanged."""
+    m, heads, hd, k = 2304, 16, 128, 256
+    x = torch.randn(m, k, generator=g(73)).bfloat16().to(dev)
+    w = (torch.randn(2 * heads * hd, k, generator=g(74)) * 0.05).bfloat16()
+    cos, sin = oracle.precompute_freqs(hd, m)
+    cos, sin = cos.bfloat16().to(dev), sin.bfloat16().to(dev)
+    half_split = ops.linear_rotary(x, w.to(dev), cos, sin, 2 * heads * hd, hd, interleaved=False)
+    wp = ops.interleave_rotary_rows(w, hd).to(dev)
+    inter = ops.linear_rotary(x, wp, cos, sin, 2 * heads * hd, hd, interleaved=True)
+    perm = inter.view(m, 2 * heads, hd // 2, 2).transpose(2, 3).reshape(m, 2 * heads * hd)  # back to half-split order
+    assert_half(perm, half_split.float().cpu(), rel=2e-2, abs_=3e-2)
+
+
 @pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 128), (torch.float16, 128), (torch.bfloat16, 64),
                                      (torch.float32, 64), (torch.float32, 40)])
 def test_context_attention(ops, dev, dtype, d):
@@ -360,6 +409,10 @@ def test_tiny_decoder_block_fp32_every_intermediate(ops, dev, pkg):
     got4, gi4 = run_decoder_block(ops, x.to(dev), {k: v.to(dev) for k, v in p.items()}, cfg, stacked_gate_up="interleaved")
     assert_fp32(gi4["act"].cpu().reshape(wi["act"].shape), wi["act"], rel=1e-5)
     assert_fp32(got4, want)
+    # rotary inside the stacked projection, on q / k weight rows permuted to the adjacent-pair convention
+    got5, gi5 = run_decoder_block(ops, x.to(dev), {k: v.to(dev) for k, v in p.items()}, cfg, fused_rotary=True)
+    assert_fp32(gi5["attn"].cpu().reshape(wi["attn"].shape), wi["attn"], rel=2e-5)
+    assert_fp32(got5, want, rel=2e-5)
 
 
 def test_small_decoder_block_bf16(ops, dev, pkg):
@@ -372,6 +425,20 @@ def test_small_decoder_block_bf16(ops, dev, pkg):
     assert_half(got, want, rel=3e-2, abs_=3e-2)
     got, _ = run_decoder_block(ops, x.to(dev), {k: v.to(dev) for k, v in p.items()}, cfg, stacked_gate_up="interleaved")
     assert_half(got, want, rel=3e-2, abs_=3e-2)
+    got, _ = run_decoder_block(ops, x.to(dev), {k: v.to(dev) for k, v in p.items()}, cfg, stacked_gate_up="interleaved", fused_rotary=True)
+    assert_half(got, want, rel=3e-2, abs_=3e-2)
+
+
+def test_decoder_block_bf16_with_both_fused_projections_in_one_launch_each(ops, dev, pkg):
+    """The benchmark's configuration of the layer at a size where both fused projections take their single-launch
+    form (2304 tokens, hidden 2048: 216 and 198 tiles of 256 x 256): rotary in the QKV epilogue on permuted weight
+    rows, silu * mul in the gate / up epilogue, residuals through addmm-free adds."""
+    x, p, cfg = pkg.workloads.llama7b_layer(seed=3, batch=3, seq=768, hidden=2048, heads=16, ffn=2816)
+    want, _ = oracle.decoder_block(x.float(), {k: v.float() for k, v in p.items()}, cfg["heads"], cfg["eps"], cfg["theta"])
+    got, _ = run_decoder_block(ops, x.to(dev), {k: v.to(dev) for k, v in p.items()}, cfg, stacked_gate_up="interleaved", fused_rotary=True)
+    assert_half(got, want, rel=3e-2, abs_=3e-2)
+    ref, _ = run_decoder_block(ops, x.to(dev), {k: v.to(dev) for k, v in p.items()}, cfg, fused_ffn=True)
+    assert_half(got, ref.float().cpu(), rel=3e-2, abs_=3e-2)
 
 
 def test_decoder_block_from_primitive_ops_only(ops, dev, pkg):
