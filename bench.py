@@ -29,10 +29,10 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TF = 2500.0   # MI355X dense bf16, published
 # Bytes that leave L2 per GEMM launch (call-weighted mean of the layer's 4 GEMM launches), from two
 # rocprofv3 --pmc runs of `bench.py --only-layer` (FETCH_SIZE, then WRITE_SIZE), scaled by what the same
-# counters read for a 64 MiB device copy: (2 x 613 829 + 125 953) KiB. The summary is
+# counters read for a 64 MiB device copy: (2 x 617 006 + 125 999) KiB. The summary is
 # profiles/decoder_layer_hbm_traffic_counters.md;
 # a counter cannot be read from inside this process, so the figure is carried here as measured.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 1_386_000_000
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 1_393_000_000
 
 
 def parse():
