@@ -531,8 +531,9 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
     // a piece outside the matrix gets an offset past the end, which the hardware drops (stores) or
     // answers with zeros (loads), so the instruction stream has no branches and the compiler can count
     // outstanding accesses exactly. Loads and stores share one in-order counter: a wait for an addend
-    // piece also waits for every store before it, so the pieces of fragment row i + 1 are requested
-    // before the stores of row i, and without an addend there is no load (and no wait) in the stream.
+    // piece also waits for every store before it, so the pieces of four fragment rows are requested
+    // together before the first store of the four (one exposed round trip per four rows instead of one per
+    // row), and without an addend there is no load (and no wait) in the stream.
     const int cperm = (kq & 1) * 16 + (kq >> 1) * 8;
     auto swapPair = [](f32x4& x0, f32x4& x1) {
 #pragma unroll
@@ -576,7 +577,6 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
     } else if constexpr (EPI == kEpiRotary) {
       // A lane's 8 consecutive columns are 4 adjacent pairs of one head; their angles are 4 consecutive table
       // entries of the lane's row. Pieces at or past rotCols (the v heads) pass through with cos = 1, sin = 0.
-      // The table entries of fragment row i + 1 are requested before the stores of row i (one in-order counter).
       float bv[TN / 2][8];
       int pair0[TN / 2];
       bool rot[TN / 2];
@@ -596,7 +596,9 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
           const_cast<void*>(g.rotCos), 0, (int)((int64_t)g.rotTableRows * half * tsz), 0x00020000);
       const __amdgpu_buffer_rsrc_t rsSin = __builtin_amdgcn_make_buffer_rsrc(
           const_cast<void*>(g.rotSin), 0, (int)((int64_t)g.rotTableRows * half * tsz), 0x00020000);
-      float cs[2][TN / 2][4], sn[2][TN / 2][4];
+      // Table entries are requested four fragment rows at a time,
+      // before any store of the batch: a request one row ahead would expose the L2 round trip once per row.
+      float cs[TM][TN / 2][4], sn[TM][TN / 2][4];
       auto fetch = [&](int i) {
         const int row = tm * BM + wm * WM + i * 16 + frow;
 #pragma unroll
@@ -606,21 +608,23 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
             const u32x4 c4 = __builtin_amdgcn_raw_buffer_load_b128(rsCos, off, 0, 0);
             const u32x4 s4 = __builtin_amdgcn_raw_buffer_load_b128(rsSin, off, 0, 0);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) cs[i & 1][jp][e] = __uint_as_float(c4[e]), sn[i & 1][jp][e] = __uint_as_float(s4[e]);
+            for (int e = 0; e < 4; ++e) cs[i][jp][e] = __uint_as_float(c4[e]), sn[i][jp][e] = __uint_as_float(s4[e]);
           } else {
             typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
             typedef T T4 __attribute__((ext_vector_type(4)));
             const T4 c4 = __builtin_bit_cast(T4, __builtin_amdgcn_raw_buffer_load_b64(rsCos, off, 0, 0));
             const T4 s4 = __builtin_bit_cast(T4, __builtin_amdgcn_raw_buffer_load_b64(rsSin, off, 0, 0));
 #pragma unroll
-            for (int e = 0; e < 4; ++e) cs[i & 1][jp][e] = static_cast<float>(c4[e]), sn[i & 1][jp][e] = static_cast<float>(s4[e]);
+            for (int e = 0; e < 4; ++e) cs[i][jp][e] = static_cast<float>(c4[e]), sn[i][jp][e] = static_cast<float>(s4[e]);
           }
         }
       };
-      fetch(0);
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
-        if (i + 1 < TM) fetch(i + 1);
+        if (i % 4 == 0) {
+#pragma unroll
+          for (int ii = i; ii < i + 4; ++ii) fetch(ii);
+        }
 #pragma unroll
         for (int jp = 0; jp < TN / 2; ++jp) {
           f32x4 x0 = acc[i][2 * jp], x1 = acc[i][2 * jp + 1];
@@ -630,8 +634,8 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
           Frag o;
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const float c = rot[jp] ? cs[i & 1][jp][e] : 1.f;
-            const float sv = rot[jp] ? sn[i & 1][jp][e] * g.rotSinSign : 0.f;
+            const float c = rot[jp] ? cs[i][jp][e] : 1.f;
+            const float sv = rot[jp] ? sn[i][jp][e] * g.rotSinSign : 0.f;
             o[2 * e] = static_cast<T>(v[2 * e] * c - v[2 * e + 1] * sv);
             o[2 * e + 1] = static_cast<T>(v[2 * e] * sv + v[2 * e + 1] * c);
           }
@@ -652,24 +656,26 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
         constexpr bool kAddend = decltype(withAddend)::value;
         const __amdgpu_buffer_rsrc_t rsC = __builtin_amdgcn_make_buffer_rsrc(
             const_cast<T*>(kAddend ? cin : out), 0, (int)(((int64_t)(g.M - 1) * g.sCm + g.N) * sizeof(T)), 0x00020000);
-        u32x4 cv[2][TN / 2];
+        u32x4 cv[TM][TN / 2];
         auto fetch = [&](int i) {
 #pragma unroll
           for (int jp = 0; jp < TN / 2; ++jp)
-            cv[i & 1][jp] = __builtin_amdgcn_raw_buffer_load_b128(rsC, offsetOf(i, jp, g.sCm), 0, 0);
+            cv[i][jp] = __builtin_amdgcn_raw_buffer_load_b128(rsC, offsetOf(i, jp, g.sCm), 0, 0);
         };
-        if constexpr (kAddend) fetch(0);
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
           if constexpr (kAddend)
-            if (i + 1 < TM) fetch(i + 1);
+            if (i % 4 == 0) {
+#pragma unroll
+              for (int ii = i; ii < i + 4; ++ii) fetch(ii);
+            }
 #pragma unroll
           for (int jp = 0; jp < TN / 2; ++jp) {
             f32x4 x0 = acc[i][2 * jp], x1 = acc[i][2 * jp + 1];
             swapPair(x0, x1);
             const float v[8] = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
             Frag o, c8;
-            if constexpr (kAddend) c8 = __builtin_bit_cast(Frag, cv[i & 1][jp]);
+            if constexpr (kAddend) c8 = __builtin_bit_cast(Frag, cv[i][jp]);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
               float x = v[e] * g.alpha + bv[jp][e];
