@@ -287,15 +287,34 @@ def single_kernel(pkg, torch, dev, rt, stream, args):
                       "achieved": round(work / (us * 1e-6), 1), "unit": unit}), flush=True)
 
 
-def cpu_baseline(pkg, torch):
-    """The oracle's decoder layer on the host cores, on the same batch of four 2048-token sequences."""
+def cpu_baseline(pkg, torch, gpu_out=None):
+    """The oracle's decoder layer on the host cores, on the same batch of four 2048-token sequences. gpu_out (the
+    layer output of the timed GPU run, same seed) is checked against the oracle's output: the oracle as the checker."""
     from oracle import cpu_fallback as oracle
     x, p, cfg = pkg.workloads.llama7b_layer(seed=0, batch=4)
     threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
     torch.set_num_threads(threads)
     t0 = time.perf_counter()
-    oracle.decoder_block(x, p, cfg["heads"], cfg["eps"], cfg["theta"])   # warm-up (thread pool, allocations)
+    host_bf16, _ = oracle.decoder_block(x, p, cfg["heads"], cfg["eps"], cfg["theta"])   # warm-up (thread pool, allocations)
     warm = time.perf_counter() - t0
+    parity = None
+    if gpu_out is not None:
+        # the first sequence of the batch (its output depends on no other) through the oracle in fp32, from the same
+        # bf16 weights and input; eleven chained bf16 roundings on the GPU side: 3e-2 relative + 3e-2 absolute
+        # The same layer run by the host in bf16 (what the timing passes below compute) is measured against the
+        # same fp32 result: the error a bf16 pipeline carries at this size, whoever runs it.
+        want, _ = oracle.decoder_block(x[:1].float(), {k: v.float() for k, v in p.items()}, cfg["heads"], cfg["eps"], cfg["theta"])
+        ref = want.reshape(-1)
+
+        def against_fp32(t):
+            err = (t.float().cpu().reshape(-1) - ref).abs()
+            return {"max_abs_err": round(float(err.max()), 5), "mean_abs_err": round(float(err.mean()), 6),
+                    "out_of_tolerance": int((err > 3e-2 + 3e-2 * ref.abs()).sum())}
+        parity = {"against": "oracle layer output in fp32, first sequence [1, 2048, 4096]", "tolerance": "3e-2 abs + 3e-2 rel",
+                  "elements": int(ref.numel()), "gpu_bf16": against_fp32(gpu_out.reshape(x.shape)[:1]),
+                  "host_bf16": against_fp32(host_bf16[:1])}
+        del want
+    del host_bf16
     reps = 1 if warm > 12 else (3 if warm > 4 else 8)
     times = []
     for _ in range(reps):
@@ -317,7 +336,7 @@ def cpu_baseline(pkg, torch):
     xh.to(dev)
     torch.cuda.synchronize()
     h2d = time.perf_counter() - t0
-    return {"value": round(8192 / t, 2), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+    return {"value": round(8192 / t, 2), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port", "layer_parity": parity,
             "sample": f"the same layer and batch (4 x 2048 tokens) through the oracle: stock ATen CPU kernels in bf16, best of {reps} "
                       f"passes after a warm-up, {t:.2f} s per pass",
             "fallback_copy_ms": {"tensor": "bf16 [4, 2048, 4096] (64 MiB), pageable host memory", "d2h": round(d2h * 1e3, 2),
@@ -408,9 +427,10 @@ def main():
     if not args.no_ops:
         result["ops"] = op_microbench(pkg, torch, dev, rt, stream)
     if not args.no_cpu:
+        gpu_out = out.clone()
         del plan, keep
         torch.cuda.empty_cache()
-        result["cpu_baseline"] = cpu_baseline(pkg, torch)
+        result["cpu_baseline"] = cpu_baseline(pkg, torch, gpu_out)
     else:
         result["cpu_baseline"] = None
     print(json.dumps(result), flush=True)
