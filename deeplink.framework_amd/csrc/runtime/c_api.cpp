@@ -75,7 +75,7 @@ struct SimBackend {
 
 struct SimAllocator {
   SimBackend backend;
-  std::unique_ptr<DeviceCachingAllocator> alloc;
+  std::unique_ptr<DeviceAllocator> alloc;
 };
 
 RawBackend makeSimBackend(SimBackend* sb) {
@@ -265,6 +265,14 @@ int dipuAmdSimAllocatorCreate(void** handle, uint64_t capacity_bytes, const char
     AllocatorConfig cfg = AllocatorConfig::parse(conf ? conf : "");
     cfg.deviceCapacity = capacity_bytes;
     sim->alloc = std::make_unique<DeviceCachingAllocator>(makeSimBackend(&sim->backend), cfg);
+    *handle = sim.release();
+  });
+}
+int dipuAmdSimAllocatorCreateBF(void** handle, uint64_t capacity_bytes, uint64_t max_extend_bytes) {
+  return guarded([&] {
+    auto sim = std::make_unique<SimAllocator>();
+    sim->backend.capacity = capacity_bytes;
+    sim->alloc = std::make_unique<BFCachingAllocator>(makeSimBackend(&sim->backend), max_extend_bytes);
     *handle = sim.release();
   });
 }

@@ -111,25 +111,40 @@ struct SegmentInfo {
   int numBlocks;
 };
 
-class DeviceCachingAllocator {
+// What the runtime needs from a device allocator, whichever algorithm DIPU_DEVICE_MEMCACHING_ALGORITHM selects.
+class DeviceAllocator {
+ public:
+  virtual ~DeviceAllocator() = default;
+  // Never returns nullptr for size > 0; throws OutOfMemory once every way of finding the bytes has failed.
+  virtual void* malloc(size_t size, StreamHandle stream) = 0;
+  virtual void free(void* ptr) = 0;
+  // `ptr` is also being used on `stream`; its reuse waits for an event on that stream.
+  virtual void recordStream(void* ptr, StreamHandle stream) = 0;
+  virtual void emptyCache() = 0;
+  virtual void processEvents() = 0;
+  virtual DeviceStats stats() const = 0;
+  virtual void resetPeakStats() = 0;
+};
+
+class DeviceCachingAllocator : public DeviceAllocator {
  public:
   explicit DeviceCachingAllocator(RawBackend backend, AllocatorConfig config = AllocatorConfig());
-  ~DeviceCachingAllocator();
+  ~DeviceCachingAllocator() override;
 
   // Never returns nullptr for size > 0; throws std::bad_alloc-derived OutOfMemory after the
   // full retry ladder (reuse -> device malloc -> release enough cached -> release all cached).
-  void* malloc(size_t size, StreamHandle stream);
-  void free(void* ptr);
+  void* malloc(size_t size, StreamHandle stream) override;
+  void free(void* ptr) override;
   // `ptr` is also being used on `stream`; its reuse waits for an event on that stream.
-  void recordStream(void* ptr, StreamHandle stream);
-  void emptyCache();
-  void processEvents();
+  void recordStream(void* ptr, StreamHandle stream) override;
+  void emptyCache() override;
+  void processEvents() override;
 
   static size_t roundSize(size_t size, const AllocatorConfig& cfg);
   static size_t allocationSize(size_t size, const AllocatorConfig& cfg);
 
-  DeviceStats stats() const;
-  void resetPeakStats();
+  DeviceStats stats() const override;
+  void resetPeakStats() override;
   std::vector<SegmentInfo> snapshot() const;
   size_t blockSize(void* ptr) const;  // rounded size of a live allocation (0 if unknown)
 
@@ -163,6 +178,68 @@ struct OutOfMemory : std::bad_alloc {
   std::string msg;
   explicit OutOfMemory(std::string m) : msg(std::move(m)) {}
   const char* what() const noexcept override { return msg.c_str(); }
+};
+
+// BF algorithm (dipu/torch_dipu/csrc_dipu/runtime/core/allocator/DIPUBFCachingAllocator.cpp:21-405): free chunks
+// sit in 32 x 4 size classes (powers of two of 512-byte units, each split four ways) with one occupancy bit per
+// class; a request takes the first chunk of its own class if that is large enough, else the first chunk of the
+// next occupied class; a chunk at least twice the request, or 8 MiB larger, is split; freed chunks merge with
+// free neighbours; when nothing fits the cache is emptied and the device is asked for max(request, extend size),
+// the extend size doubling from 8 MiB up to DIPU_MAX_EXTEND_SIZE MiB (1024). All streams share one set of
+// chunks, as in the reference (:357 uses stream set 0): a freed chunk becomes reusable once events recorded at
+// free() on its allocation stream and on every stream given to recordStream() have completed (:525-548).
+class BFCachingAllocator : public DeviceAllocator {
+ public:
+  explicit BFCachingAllocator(RawBackend backend, size_t maxExtendBytes = 0);  // 0: read DIPU_MAX_EXTEND_SIZE
+  ~BFCachingAllocator() override;
+  void* malloc(size_t size, StreamHandle stream) override;
+  void free(void* ptr) override;
+  void recordStream(void* ptr, StreamHandle stream) override;
+  void emptyCache() override;
+  void processEvents() override;
+  DeviceStats stats() const override;
+  void resetPeakStats() override;
+
+  static constexpr int kBigBins = 32, kSubBins = 4, kBins = kBigBins * kSubBins;
+  static constexpr size_t kMaxInternalFragmentation = size_t(8) << 20, kMinExtend = size_t(8) << 20;
+  static int binOf(size_t nbytes);  // size class of a 512-byte-rounded size
+
+ private:
+  struct Chunk {
+    char* ptr = nullptr;
+    size_t size = 0, requested = 0;
+    bool allocated = false;
+    Chunk* before = nullptr;  // neighbours inside the device allocation this chunk was cut from
+    Chunk* after = nullptr;
+    Chunk* binPrev = nullptr;  // neighbours in the free list of its size class
+    Chunk* binNext = nullptr;
+    int bin = -1;
+    StreamHandle stream = nullptr;
+    std::vector<StreamHandle> extraStreams;
+    bool whole() const { return before == nullptr && after == nullptr; }
+  };
+  struct Pending {
+    Chunk* chunk;
+    std::vector<EventHandle> events;
+  };
+  Chunk* take(size_t nbytes);
+  Chunk* extend(size_t nbytes);
+  void pushFree(Chunk* c);
+  void popFree(Chunk* c);
+  void giveBack(Chunk* c);
+  void releaseWholeChunks();
+  bool drainPending(bool wait);
+  EventHandle newEvent();
+
+  mutable std::mutex mutex_;
+  RawBackend backend_;
+  size_t maxExtend_, extendSize_ = kMinExtend;
+  Chunk* heads_[kBins] = {};
+  unsigned __int128 occupied_ = 0;
+  std::unordered_map<void*, Chunk*> live_;
+  std::vector<Pending> pending_;
+  std::vector<EventHandle> eventPool_;
+  DeviceStats stats_;
 };
 
 // RAW algorithm: one device allocation per request, freed when its stream work is known

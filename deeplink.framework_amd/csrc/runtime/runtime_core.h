@@ -79,7 +79,7 @@ struct Runtime {
   EventPool events;
   HostCachingAllocator host;
   // device allocators are created lazily per device according to the environment
-  DeviceCachingAllocator* caching(int device);
+  DeviceAllocator* caching(int device);  // TORCH or BF, whichever the environment selects
   RawAllocator* raw(int device);
   bool useRaw();
   void* deviceMalloc(size_t nbytes, deviceStream_t stream);
@@ -89,10 +89,10 @@ struct Runtime {
 
  private:
   std::mutex mu_;
-  std::array<std::unique_ptr<DeviceCachingAllocator>, kMaxDevices> caching_;
+  std::array<std::unique_ptr<DeviceAllocator>, kMaxDevices> caching_;
   std::array<std::unique_ptr<RawAllocator>, kMaxDevices> raw_;
   std::unordered_map<void*, int> ownerDevice_;
-  int algorithm_ = -1;  // 0 TORCH, 1 RAW
+  int algorithm_ = -1;  // 0 TORCH, 1 RAW, 2 BF
 };
 
 }  // namespace amdrt

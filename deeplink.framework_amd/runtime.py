@@ -275,9 +275,12 @@ class SimAllocator:
     """The caching allocator's state machine over a capacity-limited host stand-in for the
     device, with events that complete only on request. Needs no GPU."""
 
-    def __init__(self, capacity, conf=""):
+    def __init__(self, capacity, conf="", algorithm="TORCH", max_extend=0):
         self.h = c_void_p()
-        _check(_rt().dipuAmdSimAllocatorCreate(byref(self.h), c_uint64(capacity), conf.encode()))
+        if algorithm == "BF":
+            _check(_rt().dipuAmdSimAllocatorCreateBF(byref(self.h), c_uint64(capacity), c_uint64(max_extend)))
+        else:
+            _check(_rt().dipuAmdSimAllocatorCreate(byref(self.h), c_uint64(capacity), conf.encode()))
 
     def close(self):
         if self.h:

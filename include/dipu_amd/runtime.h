@@ -103,6 +103,10 @@ DIPU_AMD_API int dipuAmdCachingHostEmptyCache(void);
 /* The same allocator state machine over a host-memory backend with a capacity limit and
  * manually completed events: lets the allocator be driven on a machine without a GPU. */
 DIPU_AMD_API int dipuAmdSimAllocatorCreate(void** handle, uint64_t capacity_bytes, const char* conf);
+/* The same stand-in driving the BF algorithm (DIPU_DEVICE_MEMCACHING_ALGORITHM=BF,
+ * dipu/torch_dipu/csrc_dipu/runtime/core/allocator/DIPUBFCachingAllocator.cpp:21-405); max_extend_bytes = 0 reads
+ * DIPU_MAX_EXTEND_SIZE (MiB, default 1024). The other dipuAmdSimAllocator* calls work on either kind. */
+DIPU_AMD_API int dipuAmdSimAllocatorCreateBF(void** handle, uint64_t capacity_bytes, uint64_t max_extend_bytes);
 DIPU_AMD_API int dipuAmdSimAllocatorDestroy(void* handle);
 DIPU_AMD_API int dipuAmdSimAllocatorMalloc(void* handle, void** p, size_t nbytes, void* stream);
 DIPU_AMD_API int dipuAmdSimAllocatorFree(void* handle, void* p);

@@ -182,3 +182,149 @@ def test_double_free_is_an_error(pkg, sim):
     a.free(p)
     with pytest.raises(pkg.runtime.RuntimeError_):
         a.free(p)
+
+
+# ------------------------------------------------------------------ BF algorithm
+# DIPU_DEVICE_MEMCACHING_ALGORITHM=BF: dipu/torch_dipu/csrc_dipu/runtime/core/allocator/DIPUBFCachingAllocator.cpp
+@pytest.fixture()
+def bf(pkg):
+    made = []
+
+    def make(capacity=8 << 30, max_extend=0):
+        a = pkg.runtime.SimAllocator(capacity, algorithm="BF", max_extend=max_extend)
+        made.append(a)
+        return a
+
+    yield make
+    for a in made:
+        a.close()
+
+
+def bf_round(n):
+    return ((n - 1) | 511) + 1
+
+
+def test_bf_accounting_matches_the_reference_invariant(bf):
+    """test_memory_stats.py:29-45: allocated == sum(((n - 1) | 511) + 1), reserved >= allocated, and everything
+    returns to zero after the frees (events complete at once here: nothing else uses the blocks)."""
+    a = bf()
+    ptrs, want = [], 0
+    for n in list(range(1, 3000, 7)) + [32767, 65536, MiB, MiB + 1, 3 * MiB, 40 * MiB]:
+        p = a.malloc(n)
+        assert p % 512 == 0
+        ptrs.append((p, bf_round(n)))
+        want += bf_round(n)
+        st = a.stats()
+        assert st["allocated_bytes"] == want
+        assert st["reserved_bytes"] >= st["allocated_bytes"]
+    spans = sorted(ptrs)
+    for (p0, n0), (p1, _) in zip(spans, spans[1:]):
+        assert p0 + n0 <= p1, "live chunks overlap"
+    for p, _ in ptrs:
+        a.free(p)
+    a.complete_events()
+    assert a.stats()["allocated_bytes"] == 0
+    a.empty_cache()
+    assert a.stats()["reserved_bytes"] == 0 and a.backend_usage() == (0, 0)
+
+
+def test_bf_extend_sizes_double_from_8_mib(bf):
+    """extend(): the first device request is max(n, 8 MiB) and the extend size doubles after every success
+    (DIPUBFCachingAllocator.cpp:303-331), up to the cap."""
+    a = bf(max_extend=32 * MiB)
+    a.malloc(512)
+    assert a.backend_usage() == (8 * MiB, 1)
+    held = [a.malloc(6 * MiB)]          # fits in what is left of the first 8 MiB
+    assert a.backend_usage() == (8 * MiB, 1)
+    held.append(a.malloc(6 * MiB))      # nothing fits: second extend is 16 MiB
+    assert a.backend_usage() == (24 * MiB, 2)
+    held.append(a.malloc(30 * MiB))     # third: 32 MiB (the cap)
+    assert a.backend_usage() == (56 * MiB, 3)
+    held.append(a.malloc(31 * MiB))     # capped: stays 32 MiB
+    assert a.backend_usage() == (88 * MiB, 4)
+    held.append(a.malloc(100 * MiB))    # larger than the cap: exactly the rounded request
+    assert a.backend_usage() == (188 * MiB, 5)
+
+
+def test_bf_split_rule_and_merge_on_free(bf):
+    """A chunk at least twice the request (or 8 MiB larger) is split, the rest stays cached; freed neighbours
+    merge back into one chunk that serves a request of the whole size (:375-378, :284-301)."""
+    a = bf()
+    p = a.malloc(3 * MiB)               # 8 MiB from the device, split 3 + 5
+    q = a.malloc(5 * MiB)               # exactly the rest: not split
+    assert q == p + 3 * MiB and a.backend_usage() == (8 * MiB, 1)
+    a.free(p)
+    a.free(q)
+    a.complete_events()
+    r = a.malloc(8 * MiB)               # only possible if the two halves merged
+    assert r == p and a.backend_usage() == (8 * MiB, 1)
+    a.free(r)
+    a.complete_events()
+    s = a.malloc(5 * MiB)               # 8 MiB chunk, 5 MiB request: < 2x and < +8 MiB, handed out whole
+    t = a.malloc(2 * MiB)
+    assert a.backend_usage()[1] == 2, "the 3 MiB tail of an unsplit chunk is not available"
+    assert a.stats()["allocated_bytes"] == 7 * MiB
+    a.free(s), a.free(t)
+
+
+def test_bf_reuse_waits_for_events_on_every_stream(bf):
+    """free() records an event on the allocation stream and on every recordStream() stream; the chunk is reusable
+    only after all of them completed (:525-548). Streams share one set of chunks (:357)."""
+    a = bf()
+    s1, s2 = 0x10, 0x20
+    p = a.malloc(6 * MiB, stream=s1)
+    a.record_stream(p, s2)
+    a.free(p)
+    q = a.malloc(6 * MiB, stream=s1)
+    assert q != p, "reused while its events are outstanding"
+    a.complete_events(s1)
+    q2 = a.malloc(6 * MiB, stream=s1)
+    assert q2 != p, "the other stream's event is still outstanding"
+    a.complete_events(s2)
+    q3 = a.malloc(6 * MiB, stream=s2)   # another stream may take it: one shared set
+    assert q3 == p
+    for x in (q, q2, q3):
+        a.free(x)
+
+
+def test_bf_out_of_memory_ladder(bf, pkg):
+    """Nothing cached fits and the device is full: pending frees are waited for, whole cached chunks go back to the
+    device, and only then the request fails."""
+    a = bf(capacity=64 * MiB, max_extend=8 * MiB)
+    p = a.malloc(40 * MiB)
+    a.free(p)                            # pending: its event is not complete
+    q = a.malloc(48 * MiB)               # needs the 40 MiB released first
+    assert a.backend_usage() == (48 * MiB, 1)
+    with pytest.raises(RuntimeError, match="no memory available"):
+        a.malloc(32 * MiB)
+    assert a.stats()["num_ooms"] == 1
+    a.free(q)
+
+
+def test_bf_size_classes_and_random_stress(bf):
+    a = bf(capacity=2 << 30)
+    rnd = random.Random(7)
+    live = {}
+    for step in range(4000):
+        if live and (rnd.random() < 0.45 or len(live) > 200):
+            p = rnd.choice(list(live))
+            a.free(p)
+            del live[p]
+            if rnd.random() < 0.5:
+                a.complete_events()
+        else:
+            n = rnd.choice([1, 511, 513, 4096, 70000, MiB - 1, 3 * MiB + 5, 9 * MiB])
+            p = a.malloc(n, stream=rnd.choice([0, 0x10]))
+            assert p % 512 == 0 and p not in live
+            live[p] = bf_round(n)
+        if step % 500 == 0:
+            spans = sorted(live.items())
+            for (p0, n0), (p1, _) in zip(spans, spans[1:]):
+                assert p0 + n0 <= p1
+            st = a.stats()
+            assert st["allocated_bytes"] == sum(live.values()) and st["reserved_bytes"] >= st["allocated_bytes"]
+    for p in list(live):
+        a.free(p)
+    a.complete_events()
+    a.empty_cache()
+    assert a.backend_usage() == (0, 0)

@@ -144,3 +144,46 @@ def test_errors_are_reported_not_thrown(pkg, ops, dev):
         ops.mm(a, b, out=torch.empty(4, 6, device=dev))
     with pytest.raises(pkg.diopi.DiopiError, match="host"):
         ops.add(a, torch.randn(4, 5), out=torch.empty(4, 5, device=dev))
+
+
+def test_bf_algorithm_on_device_in_a_fresh_process(pkg):
+    """DIPU_DEVICE_MEMCACHING_ALGORITHM=BF is read once per process (dipu/torch_dipu/csrc_dipu/base/environ.hpp:88-92),
+    so the BF allocator gets a process of its own: accounting invariant of test_memory_stats.py:29-45, real memory,
+    reuse after the stream's work is done, workspace of an op (a transposed GEMM operand) served by it."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = r'''
+import ctypes, sys
+sys.path.insert(0, %r)
+import torch
+from __graft_entry__ import load_package
+pkg = load_package(); rt = pkg.runtime; ops = pkg.ops
+ptrs, want = [], 0
+for n in list(range(1, 32768, 997)) + [1 << 20, (1 << 20) + 1, 64 << 20]:
+    p = rt.cachingMalloc(n); assert p %% 512 == 0
+    ptrs.append(p); want += ((n - 1) | 511) + 1
+st = rt.cachingStats()
+assert st["allocated_bytes"] == want and st["reserved_bytes"] >= want, st
+rt.memSetAsync(0, ptrs[-1], 0x22, 64 << 20); rt.syncDevice()
+out = (ctypes.c_ubyte * 8)(); rt.memCopyD2H(8, ctypes.addressof(out), ptrs[-1] + (64 << 20) - 8)
+assert bytes(out) == b"\x22" * 8
+for p in ptrs: rt.cachingFree(p)
+rt.syncDevice()
+assert rt.cachingStats()["allocated_bytes"] == 0
+q = rt.cachingMalloc(64 << 20); assert q == ptrs[-1], "not served from the cache"
+rt.cachingFree(q)
+dev = torch.device("cuda:0")
+a = torch.randn(300, 200, device=dev).bfloat16(); b = torch.randn(200, 136, device=dev).bfloat16()
+got = ops.mm(a, b).float().cpu(); ref = a.float().cpu() @ b.float().cpu()
+assert float((got - ref).abs().max()) < 0.5
+rt.syncDevice(); rt.cachingEmptyCache()
+assert rt.cachingStats()["reserved_bytes"] == 0
+print("BF ok")
+''' % root
+    env = dict(os.environ, DIPU_DEVICE_MEMCACHING_ALGORITHM="BF")
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300, env=env)
+    assert out.returncode == 0 and "BF ok" in out.stdout, out.stderr[-2000:]
