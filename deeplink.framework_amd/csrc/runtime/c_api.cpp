@@ -276,6 +276,14 @@ int dipuAmdSimAllocatorCreateBF(void** handle, uint64_t capacity_bytes, uint64_t
     *handle = sim.release();
   });
 }
+int dipuAmdSimAllocatorCreateBS(void** handle, uint64_t capacity_bytes, uint64_t min_allocate_bytes, int power_of_two) {
+  return guarded([&] {
+    auto sim = std::make_unique<SimAllocator>();
+    sim->backend.capacity = capacity_bytes;
+    sim->alloc = std::make_unique<BSCachingAllocator>(makeSimBackend(&sim->backend), min_allocate_bytes, power_of_two ? 1 : 0);
+    *handle = sim.release();
+  });
+}
 int dipuAmdSimAllocatorDestroy(void* handle) {
   return guarded([&] {
     auto* sim = static_cast<SimAllocator*>(handle);

@@ -242,6 +242,51 @@ class BFCachingAllocator : public DeviceAllocator {
   DeviceStats stats_;
 };
 
+// BS algorithm (dipu/torch_dipu/csrc_dipu/runtime/core/allocator/DIPUBSCachingAllocator.cpp:18-242): one device
+// allocation per distinct size, kept in a free list of exactly that size. Sizes round up to a multiple of
+// DIPU_BS_ALLOCATOR_MIN_ALLOCATE_SIZE (512), or with DIPU_BS_MORE_ADAPTABLE set to the next power of two (:36-70).
+// Nothing is split or merged; when the device refuses, every idle block is returned to it and the request is tried
+// once more (:84-113). Reuse of a freed block waits for events on its streams (:205-222).
+class BSCachingAllocator : public DeviceAllocator {
+ public:
+  // minAllocate = 0 / powerOfTwo < 0: read the two environment variables
+  explicit BSCachingAllocator(RawBackend backend, size_t minAllocate = 0, int powerOfTwo = -1);
+  ~BSCachingAllocator() override;
+  void* malloc(size_t size, StreamHandle stream) override;
+  void free(void* ptr) override;
+  void recordStream(void* ptr, StreamHandle stream) override;
+  void emptyCache() override;
+  void processEvents() override;
+  DeviceStats stats() const override;
+  void resetPeakStats() override;
+  size_t allocateSize(size_t nbytes) const;
+
+ private:
+  struct Live {
+    size_t size = 0;
+    StreamHandle stream = nullptr;
+    std::vector<StreamHandle> extraStreams;
+  };
+  struct Pending {
+    void* ptr;
+    size_t size;
+    std::vector<EventHandle> events;
+  };
+  bool drainPending(bool wait);
+  void releaseIdle();
+  EventHandle newEvent();
+
+  mutable std::mutex mutex_;
+  RawBackend backend_;
+  size_t minAllocate_;
+  bool powerOfTwo_;
+  std::unordered_map<size_t, std::vector<void*>> idle_;
+  std::unordered_map<void*, Live> live_;
+  std::vector<Pending> pending_;
+  std::vector<EventHandle> eventPool_;
+  DeviceStats stats_;
+};
+
 // RAW algorithm: one device allocation per request, freed when its stream work is known
 // to be finished (synchronous free after a device sync is the conservative choice made here).
 class RawAllocator {

@@ -233,10 +233,12 @@ bool Runtime::useRaw() {
   if (algorithm_ < 0) {
     const char* env = std::getenv("DIPU_DEVICE_MEMCACHING_ALGORITHM");
     std::string a = env ? env : "TORCH";
-    if (a == "TORCH" || a == "BS") {
-      algorithm_ = 0;  // BS requests are served by the TORCH-style allocator on this backend
+    if (a == "TORCH") {
+      algorithm_ = 0;
     } else if (a == "BF") {
       algorithm_ = 2;
+    } else if (a == "BS") {
+      algorithm_ = 3;
     } else if (a == "RAW") {
       algorithm_ = 1;
     } else {
@@ -251,6 +253,7 @@ DeviceAllocator* Runtime::caching(int device) {
   useRaw();  // reads the algorithm selection once
   std::lock_guard<std::mutex> lock(mu_);
   if (!caching_[device] && algorithm_ == 2) caching_[device] = std::make_unique<BFCachingAllocator>(RawBackend::hip());
+  if (!caching_[device] && algorithm_ == 3) caching_[device] = std::make_unique<BSCachingAllocator>(RawBackend::hip());
   if (!caching_[device]) {
     const char* conf = std::getenv("DIPU_TORCH_ALLOCATOR_CONF");
     AllocatorConfig cfg = AllocatorConfig::parse(conf ? conf : "");

@@ -92,7 +92,7 @@ struct Runtime {
   std::array<std::unique_ptr<DeviceAllocator>, kMaxDevices> caching_;
   std::array<std::unique_ptr<RawAllocator>, kMaxDevices> raw_;
   std::unordered_map<void*, int> ownerDevice_;
-  int algorithm_ = -1;  // 0 TORCH, 1 RAW, 2 BF
+  int algorithm_ = -1;  // 0 TORCH, 1 RAW, 2 BF, 3 BS
 };
 
 }  // namespace amdrt

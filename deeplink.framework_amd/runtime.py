@@ -275,10 +275,12 @@ class SimAllocator:
     """The caching allocator's state machine over a capacity-limited host stand-in for the
     device, with events that complete only on request. Needs no GPU."""
 
-    def __init__(self, capacity, conf="", algorithm="TORCH", max_extend=0):
+    def __init__(self, capacity, conf="", algorithm="TORCH", max_extend=0, min_allocate=0, power_of_two=False):
         self.h = c_void_p()
         if algorithm == "BF":
             _check(_rt().dipuAmdSimAllocatorCreateBF(byref(self.h), c_uint64(capacity), c_uint64(max_extend)))
+        elif algorithm == "BS":
+            _check(_rt().dipuAmdSimAllocatorCreateBS(byref(self.h), c_uint64(capacity), c_uint64(min_allocate), c_int(int(power_of_two))))
         else:
             _check(_rt().dipuAmdSimAllocatorCreate(byref(self.h), c_uint64(capacity), conf.encode()))
 

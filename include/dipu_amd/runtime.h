@@ -107,6 +107,10 @@ DIPU_AMD_API int dipuAmdSimAllocatorCreate(void** handle, uint64_t capacity_byte
  * dipu/torch_dipu/csrc_dipu/runtime/core/allocator/DIPUBFCachingAllocator.cpp:21-405); max_extend_bytes = 0 reads
  * DIPU_MAX_EXTEND_SIZE (MiB, default 1024). The other dipuAmdSimAllocator* calls work on either kind. */
 DIPU_AMD_API int dipuAmdSimAllocatorCreateBF(void** handle, uint64_t capacity_bytes, uint64_t max_extend_bytes);
+/* ... and the BS algorithm (DIPUBSCachingAllocator.cpp:18-242): one free list per exact size; sizes are multiples of
+ * min_allocate_bytes (0 = 512) or, with power_of_two != 0, the next power of two (DIPU_BS_MORE_ADAPTABLE). */
+DIPU_AMD_API int dipuAmdSimAllocatorCreateBS(void** handle, uint64_t capacity_bytes, uint64_t min_allocate_bytes,
+                                             int power_of_two);
 DIPU_AMD_API int dipuAmdSimAllocatorDestroy(void* handle);
 DIPU_AMD_API int dipuAmdSimAllocatorMalloc(void* handle, void** p, size_t nbytes, void* stream);
 DIPU_AMD_API int dipuAmdSimAllocatorFree(void* handle, void* p);

@@ -328,3 +328,55 @@ def test_bf_size_classes_and_random_stress(bf):
     a.complete_events()
     a.empty_cache()
     assert a.backend_usage() == (0, 0)
+
+
+# ------------------------------------------------------------------ BS algorithm
+# DIPU_DEVICE_MEMCACHING_ALGORITHM=BS: dipu/torch_dipu/csrc_dipu/runtime/core/allocator/DIPUBSCachingAllocator.cpp
+def test_bs_exact_size_lists_and_accounting(pkg):
+    a = pkg.runtime.SimAllocator(1 << 30, algorithm="BS")
+    try:
+        p = a.malloc(1000)                       # 1024: a multiple of 512
+        q = a.malloc(1024)                       # same size, second device block
+        assert a.backend_usage() == (2048, 2) and a.stats()["allocated_bytes"] == 2048
+        a.free(p)
+        a.complete_events()
+        assert a.malloc(1500) not in (p, q)      # 1536: another size, never served from the 1024 list
+        assert a.malloc(513) == p                # 1024 again: the idle block of exactly that size
+        assert a.backend_usage() == (2048 + 1536, 3)
+        st = a.stats()
+        assert st["allocated_bytes"] == 1024 * 2 + 1536 and st["reserved_bytes"] == st["allocated_bytes"]
+        a.free(q)
+        a.empty_cache()                          # waits for the pending free, then returns idle blocks
+        assert a.backend_usage() == (1024 + 1536, 2)
+    finally:
+        a.close()
+
+
+def test_bs_power_of_two_sizes(pkg):
+    """DIPU_BS_MORE_ADAPTABLE: 1 << bit_length(n), at least 512 (DIPUBSCachingAllocator.cpp:36-52): a power of two
+    itself doubles."""
+    a = pkg.runtime.SimAllocator(1 << 30, algorithm="BS", power_of_two=True)
+    try:
+        for n, want in [(1, 512), (511, 512), (512, 1024), (1000, 1024), (1024, 2048), (70000, 131072)]:
+            before = a.backend_usage()[0]
+            a.malloc(n)
+            assert a.backend_usage()[0] - before == want, (n, want)
+    finally:
+        a.close()
+
+
+def test_bs_reuse_waits_for_events_and_oom_empties_the_cache(pkg):
+    a = pkg.runtime.SimAllocator(64 * MiB, algorithm="BS")
+    try:
+        p = a.malloc(20 * MiB, stream=0x10)
+        a.record_stream(p, 0x20)
+        a.free(p)
+        q = a.malloc(24 * MiB)                   # another size; the pending 20 MiB is waited for and parked idle
+        assert a.backend_usage() == (44 * MiB, 2)
+        r = a.malloc(30 * MiB)                   # device full: the idle 20 MiB block goes back, then it fits
+        assert a.backend_usage() == (54 * MiB, 2) and a.stats()["num_alloc_retries"] == 1
+        with pytest.raises(RuntimeError, match="no memory available"):
+            a.malloc(40 * MiB)
+        a.free(q), a.free(r)
+    finally:
+        a.close()

@@ -146,9 +146,10 @@ def test_errors_are_reported_not_thrown(pkg, ops, dev):
         ops.add(a, torch.randn(4, 5), out=torch.empty(4, 5, device=dev))
 
 
-def test_bf_algorithm_on_device_in_a_fresh_process(pkg):
-    """DIPU_DEVICE_MEMCACHING_ALGORITHM=BF is read once per process (dipu/torch_dipu/csrc_dipu/base/environ.hpp:88-92),
-    so the BF allocator gets a process of its own: accounting invariant of test_memory_stats.py:29-45, real memory,
+@pytest.mark.parametrize("algorithm", ["BF", "BS"])
+def test_other_caching_algorithms_on_device_in_a_fresh_process(pkg, algorithm):
+    """DIPU_DEVICE_MEMCACHING_ALGORITHM is read once per process (dipu/torch_dipu/csrc_dipu/base/environ.hpp:88-92),
+    so the BF and BS allocators each get a process of their own: accounting invariant of test_memory_stats.py:29-45, real memory,
     reuse after the stream's work is done, workspace of an op (a transposed GEMM operand) served by it."""
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
@@ -182,8 +183,8 @@ got = ops.mm(a, b).float().cpu(); ref = a.float().cpu() @ b.float().cpu()
 assert float((got - ref).abs().max()) < 0.5
 rt.syncDevice(); rt.cachingEmptyCache()
 assert rt.cachingStats()["reserved_bytes"] == 0
-print("BF ok")
+print("allocator ok")
 ''' % root
-    env = dict(os.environ, DIPU_DEVICE_MEMCACHING_ALGORITHM="BF")
+    env = dict(os.environ, DIPU_DEVICE_MEMCACHING_ALGORITHM=algorithm)
     out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300, env=env)
-    assert out.returncode == 0 and "BF ok" in out.stdout, out.stderr[-2000:]
+    assert out.returncode == 0 and "allocator ok" in out.stdout, out.stderr[-2000:]
