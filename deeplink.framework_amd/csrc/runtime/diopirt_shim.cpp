@@ -3,7 +3,9 @@
 // Same symbol set and behaviour as DIPU's provider,
 // dipu/torch_dipu/csrc_dipu/diopirt/diopirt_impl.cpp:15-239 (an at::Tensor* there,
 // a dipuAmdTensor* here; the impl library cannot tell the difference).
+#include <cstring>
 #include <list>
+#include <mutex>
 #include <string>
 
 #include <diopi/diopirt.h>
@@ -14,6 +16,13 @@
 using dipu::amdrt::Runtime;
 
 struct diopiTensor : dipuAmdTensor {};
+
+struct diopiGenerator {
+  mutable std::mutex mutex;
+  uint64_t seed = 67280421310721ull;
+  uint64_t offset = 0;
+  int device_index = 0;
+};
 
 struct WorkspaceTensor {
   diopiTensor desc;
@@ -183,20 +192,61 @@ DIOPI_RT_API diopiError_t diopiRequireBuffer(diopiContextHandle_t ctx, diopiTens
   return diopiRequireTensor(ctx, tensor, &size, nullptr, diopi_dtype_int8, device);
 }
 
-// The inference path draws no random numbers on the device; generators are a
-// link-time requirement only (dipu/torch_dipu/csrc_dipu/runtime/core/DIPUGeneratorImpl.h:62).
-DIOPI_RT_API diopiError_t diopiGeneratorGetState(diopiContextHandle_t, diopiConstGeneratorHandle_t,
-                                                 diopiTensorHandle_t*) {
-  return diopiNoImplement;
+// Generator state as the reference's CUDA vendor keeps it (dipu/torch_dipu/csrc_dipu/vendor/cuda/CudaGeneratorImpl.cpp:
+// 17-76): a Philox seed and offset, serialised as 16 bytes on the host (seed, then offset; an 8-byte state is a seed
+// with offset 0), the offset a multiple of 4. The inference path draws no random numbers; the callbacks are here so
+// that an operator library that does can keep its counter (diopirt_impl.cpp:175-226).
+DIOPI_RT_API diopiError_t diopiGeneratorGetState(diopiContextHandle_t ctx, diopiConstGeneratorHandle_t gen,
+                                                 diopiTensorHandle_t* data) {
+  if (!ctx || !gen || !data) return diopiErrorOccurred;
+  const int64_t n = 16;
+  diopiSize_t size{&n, 1};
+  diopiError_t err = diopiRequireTensor(ctx, data, &size, nullptr, diopi_dtype_uint8, diopi_host);
+  if (err != diopiSuccess) return err;
+  uint64_t words[2];
+  {
+    std::lock_guard<std::mutex> lock(gen->mutex);
+    words[0] = gen->seed, words[1] = gen->offset;
+  }
+  std::memcpy((*data)->data, words, sizeof(words));
+  return diopiSuccess;
 }
-DIOPI_RT_API diopiError_t diopiGeneratorSetState(diopiGeneratorHandle_t, diopiConstTensorHandle_t) {
-  return diopiNoImplement;
+DIOPI_RT_API diopiError_t diopiGeneratorSetState(diopiGeneratorHandle_t gen, diopiConstTensorHandle_t state) {
+  if (!gen || !state || state->device != diopi_host || state->dtype != diopi_dtype_uint8 || state->ndim != 1 ||
+      state->stride[0] != 1 || (state->shape[0] != 16 && state->shape[0] != 8))
+    return diopiErrorOccurred;  // "RNG state is wrong size" / not a byte tensor on the host
+  uint64_t words[2] = {0, 0};
+  std::memcpy(words, state->data, static_cast<size_t>(state->shape[0]));
+  if (words[1] % 4 != 0) return diopiErrorOccurred;  // offset must be a multiple of 4
+  std::lock_guard<std::mutex> lock(gen->mutex);
+  gen->seed = words[0], gen->offset = words[1];
+  return diopiSuccess;
 }
-DIOPI_RT_API diopiError_t diopiGeneratorGetSeedAndOffset(diopiGeneratorHandle_t, uint64_t*, uint64_t*) {
-  return diopiNoImplement;
+DIOPI_RT_API diopiError_t diopiGeneratorGetSeedAndOffset(diopiGeneratorHandle_t gen, uint64_t* seed, uint64_t* offset) {
+  if (!gen || !seed || !offset) return diopiErrorOccurred;
+  std::lock_guard<std::mutex> lock(gen->mutex);
+  *seed = gen->seed, *offset = gen->offset;
+  return diopiSuccess;
 }
-DIOPI_RT_API diopiError_t diopiGeneratorSetSeedAndOffset(diopiGeneratorHandle_t, uint64_t, uint64_t) {
-  return diopiNoImplement;
+DIOPI_RT_API diopiError_t diopiGeneratorSetSeedAndOffset(diopiGeneratorHandle_t gen, uint64_t seed, uint64_t offset) {
+  if (!gen || offset % 4 != 0) return diopiErrorOccurred;
+  std::lock_guard<std::mutex> lock(gen->mutex);
+  gen->seed = seed, gen->offset = offset;
+  return diopiSuccess;
+}
+
+// The object vendorMakeGenerator hands out (runtime/core/DIPUGeneratorImpl.h:62), without libtorch: seed 67280421310721
+// is torch's default_rng_seed_val.
+int dipuAmdGeneratorCreate(diopiGeneratorHandle_t* gen, int device_index) {
+  if (!gen) return 1;
+  auto* g = new diopiGenerator();
+  g->device_index = device_index;
+  *gen = g;
+  return 0;
+}
+int dipuAmdGeneratorDestroy(diopiGeneratorHandle_t gen) {
+  delete gen;
+  return 0;
 }
 
 // Named host ranges: ROCTX ranges while devapis::enableProfiler is in effect, nothing otherwise

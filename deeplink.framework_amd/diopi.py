@@ -118,6 +118,51 @@ def handle(t):
     return h, h.ptr
 
 
+class Generator:
+    """The generator object behind the diopiGenerator* runtime callbacks (what vendorMakeGenerator returns in DIPU,
+    runtime/core/DIPUGeneratorImpl.h:62): a Philox seed and offset, state = 16 host bytes (seed, offset)."""
+
+    def __init__(self, device_index=0):
+        self.ptr = c_void_p()
+        if _native.runtime().dipuAmdGeneratorCreate(byref(self.ptr), c_int(device_index)) != 0:
+            raise DiopiError("dipuAmdGeneratorCreate failed")
+
+    def close(self):
+        if self.ptr:
+            _native.runtime().dipuAmdGeneratorDestroy(self.ptr)
+            self.ptr = None
+
+    def seed_and_offset(self):
+        seed, off = c_uint64(), c_uint64()
+        rc = _native.runtime().diopiGeneratorGetSeedAndOffset(self.ptr, byref(seed), byref(off))
+        if rc != 0:
+            raise DiopiError(f"diopiGeneratorGetSeedAndOffset returned {rc}")
+        return seed.value, off.value
+
+    def set_seed_and_offset(self, seed, offset):
+        rc = _native.runtime().diopiGeneratorSetSeedAndOffset(self.ptr, c_uint64(seed), c_uint64(offset))
+        if rc != 0:
+            raise DiopiError(f"diopiGeneratorSetSeedAndOffset returned {rc} (the offset must be a multiple of 4)")
+
+    def get_state(self):
+        """The state as a uint8 CPU tensor of 16 bytes (copied out of the context's workspace before it closes)."""
+        import torch
+        with Context(0) as ctx:  # the state lives on the host: no stream is involved
+            th = c_void_p()
+            rc = _native.runtime().diopiGeneratorGetState(ctx.ptr, self.ptr, byref(th))
+            if rc != 0:
+                raise DiopiError(f"diopiGeneratorGetState returned {rc}")
+            desc = ctypes.cast(th, POINTER(dipuAmdTensor)).contents
+            raw = ctypes.string_at(desc.data, int(desc.shape[0]))
+        return torch.frombuffer(bytearray(raw), dtype=torch.uint8)
+
+    def set_state(self, state):
+        h, p = handle(state)
+        rc = _native.runtime().diopiGeneratorSetState(self.ptr, p)
+        if rc != 0:
+            raise DiopiError(f"diopiGeneratorSetState returned {rc} (state must be 16 or 8 host bytes, offset a multiple of 4)")
+
+
 class Context:
     """diopiContext bound to a stream (diopirt_impl.h:19-26). Workspace the impl library
     requests lives until the context is closed; DIPU closes it when the wrapper returns."""

@@ -100,6 +100,12 @@ DIPU_AMD_API int dipuAmdCachingHostFree(void* p);
 DIPU_AMD_API int dipuAmdCachingHostRecordStream(void* p, void* stream);
 DIPU_AMD_API int dipuAmdCachingHostEmptyCache(void);
 
+/* A generator object for the diopiGenerator* callbacks of diopirt.h: what vendorMakeGenerator returns in DIPU
+ * (runtime/core/DIPUGeneratorImpl.h:62; state layout of vendor/cuda/CudaGeneratorImpl.cpp:17-76), without libtorch. */
+struct diopiGenerator;
+DIPU_AMD_API int dipuAmdGeneratorCreate(struct diopiGenerator** gen, int device_index);
+DIPU_AMD_API int dipuAmdGeneratorDestroy(struct diopiGenerator* gen);
+
 /* The same allocator state machine over a host-memory backend with a capacity limit and
  * manually completed events: lets the allocator be driven on a machine without a GPU. */
 DIPU_AMD_API int dipuAmdSimAllocatorCreate(void** handle, uint64_t capacity_bytes, const char* conf);

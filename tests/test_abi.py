@@ -106,3 +106,32 @@ def test_profiler_hooks_count_ranges_only_while_enabled(pkg):
         assert (s2 - s0, e2 - e0) == (3, 3)
     finally:
         rt.disableProfiler()
+
+
+def test_generator_state_round_trip(pkg):
+    """The diopiGenerator* runtime callbacks with the CUDA vendor's state layout
+    (dipu/torch_dipu/csrc_dipu/vendor/cuda/CudaGeneratorImpl.cpp:17-76; callbacks diopirt_impl.cpp:175-226): 16 host
+    bytes = seed then Philox offset, an 8-byte state sets offset 0, offsets must be multiples of 4."""
+    import struct
+    import torch
+    d = pkg.diopi
+    g = d.Generator()
+    try:
+        assert g.seed_and_offset() == (67280421310721, 0)          # torch's default seed
+        g.set_seed_and_offset(1234, 8)
+        assert g.seed_and_offset() == (1234, 8)
+        st = g.get_state()
+        assert st.dtype == torch.uint8 and st.numel() == 16
+        assert struct.unpack("<QQ", bytes(st.tolist())) == (1234, 8)
+        h = d.Generator()
+        h.set_state(st)
+        assert h.seed_and_offset() == (1234, 8)
+        h.set_state(torch.tensor(list(struct.pack("<Q", 99)), dtype=torch.uint8))   # seed only
+        assert h.seed_and_offset() == (99, 0)
+        with pytest.raises(d.DiopiError):
+            g.set_seed_and_offset(1, 6)                               # offset not a multiple of 4
+        with pytest.raises(d.DiopiError):
+            h.set_state(torch.zeros(12, dtype=torch.uint8))           # wrong size
+        h.close()
+    finally:
+        g.close()
