@@ -6,6 +6,7 @@
 
 #include <dipu_amd/runtime.h>
 
+#include "expandable_segment.h"
 #include "runtime_core.h"
 
 using namespace dipu;
@@ -73,6 +74,47 @@ struct SimBackend {
   }
 };
 
+// A 1 GiB synthetic address range whose segments count against the simulated capacity while mapped.
+struct SimExpandableRange final : ExpandableRange {
+  SimBackend* sb;
+  size_t segmentSize;
+  char* base;
+  std::vector<bool> mapped;
+  SimExpandableRange(SimBackend* b, size_t segSize) : sb(b), segmentSize(segSize), mapped((size_t(1) << 30) / segSize, false) {
+    base = reinterpret_cast<char*>(sb->nextAddr);
+    sb->nextAddr += size_t(1) << 30;
+  }
+  ~SimExpandableRange() override {
+    for (bool m : mapped)
+      if (m) sb->inUse -= segmentSize, --sb->segments;
+  }
+  void map(char* p, size_t n, char** mp, size_t* ms) override {
+    const size_t begin = static_cast<size_t>(p - base) / segmentSize;
+    const size_t end = std::min(mapped.size(), (static_cast<size_t>(p - base) + n + segmentSize - 1) / segmentSize);
+    if (static_cast<size_t>(p - base) % segmentSize) throw std::invalid_argument("sim expandable range: map must start at a segment");
+    *mp = p, *ms = 0;
+    if (sb->inUse + (end - begin) * segmentSize > sb->capacity) return;
+    for (size_t i = begin; i < end; ++i) {
+      if (mapped[i]) throw std::invalid_argument("sim expandable range: segment mapped twice");
+      mapped[i] = true, sb->inUse += segmentSize, ++sb->segments;
+    }
+    *ms = (end - begin) * segmentSize;
+  }
+  void unmap(char* p, size_t n, char** up, size_t* us) override {
+    const size_t begin = (static_cast<size_t>(p - base) + segmentSize - 1) / segmentSize;
+    const size_t end = std::min(mapped.size(), (static_cast<size_t>(p - base) + n) / segmentSize);
+    *up = base + begin * segmentSize, *us = 0;
+    if (begin >= end) return;
+    for (size_t i = begin; i < end; ++i) {
+      if (!mapped[i]) throw std::invalid_argument("sim expandable range: segment was not mapped");
+      mapped[i] = false, sb->inUse -= segmentSize, --sb->segments;
+    }
+    *us = (end - begin) * segmentSize;
+  }
+  char* ptr() const override { return base; }
+  size_t size() const override { return mapped.size() * segmentSize; }
+};
+
 struct SimAllocator {
   SimBackend backend;
   std::unique_ptr<DeviceAllocator> alloc;
@@ -80,6 +122,7 @@ struct SimAllocator {
 
 RawBackend makeSimBackend(SimBackend* sb) {
   RawBackend b;
+  b.createExpandable = [sb](StreamHandle, size_t segmentSize) -> ExpandableRange* { return new SimExpandableRange(sb, segmentSize); };
   b.mallocDevice = [sb](void** p, size_t n) {
     if (sb->inUse + n > sb->capacity) return false;
     // Addresses are synthetic and never dereferenced: a monotonically growing, 2 MiB
@@ -274,6 +317,32 @@ int dipuAmdSimAllocatorCreateBF(void** handle, uint64_t capacity_bytes, uint64_t
     sim->backend.capacity = capacity_bytes;
     sim->alloc = std::make_unique<BFCachingAllocator>(makeSimBackend(&sim->backend), max_extend_bytes);
     *handle = sim.release();
+  });
+}
+int dipuAmdExpandableSegmentCreate(void** handle, int device, void* stream, uint64_t segment_bytes) {
+  return guarded([&] { *handle = new HipExpandableSegment(device, S(stream), segment_bytes); });
+}
+int dipuAmdExpandableSegmentDestroy(void* handle) {
+  return guarded([&] { delete static_cast<HipExpandableSegment*>(handle); });
+}
+int dipuAmdExpandableSegmentInfo(void* handle, void** base, uint64_t* reserved_bytes, uint64_t* mapped_bytes) {
+  return guarded([&] {
+    auto* s = static_cast<HipExpandableSegment*>(handle);
+    *base = s->ptr(), *reserved_bytes = s->size(), *mapped_bytes = s->mappedBytes();
+  });
+}
+int dipuAmdExpandableSegmentMap(void* handle, uint64_t offset, uint64_t nbytes, uint64_t* mapped_offset, uint64_t* mapped_bytes) {
+  return guarded([&] {
+    auto* s = static_cast<HipExpandableSegment*>(handle);
+    const SegmentRange r = s->map({s->ptr() + offset, nbytes});
+    *mapped_offset = static_cast<uint64_t>(r.ptr - s->ptr()), *mapped_bytes = r.size;
+  });
+}
+int dipuAmdExpandableSegmentUnmap(void* handle, uint64_t offset, uint64_t nbytes, uint64_t* unmapped_offset, uint64_t* unmapped_bytes) {
+  return guarded([&] {
+    auto* s = static_cast<HipExpandableSegment*>(handle);
+    const SegmentRange r = s->unmap({s->ptr() + offset, nbytes});
+    *unmapped_offset = static_cast<uint64_t>(r.ptr - s->ptr()), *unmapped_bytes = r.size;
   });
 }
 int dipuAmdSimAllocatorCreateBS(void** handle, uint64_t capacity_bytes, uint64_t min_allocate_bytes, int power_of_two) {

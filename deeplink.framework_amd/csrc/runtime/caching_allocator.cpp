@@ -15,6 +15,11 @@ bool BlockLess::operator()(const Block* a, const Block* b) const {
 }
 
 // ---------------------------------------------------------------- config ----
+bool BlockAddressLess::operator()(const Block* a, const Block* b) const {
+  if (a->stream != b->stream) return reinterpret_cast<uintptr_t>(a->stream) < reinterpret_cast<uintptr_t>(b->stream);
+  return reinterpret_cast<uintptr_t>(a->ptr) < reinterpret_cast<uintptr_t>(b->ptr);
+}
+
 AllocatorConfig AllocatorConfig::parse(const std::string& conf) {
   AllocatorConfig cfg;
   std::stringstream ss(conf);
@@ -46,7 +51,8 @@ AllocatorConfig AllocatorConfig::parse(const std::string& conf) {
     } else if (key == "huge_segments") {
       cfg.hugeSegments = (val == "1" || val == "true" || val == "True");
     } else if (key == "expandable_segments") {
-      // accepted for configuration compatibility; this backend sizes segments instead
+      if (val != "True" && val != "False") throw std::invalid_argument("allocator conf: expandable_segments expects True or False");
+      cfg.expandableSegments = val == "True";
     } else {
       throw std::invalid_argument("allocator conf: unknown option '" + key + "'");
     }
@@ -86,6 +92,7 @@ DeviceCachingAllocator::~DeviceCachingAllocator() {
     releaseBlocks(large_);
     releaseBlocks(small_);
     for (auto e : eventPool_) backend_.destroyEvent(e);
+    for (ExpandableRange* es : expandables_) delete es;  // ranges that still hold live blocks at teardown
   } catch (...) {
   }
   for (auto& kv : active_) delete kv.second;
@@ -115,7 +122,143 @@ Block* DeviceCachingAllocator::getFreeBlock(BlockPool& pool, size_t size, Stream
   return b;
 }
 
-bool DeviceCachingAllocator::allocBlock(BlockPool& pool, size_t allocSize, StreamHandle stream, Block** out) {
+// ---- expandable segments (DIPUCachingDeviceAllocator.cpp:1086-1215, 1633-1705) ----
+// One address range per (stream, pool) grows at its end instead of new fixed-size segments being requested: a
+// request is served by free mapped blocks followed by enough freshly mapped segments, so a large block can always
+// be assembled from what smaller ones left behind.
+Block* DeviceCachingAllocator::findExpandableBlock(BlockPool& pool, size_t size, StreamHandle stream) {
+  auto allocatable = [](const Block* b) { return b && !b->allocated && b->eventCount == 0 && b->streamUses.empty(); };
+  auto roomFrom = [&](const Block* b) {
+    size_t bytes = 0;
+    while (bytes < size && allocatable(b)) bytes += b->size, b = b->next;
+    return bytes >= size;
+  };
+  Block key;
+  key.stream = stream;
+  key.ptr = nullptr;
+  for (auto it = pool.unmapped.lower_bound(&key); it != pool.unmapped.end() && (*it)->stream == stream; ++it) {
+    Block* c = *it;
+    if (allocatable(c->prev)) c = c->prev;  // a free mapped block right before the unmapped range is used first
+    if (roomFrom(c)) return c;
+  }
+  ExpandableRange* es = backend_.createExpandable(stream, pool.isSmall ? kSmallBuffer : kLargeBuffer);
+  expandables_.push_back(es);
+  stats_.segment.add(1);
+  Block* candidate = new Block();
+  candidate->stream = stream;
+  candidate->size = es->size();
+  candidate->pool = &pool;
+  candidate->ptr = es->ptr();
+  candidate->mapped = false;
+  candidate->expandable = es;
+  pool.unmapped.insert(candidate);
+  return candidate;
+}
+
+bool DeviceCachingAllocator::mapBlock(Block* toMap, size_t size) {
+  char* mp = nullptr;
+  size_t ms = 0;
+  toMap->expandable->map(static_cast<char*>(toMap->ptr), size, &mp, &ms);
+  if (ms == 0) return false;
+  BlockPool& pool = *toMap->pool;
+  pool.unmapped.erase(toMap);
+  toMap->mapped = true;
+  if (ms < toMap->size) {  // the rest of the range stays unmapped behind it
+    Block* rest = new Block();
+    rest->stream = toMap->stream;
+    rest->pool = &pool;
+    rest->ptr = static_cast<char*>(toMap->ptr) + ms;
+    rest->size = toMap->size - ms;
+    rest->mapped = false;
+    rest->expandable = toMap->expandable;
+    rest->prev = toMap;
+    rest->next = toMap->next;
+    if (rest->next) rest->next->prev = rest;
+    toMap->next = rest;
+    toMap->size = ms;
+    pool.unmapped.insert(rest);
+  }
+  tryMerge(toMap, toMap->prev, pool);
+  tryMerge(toMap, toMap->next, pool);
+  pool.blocks.insert(toMap);
+  totalReserved_ += ms;
+  stats_.reservedBytes.add(static_cast<int64_t>(ms));
+  return true;
+}
+
+Block* DeviceCachingAllocator::tryAllocateExpandableBlock(BlockPool& pool, size_t size, StreamHandle stream) {
+  Block* candidate = findExpandableBlock(pool, size, stream);
+  // candidate heads a run of free / unmapped blocks with room for `size`: unmapped, unmapped -> free, free -> unmapped
+  if (!candidate->mapped && !mapBlock(candidate, std::min(candidate->size, size))) return nullptr;
+  while (candidate->size < size) {  // free -> unmapped: map some of the unmapped part, it merges into the free one
+    Block* next = candidate->next;
+    if (!mapBlock(next, std::min(size - candidate->size, next->size))) return nullptr;
+    candidate = next;  // the free block in front was merged into the newly mapped one
+  }
+  pool.blocks.erase(candidate);
+  return candidate;
+}
+
+// Gives the whole segments inside a free block of an expandable range back to the device.
+void DeviceCachingAllocator::unmapBlock(Block* block) {
+  char* up = nullptr;
+  size_t us = 0;
+  block->expandable->unmap(static_cast<char*>(block->ptr), block->size, &up, &us);
+  if (us == 0) return;
+  BlockPool& pool = *block->pool;
+  pool.blocks.erase(block);
+  const size_t before = static_cast<size_t>(up - static_cast<char*>(block->ptr));
+  const size_t after = block->size - before - us;
+  auto piece = [&](char* p, size_t n) {
+    Block* b = new Block();
+    b->stream = block->stream;
+    b->pool = &pool;
+    b->ptr = p;
+    b->size = n;
+    b->expandable = block->expandable;
+    return b;
+  };
+  if (before > 0) {  // prev? -> beforeFree -> block
+    Block* b = piece(static_cast<char*>(block->ptr), before);
+    b->prev = block->prev;
+    if (b->prev) b->prev->next = b;
+    b->next = block;
+    block->prev = b;
+    pool.blocks.insert(b);
+  }
+  if (after > 0) {  // block -> afterFree -> next?
+    Block* b = piece(up + us, after);
+    b->next = block->next;
+    if (b->next) b->next->prev = b;
+    b->prev = block;
+    block->next = b;
+    pool.blocks.insert(b);
+  }
+  block->ptr = up;
+  block->size = us;
+  block->mapped = false;
+  tryMerge(block, block->prev, pool);
+  tryMerge(block, block->next, pool);
+  pool.unmapped.insert(block);
+  totalReserved_ -= us;
+  stats_.reservedBytes.add(-static_cast<int64_t>(us));
+}
+
+void DeviceCachingAllocator::releaseExpandable(Block* block) {
+  // the block is the range's only one and nothing of it is mapped
+  auto it = std::find(expandables_.begin(), expandables_.end(), block->expandable);
+  if (it != expandables_.end()) expandables_.erase(it);
+  block->pool->unmapped.erase(block);
+  delete block->expandable;
+  stats_.segment.add(-1);
+  delete block;
+}
+
+bool DeviceCachingAllocator::allocBlock(BlockPool& pool, size_t size, size_t allocSize, StreamHandle stream, Block** out) {
+  if (config_.expandableSegments && backend_.createExpandable) {
+    *out = tryAllocateExpandableBlock(pool, size, stream);
+    return *out != nullptr;
+  }
   void* p = nullptr;
   ++stats_.numDeviceMalloc;
   if (!backend_.mallocDevice(&p, allocSize) || p == nullptr) return false;
@@ -142,14 +285,14 @@ void* DeviceCachingAllocator::malloc(size_t origSize, StreamHandle stream) {
   Block* block = getFreeBlock(pool, size, stream);
   if (!block) {
     if (config_.gcThreshold > 0.0) garbageCollect();
-    bool ok = allocBlock(pool, allocSize, stream, &block);
+    bool ok = allocBlock(pool, size, allocSize, stream, &block);
     if (!ok) {
       ++stats_.numAllocRetries;
-      ok = releaseAvailableCachedBlocks(pool, allocSize, stream) && allocBlock(pool, allocSize, stream, &block);
+      ok = releaseAvailableCachedBlocks(pool, allocSize, stream) && allocBlock(pool, size, allocSize, stream, &block);
     }
     if (!ok) {
       ++stats_.numAllocRetries;
-      ok = releaseCachedBlocks() && allocBlock(pool, allocSize, stream, &block);
+      ok = releaseCachedBlocks() && allocBlock(pool, size, allocSize, stream, &block);
     }
     if (!ok) {
       ++stats_.numOoms;
@@ -177,6 +320,7 @@ void* DeviceCachingAllocator::malloc(size_t origSize, StreamHandle stream) {
     rem->pool = block->pool;
     rem->ptr = static_cast<char*>(block->ptr) + size;
     rem->size = block->size - size;
+    rem->expandable = block->expandable;
     rem->prev = block;
     rem->next = block->next;
     if (rem->next) rem->next->prev = rem;
@@ -217,7 +361,7 @@ void DeviceCachingAllocator::free(void* ptr) {
 }
 
 size_t DeviceCachingAllocator::tryMerge(Block* dst, Block* src, BlockPool& pool) {
-  if (!src || src->allocated || src->eventCount > 0 || !src->streamUses.empty()) return 0;
+  if (!src || src->allocated || src->eventCount > 0 || !src->streamUses.empty() || dst->mapped != src->mapped) return 0;
   if (dst->prev == src) {
     dst->ptr = src->ptr;
     dst->prev = src->prev;
@@ -228,7 +372,7 @@ size_t DeviceCachingAllocator::tryMerge(Block* dst, Block* src, BlockPool& pool)
   }
   size_t subsumed = src->size;
   dst->size += subsumed;
-  pool.blocks.erase(src);
+  if (src->mapped) pool.blocks.erase(src); else pool.unmapped.erase(src);
   delete src;
   return subsumed;
 }
@@ -322,10 +466,16 @@ void DeviceCachingAllocator::releaseBlock(Block* block) {
 }
 
 void DeviceCachingAllocator::releaseBlocks(BlockPool& pool) {
+  std::vector<Block*> toUnmap;  // unmapping changes the pool: collect first
   for (auto it = pool.blocks.begin(); it != pool.blocks.end();) {
     Block* b = *it;
     ++it;
-    if (!b->prev && !b->next) releaseBlock(b);  // only whole segments go back to the device
+    if (b->expandable) toUnmap.push_back(b);
+    else if (!b->prev && !b->next) releaseBlock(b);  // only whole segments go back to the device
+  }
+  for (Block* b : toUnmap) {
+    unmapBlock(b);
+    if (!b->mapped && !b->prev && !b->next) releaseExpandable(b);  // nothing of the range is in use any more
   }
 }
 
@@ -345,7 +495,7 @@ bool DeviceCachingAllocator::releaseAvailableCachedBlocks(BlockPool& pool, size_
       Block* cur = *it;
       bool atBegin = it == pool.blocks.begin();
       if (!atBegin) --it;
-      if (!cur->prev && !cur->next) {
+      if (!cur->prev && !cur->next && !cur->expandable) {
         freed += cur->size;
         releaseBlock(cur);
       }
@@ -353,7 +503,7 @@ bool DeviceCachingAllocator::releaseAvailableCachedBlocks(BlockPool& pool, size_
     }
     return freed >= size;
   }
-  if ((*it)->prev || (*it)->next) return false;
+  if ((*it)->prev || (*it)->next || (*it)->expandable) return false;
   releaseBlock(*it);
   return true;
 }
@@ -379,7 +529,7 @@ void DeviceCachingAllocator::garbageCollect() {
   size_t target = totalReserved_ - limit, freed = 0;
   int64_t totalAge = 0, count = 0;
   for (Block* b : large_.blocks)
-    if (!b->isSplit()) totalAge += ++b->gcCount, ++count;
+    if (!b->isSplit() && !b->expandable) totalAge += ++b->gcCount, ++count;  // parts of expandable ranges stay
   if (count == 0) return;
   bool progressed = true;
   while (freed < target && progressed && count > 0) {
@@ -388,7 +538,7 @@ void DeviceCachingAllocator::garbageCollect() {
     for (auto it = large_.blocks.begin(); it != large_.blocks.end() && freed < target;) {
       Block* b = *it;
       ++it;
-      if (!b->isSplit() && static_cast<double>(b->gcCount) >= avg) {
+      if (!b->isSplit() && !b->expandable && static_cast<double>(b->gcCount) >= avg) {
         freed += b->size;
         totalAge -= b->gcCount;
         --count;
@@ -436,6 +586,7 @@ std::vector<SegmentInfo> DeviceCachingAllocator::snapshot() const {
   for (const Block* h : heads) {
     SegmentInfo s{h->ptr, 0, 0, 0, !h->pool->isSmall, 0};
     for (const Block* b = h; b; b = b->next) {
+      if (!b->mapped) continue;  // address space only
       s.totalSize += b->size;
       if (b->allocated) s.allocatedSize += b->size;
       if (b->allocated || b->eventCount > 0) s.activeSize += b->size;

@@ -30,9 +30,23 @@ namespace amdrt {
 using StreamHandle = void*;
 using EventHandle = void*;
 
+// A reserved address range whose segments are backed and released on demand (DIPU's ExpandableSegment,
+// runtime/core/allocator/ExpandableSegment.h:114-136). map() backs every segment the range touches and reports what
+// is mapped now (size 0: out of memory, nothing changed); unmap() releases the segments entirely inside the range.
+struct ExpandableRange {
+  virtual ~ExpandableRange() = default;
+  virtual void map(char* ptr, size_t size, char** mappedPtr, size_t* mappedSize) = 0;
+  virtual void unmap(char* ptr, size_t size, char** unmappedPtr, size_t* unmappedSize) = 0;
+  virtual char* ptr() const = 0;
+  virtual size_t size() const = 0;
+};
+
 struct RawBackend {
   // returns false on out-of-memory (never throws for OOM)
   std::function<bool(void** p, size_t nbytes)> mallocDevice;
+  // null when the device has no virtual memory management: expandable_segments:True is then ignored, as the
+  // reference ignores it without vendorCreateExpandableSegment (DIPUCachingDeviceAllocator.cpp:481-487)
+  std::function<ExpandableRange*(StreamHandle stream, size_t segmentSize)> createExpandable;
   std::function<void(void* p)> freeDevice;
   std::function<EventHandle()> createEvent;
   std::function<void(EventHandle)> destroyEvent;
@@ -58,6 +72,7 @@ struct AllocatorConfig {
   double gcThreshold = 0.0;              // fraction of device capacity; 0 = off
   size_t roundupPower2Divisions = 0;     // 0 = plain 512 B rounding
   bool hugeSegments = true;
+  bool expandableSegments = false;       // expandable_segments:True
   size_t deviceCapacity = 0;             // for gcThreshold; 0 = unknown
   // Parses DIPU's "max_split_size_mb:N,garbage_collection_threshold:F,roundup_power2_divisions:N"
   // (dipu/.../DIPUCachingDeviceAllocator.cpp:454-496). Unknown keys raise std::invalid_argument.
@@ -83,8 +98,12 @@ struct Block;
 struct BlockLess {
   bool operator()(const Block* a, const Block* b) const;
 };
+struct BlockAddressLess {
+  bool operator()(const Block* a, const Block* b) const;
+};
 struct BlockPool {
   std::set<Block*, BlockLess> blocks;
+  std::set<Block*, BlockAddressLess> unmapped;  // address ranges of expandable segments with nothing behind them
   bool isSmall;
   explicit BlockPool(bool small) : isSmall(small) {}
 };
@@ -101,6 +120,8 @@ struct Block {
   Block* next = nullptr;
   int eventCount = 0;
   int gcCount = 0;
+  bool mapped = true;                  // false: part of an expandable segment's range with no memory behind it
+  ExpandableRange* expandable = nullptr;
   bool isSplit() const { return prev != nullptr || next != nullptr; }
 };
 
@@ -150,7 +171,12 @@ class DeviceCachingAllocator : public DeviceAllocator {
 
  private:
   Block* getFreeBlock(BlockPool& pool, size_t size, StreamHandle stream);
-  bool allocBlock(BlockPool& pool, size_t allocSize, StreamHandle stream, Block** out);
+  bool allocBlock(BlockPool& pool, size_t size, size_t allocSize, StreamHandle stream, Block** out);
+  Block* findExpandableBlock(BlockPool& pool, size_t size, StreamHandle stream);
+  bool mapBlock(Block* toMap, size_t size);
+  Block* tryAllocateExpandableBlock(BlockPool& pool, size_t size, StreamHandle stream);
+  void unmapBlock(Block* block);
+  void releaseExpandable(Block* block);
   bool releaseAvailableCachedBlocks(BlockPool& pool, size_t size, StreamHandle stream);
   bool releaseCachedBlocks();
   void releaseBlocks(BlockPool& pool);
@@ -171,6 +197,7 @@ class DeviceCachingAllocator : public DeviceAllocator {
   std::unordered_map<void*, Block*> active_;
   std::unordered_map<StreamHandle, std::vector<std::pair<EventHandle, Block*>>> events_;
   std::vector<EventHandle> eventPool_;
+  std::vector<ExpandableRange*> expandables_;
   size_t totalReserved_ = 0;
 };
 

@@ -1,4 +1,5 @@
 #include "runtime_core.h"
+#include "expandable_segment.h"
 
 #include <cstdlib>
 #include <cstring>
@@ -31,8 +32,29 @@ struct DeviceSwitch {  // sets the device for the scope and restores the previou
 };
 }  // namespace
 
+namespace {
+// The caching allocator's view of a HipExpandableSegment.
+struct HipExpandableRange final : ExpandableRange {
+  HipExpandableSegment seg;
+  HipExpandableRange(int device, deviceStream_t stream, size_t segmentSize) : seg(device, stream, segmentSize) {}
+  void map(char* ptr, size_t size, char** mappedPtr, size_t* mappedSize) override {
+    const SegmentRange r = seg.map({ptr, size});
+    *mappedPtr = r.ptr, *mappedSize = r.size;
+  }
+  void unmap(char* ptr, size_t size, char** unmappedPtr, size_t* unmappedSize) override {
+    const SegmentRange r = seg.unmap({ptr, size});
+    *unmappedPtr = r.ptr, *unmappedSize = r.size;
+  }
+  char* ptr() const override { return seg.ptr(); }
+  size_t size() const override { return seg.size(); }
+};
+}  // namespace
+
 RawBackend RawBackend::hip() {
   RawBackend b;
+  b.createExpandable = [](StreamHandle s, size_t segmentSize) -> ExpandableRange* {
+    return new HipExpandableRange(static_cast<int>(devapis::current_device()), static_cast<deviceStream_t>(s), segmentSize);
+  };
   b.mallocDevice = [](void** p, size_t n) { return devapis::mallocDevice(p, n, false) == devapis::OpStatus::SUCCESS; };
   b.freeDevice = [](void* p) { devapis::freeDevice(p); };
   b.createEvent = []() {

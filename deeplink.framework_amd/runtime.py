@@ -348,3 +348,32 @@ def recordEnd(rec):
     f.argtypes = [ctypes.POINTER(c_void_p)]
     if f(byref(rec)) != 0:
         raise RuntimeError_("diopiRecordEnd failed")
+
+
+class ExpandableSegment:
+    """An address range backed segment by segment through HIP virtual memory management (the vendor half of DIPU's
+    expandable segments, runtime/core/allocator/ExpandableSegment.h:114-136). Offsets are relative to `base`."""
+
+    def __init__(self, segment_bytes, device=0, stream=0):
+        self.h = c_void_p()
+        _check(_rt().dipuAmdExpandableSegmentCreate(byref(self.h), c_int(device), c_void_p(stream), c_uint64(segment_bytes)))
+
+    def close(self):
+        if self.h:
+            _check(_rt().dipuAmdExpandableSegmentDestroy(self.h))
+            self.h = None
+
+    def info(self):
+        base, res, mapped = c_void_p(), c_uint64(), c_uint64()
+        _check(_rt().dipuAmdExpandableSegmentInfo(self.h, byref(base), byref(res), byref(mapped)))
+        return base.value, res.value, mapped.value
+
+    def map(self, offset, nbytes):
+        o, n = c_uint64(), c_uint64()
+        _check(_rt().dipuAmdExpandableSegmentMap(self.h, c_uint64(offset), c_uint64(nbytes), byref(o), byref(n)))
+        return o.value, n.value
+
+    def unmap(self, offset, nbytes):
+        o, n = c_uint64(), c_uint64()
+        _check(_rt().dipuAmdExpandableSegmentUnmap(self.h, c_uint64(offset), c_uint64(nbytes), byref(o), byref(n)))
+        return o.value, n.value

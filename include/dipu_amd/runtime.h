@@ -100,6 +100,20 @@ DIPU_AMD_API int dipuAmdCachingHostFree(void* p);
 DIPU_AMD_API int dipuAmdCachingHostRecordStream(void* p, void* stream);
 DIPU_AMD_API int dipuAmdCachingHostEmptyCache(void);
 
+/* Expandable segment over HIP virtual memory management: the vendor half of DIPU's expandable segments
+ * (runtime/core/allocator/ExpandableSegment.h:114-136; CUDA form vendor/cuda/CUDAExpandableSegment.cpp:15-176).
+ * A reserved address range of 9/8 of the device's memory whose segments of segment_bytes are backed on map and given
+ * back on unmap; offsets are relative to the range's base. map starts at a segment boundary and maps every segment
+ * the range touches (mapped_bytes == 0: out of memory); unmap releases the segments entirely inside the range after
+ * synchronising the stream. */
+DIPU_AMD_API int dipuAmdExpandableSegmentCreate(void** handle, int device, void* stream, uint64_t segment_bytes);
+DIPU_AMD_API int dipuAmdExpandableSegmentDestroy(void* handle);
+DIPU_AMD_API int dipuAmdExpandableSegmentInfo(void* handle, void** base, uint64_t* reserved_bytes, uint64_t* mapped_bytes);
+DIPU_AMD_API int dipuAmdExpandableSegmentMap(void* handle, uint64_t offset, uint64_t nbytes, uint64_t* mapped_offset,
+                                             uint64_t* mapped_bytes);
+DIPU_AMD_API int dipuAmdExpandableSegmentUnmap(void* handle, uint64_t offset, uint64_t nbytes, uint64_t* unmapped_offset,
+                                               uint64_t* unmapped_bytes);
+
 /* A generator object for the diopiGenerator* callbacks of diopirt.h: what vendorMakeGenerator returns in DIPU
  * (runtime/core/DIPUGeneratorImpl.h:62; state layout of vendor/cuda/CudaGeneratorImpl.cpp:17-76), without libtorch. */
 struct diopiGenerator;

@@ -380,3 +380,137 @@ def test_bs_reuse_waits_for_events_and_oom_empties_the_cache(pkg):
         a.free(q), a.free(r)
     finally:
         a.close()
+
+
+# ---- expandable_segments:True (DIPUCachingDeviceAllocator.cpp:1086-1215, 1633-1705) ----
+# The stand-in range is 1 GiB of address space per (stream, pool); its 2 MiB / 20 MiB segments count against the
+# capacity only while mapped.
+ES = "expandable_segments:True"
+
+
+def test_expandable_conf_is_parsed(pkg, sim):
+    sim(conf="expandable_segments:False")
+    with pytest.raises(pkg.runtime.RuntimeError_, match="expandable_segments"):
+        sim(conf="expandable_segments:yes")
+
+
+def test_expandable_range_grows_at_its_end_in_whole_segments(sim):
+    a = sim(conf=ES)
+    p1 = a.malloc(30 * MiB)                     # two 20 MiB segments mapped
+    st = a.stats()
+    assert st["reserved_bytes"] == 40 * MiB and st["segments"] == 1
+    assert a.backend_usage()[0] == 40 * MiB
+    p2 = a.malloc(5 * MiB)                      # fits the mapped remainder
+    assert p2 == p1 + 30 * MiB and a.stats()["reserved_bytes"] == 40 * MiB
+    p3 = a.malloc(25 * MiB)                     # 5 MiB free + one more segment, contiguous with the rest
+    assert p3 == p2 + 5 * MiB
+    st = a.stats()
+    assert st["reserved_bytes"] == 60 * MiB and st["segments"] == 1
+    assert st["allocated_bytes"] == 60 * MiB
+
+
+def test_expandable_assembles_a_large_block_from_freed_small_ones(sim):
+    # the point of the mode: ten 18 MiB blocks freed leave one free run that serves 170 MiB without new memory;
+    # fixed segments would hold ten separate 20 MiB segments and need 170 MiB more
+    a = sim(capacity=200 * MiB, conf=ES)
+    ps = [a.malloc(18 * MiB) for _ in range(10)]
+    assert ps == [ps[0] + i * 18 * MiB for i in range(10)]
+    assert a.stats()["reserved_bytes"] == 180 * MiB
+    for p in ps:
+        a.free(p)
+    big = a.malloc(170 * MiB)
+    assert big == ps[0]
+    st = a.stats()
+    assert st["reserved_bytes"] == 180 * MiB and st["num_alloc_retries"] == 0
+
+    b = sim(capacity=200 * MiB)                 # same trace without the mode: only after releasing the cache
+    qs = [b.malloc(18 * MiB) for _ in range(10)]
+    for q in qs:
+        b.free(q)
+    b.malloc(170 * MiB)
+    assert b.stats()["num_alloc_retries"] >= 1
+
+
+def test_expandable_empty_cache_unmaps_whole_free_segments_only(sim):
+    a = sim(conf=ES)
+    p1 = a.malloc(30 * MiB)
+    p2 = a.malloc(30 * MiB)
+    p3 = a.malloc(30 * MiB)                     # 90 MiB -> five segments mapped
+    assert a.stats()["reserved_bytes"] == 100 * MiB
+    a.free(p2)                                  # [30, 60) free: only segment [40, 60) lies inside it
+    a.empty_cache()
+    st = a.stats()
+    assert st["reserved_bytes"] == 80 * MiB and a.backend_usage()[0] == 80 * MiB
+    assert st["segments"] == 1
+    q = a.malloc(30 * MiB)                      # maps the hole again, same address
+    assert q == p2 and a.stats()["reserved_bytes"] == 100 * MiB
+    for p in (p1, p3, q):
+        a.free(p)
+    a.empty_cache()                             # nothing in use: the range itself goes
+    st = a.stats()
+    assert st["reserved_bytes"] == 0 and st["segments"] == 0 and a.backend_usage()[0] == 0
+    assert a.malloc(30 * MiB) != 0              # and a new one is made on demand
+    assert a.stats()["segments"] == 1
+
+
+def test_expandable_small_pool_streams_and_events(sim):
+    a = sim(conf=ES)
+    s1, s2 = 0x1000, 0x2000
+    p = a.malloc(4096, s1)                      # small pool: 2 MiB segments
+    assert a.stats()["reserved_bytes"] == 2 * MiB
+    q = a.malloc(4096, s2)                      # another stream gets a range of its own
+    assert abs(q - p) >= (1 << 30) and a.stats()["segments"] == 2
+    a.record_stream(p, s2)
+    a.free(p)
+    r = a.malloc(MiB, s1)                       # p still waits for s2's event: served behind it
+    assert r == p + 4096
+    a.complete_events(s2)
+    a.free(r)
+    assert a.malloc(MiB, s1) == p               # merged back once the event is done
+    assert a.malloc(MiB, s1) == p + MiB         # the first segment is full now
+    assert a.malloc(MiB, s1) == p + 2 * MiB     # one more small segment, contiguous
+    assert a.stats()["reserved_bytes"] == 4 * MiB + 2 * MiB and a.stats()["segments"] == 2
+
+
+def test_expandable_out_of_memory_ladder(pkg, sim):
+    a = sim(capacity=100 * MiB, conf=ES)
+    s1, s2 = 0x1000, 0x2000
+    p = a.malloc(60 * MiB, s1)
+    a.free(p)                                   # 60 MiB cached on s1's range
+    q = a.malloc(50 * MiB, s2)                  # s2's range needs 60 MiB: s1's cache has to be unmapped first
+    st = a.stats()
+    assert st["num_alloc_retries"] >= 1 and st["num_ooms"] == 0
+    assert st["reserved_bytes"] == 60 * MiB
+    with pytest.raises(pkg.runtime.RuntimeError_, match="out of memory"):
+        a.malloc(60 * MiB, s2)
+    a.free(q)
+    assert a.malloc(90 * MiB, s2) == q
+
+
+def test_expandable_random_stress_keeps_the_books(sim):
+    rng = random.Random(7)
+    a = sim(capacity=900 * MiB, conf=ES)
+    live = {}
+    for step in range(3000):
+        if live and (rng.random() < 0.45 or len(live) > 60):
+            p = rng.choice(list(live))
+            a.free(p)
+            del live[p]
+        else:
+            n = rng.choice([rng.randint(1, 4096), rng.randint(4096, MiB), rng.randint(MiB, 12 * MiB)])
+            p = a.malloc(n)
+            assert p not in live
+            live[p] = n
+        if step % 500 == 499:
+            a.empty_cache()
+        if step % 100 == 0:
+            spans = sorted((p, p + n) for p, n in live.items())
+            assert all(x[1] <= y[0] for x, y in zip(spans, spans[1:]))
+            st = a.stats()
+            want = sum(round512(n) for n in live.values())  # a large block keeps a remainder of up to 1 MiB
+            assert want <= st["allocated_bytes"] <= want + len(live) * MiB
+            assert st["reserved_bytes"] == a.backend_usage()[0] >= st["allocated_bytes"]
+    for p in list(live):
+        a.free(p)
+    a.empty_cache()
+    assert a.stats()["reserved_bytes"] == 0 and a.backend_usage()[0] == 0

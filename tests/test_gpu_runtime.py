@@ -188,3 +188,92 @@ print("allocator ok")
     env = dict(os.environ, DIPU_DEVICE_MEMCACHING_ALGORITHM=algorithm)
     out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300, env=env)
     assert out.returncode == 0 and "allocator ok" in out.stdout, out.stderr[-2000:]
+
+
+def test_torch_algorithm_with_expandable_segments_on_device_in_a_fresh_process(pkg):
+    """DIPU_TORCH_ALLOCATOR_CONF=expandable_segments:True (DIPUCachingDeviceAllocator.cpp:1086-1215) over HIP virtual
+    memory: blocks are contiguous in one growing range, a large request is assembled from freed small ones without
+    new memory, contents survive, empty_cache gives everything back, an op's workspace is served by it."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = r"""
+import ctypes, sys
+sys.path.insert(0, %r)
+import torch
+from __graft_entry__ import load_package
+pkg = load_package(); rt = pkg.runtime; ops = pkg.ops
+MiB = 1 << 20
+ps = [rt.cachingMalloc(18 * MiB) for _ in range(10)]
+assert ps == [ps[0] + i * 18 * MiB for i in range(10)], ps
+st = rt.cachingStats()
+assert st["reserved_bytes"] == 180 * MiB and st["segments"] == 1 and st["allocated_bytes"] == 180 * MiB, st
+for i, p in enumerate(ps): rt.memSetAsync(0, p, 0x30 + i, 18 * MiB)
+rt.syncDevice()
+for p in ps: rt.cachingFree(p)
+big = rt.cachingMalloc(170 * MiB)
+assert big == ps[0]
+st = rt.cachingStats()
+assert st["reserved_bytes"] == 180 * MiB and st["num_device_malloc"] == 0, st
+out = (ctypes.c_ubyte * 4)()
+for i in (0, 3, 9):
+    rt.memCopyD2H(4, ctypes.addressof(out), big + i * 18 * MiB + 12345)
+    assert bytes(out) == bytes([0x30 + i]) * 4, (i, bytes(out))
+small = rt.cachingMalloc(1000)
+rt.cachingFree(big)
+rt.cachingEmptyCache()
+st = rt.cachingStats()
+assert st["reserved_bytes"] == 2 * MiB and st["segments"] == 1, st   # only the small pool's range is left
+again = rt.cachingMalloc(170 * MiB)
+rt.memSetAsync(0, again, 0x11, 170 * MiB); rt.syncDevice()
+rt.cachingFree(again); rt.cachingFree(small)
+dev = torch.device("cuda:0")
+a = torch.randn(300, 200, device=dev).bfloat16(); b = torch.randn(200, 136, device=dev).bfloat16()
+got = ops.mm(a, b).float().cpu(); ref = a.float().cpu() @ b.float().cpu()
+assert float((got - ref).abs().max()) < 0.5
+rt.syncDevice(); rt.cachingEmptyCache()
+st = rt.cachingStats()
+assert st["reserved_bytes"] == 0 and st["segments"] == 0, st
+print("allocator ok")
+""" % root
+    env = dict(os.environ, DIPU_TORCH_ALLOCATOR_CONF="expandable_segments:True")
+    env.pop("DIPU_DEVICE_MEMCACHING_ALGORITHM", None)
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300, env=env)
+    assert out.returncode == 0 and "allocator ok" in out.stdout, out.stderr[-2000:]
+
+
+def test_expandable_segment_over_hip_virtual_memory(rt):
+    """The vendor half of expandable segments (runtime/core/allocator/ExpandableSegment.h:114-136): map backs whole
+    segments, the memory is real and keeps its contents while neighbours come and go, unmap releases only the
+    segments entirely inside the range, misuse raises."""
+    MiB = 1 << 20
+    seg = rt.ExpandableSegment(2 * MiB)
+    try:
+        base, reserved, mapped = seg.info()
+        assert base and reserved >= rt.getDeviceProperties(0)["totalGlobalMem"] and mapped == 0
+        assert seg.map(0, 5 * MiB) == (0, 6 * MiB)              # three segments cover 5 MiB
+        assert seg.info()[2] == 6 * MiB
+        rt.memSetAsync(0, base, 0x5a, 6 * MiB)
+        rt.syncDevice()
+        out = (ctypes.c_ubyte * 8)()
+        rt.memCopyD2H(8, ctypes.addressof(out), base + 6 * MiB - 8)
+        assert bytes(out) == b"\x5a" * 8
+        assert seg.unmap(1 * MiB, 4 * MiB) == (2 * MiB, 2 * MiB)   # only the middle segment lies inside [1, 5) MiB
+        assert seg.info()[2] == 4 * MiB
+        assert seg.unmap(3 * MiB, 512) == (3 * MiB, 0)              # nothing entirely inside
+        assert seg.map(2 * MiB, 2 * MiB) == (2 * MiB, 2 * MiB)      # the hole is filled again
+        rt.memCopyD2H(8, ctypes.addressof(out), base + 8)           # the first segment kept its contents
+        assert bytes(out) == b"\x5a" * 8
+        assert seg.map(6 * MiB, 1) == (6 * MiB, 2 * MiB)            # grows at the end
+        with pytest.raises(RuntimeError, match="already mapped"):
+            seg.map(0, 2 * MiB)
+        with pytest.raises(RuntimeError, match="segment boundary"):
+            seg.map(8 * MiB + 4096, 2 * MiB)
+        assert seg.unmap(0, 8 * MiB) == (0, 8 * MiB) and seg.info()[2] == 0
+    finally:
+        seg.close()
+    with pytest.raises(RuntimeError, match="granularity"):
+        rt.ExpandableSegment(3000)
