@@ -54,8 +54,9 @@ class Prepared:
     """A DIOPI call with its arguments marshalled once: per launch it costs two C calls
     (the op and the release of the context's workspace), so short kernels are not host-bound."""
 
-    def __init__(self, pkg, name, *args):
+    def __init__(self, pkg, name, *args, hold=False):
         d = pkg.diopi
+        self.hold = hold  # keep the workspace until close(): for calls recorded into a HIP graph
         self.keep = []
         self.cargs = []
         for a in args:
@@ -74,12 +75,17 @@ class Prepared:
         self.name = name
         self.reset = pkg._native.runtime().dipuAmdContextReset
         self.err = d.last_error
+        self.rt_err = d.rt_error
 
     def __call__(self):
         rc = self.fn(self.ctx.ptr, *self.cargs)
         if rc != 0:
-            raise RuntimeError(f"{self.name} failed: {self.err()}")
-        self.reset(self.ctx.ptr)
+            raise RuntimeError(f"{self.name} failed: {self.err()} {self.rt_err()}")
+        if not self.hold:
+            self.reset(self.ctx.ptr)
+
+    def close(self):
+        self.ctx.close()
 
 
 def layer_plan(pkg, torch, dev, x, p, cfg):
@@ -145,6 +151,79 @@ def time_ops(rt, stream, calls, iters, warm):
         rt.destroyEvent(e0)
         rt.destroyEvent(e1)
     return out
+
+
+def decode_layer_step(pkg, torch, dev, rt, stream, g):
+    """One decode step of a 7B-shaped layer at batch 64 (every op launch-bound except the attention): the same
+    prepared calls launched one by one, and recorded once into a HIP graph and replayed."""
+    d = pkg.diopi
+    bf = torch.bfloat16
+    B, hidden, heads, hd, ffn = 64, 4096, 32, 128, 11008
+    gen = torch.Generator(device=dev).manual_seed(3)
+    rnd = lambda *shape, scale=0.02: (torch.randn(*shape, generator=gen, device=dev) * scale).to(bf)
+    x, n1, n2 = rnd(B, hidden, scale=1.0), rnd(hidden) + 1, rnd(hidden) + 1
+    wqkv = torch.cat([pkg.ops.interleave_rotary_rows(rnd(hidden, hidden), hd), pkg.ops.interleave_rotary_rows(rnd(hidden, hidden), hd),
+                      rnd(hidden, hidden)], dim=0)
+    wo, wgu, wdown = rnd(hidden, hidden), rnd(2 * ffn, hidden), rnd(hidden, ffn)
+    cos, sin = pkg.workloads.rotary_tables(hd, int(g["max_input_len"]), dtype=torch.float32)
+    at = (g["b_seq_len"].long() - 1).cpu()
+    cos, sin = cos[at].to(bf).to(dev), sin[at].to(bf).to(dev)
+    new = lambda *shape: torch.empty(*shape, dtype=bf, device=dev)
+    h1, qkv, att, x1, h2, act, out = new(B, hidden), new(B, 3 * hidden), new(B, heads, hd), new(B, hidden), new(B, hidden), new(B, ffn), new(B, hidden)
+    q, k, v = (qkv[:, i * hidden:(i + 1) * hidden].view(B, heads, hd) for i in range(3))
+    one = d.scalar(1)
+
+    def calls(hold):
+        P = lambda name, *a: Prepared(pkg, name, *a, hold=hold)
+        return [P("diopiRMSNorm", h1, None, x, d.size([hidden]), n1, None, 1e-5),
+                P("diopiLinearRotary", qkv, h1, wqkv, None, cos, sin, 2 * hidden, hd, False, True),
+                P("diopiDestIndexCopyKV", g["k_pool"], k, g["dest_loc"]),
+                P("diopiDestIndexCopyKV", g["v_pool"], v, g["dest_loc"]),
+                P("diopiTokenDecodeAttentionInference", att, q, g["k_pool"], g["v_pool"], g["b_loc"], g["b_start_loc"],
+                  g["b_seq_len"], int(g["max_input_len"])),
+                P("diopiAddmm", x1, x, att.view(B, hidden), wo.t(), one, one),
+                P("diopiRMSNorm", h2, None, x1, d.size([hidden]), n2, None, 1e-5),
+                P("diopiLinearSiluMul", act, h2, wgu),
+                P("diopiAddmm", out, x1, act, wdown.t(), one, one)]
+
+    eager = calls(False)
+
+    def step():
+        for c in eager:
+            c()
+    (t_eager,) = time_ops(rt, stream, [step], 30, 6)
+    want = out.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        # Recording may not allocate device memory, so the capture stream's workspace cache is filled first: passes
+        # that hold all their workspace, like the recording will, until one finds everything in the cache (the pass
+        # after it starts from the same cache and makes the same choices).
+        for _ in range(6):
+            before = pkg.runtime.cachingStats()["num_device_malloc"]
+            warm = calls(True)
+            for c in warm:
+                c()
+            side.synchronize()
+            for c in warm:
+                c.close()
+            if pkg.runtime.cachingStats()["num_device_malloc"] == before:
+                break
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        recorded = calls(True)
+        for c in recorded:
+            c()
+    out.zero_()
+    (t_graph,) = time_ops(rt, stream, [graph.replay], 30, 6)
+    torch.cuda.synchronize()
+    same = bool(torch.equal(out, want))
+    del graph
+    for c in recorded:
+        c.close()
+    return {"op": "decode layer step, 9 DIOPI calls", "workload": "7B-shaped layer, batch 64, paged KV as above",
+            "us_eager_launches": round(t_eager, 2), "us_hip_graph_replay": round(t_graph, 2),
+            "tokens_per_s_graph": round(B / (t_graph * 1e-6), 1), "replay_equals_eager": same}
 
 
 def op_microbench(pkg, torch, dev, rt, stream):
@@ -223,6 +302,7 @@ def op_microbench(pkg, torch, dev, rt, stream):
                 "us_cold": round(t_at, 2), "GBs_cold": round(attn_bytes / t_at / 1e3, 1), "frac_cold": round(attn_bytes / t_at / 1e3 / HBM_PEAK_GBS, 3)})
     res.append({"op": "decode step (scatter + attention)", "workload": "batch 64", "us_cold": round(t_step, 2),
                 "tokens_per_s": round(64 / (t_step * 1e-6), 1)})
+    res.append(decode_layer_step(pkg, torch, dev, rt, stream, g))
     del g, pd
     # int8 weight-only linear: weights rotate through 8 copies (360 MB) for the cold figure
     for m in (1, 4, 16):

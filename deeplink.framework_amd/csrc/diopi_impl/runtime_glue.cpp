@@ -133,7 +133,8 @@ diopiError_t getStream(diopiContextHandle_t ctx, hipStream_t* stream) {
 diopiError_t requireWorkspace(diopiContextHandle_t ctx, int64_t nbytes, void** ptr) {
   diopiTensorHandle_t th = nullptr;
   if (nbytes < 1) nbytes = 1;
-  AMD_TRY(diopiRequireBuffer(ctx, &th, nbytes, diopi_device));
+  AMD_CHECK(diopiRequireBuffer(ctx, &th, nbytes, diopi_device) == diopiSuccess,
+            "diopiRequireBuffer failed for %ld bytes of workspace (the runtime holds the cause)", (long)nbytes);
   AMD_CHECK(th != nullptr, "diopiRequireBuffer returned a null handle for %ld bytes", (long)nbytes);
   AMD_TRY(diopiGetTensorData(th, ptr));
   AMD_CHECK(*ptr != nullptr, "diopiRequireBuffer returned null data for %ld bytes", (long)nbytes);
@@ -144,7 +145,8 @@ diopiError_t requireTensor(diopiContextHandle_t ctx, const int64_t* shape, int n
                            diopiTensorHandle_t* th, TensorView* view) {
   diopiSize_t size{shape, ndim};
   *th = nullptr;
-  AMD_TRY(diopiRequireTensor(ctx, th, &size, nullptr, dtype, diopi_device));
+  AMD_CHECK(diopiRequireTensor(ctx, th, &size, nullptr, dtype, diopi_device) == diopiSuccess,
+            "diopiRequireTensor failed for a workspace tensor (the runtime holds the cause)");
   AMD_CHECK(*th != nullptr, "diopiRequireTensor returned a null handle");
   return getView(*th, view, "workspace tensor");
 }

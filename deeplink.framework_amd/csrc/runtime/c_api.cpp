@@ -18,6 +18,7 @@ void* contextCreate(deviceStream_t s);
 void contextDestroy(void* c);
 void contextReset(void* c);
 void contextWorkspace(void* c, uint64_t* tensors, uint64_t* bytes);
+void noteError(const char* what);
 }  // namespace amdrt
 }  // namespace dipu
 
@@ -165,6 +166,10 @@ RawBackend makeSimBackend(SimBackend* sb) {
 extern "C" {
 
 const char* dipuAmdGetLastError(void) { return g_err.c_str(); }
+}
+// what a diopirt callback could not report through its return code (it has no message channel of its own)
+void dipu::amdrt::noteError(const char* what) { g_err = what; }
+extern "C" {
 
 int dipuAmdInitializeVendor(void) { return guarded([] { devapis::initializeVendor(); }); }
 int dipuAmdFinalizeVendor(void) {

@@ -13,6 +13,12 @@
 
 #include "runtime_core.h"
 
+namespace dipu {
+namespace amdrt {
+void noteError(const char* what);  // c_api.cpp: text for dipuAmdGetLastError
+}  // namespace amdrt
+}  // namespace dipu
+
 using dipu::amdrt::Runtime;
 
 struct diopiTensor : dipuAmdTensor {};
@@ -176,7 +182,11 @@ DIOPI_RT_API diopiError_t diopiRequireTensor(diopiContextHandle_t ctx, diopiTens
       w.desc.device_index = -1;
       w.allocation = span > 0 ? ::malloc(static_cast<size_t>(span * item)) : nullptr;
     }
+  } catch (const std::exception& e) {
+    dipu::amdrt::noteError(e.what());
+    return diopiErrorOccurred;
   } catch (...) {
+    dipu::amdrt::noteError("diopiRequireTensor: unknown C++ exception");
     return diopiErrorOccurred;
   }
   w.desc.data = w.allocation;

@@ -305,4 +305,5 @@ def call(name, ctx, *args):
     which is what the generated wrappers' TORCH_CHECK does (autogen_diopi_wrapper.py:1001)."""
     ret = fn(name)(ctx.ptr, *args)
     if ret != DIOPI_SUCCESS:
-        raise DiopiError(f"{name} failed, ret = {ret}: {last_error()}")
+        why = rt_error()
+        raise DiopiError(f"{name} failed, ret = {ret}: {last_error()}" + (f" [runtime: {why}]" if why else ""))

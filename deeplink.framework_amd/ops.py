@@ -40,7 +40,37 @@ def _binary_out(a, b, out):
     return torch.empty(shape, dtype=dtype, device=a.device)
 
 
+_scope = None
+
+
+class WorkspaceScope:
+    """One diopiContext shared by every op called inside `with scope:`; the workspace those ops request stays
+    allocated until close(), as a context keeps its arrays until it is destroyed (diopirt_impl.h:19-26). For work
+    recorded into a HIP graph: the graph's kernels keep the workspace addresses they were recorded with, so the scope
+    is created on the capturing stream and closed only after the last replay. Recording may not allocate device
+    memory: run the same calls under a scope on that stream beforehand, and again until a pass leaves the
+    allocator's num_device_malloc unchanged; the recording then finds every block in the cache."""
+
+    def __init__(self, stream=None):
+        self.ctx = Context(stream)
+
+    def __enter__(self):
+        global _scope
+        self._outer, _scope = _scope, self
+        return self
+
+    def __exit__(self, *exc):
+        global _scope
+        _scope = self._outer
+
+    def close(self):
+        self.ctx.close()
+
+
 def _call(name, *args, stream=None):
+    if _scope is not None and stream is None:
+        call(name, _scope.ctx, *args)
+        return
     with Context(stream) as ctx:
         call(name, ctx, *args)
 
