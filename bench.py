@@ -323,7 +323,7 @@ def op_microbench(pkg, torch, dev, rt, stream):
                     "frac_hot": round(nbytes / hot / 1e3 / HBM_PEAK_GBS, 3), "frac_cold": round(nbytes / cold / 1e3 / HBM_PEAK_GBS, 3)})
         del W
     # bf16 linear at decode shapes (a handful of rows against a [11008, 4096] weight): the weight stream is the traffic
-    for m in (1, 16):
+    for m in (1, 16, 64):
         gq = torch.Generator().manual_seed(7)
         x = torch.randn(m, 4096, generator=gq).bfloat16().to(dev)
         W = [(torch.randn(11008, 4096, generator=gq) * 0.02).bfloat16().to(dev) for _ in range(4)]

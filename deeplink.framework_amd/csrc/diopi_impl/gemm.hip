@@ -863,6 +863,104 @@ __global__ __launch_bounds__(NTW * KS * 64) void gemmSkinnyKernel(SkinnyArgs a) 
   }
 }
 
+// 33 to 64 rows against a wide weight (at least 512 column tiles): no K split over the grid, so no partial products
+// and no reduction pass. One workgroup owns NTW column tiles for the whole of K and walks it in chunks of 512: the
+// four waves of a tile each take one 128-column step of the chunk. The activations of chunk c + 1 travel through
+// registers into the second LDS buffer while chunk c is multiplied, the weights are fetched two chunks ahead, and
+// every load is an ordinary one at a clamped (always valid) address, so the compiler counts outstanding loads
+// exactly and nothing in the loop waits for more than it needs.
+template <typename T, int NTW>
+__global__ __launch_bounds__(NTW * 4 * 64) void gemmSkinnyWideKernel(SkinnyArgs a) {
+  using Frag = typename MfmaOp<T>::Frag;
+  constexpr int KS = 4, G = 4, THREADS = NTW * KS * 64, CHUNK = KS * kSkinnyStep, LDX = CHUNK + kSkinnyPad;
+  constexpr int PIECES = 16 * G * (CHUNK / 8), PER = (PIECES + THREADS - 1) / THREADS;  // 16-byte pieces of a chunk
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  T* sx = reinterpret_cast<T*>(smem);  // two buffers of 64 rows x LDX
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = wave / KS, ks = wave % KS;
+  const int r16 = lane & 15, kgrp = lane >> 4;
+  const int n0 = (blockIdx.x * NTW + tile) * 16;
+  const T* wbase = reinterpret_cast<const T*>(a.B) + (int64_t)min(n0 + r16, a.N - 1) * a.ldb + kgrp * 32;
+  const T* xbase = reinterpret_cast<const T*>(a.A);
+  const int nChunks = (a.K + CHUNK - 1) / CHUNK;
+  f32x4 acc[G];
+#pragma unroll
+  for (int gi = 0; gi < G; ++gi) acc[gi] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  u32x4 xa[PER];
+  auto loadW = [&](int c, Frag (&w)[4]) {  // a step past the end of K reads the last step instead and is not used
+    const T* src = wbase + min(min(c, nChunks - 1) * CHUNK + ks * kSkinnyStep, a.K - kSkinnyStep);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) w[t] = *reinterpret_cast<const Frag*>(src + 8 * t);
+  };
+  auto loadX = [&](int c) {  // rows past M and columns past K repeat valid ones; nothing multiplies them
+    const int kc = min(c, nChunks - 1) * CHUNK, len = min(CHUNK, a.K - kc);
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int p = threadIdx.x + i * THREADS, r = min(p >> 6, a.M - 1), q = min((p & 63) * 8, len - 8);
+      xa[i] = *reinterpret_cast<const u32x4*>(xbase + (int64_t)r * a.lda + kc + q);
+    }
+  };
+  auto storeX = [&](int buf) {
+    T* dst = sx + buf * (16 * G * LDX);
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int p = threadIdx.x + i * THREADS;
+      if (PIECES % THREADS == 0 || p < PIECES) *reinterpret_cast<u32x4*>(dst + (p >> 6) * LDX + (p & 63) * 8) = xa[i];
+    }
+  };
+
+  Frag wc[4], w0[4], w1[4];
+  loadW(0, w0);
+  loadW(1, w1);
+  loadX(0);
+  storeX(0);
+  __syncthreads();
+  for (int c = 0; c < nChunks; ++c) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) wc[t] = w0[t], w0[t] = w1[t];
+    loadX(c + 1);
+    loadW(c + 2, w1);
+    if (c * CHUNK + ks * kSkinnyStep < a.K) {  // wave-uniform: this wave's step of the chunk exists
+      const T* xs = sx + (c & 1) * (16 * G * LDX) + ks * kSkinnyStep + kgrp * 32;
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int gi = 0; gi < G; ++gi)
+          acc[gi] = MfmaOp16<T>::run(*reinterpret_cast<const Frag*>(xs + min(gi * 16 + r16, a.M - 1) * LDX + 8 * t), wc[t], acc[gi]);
+    }
+    storeX((c + 1) & 1);  // the buffer chunk c - 1 was read from; every wave left it at the last barrier
+    __syncthreads();
+  }
+  // the four K shares of a tile meet where the activations were
+  float* red = reinterpret_cast<float*>(smem);  // [NTW * KS][G][4][64]
+#pragma unroll
+  for (int gi = 0; gi < G; ++gi)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[((wave * G + gi) * 4 + r) * 64 + lane] = acc[gi][r];
+  __syncthreads();
+  const int col = n0 + r16;
+  if (ks == 0 && col < a.N) {
+    T* out = reinterpret_cast<T*>(a.out);
+    const T* cin = reinterpret_cast<const T*>(a.Cin);
+    const float bv = a.bias ? static_cast<float>(reinterpret_cast<const T*>(a.bias)[col]) : 0.f;
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = gi * 16 + kgrp * 4 + r;
+        if (row < a.M) {
+          float v = 0.f;
+#pragma unroll
+          for (int w2 = 0; w2 < KS; ++w2) v += red[(((tile * KS + w2) * G + gi) * 4 + r) * 64 + lane];
+          v = v * a.alpha + bv;
+          if (cin) v += a.beta * static_cast<float>(cin[(int64_t)row * a.sCm + (int64_t)col * a.sCn]);
+          out[(int64_t)row * a.ldo + col] = static_cast<T>(v);
+        }
+      }
+  }
+}
+
 // -------------------------------------------------------------- transpose ----
 // dst[b, c, r] = src[b, r, c] for 2-byte or 4-byte elements, 64x64 tiles through LDS.
 template <typename U>
@@ -1097,6 +1195,17 @@ static diopiError_t launchSkinny(hipStream_t stream, const SkinnyArgs& a) {
   return diopiSuccess;
 }
 
+template <typename T, int NTW>
+static diopiError_t launchSkinnyWide(hipStream_t stream, const SkinnyArgs& a) {
+  constexpr int CHUNK = 4 * kSkinnyStep;
+  const int lds = std::max(2 * 64 * (CHUNK + kSkinnyPad) * (int)sizeof(T), NTW * 4 * 4 * 4 * 64 * (int)sizeof(float));
+  AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmSkinnyWideKernel<T, NTW>), lds));
+  const int tiles = (a.N + 15) / 16;
+  hipLaunchKernelGGL((gemmSkinnyWideKernel<T, NTW>), dim3((unsigned)((tiles + NTW - 1) / NTW)), dim3(NTW * 4 * 64), lds, stream, a);
+  AMD_LAUNCH_CHECK();
+  return diopiSuccess;
+}
+
 static bool mult8(int64_t v) { return (v & 7) == 0; }
 static bool ptr16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
@@ -1120,6 +1229,16 @@ static diopiError_t launchSkinnyForShape(diopiContextHandle_t ctx, hipStream_t s
   // activations would be 2-4 times the weight bytes on the L2 -> CU path. Wider workgroups (up to 4 tiles) bring
   // that to 1:1, and K is split over grid.y as well, one staged chunk per workgroup, to keep the chip full; the
   // slices meet in fp32 workspace and the split-K reduction pass applies the epilogue.
+  if (a.M > 32 && tiles >= 3 * cus && a.K >= 2048) {
+    // Wide weights and a long K: whole-K workgroups with double-buffered activations, no partial products. Measured
+    // at 64 rows, K = 4096, against the K-split form below: 24.8 against 34.6 us at N = 12288, 30.9 against 44.4 at
+    // 16384, 57 against 61 at 22016 (66.6 against 110 at N = 12288, K = 11008); slower at N = 8192 (26.3 against 25.2)
+    // and at K = 640 (10.1 against 8.3). One workgroup per CU at a time, each paying for its tiles' weights and once
+    // for the activations (about one and a half tiles' worth): four tiles per workgroup, or three when that saves
+    // rounds (768 tiles on 256 CUs: one round of three tiles instead of one of four).
+    const int cost4 = ((tiles + 3) / 4 + cus - 1) / cus * (2 * 4 + 3), cost3 = ((tiles + 2) / 3 + cus - 1) / cus * (2 * 3 + 3);
+    return cost3 < cost4 ? launchSkinnyWide<T, 3>(stream, a) : launchSkinnyWide<T, 4>(stream, a);
+  }
   const int groups = a.M <= 32 ? 2 : 4, chunk = kSkinnyRowsK / (16 * groups);
   const bool canSplit = a.N % 8 == 0 && mult8(p.sOm) && ptr16(p.out) && (!p.bias || ptr16(p.bias)) &&
                         (!p.Cin || (p.sCn == 1 && mult8(p.sCm) && ptr16(p.Cin)));
@@ -1176,10 +1295,10 @@ diopiError_t runGemm(diopiContextHandle_t ctx, hipStream_t stream, GemmProblem p
       AMD_TRY(launchTranspose<uint16_t>(stream, ws, p.B, nb, p.K, p.N, p.sBk, p.sBn, sbb));
       p.B = ws, p.sBk = 1, p.sBn = p.K, p.sBb = (sbb == 0) ? 0 : p.N * p.K;
     }
-    // up to 32 rows always; up to 64 while N is moderate (measured at 64 rows, K = 4096, kernel + reduction
-    // pass: 16 us against 50 us for the split-K tiled kernel at N = 4096, 36 against 52 at N = 12288, 63 against 51
-    // at N = 22016)
-    if (p.batch == 1 && (p.M <= 32 || (p.M <= kSkinnyMaxM && p.N <= 16384)) && p.K % kSkinnyStep == 0 && p.N >= 16 &&
+    // up to 32 rows always; up to 64 while N is moderate or K is long enough for the whole-K form (measured at 64
+    // rows, K = 4096: K-split form + reduction pass 16 us against 50 us for the split-K tiled kernel at N = 4096, 36
+    // against 52 at N = 12288, 63 against 51 at N = 22016, where the whole-K form takes 46)
+    if (p.batch == 1 && (p.M <= 32 || (p.M <= kSkinnyMaxM && (p.N <= 16384 || p.K >= 2048))) && p.K % kSkinnyStep == 0 && p.N >= 16 &&
         ((p.M - 1) * p.sAm + p.K) * item < (int64_t(1) << 31))
       return p.dtype == diopi_dtype_bfloat16 ? launchSkinnyForShape<bf16_t>(ctx, stream, p)
                                              : launchSkinnyForShape<half_t>(ctx, stream, p);
