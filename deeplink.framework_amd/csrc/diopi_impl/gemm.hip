@@ -882,19 +882,20 @@ __global__ __launch_bounds__(NTW * 4 * 64) void gemmSkinnyWideKernel(SkinnyArgs 
   const int n0 = (blockIdx.x * NTW + tile) * 16;
   const T* wbase = reinterpret_cast<const T*>(a.B) + (int64_t)min(n0 + r16, a.N - 1) * a.ldb + kgrp * 32;
   const T* xbase = reinterpret_cast<const T*>(a.A);
-  const int nChunks = (a.K + CHUNK - 1) / CHUNK;
+  const int kBegin = blockIdx.y * a.kPerWg, kEnd = min(a.K, kBegin + a.kPerWg);  // grid.y slices K (whole chunks)
+  const int nChunks = (kEnd - kBegin + CHUNK - 1) / CHUNK;
   f32x4 acc[G];
 #pragma unroll
   for (int gi = 0; gi < G; ++gi) acc[gi] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   u32x4 xa[PER];
   auto loadW = [&](int c, Frag (&w)[4]) {  // a step past the end of K reads the last step instead and is not used
-    const T* src = wbase + min(min(c, nChunks - 1) * CHUNK + ks * kSkinnyStep, a.K - kSkinnyStep);
+    const T* src = wbase + min(kBegin + min(c, nChunks - 1) * CHUNK + ks * kSkinnyStep, kEnd - kSkinnyStep);
 #pragma unroll
     for (int t = 0; t < 4; ++t) w[t] = *reinterpret_cast<const Frag*>(src + 8 * t);
   };
   auto loadX = [&](int c) {  // rows past M and columns past K repeat valid ones; nothing multiplies them
-    const int kc = min(c, nChunks - 1) * CHUNK, len = min(CHUNK, a.K - kc);
+    const int kc = kBegin + min(c, nChunks - 1) * CHUNK, len = min(CHUNK, kEnd - kc);
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int p = threadIdx.x + i * THREADS, r = min(p >> 6, a.M - 1), q = min((p & 63) * 8, len - 8);
@@ -921,7 +922,7 @@ __global__ __launch_bounds__(NTW * 4 * 64) void gemmSkinnyWideKernel(SkinnyArgs 
     for (int t = 0; t < 4; ++t) wc[t] = w0[t], w0[t] = w1[t];
     loadX(c + 1);
     loadW(c + 2, w1);
-    if (c * CHUNK + ks * kSkinnyStep < a.K) {  // wave-uniform: this wave's step of the chunk exists
+    if (kBegin + c * CHUNK + ks * kSkinnyStep < kEnd) {  // wave-uniform: this wave's step of the chunk exists
       const T* xs = sx + (c & 1) * (16 * G * LDX) + ks * kSkinnyStep + kgrp * 32;
 #pragma unroll
       for (int t = 0; t < 4; ++t)
@@ -953,6 +954,10 @@ __global__ __launch_bounds__(NTW * 4 * 64) void gemmSkinnyWideKernel(SkinnyArgs 
           float v = 0.f;
 #pragma unroll
           for (int w2 = 0; w2 < KS; ++w2) v += red[(((tile * KS + w2) * G + gi) * 4 + r) * 64 + lane];
+          if (a.partial) {  // this slice's sum; the reduction pass applies the epilogue
+            a.partial[((int64_t)blockIdx.y * a.M + row) * a.N + col] = v;
+            continue;
+          }
           v = v * a.alpha + bv;
           if (cin) v += a.beta * static_cast<float>(cin[(int64_t)row * a.sCm + (int64_t)col * a.sCn]);
           out[(int64_t)row * a.ldo + col] = static_cast<T>(v);
@@ -1201,8 +1206,19 @@ static diopiError_t launchSkinnyWide(hipStream_t stream, const SkinnyArgs& a) {
   const int lds = std::max(2 * 64 * (CHUNK + kSkinnyPad) * (int)sizeof(T), NTW * 4 * 4 * 4 * 64 * (int)sizeof(float));
   AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmSkinnyWideKernel<T, NTW>), lds));
   const int tiles = (a.N + 15) / 16;
-  hipLaunchKernelGGL((gemmSkinnyWideKernel<T, NTW>), dim3((unsigned)((tiles + NTW - 1) / NTW)), dim3(NTW * 4 * 64), lds, stream, a);
+  const int splits = (a.K + a.kPerWg - 1) / a.kPerWg;
+  hipLaunchKernelGGL((gemmSkinnyWideKernel<T, NTW>), dim3((unsigned)((tiles + NTW - 1) / NTW), (unsigned)splits), dim3(NTW * 4 * 64), lds,
+                     stream, a);
   AMD_LAUNCH_CHECK();
+  if (a.partial) {
+    MfmaArgs g;
+    g.out = a.out, g.Cin = a.Cin, g.bias = a.bias, g.partial = a.partial;
+    g.ldo = a.ldo, g.sCm = a.sCm, g.sCn = a.sCn;
+    g.M = a.M, g.N = a.N, g.K = a.K, g.alpha = a.alpha, g.beta = a.beta;
+    hipLaunchKernelGGL(splitKReduceKernel<T>, dim3((unsigned)ceilDiv((int64_t)a.M * (a.N / 8), 256)), dim3(256), 0, stream, g,
+                       splits);
+    AMD_LAUNCH_CHECK();
+  }
   return diopiSuccess;
 }
 
@@ -1239,9 +1255,24 @@ static diopiError_t launchSkinnyForShape(diopiContextHandle_t ctx, hipStream_t s
     const int cost4 = ((tiles + 3) / 4 + cus - 1) / cus * (2 * 4 + 3), cost3 = ((tiles + 2) / 3 + cus - 1) / cus * (2 * 3 + 3);
     return cost3 < cost4 ? launchSkinnyWide<T, 3>(stream, a) : launchSkinnyWide<T, 4>(stream, a);
   }
-  const int groups = a.M <= 32 ? 2 : 4, chunk = kSkinnyRowsK / (16 * groups);
   const bool canSplit = a.N % 8 == 0 && mult8(p.sOm) && ptr16(p.out) && (!p.bias || ptr16(p.bias)) &&
                         (!p.Cin || (p.sCn == 1 && mult8(p.sCm) && ptr16(p.Cin)));
+  if (a.M > 32 && canSplit) {
+    // Narrower weights with a long K: the same whole-chunk pipeline on K slices of at least 2048 (four chunks), four
+    // tiles per workgroup, when the slices fill at least three quarters of the CUs; the slices meet in fp32 workspace.
+    // 64 rows, against the single-chunk K-split form below: N = 4096 26.2 -> 24.2 us at K = 8192 and 37.6 -> 30.6 at
+    // K = 11008 (four slices), N = 8192 25.0 -> 23.6 at K = 4096 and 45.4 -> 35.3 at K = 8192 (two slices); with
+    // slices of 1024 or half the CUs idle (N = 4096, K = 4096: 17.9 and 22.2 against 15.1) it loses.
+    const int wgs = (tiles + 3) / 4, ways = std::min(cus / std::max(wgs, 1), a.K / 2048);
+    if (ways >= 2 && wgs * ways * 4 >= cus * 3) {
+      const int per = ((a.K + ways - 1) / ways + 511) / 512 * 512, slices = (a.K + per - 1) / per;
+      void* ws = nullptr;
+      AMD_TRY(requireWorkspace(ctx, (int64_t)slices * a.M * a.N * 4, &ws));
+      a.partial = static_cast<float*>(ws), a.kPerWg = per;
+      return launchSkinnyWide<T, 4>(stream, a);
+    }
+  }
+  const int groups = a.M <= 32 ? 2 : 4, chunk = kSkinnyRowsK / (16 * groups);
   const int splits = canSplit && groups == 4 ? (a.K + chunk - 1) / chunk : 1;  // two groups: measured no gain
   if (splits > 1) {
     void* ws = nullptr;
