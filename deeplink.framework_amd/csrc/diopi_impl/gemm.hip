@@ -1245,11 +1245,12 @@ static diopiError_t launchSkinnyForShape(diopiContextHandle_t ctx, hipStream_t s
   // activations would be 2-4 times the weight bytes on the L2 -> CU path. Wider workgroups (up to 4 tiles) bring
   // that to 1:1, and K is split over grid.y as well, one staged chunk per workgroup, to keep the chip full; the
   // slices meet in fp32 workspace and the split-K reduction pass applies the epilogue.
-  if (a.M > 32 && tiles >= 3 * cus && a.K >= 2048) {
+  if (a.M > 32 && tiles >= 2 * cus && a.K >= 4096) {
     // Wide weights and a long K: whole-K workgroups with double-buffered activations, no partial products. Measured
-    // at 64 rows, K = 4096, against the K-split form below: 24.8 against 34.6 us at N = 12288, 30.9 against 44.4 at
-    // 16384, 57 against 61 at 22016 (66.6 against 110 at N = 12288, K = 11008); slower at N = 8192 (26.3 against 25.2)
-    // and at K = 640 (10.1 against 8.3). One workgroup per CU at a time, each paying for its tiles' weights and once
+    // at 64 rows, K = 4096, against the K-split form below: 24.2 against 25.4 us at N = 8192, 24.1 against 32.3 at
+    // 9216, 24.2 against 33.5 at 11008, 24.8 against 34.6 at 12288, 30.9 against 44.4 at 16384, 46 against 61 at 22016
+    // (66.6 against 110 at N = 12288, K = 11008); slower at K = 2048 (14.9 against 13.6 at N = 8192) and at K = 640
+    // (10.1 against 8.3). One workgroup per CU at a time, each paying for its tiles' weights and once
     // for the activations (about one and a half tiles' worth): four tiles per workgroup, or three when that saves
     // rounds (768 tiles on 256 CUs: one round of three tiles instead of one of four).
     const int cost4 = ((tiles + 3) / 4 + cus - 1) / cus * (2 * 4 + 3), cost3 = ((tiles + 2) / 3 + cus - 1) / cus * (2 * 3 + 3);
@@ -1329,7 +1330,7 @@ diopiError_t runGemm(diopiContextHandle_t ctx, hipStream_t stream, GemmProblem p
     // up to 32 rows always; up to 64 while N is moderate or K is long enough for the whole-K form (measured at 64
     // rows, K = 4096: K-split form + reduction pass 16 us against 50 us for the split-K tiled kernel at N = 4096, 36
     // against 52 at N = 12288, 63 against 51 at N = 22016, where the whole-K form takes 46)
-    if (p.batch == 1 && (p.M <= 32 || (p.M <= kSkinnyMaxM && (p.N <= 16384 || p.K >= 2048))) && p.K % kSkinnyStep == 0 && p.N >= 16 &&
+    if (p.batch == 1 && (p.M <= 32 || (p.M <= kSkinnyMaxM && (p.N <= 16384 || p.K >= 4096))) && p.K % kSkinnyStep == 0 && p.N >= 16 &&
         ((p.M - 1) * p.sAm + p.K) * item < (int64_t(1) << 31))
       return p.dtype == diopi_dtype_bfloat16 ? launchSkinnyForShape<bf16_t>(ctx, stream, p)
                                              : launchSkinnyForShape<half_t>(ctx, stream, p);

@@ -144,16 +144,16 @@ def test_split_k_gemm(ops, dev, dtype, m, n, k):
 @pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (5, 100, 8192 + 128), (16, 11008, 4096), (17, 4096, 11008),
                                    (40, 16 * 7 + 3, 384), (64, 16000, 128), (1, 16, 128), (64, 4096, 4096),
                                    (48, 12288, 1024 + 768), (33, 2056, 11008),
-                                   (64, 12288, 2048), (33, 12296, 2048 + 128), (50, 16384, 2048 + 384), (64, 22016, 2048),
-                                   (64, 4096, 8192), (40, 4104, 11008), (64, 8192, 4096 + 640)])
+                                   (64, 12288, 4096), (33, 12296, 4096 + 128), (50, 16384, 4096 + 384), (64, 22016, 4096), (64, 9216, 4096),
+                                   (64, 4096, 8192), (40, 4104, 11008), (64, 6144, 4096 + 640)])
 def test_skinny_m_linear_and_addmm(ops, dev, dtype, m, n, k):
     """At most 64 rows against a K-contiguous weight with K a multiple of 128 select the weight-streaming kernel:
     one, two and four 16-column tiles per workgroup (N = 4096, 11008, 32000), K in one and in two staged chunks
     and down to a single step per wave, row groups of 16 with a ragged last group, ragged N, bias, and the
     alpha / beta epilogue with a full and a broadcast addend. With more than 32 rows K is also split over the grid
     in slices of 1024 (4, 2 with a ragged second, and 11 slices here; N = 16 * 7 + 3 is not a multiple of 8 and
-    stays unsplit) and a reduction pass applies the epilogue. Four cases (more than 32 rows, at least 768
-    column tiles, K from 2048) take the whole-K form with double-buffered activations: three and four tiles per
+    stays unsplit) and a reduction pass applies the epilogue. Five cases (more than 32 rows, at least 512
+    column tiles, K from 4096) take the whole-K form with double-buffered activations: three and four tiles per
     workgroup, a last chunk of one and of three steps, a ragged last tile and a last workgroup with a tile past N;
     the three after them run it on K slices (four even slices, four with a short last one, two with a ragged
     second) that meet in the reduction pass."""
