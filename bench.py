@@ -80,7 +80,8 @@ class Prepared:
     def __call__(self):
         rc = self.fn(self.ctx.ptr, *self.cargs)
         if rc != 0:
-            raise RuntimeError(f"{self.name} failed: {self.err()} {self.rt_err()}")
+            msg = self.err()
+            raise RuntimeError(f"{self.name} failed: {msg}" + (f" [{self.rt_err()}]" if "runtime holds the cause" in msg else ""))
         if not self.hold:
             self.reset(self.ctx.ptr)
 

@@ -305,5 +305,7 @@ def call(name, ctx, *args):
     which is what the generated wrappers' TORCH_CHECK does (autogen_diopi_wrapper.py:1001)."""
     ret = fn(name)(ctx.ptr, *args)
     if ret != DIOPI_SUCCESS:
-        why = rt_error()
-        raise DiopiError(f"{name} failed, ret = {ret}: {last_error()}" + (f" [runtime: {why}]" if why else ""))
+        msg = last_error()
+        if "runtime holds the cause" in msg:  # a workspace request failed: the runtime library knows why
+            msg += f" [{rt_error()}]"
+        raise DiopiError(f"{name} failed, ret = {ret}: {msg}")
