@@ -22,7 +22,10 @@ Pinning (tests/test_oracle.py): reference known-answer tests
 (dipu/tests/python/unittests/test_rsqrt.py:11, test_silu.py:31-34, test_linear.py:14-46,
 test_index.py:78-104), float64 brute-force loops on tiny inputs, torch library routines
 (F.rms_norm, F.scaled_dot_product_attention) and algebraic invariants (rotation composes
-and preserves norms, position 0 is the identity, first causal row equals V[0], ...).
+and preserves norms, position 0 is the identity, first causal row equals V[0], ...);
+precompute_freqs by the closed form cos/sin(t * theta^(-2i/dim)) evaluated element by element for
+two bases, token_logits by a float64 loop over every (sequence, head, token) with grouped KV heads
+and gapped start columns, and by softmax(logits) @ V == token_attention.
 Parity unpinned: the C signatures of the ext ops (nothing in the reference states them).
 """
 import math

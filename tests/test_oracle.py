@@ -105,6 +105,26 @@ def test_rotary_invariants():
     assert torch.allclose(oracle.rotary_emb(oracle.rotary_emb(x, c3, s3), c4, s4), oracle.rotary_emb(x, c7, s7), atol=1e-6)
 
 
+def test_precompute_freqs_closed_form():
+    # dicp/test/model/llama/model.py:42-47: angle[t, i] = t * theta ** (-2 i / dim), evaluated here in
+    # Python float arithmetic, element by element, for two bases and two head dims.
+    for dim, end, theta in [(8, 9, 10000.0), (16, 33, 10000.0), (12, 7, 500.0), (128, 5, 10000.0)]:
+        cos, sin = oracle.precompute_freqs(dim, end, theta)
+        assert cos.shape == (end, dim // 2) and sin.shape == (end, dim // 2)
+        for t in range(end):
+            for i in range(dim // 2):
+                ang = t * theta ** (-2.0 * i / dim)
+                assert abs(float(cos[t, i]) - math.cos(ang)) < 2e-6, (dim, t, i)
+                assert abs(float(sin[t, i]) - math.sin(ang)) < 2e-6, (dim, t, i)
+    # known values: pair 0 turns by one radian per position; the last pair of a 128-wide head by 10000^(-126/128)
+    cos, sin = oracle.precompute_freqs(128, 3)
+    assert abs(float(cos[1, 0]) - 0.5403023058681398) < 1e-6 and abs(float(sin[2, 0]) - 0.9092974268256817) < 1e-6
+    assert abs(float(sin[2, 63]) - math.sin(2 * 10000.0 ** (-126.0 / 128.0))) < 1e-9
+    # the default base is 10000
+    c2, s2 = oracle.precompute_freqs(128, 3, 10000.0)
+    assert torch.equal(cos, c2) and torch.equal(sin, s2)
+
+
 def test_rotary_half_split_equals_interleaved_under_permutation():
     g = torch.Generator().manual_seed(3)
     seq, heads, d = 12, 2, 16
@@ -212,11 +232,49 @@ def test_token_attention_brute_force_and_len_one():
             assert torch.allclose(out[b, h].double(), want, atol=1e-5)
     # a sequence of length one returns its only value row
     assert torch.allclose(out[1], vp[int(b_loc[1, -1])], atol=1e-6)
-    # the two-call form's logits agree with the fused definition's scores
-    starts = torch.tensor([0, 5, 6])
-    att = oracle.token_logits(q, kp, b_loc, starts, lens, max_len, 15)
-    s0 = b_loc[0, max_len - 5:].tolist()
-    assert abs(float(att[1, 2]) - float(torch.dot(q[0, 1], kp[s0[2], 1])) / math.sqrt(d)) < 1e-5
+
+
+def test_token_logits_brute_force_every_element_and_two_call_identity():
+    # ext_ops.py:116-118 split in two calls: logits [heads, total] with sequence b's scores at columns
+    # b_start_loc[b] .. +len_b, then softmax over that range times V. Grouped KV heads, starts that leave a gap.
+    g = torch.Generator().manual_seed(17)
+    batch, heads, kvh, d, slots = 3, 4, 2, 8, 64
+    lens = torch.tensor([5, 1, 9])
+    starts = torch.tensor([0, 6, 8])          # a one-column gap after sequence 0 and after sequence 1
+    total = 17
+    max_len = 11
+    perm = torch.randperm(slots, generator=g)
+    b_loc = torch.full((batch, max_len), -1, dtype=torch.int64)
+    off = 0
+    for b in range(batch):
+        n = int(lens[b])
+        b_loc[b, max_len - n:] = perm[off:off + n]
+        off += n
+    kp = torch.randn(slots, kvh, d, generator=g)
+    vp = torch.randn(slots, kvh, d, generator=g)
+    q = torch.randn(batch, heads, d, generator=g)
+    att = oracle.token_logits(q, kp, b_loc, starts, lens, max_len, total)
+    assert att.shape == (heads, total)
+    want = np.zeros((heads, total))
+    for b in range(batch):
+        n, s = int(lens[b]), int(starts[b])
+        sl = b_loc[b, max_len - n:].tolist()
+        for h in range(heads):
+            for j in range(n):
+                acc = 0.0
+                for t in range(d):
+                    acc += float(q[b, h, t]) * float(kp[sl[j], h // (heads // kvh), t])
+                want[h, s + j] = acc / math.sqrt(d)
+    assert np.allclose(att.double().numpy(), want, atol=1e-5)
+    assert float(att[:, 5].abs().max()) == 0.0 and float(att[:, 7].abs().max()) == 0.0
+    # softmax over a sequence's own columns times its V rows is the fused definition's output
+    fused = oracle.token_attention(q, kp, vp, b_loc, lens, max_len)
+    for b in range(batch):
+        n, s = int(lens[b]), int(starts[b])
+        sl = b_loc[b, max_len - n:]
+        v = vp[sl].repeat_interleave(heads // kvh, dim=1)            # n, heads, d
+        p = att[:, s:s + n].softmax(-1)                              # heads, n
+        assert torch.allclose(torch.einsum("hn,nhd->hd", p, v), fused[b], atol=1e-5)
 
 
 # ---- int8 weight-only linear ----------------------------------------------------------------
