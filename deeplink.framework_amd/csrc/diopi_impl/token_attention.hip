@@ -78,7 +78,7 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   const int h = blockIdx.x, split = blockIdx.y, b = blockIdx.z;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int sub = lane % LPT, grp = lane / LPT;
-  const int len = (int)ldIndex(a.bLen, b, a.len64);
+  const int len = min(max((int)ldIndex(a.bLen, b, a.len64), 0), a.maxLen);  // a length beyond the table's width is cut to it
   const int begin = split * a.chunk;
   if (begin >= len && !(split == 0)) return;  // nothing to do; split 0 still writes zeros for len == 0
   const int end = min(len, begin + a.chunk);
@@ -269,7 +269,7 @@ __global__ __launch_bounds__(256) void tokenLogitsKernel(TaArgs a, OT* __restric
   const int h = blockIdx.x, b = blockIdx.z;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int sub = lane % LPT, grp = lane / LPT;
-  const int len = (int)ldIndex(a.bLen, b, a.len64);
+  const int len = min(max((int)ldIndex(a.bLen, b, a.len64), 0), a.maxLen);  // a length beyond the table's width is cut to it
   const int64_t start = ldIndex(a.bStart, b, a.start64);
   const int begin = blockIdx.y * a.chunk;
   if (begin >= len) return;
@@ -320,7 +320,7 @@ __global__ __launch_bounds__(256) void softmaxReduceVKernel(TaArgs a, T* __restr
   const int h = blockIdx.x, b = blockIdx.z;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int sub = lane % LPT, grp = lane / LPT;
-  const int len = (int)ldIndex(a.bLen, b, a.len64);
+  const int len = min(max((int)ldIndex(a.bLen, b, a.len64), 0), a.maxLen);  // a length beyond the table's width is cut to it
   const int64_t start = ldIndex(a.bStart, b, a.start64);
   const int kvh = h / (a.heads / a.kvHeads);
   const int64_t locBase = (int64_t)b * a.locRowStride + (a.maxLen - len);

@@ -46,6 +46,8 @@ DIOPI_API diopiError_t diopiDestIndexCopyKV(diopiContextHandle_t ctx, diopiTenso
 /* Decode attention, first half: attention_out[h, b_start_loc[b] + t] = q[b,h,:] . k[slot,h,:] / sqrt(d)
  * for t in [0, b_seq_len[b]), slot = b_loc[b, max_input_len - b_seq_len[b] + t] (right-aligned slot table).
  * q [batch, heads, d]; k [slots, kv_heads, d]; attention_out [heads, total_tokens] (fp32 or q dtype).
+ * In all three decode entry points a b_seq_len[b] outside [0, max_input_len] is cut to that range (the table row
+ * holds no more), and slots outside the pool are skipped, never dereferenced.
  * Semantics: the q.K^T/sqrt(d) step of ext_ops.py:100-133. */
 DIOPI_API diopiError_t diopiTokenAttentionInference(diopiContextHandle_t ctx, diopiTensorHandle_t attention_out,
                                                     diopiConstTensorHandle_t q, diopiConstTensorHandle_t k,
