@@ -24,6 +24,7 @@
 //     tokens and at most 64 per sequence); states are merged by wave butterflies, then through
 //     LDS, then across chunks by a small lane-parallel second kernel.
 #include <algorithm>
+#include <mutex>
 
 #include "common.hpp"
 
@@ -483,14 +484,41 @@ static diopiError_t fillArgs(const TaViews& t, bool needK, bool needV, int maxLe
     }                                                                                          \
   } while (0)
 
+// Split-KV partial results for the entry point that allocates nothing. Every device the library's code object is
+// loaded on holds its own copy of this array, at its own address, until the process ends.
+constexpr int64_t kDecodeScratchBytes = 32ll << 20;
+static __device__ __align__(256) unsigned char scratch[kDecodeScratchBytes];
+
+// The array's name is a host-side stand-in; its device address is looked up once per device, with that device
+// current, and only that address is ever handed to a kernel.
+static diopiError_t decodeScratch(float** out) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mu;
+  static void* addr[kMaxDevices] = {};
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  AMD_CHECK(e == hipSuccess && dev >= 0 && dev < kMaxDevices, "token attention: no current device (%s)", hipGetErrorString(e));
+  std::lock_guard<std::mutex> lock(mu);
+  if (addr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    AMD_CHECK(e == hipSuccess && p != nullptr, "token attention: hipGetSymbolAddress of the scratch array failed on device %d (%s)",
+              dev, hipGetErrorString(e));
+    addr[dev] = p;
+  }
+  *out = static_cast<float*>(addr[dev]);
+  return diopiSuccess;
+}
+
 }  // namespace amd
 
 using namespace amd;
 
-extern "C" __attribute__((visibility("default"))) diopiError_t diopiTokenDecodeAttentionInference(
-    diopiContextHandle_t ctx, diopiTensorHandle_t outH, diopiConstTensorHandle_t qH, diopiConstTensorHandle_t kH,
-    diopiConstTensorHandle_t vH, diopiConstTensorHandle_t locH, diopiConstTensorHandle_t startH,
-    diopiConstTensorHandle_t lenH, int maxInputLen) {
+// staticScratch: partial results go to the library's own device array instead of workspace from the context.
+static diopiError_t decodeAttention(diopiContextHandle_t ctx, diopiTensorHandle_t outH, diopiConstTensorHandle_t qH,
+                                    diopiConstTensorHandle_t kH, diopiConstTensorHandle_t vH, diopiConstTensorHandle_t locH,
+                                    diopiConstTensorHandle_t startH, diopiConstTensorHandle_t lenH, int maxInputLen,
+                                    bool staticScratch) {
   hipStream_t stream;
   AMD_TRY(getStream(ctx, &stream));
   TaViews t;
@@ -513,9 +541,20 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiTokenDecodeA
             a.nsplit);
   float* partial = nullptr;
   if (a.nsplit > 1) {
-    void* ws = nullptr;
-    AMD_TRY(requireWorkspace(ctx, (int64_t)batch * a.heads * a.nsplit * (2 + a.d) * (int64_t)sizeof(float), &ws));
-    partial = static_cast<float*>(ws);
+    const int64_t need = (int64_t)batch * a.heads * a.nsplit * (2 + a.d) * (int64_t)sizeof(float);
+    if (staticScratch) {
+      AMD_CHECK(need <= kDecodeScratchBytes,
+                "token attention: batch %ld x %d heads x %d splits of %d tokens needs %ld bytes of partial results, the "
+                "entry point that allocates nothing holds %ld; use diopiTokenDecodeAttentionInference",
+                (long)batch, a.heads, a.nsplit, a.chunk, (long)need, (long)kDecodeScratchBytes);
+      // Nothing has to start at zero: the split kernel writes every (max, sum, acc) row the merge kernel uses, and
+      // rows of splits that hold no tokens are read but discarded by a select.
+      AMD_TRY(decodeScratch(&partial));
+    } else {
+      void* ws = nullptr;
+      AMD_TRY(requireWorkspace(ctx, need, &ws));
+      partial = static_cast<float*>(ws);
+    }
   }
   dim3 grid(a.heads, a.nsplit, (unsigned)batch), block(kTaWaves * 64);
   const int64_t bytes = t.q.shape[2] * t.q.itemsize;
@@ -535,6 +574,22 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiTokenDecodeA
     AMD_LAUNCH_CHECK();
   }
   return diopiSuccess;
+}
+
+extern "C" __attribute__((visibility("default"))) diopiError_t diopiTokenDecodeAttentionInference(
+    diopiContextHandle_t ctx, diopiTensorHandle_t outH, diopiConstTensorHandle_t qH, diopiConstTensorHandle_t kH,
+    diopiConstTensorHandle_t vH, diopiConstTensorHandle_t locH, diopiConstTensorHandle_t startH,
+    diopiConstTensorHandle_t lenH, int maxInputLen) {
+  return decodeAttention(ctx, outH, qH, kH, vH, locH, startH, lenH, maxInputLen, false);
+}
+
+// The same kernels with the split-KV partial results in the library's own device array: no hipMalloc, no hipFree, no
+// workspace request. Calls that overlap on one device (two streams, two threads) share the array and race.
+extern "C" __attribute__((visibility("default"))) diopiError_t diopiTokenDecodeAttentionInferenceNoAlloc(
+    diopiContextHandle_t ctx, diopiTensorHandle_t outH, diopiConstTensorHandle_t qH, diopiConstTensorHandle_t kH,
+    diopiConstTensorHandle_t vH, diopiConstTensorHandle_t locH, diopiConstTensorHandle_t startH,
+    diopiConstTensorHandle_t lenH, int maxInputLen) {
+  return decodeAttention(ctx, outH, qH, kH, vH, locH, startH, lenH, maxInputLen, true);
 }
 
 extern "C" __attribute__((visibility("default"))) diopiError_t diopiTokenAttentionInference(

@@ -281,6 +281,7 @@ SIGNATURES = {
     "diopiTokenSoftmaxReduceVInference": [_T, _T, _T, _T, _T, _T, c_int, c_int],
     "diopiContextAttentionInference": [_T, _T, _T, _T, _T, _T, c_int],
     "diopiTokenDecodeAttentionInference": [_T, _T, _T, _T, _T, _T, _T, c_int],
+    "diopiTokenDecodeAttentionInferenceNoAlloc": [_T, _T, _T, _T, _T, _T, _T, c_int],
     "diopiWeightOnlyInt8Linear": [_T, _T, _T, _T, _T],
     "diopiSiluMul": [_T, _T, _T],
     "diopiLinearSiluMul": [_T, _T, _T],

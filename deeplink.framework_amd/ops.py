@@ -646,8 +646,9 @@ def token_softmax_reducev(logics, v, out, b_loc, b_start_loc, b_seq_len, max_inp
     return out
 
 
-def token_decode_attention(q, k, v, b_loc, b_start_loc, b_seq_len, max_input_len, *, out=None):
-    """lightllm::flash_attention_inference (ext_ops.py:90-133) over a paged pool, fused."""
+def token_decode_attention(q, k, v, b_loc, b_start_loc, b_seq_len, max_input_len, *, out=None, no_alloc=False):
+    """lightllm::flash_attention_inference (ext_ops.py:90-133) over a paged pool, fused. no_alloc selects the entry
+    point whose partial results live in the library's own device array (the caller then passes `out`)."""
     if out is None:
         out = torch.empty_like(q)
     ho, po = handle(out)
@@ -657,7 +658,8 @@ def token_decode_attention(q, k, v, b_loc, b_start_loc, b_seq_len, max_input_len
     h1, p1 = handle(b_loc)
     h2, p2 = handle(b_start_loc)
     h3, p3 = handle(b_seq_len)
-    _call("diopiTokenDecodeAttentionInference", po, pq, pk, pv, p1, p2, p3, int(max_input_len))
+    _call("diopiTokenDecodeAttentionInferenceNoAlloc" if no_alloc else "diopiTokenDecodeAttentionInference",
+          po, pq, pk, pv, p1, p2, p3, int(max_input_len))
     return out
 
 

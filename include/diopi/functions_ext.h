@@ -86,6 +86,19 @@ DIOPI_API diopiError_t diopiTokenDecodeAttentionInference(diopiContextHandle_t c
                                                           diopiConstTensorHandle_t b_start_loc,
                                                           diopiConstTensorHandle_t b_seq_len, int max_input_len);
 
+/* diopiTokenDecodeAttentionInference for callers that cannot allocate (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): same arguments, same kernels, same result bit for bit, but the split-KV
+ * partial results live in a 32 MiB device array inside the library instead of workspace from diopiRequireBuffer, and
+ * the call makes no hipMalloc, hipFree or workspace request. It has no counterpart in the reference. Fails with a
+ * clear error when batch x heads x splits x (2 + head_dim) x 4 bytes exceeds 32 MiB (splits = ceil(max_input_len /
+ * 512), at most 64; batch 64 x 32 heads x head_dim 128 fits up to max_input_len 15872). Every call on a device
+ * shares that device's array: calls that overlap on one device (two streams, two threads) race. */
+DIOPI_API diopiError_t diopiTokenDecodeAttentionInferenceNoAlloc(diopiContextHandle_t ctx, diopiTensorHandle_t out,
+                                                                 diopiConstTensorHandle_t q, diopiConstTensorHandle_t k,
+                                                                 diopiConstTensorHandle_t v, diopiConstTensorHandle_t b_loc,
+                                                                 diopiConstTensorHandle_t b_start_loc,
+                                                                 diopiConstTensorHandle_t b_seq_len, int max_input_len);
+
 /* out[M,N] = input[M,K] @ (weight[N,K] (int8) * scale[N])^T + bias[N].
  * input/out bf16 or fp16; scale fp16/bf16/fp32 per output channel; bias nullable.
  * The int8 -> bf16/fp16 conversion happens while the MFMA operand tile is loaded; the
