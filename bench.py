@@ -31,8 +31,10 @@ MFMA_BF16_PEAK_TF = 2500.0   # MI355X dense bf16, published
 # rocprofv3 --pmc runs of `bench.py --only-layer` (FETCH_SIZE, then WRITE_SIZE), scaled by what the same
 # counters read for a 64 MiB device copy: (2 x 617 006 + 125 999) KiB. The summary is
 # profiles/decoder_layer_hbm_traffic_counters.md;
-# a counter cannot be read from inside this process, so the figure is carried here as measured.
+# a counter cannot be read from inside this process, so the figure is carried here as measured, with the commit
+# whose kernels the counters were taken on (it does not move when the kernel does; re-take it after a GEMM change).
 GEMM_TRAFFIC_BYTES_PER_LAUNCH = 1_393_000_000
+GEMM_TRAFFIC_MEASURED_AT = "11aac02"
 
 
 def parse():
@@ -154,6 +156,58 @@ def time_ops(rt, stream, calls, iters, warm):
     return out
 
 
+def host_threads(torch):
+    """Threads for the CPU legs: every core the process may use. OMP_NUM_THREADS, where the machine's owner sets it
+    (a GPU box gives each GPU a share of the host's cores that way), is that number; otherwise os.cpu_count()."""
+    n = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+    torch.set_num_threads(n)
+    return n
+
+
+def host_description(torch):
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {"cpu_model": model, "os_cpu_count": os.cpu_count(), "omp_num_threads_env": os.environ.get("OMP_NUM_THREADS"),
+            "torch_num_threads": torch.get_num_threads()}
+
+
+def host_time(fn, warm=2, runs=5):
+    """Median wall time in seconds of fn() after warm-ups (time.perf_counter)."""
+    for _ in range(warm):
+        fn()
+    ts = []
+    for _ in range(runs):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    return ts[len(ts) // 2]
+
+
+def cpu_op(torch, dev, cpu_fn, dev_inputs, warm=2, runs=5):
+    """The op as DIPU's CPU fallback runs it: (i) the stock ATen CPU kernels alone (cpu_fn on host copies of the
+    inputs), (ii) fallback-shaped: device inputs to pageable host memory, the CPU kernels, the result back to the
+    device (dipu/torch_dipu/csrc_dipu/aten/ops/DIPUCopy.hpp:282-325). Returns microseconds."""
+    host_in = [t.cpu() for t in dev_inputs]
+    pure = host_time(lambda: cpu_fn(*host_in), warm, runs)
+
+    def shaped():
+        hi = [t.cpu() for t in dev_inputs]
+        r = cpu_fn(*hi)
+        for t in (r if isinstance(r, (tuple, list)) else (r,)):
+            t.to(dev)
+        torch.cuda.synchronize()
+    full = host_time(shaped, min(warm, 1), max(1, min(runs, 3)))
+    return {"us": round(pure * 1e6, 1), "us_fallback_shaped": round(full * 1e6, 1), "runs": runs}
+
+
 def decode_layer_step(pkg, torch, dev, rt, stream, g):
     """One decode step of a 7B-shaped layer at batch 64 (every op launch-bound except the attention): the same
     prepared calls launched one by one, and recorded once into a HIP graph and replayed."""
@@ -227,9 +281,12 @@ def decode_layer_step(pkg, torch, dev, rt, stream, g):
             "tokens_per_s_graph": round(B / (t_graph * 1e-6), 1), "replay_equals_eager": same}
 
 
-def op_microbench(pkg, torch, dev, rt, stream):
+def op_microbench(pkg, torch, dev, rt, stream, with_cpu=True):
     """HBM-bound ops: algorithmic bytes / measured device time. `cold` rotates through enough
-    buffer sets to exceed the 256 MB Infinity Cache; `hot` reuses one set."""
+    buffer sets to exceed the 256 MB Infinity Cache; `hot` reuses one set. With with_cpu every row also carries
+    "cpu": the same op on the same inputs through the oracle (stock ATen CPU kernels) on the host cores, alone and
+    fallback-shaped (inputs device -> host, CPU kernels, result host -> device)."""
+    from oracle import cpu_fallback as oracle
     d = pkg.diopi
     wl = pkg.workloads
     res = []
@@ -252,17 +309,20 @@ def op_microbench(pkg, torch, dev, rt, stream):
         return run
 
     specs = [
-        ("diopiAdd", 3 * E * 2, lambda i: Prepared(pkg, "diopiAdd", O[i], A[i], B[i], one)),
-        ("diopiMul", 3 * E * 2, lambda i: Prepared(pkg, "diopiMul", O[i], A[i], B[i])),
-        ("diopiSoftmax", 2 * E * 2, lambda i: Prepared(pkg, "diopiSoftmax", O[i], A[i], -1)),
-        ("diopiRMSNorm", 2 * E * 2 + 8192, lambda i: Prepared(pkg, "diopiRMSNorm", O[i], None, A[i], d.size([4096]), rw, None, 1e-5)),
-        ("diopiSiluMul", 3 * E * 2, lambda i: Prepared(pkg, "diopiSiluMul", O[i], A[i], B[i])),
+        ("diopiAdd", 3 * E * 2, lambda i: Prepared(pkg, "diopiAdd", O[i], A[i], B[i], one), oracle.add, (A[0], B[0])),
+        ("diopiMul", 3 * E * 2, lambda i: Prepared(pkg, "diopiMul", O[i], A[i], B[i]), oracle.mul, (A[0], B[0])),
+        ("diopiSoftmax", 2 * E * 2, lambda i: Prepared(pkg, "diopiSoftmax", O[i], A[i], -1), lambda a: oracle.softmax(a, -1), (A[0],)),
+        ("diopiRMSNorm", 2 * E * 2 + 8192, lambda i: Prepared(pkg, "diopiRMSNorm", O[i], None, A[i], d.size([4096]), rw, None, 1e-5),
+         lambda a, wt: oracle.rms_norm(a, wt, 1e-5), (A[0], rw)),
+        ("diopiSiluMul", 3 * E * 2, lambda i: Prepared(pkg, "diopiSiluMul", O[i], A[i], B[i]), lambda a, b: oracle.mul(oracle.silu(a), b), (A[0], B[0])),
     ]
-    for name, nbytes, mk in specs:
+    for name, nbytes, mk, cpu_fn, cpu_in in specs:
         hot, cold = time_ops(rt, stream, [mk(0), rotating(mk)], 60, 12)
         res.append({"op": name, "workload": "bf16 [8192,4096]", "bytes": nbytes, "us_hot": round(hot, 2), "us_cold": round(cold, 2),
                     "GBs_hot": round(nbytes / hot / 1e3, 1), "GBs_cold": round(nbytes / cold / 1e3, 1),
                     "frac_hot": round(nbytes / hot / 1e3 / HBM_PEAK_GBS, 3), "frac_cold": round(nbytes / cold / 1e3 / HBM_PEAK_GBS, 3)})
+        if with_cpu:
+            res[-1]["cpu"] = cpu_op(torch, dev, cpu_fn, cpu_in)
     del A, B, O
     X = [w["rot_x"].to(dev).clone() for _ in range(nset)]
     RO = [torch.empty_like(X[0]) for _ in range(nset)]
@@ -274,6 +334,8 @@ def op_microbench(pkg, torch, dev, rt, stream):
                 "us_hot": round(hot, 2), "us_cold": round(cold, 2), "GBs_hot": round(nbytes / hot / 1e3, 1),
                 "GBs_cold": round(nbytes / cold / 1e3, 1), "frac_hot": round(nbytes / hot / 1e3 / HBM_PEAK_GBS, 3),
                 "frac_cold": round(nbytes / cold / 1e3 / HBM_PEAK_GBS, 3)})
+    if with_cpu:
+        res[-1]["cpu"] = cpu_op(torch, dev, oracle.rotary_emb, (X[0], cos, sin))
     del X, RO
     # paged decode step: scatter the new token's K and V, then fused attention (4 GiB of pool: always cold)
     pd = wl.paged_decode(seed=0)
@@ -303,6 +365,15 @@ def op_microbench(pkg, torch, dev, rt, stream):
                 "us_cold": round(t_at, 2), "GBs_cold": round(attn_bytes / t_at / 1e3, 1), "frac_cold": round(attn_bytes / t_at / 1e3 / HBM_PEAK_GBS, 3)})
     res.append({"op": "decode step (scatter + attention)", "workload": "batch 64", "us_cold": round(t_step, 2),
                 "tokens_per_s": round(64 / (t_step * 1e-6), 1)})
+    if with_cpu:
+        # The fallback moves every operand, i.e. the whole 2 GiB pool of K (and of V), to the host and the scattered pool back
+        # (dipu/torch_dipu/csrc_dipu/aten/ops/CustomFallbackFunctions.hpp:78-91); one run each, no warm-up, they take seconds.
+        def scatter_cpu(kp, vp, kn, vn, loc):
+            return oracle.dest_index_copy_kv(kp, kn, loc), oracle.dest_index_copy_kv(vp, vn, loc)
+        res[-3]["cpu"] = cpu_op(torch, dev, scatter_cpu, (g["k_pool"], g["v_pool"], g["k_new"], g["v_new"], g["dest_loc"]), warm=1, runs=3)
+        mil = int(pd["max_input_len"])
+        res[-2]["cpu"] = cpu_op(torch, dev, lambda q, kp, vp, loc, ln: oracle.token_attention(q, kp, vp, loc, ln, mil),
+                                (g["q"], g["k_pool"], g["v_pool"], g["b_loc"], g["b_seq_len"]), warm=1, runs=3)
     res.append(decode_layer_step(pkg, torch, dev, rt, stream, g))
     del g, pd
     # int8 weight-only linear: weights rotate through 8 copies (360 MB) for the cold figure
@@ -322,6 +393,8 @@ def op_microbench(pkg, torch, dev, rt, stream):
         res.append({"op": "diopiWeightOnlyInt8Linear", "workload": f"M={m}, K=4096, N=11008", "bytes": nbytes, "us_hot": round(hot, 2),
                     "us_cold": round(cold, 2), "GBs_hot": round(nbytes / hot / 1e3, 1), "GBs_cold": round(nbytes / cold / 1e3, 1),
                     "frac_hot": round(nbytes / hot / 1e3 / HBM_PEAK_GBS, 3), "frac_cold": round(nbytes / cold / 1e3 / HBM_PEAK_GBS, 3)})
+        if with_cpu:
+            res[-1]["cpu"] = cpu_op(torch, dev, oracle.weight_only_int8_linear, (x, W[0], sc))
         del W
     # bf16 linear at decode shapes (a handful of rows against a [11008, 4096] weight): the weight stream is the traffic
     for m in (1, 16, 64):
@@ -340,6 +413,8 @@ def op_microbench(pkg, torch, dev, rt, stream):
         res.append({"op": "diopiLinear (decode)", "workload": f"bf16 M={m}, K=4096, N=11008", "bytes": nbytes, "us_hot": round(hot, 2),
                     "us_cold": round(cold, 2), "GBs_hot": round(nbytes / hot / 1e3, 1), "GBs_cold": round(nbytes / cold / 1e3, 1),
                     "frac_hot": round(nbytes / hot / 1e3 / HBM_PEAK_GBS, 3), "frac_cold": round(nbytes / cold / 1e3 / HBM_PEAK_GBS, 3)})
+        if with_cpu:
+            res[-1]["cpu"] = cpu_op(torch, dev, oracle.linear, (x, W[0]))
         del W
     return res
 
@@ -373,8 +448,7 @@ def cpu_baseline(pkg, torch, gpu_out=None):
     layer output of the timed GPU run, same seed) is checked against the oracle's output: the oracle as the checker."""
     from oracle import cpu_fallback as oracle
     x, p, cfg = pkg.workloads.llama7b_layer(seed=0, batch=4)
-    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
-    torch.set_num_threads(threads)
+    host_threads(torch)
     t0 = time.perf_counter()
     host_bf16, _ = oracle.decoder_block(x, p, cfg["heads"], cfg["eps"], cfg["theta"])   # warm-up (thread pool, allocations)
     warm = time.perf_counter() - t0
@@ -390,19 +464,24 @@ def cpu_baseline(pkg, torch, gpu_out=None):
         def against_fp32(t):
             err = (t.float().cpu().reshape(-1) - ref).abs()
             return {"max_abs_err": round(float(err.max()), 5), "mean_abs_err": round(float(err.mean()), 6),
-                    "out_of_tolerance": int((err > 3e-2 + 3e-2 * ref.abs()).sum())}
-        parity = {"against": "oracle layer output in fp32, first sequence [1, 2048, 4096]", "tolerance": "3e-2 abs + 3e-2 rel",
+                    "outside_1e-2_abs_2e-2_rel": int((err > 1e-2 + 2e-2 * ref.abs()).sum()),
+                    "outside_3e-2_abs_3e-2_rel": int((err > 3e-2 + 3e-2 * ref.abs()).sum())}
+        parity = {"against": "oracle layer output in fp32, first sequence [1, 2048, 4096]",
+                  "note": "a report of how bf16 rounding chains through the seven launches, for the device and for the host's own "
+                          "bf16 run; the gate at this size is per op (each op fed the oracle's bf16 intermediate, 2e-2 relative / "
+                          "1e-2 absolute) in tests/test_gpu_full_size.py",
                   "elements": int(ref.numel()), "gpu_bf16": against_fp32(gpu_out.reshape(x.shape)[:1]),
                   "host_bf16": against_fp32(host_bf16[:1])}
         del want
     del host_bf16
-    reps = 1 if warm > 12 else (3 if warm > 4 else 8)
+    reps = 1 if warm > 12 else (3 if warm > 6 else 5)   # about 10-30 s of host work in all
     times = []
     for _ in range(reps):
         t0 = time.perf_counter()
         oracle.decoder_block(x, p, cfg["heads"], cfg["eps"], cfg["theta"])
         times.append(time.perf_counter() - t0)
-    t = min(times)
+    times.sort()
+    t = times[len(times) // 2]
     # What DIPU's CPU fallback adds per op on top of the CPU kernel: operands to the host and the result back
     # (dipu/torch_dipu/csrc_dipu/aten/ops/DIPUCopy.hpp:282-325, pageable memory, stream-synchronous). One
     # [4, 2048, 4096] bf16 activation each way is timed here; a layer run op by op through the fallback pays about
@@ -417,8 +496,9 @@ def cpu_baseline(pkg, torch, gpu_out=None):
     xh.to(dev)
     torch.cuda.synchronize()
     h2d = time.perf_counter() - t0
-    return {"value": round(8192 / t, 2), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port", "layer_parity": parity,
-            "sample": f"the same layer and batch (4 x 2048 tokens) through the oracle: stock ATen CPU kernels in bf16, best of {reps} "
+    return {"value": round(8192 / t, 2), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port", "host": host_description(torch),
+            "layer_parity": parity,
+            "sample": f"the same layer and batch (4 x 2048 tokens) through the oracle: stock ATen CPU kernels in bf16, median of {reps} "
                       f"passes after a warm-up, {t:.2f} s per pass",
             "fallback_copy_ms": {"tensor": "bf16 [4, 2048, 4096] (64 MiB), pageable host memory", "d2h": round(d2h * 1e3, 2),
                                  "h2d": round(h2d * 1e3, 2)}}
@@ -490,6 +570,7 @@ def main():
     roofline = {"bound": "mfma", "kernel": "gemmMfmaPipelinedKernel<bf16> 256x256x64 (4 launches per step: qkv with rotary, o + residual, gate+up with silu*mul, down + residual)",
                 "achieved": round(achieved_tf, 1), "peak": MFMA_BF16_PEAK_TF, "unit": "TFLOP/s",
                 "frac": round(achieved_tf / MFMA_BF16_PEAK_TF, 4), "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH,
+                "traffic_measured_at_commit": GEMM_TRAFFIC_MEASURED_AT,
                 "flops_per_step": gemm_flops, "avg_launch_us": round(gemm_time_us / len(gemm_labels), 1),
                 "per_gemm_TFLOPs": {l: round(flops[l] / (sum(per_op[l]) / args.steps * 1e-6) / 1e12, 1) for l in gemm_labels}}
 
@@ -506,7 +587,8 @@ def main():
         "layer_breakdown_us": breakdown,
     }
     if not args.no_ops:
-        result["ops"] = op_microbench(pkg, torch, dev, rt, stream)
+        host_threads(torch)
+        result["ops"] = op_microbench(pkg, torch, dev, rt, stream, with_cpu=not args.no_cpu)
     if not args.no_cpu:
         gpu_out = out.clone()
         del plan, keep
