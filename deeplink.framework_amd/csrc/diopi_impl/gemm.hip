@@ -1808,7 +1808,14 @@ GEMM_EXPORT diopiError_t diopiLinearRotary(diopiContextHandle_t ctx, diopiTensor
       v.shape[0] = rows, v.shape[1] = rotaryCols / headDim, v.shape[2] = headDim;
       v.stride[0] = n, v.stride[1] = headDim, v.stride[2] = 1;
       v.numel = rows * rotaryCols;
-      AMD_TRY(runRotary(ctx, stream, v, v, cc, cs, conj, interleaved));
+      // the tables as [t, head_dim / 2] whatever shape the caller's dense tensors have, as the one-launch form reads them
+      auto asTable = [&](TensorView t) {
+        t.ndim = 2;
+        t.shape[0] = tableRows, t.shape[1] = half;
+        t.stride[0] = half, t.stride[1] = 1;
+        return t;
+      };
+      AMD_TRY(runRotary(ctx, stream, v, v, asTable(cc), asTable(cs), conj, interleaved));
     }
   }
   if (outTemp) AMD_TRY(stridedCopy(stream, cout, out));

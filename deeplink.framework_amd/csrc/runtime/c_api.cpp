@@ -8,6 +8,7 @@
 
 #include "expandable_segment.h"
 #include "runtime_core.h"
+#include "allocator_metrics.h"
 
 using namespace dipu;
 using namespace dipu::amdrt;
@@ -247,12 +248,12 @@ int dipuAmdGetEventStatus(void* event, int* status) {
   return guarded([&] { *status = static_cast<int>(devapis::getEventStatus(E(event))); });
 }
 
-int dipuAmdMallocHost(void** p, size_t n) { return guarded([&] { devapis::mallocHost(p, n); }); }
-int dipuAmdFreeHost(void* p) { return guarded([&] { devapis::freeHost(p); }); }
+int dipuAmdMallocHost(void** p, size_t n) { return guarded([&] { devproxy::mallocHost(p, n); }); }
+int dipuAmdFreeHost(void* p) { return guarded([&] { devproxy::freeHost(p); }); }
 int dipuAmdMallocDevice(void** p, size_t n, int throw_on_oom, int* status) {
-  return guarded([&] { *status = static_cast<int>(devapis::mallocDevice(p, n, throw_on_oom != 0)); });
+  return guarded([&] { *status = static_cast<int>(devproxy::mallocDevice(p, n, throw_on_oom != 0)); });
 }
-int dipuAmdFreeDevice(void* p) { return guarded([&] { devapis::freeDevice(p); }); }
+int dipuAmdFreeDevice(void* p) { return guarded([&] { devproxy::freeDevice(p); }); }
 int dipuAmdIsPinnedPtr(const void* p, int* pinned) {
   return guarded([&] { *pinned = devapis::isPinnedPtr(p) ? 1 : 0; });
 }
@@ -423,6 +424,31 @@ int dipuAmdProfilerEnable(const char* dump_path) {
 int dipuAmdProfilerDisable() { return guarded([&] { dipu::devapis::disableProfiler(); }); }
 int dipuAmdProfilerCounts(uint64_t* started, uint64_t* stopped, int* roctx_bound) {
   return guarded([&] { dipu::profile::counts(started, stopped, roctx_bound); });
+}
+
+
+int dipuAmdMetricsEnable(int update, int* enabled) {
+  return guarded([&] {
+    const bool v = metricsEnable(update);
+    if (enabled) *enabled = v ? 1 : 0;
+  });
+}
+int dipuAmdMetricsText(char* buffer, size_t capacity, size_t* needed) {
+  return guarded([&] {
+    const std::string text = metricsText();
+    if (needed) *needed = text.size() + 1;
+    if (buffer && capacity > 0) {
+      const size_t n = text.size() < capacity - 1 ? text.size() : capacity - 1;
+      std::memcpy(buffer, text.data(), n);
+      buffer[n] = 0;
+    }
+  });
+}
+int dipuAmdMetricsRecord(const char* type, int device, int deallocate, void* data, size_t size) {
+  return guarded([&] {
+    AllocatorMetrics& m = allocatorMetrics(type ? type : "", device);
+    if (deallocate) m.deallocate(data); else m.allocate(data, size);
+  });
 }
 
 }  // extern "C"

@@ -274,6 +274,20 @@ bool DeviceCachingAllocator::allocBlock(BlockPool& pool, size_t size, size_t all
   return true;
 }
 
+void* DeviceCachingAllocator::mallocFromCache(size_t size, StreamHandle stream) {
+  std::lock_guard<std::recursive_mutex> lock(mutex_);
+  cacheOnly_ = true;
+  void* p = nullptr;
+  try {
+    p = malloc(size, stream);
+  } catch (...) {
+    cacheOnly_ = false;
+    throw;
+  }
+  cacheOnly_ = false;
+  return p;
+}
+
 void* DeviceCachingAllocator::malloc(size_t origSize, StreamHandle stream) {
   if (origSize == 0) return nullptr;
   std::lock_guard<std::recursive_mutex> lock(mutex_);
@@ -283,6 +297,7 @@ void* DeviceCachingAllocator::malloc(size_t origSize, StreamHandle stream) {
   size_t allocSize = allocationSize(size, config_);
 
   Block* block = getFreeBlock(pool, size, stream);
+  if (!block && cacheOnly_) return nullptr;
   if (!block) {
     if (config_.gcThreshold > 0.0) garbageCollect();
     bool ok = allocBlock(pool, size, allocSize, stream, &block);

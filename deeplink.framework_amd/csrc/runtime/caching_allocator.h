@@ -138,6 +138,12 @@ class DeviceAllocator {
   virtual ~DeviceAllocator() = default;
   // Never returns nullptr for size > 0; throws OutOfMemory once every way of finding the bytes has failed.
   virtual void* malloc(size_t size, StreamHandle stream) = 0;
+  // A block out of the cache or nullptr: never calls the device allocator, never synchronises, records no event.
+  // For requests made while `stream` is being captured into a graph. nullptr also means "not supported".
+  virtual void* mallocFromCache(size_t size, StreamHandle stream) {
+    (void)size, (void)stream;
+    return nullptr;
+  }
   virtual void free(void* ptr) = 0;
   // `ptr` is also being used on `stream`; its reuse waits for an event on that stream.
   virtual void recordStream(void* ptr, StreamHandle stream) = 0;
@@ -155,6 +161,7 @@ class DeviceCachingAllocator : public DeviceAllocator {
   // Never returns nullptr for size > 0; throws std::bad_alloc-derived OutOfMemory after the
   // full retry ladder (reuse -> device malloc -> release enough cached -> release all cached).
   void* malloc(size_t size, StreamHandle stream) override;
+  void* mallocFromCache(size_t size, StreamHandle stream) override;
   void free(void* ptr) override;
   // `ptr` is also being used on `stream`; its reuse waits for an event on that stream.
   void recordStream(void* ptr, StreamHandle stream) override;
@@ -170,6 +177,7 @@ class DeviceCachingAllocator : public DeviceAllocator {
   size_t blockSize(void* ptr) const;  // rounded size of a live allocation (0 if unknown)
 
  private:
+  bool cacheOnly_ = false;  // set for the duration of mallocFromCache (under mutex_)
   Block* getFreeBlock(BlockPool& pool, size_t size, StreamHandle stream);
   bool allocBlock(BlockPool& pool, size_t size, size_t allocSize, StreamHandle stream, Block** out);
   Block* findExpandableBlock(BlockPool& pool, size_t size, StreamHandle stream);

@@ -4,7 +4,11 @@
 // behaviours DIPU's callers rely on.
 #include <cstdlib>
 
+// A DIPU tree declares the contract itself (csrc_dipu/runtime/device/deviceapis.h) before it compiles these bodies
+// as vendor/amd/deviceimpl.cpp; on its own the runtime library uses the restated declarations.
+#ifndef DIPU_AMD_DEVAPIS_DECLARED
 #include "devapis_contract.h"
+#endif
 
 namespace dipu {
 namespace devapis {

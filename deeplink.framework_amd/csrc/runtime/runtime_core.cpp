@@ -1,4 +1,7 @@
+#include <sstream>
+
 #include "runtime_core.h"
+#include "allocator_metrics.h"
 #include "expandable_segment.h"
 
 #include <cstdlib>
@@ -50,13 +53,35 @@ struct HipExpandableRange final : ExpandableRange {
 };
 }  // namespace
 
+// The raw vendor calls with their metrics, as DIPU's device proxy wraps them
+// (dipu/torch_dipu/csrc_dipu/runtime/devproxy/deviceproxy.cpp:196-218): type "host" and "device".
+namespace devproxy {
+void mallocHost(void** p, size_t nbytes) {
+  devapis::mallocHost(p, nbytes);
+  allocatorMetrics("host", devapis::current_device()).allocate(p ? *p : nullptr, nbytes);
+}
+void freeHost(void* p) {
+  allocatorMetrics("host", devapis::current_device()).deallocate(p);
+  devapis::freeHost(p);
+}
+devapis::OpStatus mallocDevice(void** p, size_t nbytes, bool throwException) {
+  const devapis::OpStatus code = devapis::mallocDevice(p, nbytes, throwException);
+  allocatorMetrics("device", devapis::current_device()).allocate(p ? *p : nullptr, nbytes);
+  return code;
+}
+void freeDevice(void* p) {
+  allocatorMetrics("device", devapis::current_device()).deallocate(p);
+  devapis::freeDevice(p);
+}
+}  // namespace devproxy
+
 RawBackend RawBackend::hip() {
   RawBackend b;
   b.createExpandable = [](StreamHandle s, size_t segmentSize) -> ExpandableRange* {
     return new HipExpandableRange(static_cast<int>(devapis::current_device()), static_cast<deviceStream_t>(s), segmentSize);
   };
-  b.mallocDevice = [](void** p, size_t n) { return devapis::mallocDevice(p, n, false) == devapis::OpStatus::SUCCESS; };
-  b.freeDevice = [](void* p) { devapis::freeDevice(p); };
+  b.mallocDevice = [](void** p, size_t n) { return devproxy::mallocDevice(p, n, false) == devapis::OpStatus::SUCCESS; };
+  b.freeDevice = [](void* p) { devproxy::freeDevice(p); };
   b.createEvent = []() {
     deviceEvent_t e;
     devapis::createEvent(&e);
@@ -192,7 +217,7 @@ void* HostCachingAllocator::malloc(size_t nbytes) {
     p = fl.back();
     fl.pop_back();
   } else {
-    devapis::mallocHost(&p, size);
+    devproxy::mallocHost(&p, size);
     blocks_[p].size = size;
   }
   blocks_[p].allocated = true;
@@ -233,7 +258,7 @@ void HostCachingAllocator::emptyCache() {
   processEvents();
   for (auto& kv : freeBySize_) {
     for (void* p : kv.second) {
-      devapis::freeHost(p);
+      devproxy::freeHost(p);
       blocks_.erase(p);
     }
     kv.second.clear();
@@ -296,13 +321,42 @@ RawAllocator* Runtime::raw(int device) {
   return raw_[device].get();
 }
 
+// hipStreamIsCapturing on the null stream fails while another stream captures in global mode; that failure is not
+// this request's and is cleared.
+static bool streamIsCapturing(deviceStream_t stream) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return status == hipStreamCaptureStatusActive;
+}
+
 void* Runtime::deviceMalloc(size_t nbytes, deviceStream_t stream) {
   int device = devapis::current_device();
-  void* p = useRaw() ? raw(device)->malloc(nbytes) : caching(device)->malloc(nbytes, stream);
+  void* p = nullptr;
+  if (nbytes > 0 && streamIsCapturing(stream)) {
+    // Recording into a graph: hipMalloc, hipFree, event records and device-wide waits are all illegal, so only a
+    // block already in the TORCH algorithm's cache can serve the request.
+    if (!useRaw() && algorithm_ == 0) p = caching(device)->mallocFromCache(nbytes, stream);
+    if (!p) {
+      std::ostringstream os;
+      os << "request for " << nbytes << " bytes on a stream that is being captured into a graph";
+      if (useRaw() || algorithm_ != 0)
+        os << ": only DIPU_DEVICE_MEMCACHING_ALGORITHM=TORCH serves requests during capture";
+      else
+        os << " found no cached block: run the same calls on this stream once before capturing, holding their workspace";
+      throw std::runtime_error(os.str());
+    }
+  } else {
+    p = useRaw() ? raw(device)->malloc(nbytes) : caching(device)->malloc(nbytes, stream);
+  }
   if (p) {
     std::lock_guard<std::mutex> lock(mu_);
     ownerDevice_[p] = device;
   }
+  // type "caching" (DIPUCachingDeviceAllocator.cpp:1845-1875), with the size that was asked for
+  allocatorMetrics("caching", device).allocate(p, nbytes);
   return p;
 }
 
@@ -316,6 +370,7 @@ void Runtime::deviceFree(void* p) {
     device = it->second;
     ownerDevice_.erase(it);
   }
+  allocatorMetrics("caching", device).deallocate(p);
   if (useRaw()) raw(device)->free(p); else caching(device)->free(p);
 }
 

@@ -74,6 +74,14 @@ class HostCachingAllocator {
   std::vector<void*> pending_;
 };
 
+// devapis::malloc* / free* with the "host" and "device" allocator metrics recorded around them.
+namespace devproxy {
+void mallocHost(void** p, size_t nbytes);
+void freeHost(void* p);
+devapis::OpStatus mallocDevice(void** p, size_t nbytes, bool throwException);
+void freeDevice(void* p);
+}  // namespace devproxy
+
 struct Runtime {
   StreamPool streams;
   EventPool events;

@@ -2,6 +2,9 @@
 // dipu/torch_dipu/csrc_dipu/vendor/cuda/vendorapi.h:37-49 for gfx950.
 #pragma once
 
+// Inside a DIPU tree the vendor directory's own vendorapi.h (TORCH_CHECK-based) has already declared everything below.
+#ifndef DIPU_CALLHIP
+
 #include <hip/hip_runtime_api.h>
 
 #include <stdexcept>
@@ -33,3 +36,5 @@ struct commUniqueId {
 };
 
 }  // namespace dipu
+
+#endif  // DIPU_CALLHIP

@@ -13,7 +13,7 @@ from ctypes import POINTER, Structure, Union, byref, c_bool, c_char_p, c_double,
 
 import torch
 
-from . import _native
+from . import _native, runtime
 
 MAX_DIMS = 8
 
@@ -304,7 +304,16 @@ def fn(name):
 def call(name, ctx, *args):
     """Calls diopi<name>(ctx, *args) and raises with diopiGetLastErrorString() on failure,
     which is what the generated wrappers' TORCH_CHECK does (autogen_diopi_wrapper.py:1001)."""
-    ret = fn(name)(ctx.ptr, *args)
+    if runtime.profiler_on:
+        # the generated wrapper's RecordBlockCreator dipuRecorder("<interface>") ... dipuRecorder.end()
+        # around the call (autogen_diopi_wrapper.py:1013-1016): here a ROCTX range of that name
+        rec = runtime.recordStart(name)
+        try:
+            ret = fn(name)(ctx.ptr, *args)
+        finally:
+            runtime.recordEnd(rec)
+    else:
+        ret = fn(name)(ctx.ptr, *args)
     if ret != DIOPI_SUCCESS:
         msg = last_error()
         if "runtime holds the cause" in msg:  # a workspace request failed: the runtime library knows why

@@ -318,11 +318,18 @@ class SimAllocator:
 
 
 # ---- profiler hooks (runtime/device/profilerapis.h:12-14; diopirt_impl.cpp:224-237) ----
+profiler_on = False   # read by diopi.call on every op: a plain attribute, no C call while the profiler is off
+
+
 def enableProfiler(dump_path=""):
+    global profiler_on
     _check(_rt().dipuAmdProfilerEnable(dump_path.encode()))
+    profiler_on = True
 
 
 def disableProfiler():
+    global profiler_on
+    profiler_on = False
     _check(_rt().dipuAmdProfilerDisable())
 
 
@@ -377,3 +384,35 @@ class ExpandableSegment:
         o, n = c_uint64(), c_uint64()
         _check(_rt().dipuAmdExpandableSegmentUnmap(self.h, c_uint64(offset), c_uint64(nbytes), byref(o), byref(n)))
         return o.value, n.value
+
+
+# ---- allocator metrics ----
+def metricsEnable(update=None):
+    """torch_dipu._C.enable_metrics / is_metrics_enabled (binding/ExportRT.cpp:345-346): returns the setting."""
+    on = c_int()
+    _check(_rt().dipuAmdMetricsEnable(c_int(-1 if update is None else int(bool(update))), byref(on)))
+    return bool(on.value)
+
+
+def metricsText():
+    need = ctypes.c_size_t()
+    _check(_rt().dipuAmdMetricsText(None, ctypes.c_size_t(0), byref(need)))
+    buf = ctypes.create_string_buffer(need.value + 4096)
+    _check(_rt().dipuAmdMetricsText(buf, ctypes.c_size_t(len(buf)), byref(need)))
+    return buf.value.decode()
+
+
+def metrics():
+    """{(name, frozenset of (label, value) pairs): value} of every exported line, the lookup
+    dipu/tests/python/individual_scripts/test_metrics.py:22-26 does on torch_dipu._C.metrics()."""
+    out = {}
+    for line in metricsText().splitlines():
+        head, value = line.rsplit(" ", 1)
+        name, labels = head.split("{", 1)
+        pairs = frozenset(tuple(kv.split("=", 1)) for kv in labels.rstrip("}").split(","))
+        out[(name, frozenset((k, v.strip('"')) for k, v in pairs))] = int(value)
+    return out
+
+
+def metricsRecord(type_, device, data, size=0, deallocate=False):
+    _check(_rt().dipuAmdMetricsRecord(type_.encode(), c_int(device), c_int(1 if deallocate else 0), c_void_p(data), ctypes.c_size_t(size)))

@@ -174,6 +174,16 @@ DIPU_AMD_API int dipuAmdProfilerEnable(const char* dump_path);
 DIPU_AMD_API int dipuAmdProfilerDisable(void);
 DIPU_AMD_API int dipuAmdProfilerCounts(uint64_t* started, uint64_t* stopped, int* roctx_bound);
 
+/* ---- allocator metrics: dipu/torch_dipu/csrc_dipu/runtime/core/allocator/allocator_metrics.h:17-160 (label sets
+ * type / device / method / event) and metrics/metrics.cpp:5-11 (the switch, on by default). dipuAmdMetricsEnable:
+ * update 0 / 1 sets the switch, anything else only reads it. dipuAmdMetricsText writes the Prometheus text
+ * exposition of every value (allocator_event_count, allocator_size_bucket / _sum / _count), NUL-terminated and cut to
+ * capacity; *needed is the size of the whole text. dipuAmdMetricsRecord feeds one allocate (deallocate = 0) or
+ * deallocate event to the metrics of (type, device) directly, the call the allocators make. */
+DIPU_AMD_API int dipuAmdMetricsEnable(int update, int* enabled);
+DIPU_AMD_API int dipuAmdMetricsText(char* buffer, size_t capacity, size_t* needed);
+DIPU_AMD_API int dipuAmdMetricsRecord(const char* type, int device, int deallocate, void* data, size_t size);
+
 #if defined(__cplusplus)
 }
 #endif

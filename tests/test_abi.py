@@ -135,3 +135,41 @@ def test_generator_state_round_trip(pkg):
         h.close()
     finally:
         g.close()
+
+
+def test_allocator_metrics_labels_events_and_histogram(pkg):
+    """Label sets and event rules of dipu/torch_dipu/csrc_dipu/runtime/core/allocator/allocator_metrics.h:17-120, fed
+    through the same call the allocators make (no device needed)."""
+    rt = pkg.runtime
+    assert rt.metricsEnable() is True                       # on by default (metrics/metrics.cpp:5-11)
+    t, dev = "unit_test", 3
+    key = lambda name, **kw: (name, frozenset({("type", t), ("device", str(dev))} | set(kw.items())))
+    rt.metricsRecord(t, dev, 0x1000, 16)                    # <= 2^4: first bucket
+    rt.metricsRecord(t, dev, 0x2000, 17)                    # second bucket
+    rt.metricsRecord(t, dev, 0x3000, 1 << 31)               # last finite bucket
+    rt.metricsRecord(t, dev, 0x4000, (1 << 31) + 1)         # +Inf
+    rt.metricsRecord(t, dev, 0x5000, 0)                     # size 0: ignored
+    rt.metricsRecord(t, dev, 0, 64)                         # null pointer
+    rt.metricsRecord(t, dev, 0x1000, 32)                    # already live
+    m = rt.metrics()
+    assert m[key("allocator_event_count", method="allocate", event="nullptr")] == 1
+    assert m[key("allocator_event_count", method="allocate", event="duplicated")] == 1
+    assert m[key("allocator_size_bucket", method="allocate", le="16")] == 1
+    assert m[key("allocator_size_bucket", method="allocate", le="32")] == 2
+    assert m[key("allocator_size_bucket", method="allocate", le=str(1 << 30))] == 2
+    assert m[key("allocator_size_bucket", method="allocate", le=str(1 << 31))] == 3
+    assert m[key("allocator_size_bucket", method="allocate", le="+Inf")] == 4
+    assert m[key("allocator_size_count", method="allocate")] == 4
+    assert m[key("allocator_size_sum", method="allocate")] == 16 + 17 + (1 << 31) + (1 << 31) + 1
+    rt.metricsRecord(t, dev, 0x2000, deallocate=True)       # records the size it was allocated with
+    rt.metricsRecord(t, dev, 0x2000, deallocate=True)       # no longer live
+    rt.metricsRecord(t, dev, 0, deallocate=True)
+    m = rt.metrics()
+    assert m[key("allocator_size_sum", method="deallocate")] == 17 and m[key("allocator_size_count", method="deallocate")] == 1
+    assert m[key("allocator_event_count", method="deallocate", event="unexpected")] == 1
+    assert m[key("allocator_event_count", method="deallocate", event="nullptr")] == 1
+    # switched off nothing is recorded
+    assert rt.metricsEnable(False) is False
+    rt.metricsRecord(t, dev, 0x9000, 64)
+    assert rt.metrics()[key("allocator_size_count", method="allocate")] == 4
+    assert rt.metricsEnable(True) is True

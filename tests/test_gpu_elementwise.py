@@ -3,7 +3,7 @@ import pytest
 import torch
 
 from oracle import cpu_fallback as oracle
-from tests.parity import assert_close, assert_exact, assert_fp32, assert_half
+from tests.parity import assert_close, assert_each, assert_exact, assert_fp32, assert_half
 
 pytestmark = pytest.mark.gpu
 
@@ -17,36 +17,36 @@ def g(seed):
 def test_add_mul_vector_and_tail(ops, dev, dtype, shape):
     a = torch.randn(shape, generator=g(0)).to(dtype)
     b = torch.randn(shape, generator=g(1)).to(dtype)
-    assert_close(ops.add(a.to(dev), b.to(dev)), oracle.add(a, b))
-    assert_close(ops.add(a.to(dev), b.to(dev), alpha=2), oracle.add(a, b, alpha=2))
-    assert_close(ops.add(a.to(dev), b.to(dev), alpha=-0.5), oracle.add(a, b, alpha=-0.5))
-    assert_close(ops.mul(a.to(dev), b.to(dev)), oracle.mul(a, b))
-    assert_close(ops.sub(a.to(dev), b.to(dev), alpha=3), oracle.sub(a, b, alpha=3))
-    assert_close(ops.div(a.to(dev), (b.abs() + 1).to(dev)), oracle.div(a, b.abs() + 1))
+    assert_each(ops.add(a.to(dev), b.to(dev)), oracle.add(a, b))
+    assert_each(ops.add(a.to(dev), b.to(dev), alpha=2), oracle.add(a, b, alpha=2))
+    assert_each(ops.add(a.to(dev), b.to(dev), alpha=-0.5), oracle.add(a, b, alpha=-0.5))
+    assert_each(ops.mul(a.to(dev), b.to(dev)), oracle.mul(a, b))
+    assert_each(ops.sub(a.to(dev), b.to(dev), alpha=3), oracle.sub(a, b, alpha=3))
+    assert_each(ops.div(a.to(dev), (b.abs() + 1).to(dev)), oracle.div(a, b.abs() + 1))
 
 
 def test_broadcast_strided_mixed_and_inplace(ops, dev):
     a = torch.randn(6, 1, 33, generator=g(2))
     b = torch.randn(5, 33, generator=g(3))
-    assert_close(ops.add(a.to(dev), b.to(dev)), a + b)
+    assert_each(ops.add(a.to(dev), b.to(dev)), a + b)
     at = torch.randn(40, 24, generator=g(4))
-    assert_close(ops.mul(at.to(dev).t(), at.to(dev).t()[:, ::2].repeat(1, 2)), at.t() * at.t()[:, ::2].repeat(1, 2))
+    assert_each(ops.mul(at.to(dev).t(), at.to(dev).t()[:, ::2].repeat(1, 2)), at.t() * at.t()[:, ::2].repeat(1, 2))
     # [M,N] * [N] and [M,N] * [M,1] (the decomposed RMSNorm's broadcasts)
     x = torch.randn(64, 96, generator=g(5)).bfloat16()
     w = torch.randn(96, generator=g(6)).bfloat16()
     r = torch.rand(64, 1, generator=g(7)).bfloat16()
-    assert_close(ops.mul(x.to(dev), w.to(dev)), x * w)
-    assert_close(ops.mul(x.to(dev), r.to(dev)), x * r)
+    assert_each(ops.mul(x.to(dev), w.to(dev)), x * w)
+    assert_each(ops.mul(x.to(dev), r.to(dev)), x * r)
     # type promotion is the caller's: bf16 + fp32 -> fp32 out
-    assert_close(ops.add(x.to(dev), a[:, 0, :1].expand(6, 1).repeat(11, 96)[:64].to(dev)),
+    assert_each(ops.add(x.to(dev), a[:, 0, :1].expand(6, 1).repeat(11, 96)[:64].to(dev)),
                  x + a[:, 0, :1].expand(6, 1).repeat(11, 96)[:64])
     # in-place variants, also on a non-contiguous destination
     y = x.clone().to(dev)
     ops.add_(y, w.to(dev), alpha=2)
-    assert_close(y, x + 2 * w)
+    assert_each(y, x + 2 * w)
     z = at.clone().to(dev)
     ops.mul_(z.t(), at.to(dev).t())
-    assert_close(z, at * at)
+    assert_each(z, at * at)
     # integers
     i1 = torch.randint(-100, 100, (50, 3), generator=g(8))
     i2 = torch.randint(-100, 100, (50, 3), generator=g(9))
@@ -66,19 +66,19 @@ def test_column_slices_of_a_wider_matrix(ops, dev, dtype):
         gate, up = view[..., :ffn], view[..., ffn:]
         dgate, dup = dview[..., :ffn], dview[..., ffn:]
         assert not dgate.is_contiguous()
-        assert_close(ops.silu_mul(dgate, dup), (oracle.silu(gate).float() * up.float()).to(dtype))
-        assert_close(ops.add(dgate, dup, alpha=0.5), oracle.add(gate, up, alpha=0.5))
-        assert_close(ops.mul(dgate, dup), oracle.mul(gate, up))
-        assert_close(ops.silu(dup), oracle.silu(up))
+        assert_each(ops.silu_mul(dgate, dup), (oracle.silu(gate).float() * up.float()).to(dtype))
+        assert_each(ops.add(dgate, dup, alpha=0.5), oracle.add(gate, up, alpha=0.5))
+        assert_each(ops.mul(dgate, dup), oracle.mul(gate, up))
+        assert_each(ops.silu(dup), oracle.silu(up))
     # strided output (and untouched neighbours), in-place on a slice, copy out of / into a slice
     dst = torch.zeros(240, 2 * ffn, dtype=dtype, device=dev)
     a2, b2 = gu.reshape(240, 2 * ffn)[:, :ffn], gu.reshape(240, 2 * ffn)[:, ffn:]
     ops.mul(dgu.reshape(240, 2 * ffn)[:, :ffn], dgu.reshape(240, 2 * ffn)[:, ffn:], out=dst[:, ffn:])
-    assert_close(dst[:, ffn:], oracle.mul(a2, b2))
+    assert_each(dst[:, ffn:], oracle.mul(a2, b2))
     assert_exact(dst[:, :ffn], torch.zeros(240, ffn, dtype=dtype))
     work = dgu.reshape(240, 2 * ffn).clone()
     ops.add_(work[:, :ffn], work[:, ffn:])
-    assert_close(work[:, :ffn], oracle.add(a2, b2))
+    assert_each(work[:, :ffn], oracle.add(a2, b2))
     assert_exact(work[:, ffn:], b2)
     dense = torch.empty(240, ffn, dtype=dtype, device=dev)
     ops.copy_(dense, dgu.reshape(240, 2 * ffn)[:, ffn:])
@@ -87,23 +87,23 @@ def test_column_slices_of_a_wider_matrix(ops, dev, dtype):
     assert_exact(dst[:, :ffn], b2)
     # a slice whose start is not 16-byte aligned, or whose length is not a whole number of vectors, takes the generic path
     odd = dgu.reshape(240, 2 * ffn)[:, 3:3 + 1001]
-    assert_close(ops.mul(odd, odd), oracle.mul(gu.reshape(240, 2 * ffn)[:, 3:3 + 1001], gu.reshape(240, 2 * ffn)[:, 3:3 + 1001]))
+    assert_each(ops.mul(odd, odd), oracle.mul(gu.reshape(240, 2 * ffn)[:, 3:3 + 1001], gu.reshape(240, 2 * ffn)[:, 3:3 + 1001]))
 
 
 def test_scalar_forms(ops, dev):
     x = torch.randn(100, 3, generator=g(10))
-    assert_close(ops.add(x.to(dev), 1.5), x + 1.5)
-    assert_close(ops.add(x.to(dev), 2, alpha=3), x + 6)
-    assert_close(ops.sub(x.to(dev), 2.0, alpha=0.5), x - 1.0)
-    assert_close(ops.mul(x.to(dev), -2.5), x * -2.5)
-    assert_close(ops.div(x.to(dev), 4.0), x / 4.0)
-    assert_close(ops.add(x.to(dev), torch.tensor(0.25)), x + 0.25)  # CPU 0-dim tensor is peeled to a scalar
+    assert_each(ops.add(x.to(dev), 1.5), x + 1.5)
+    assert_each(ops.add(x.to(dev), 2, alpha=3), x + 6)
+    assert_each(ops.sub(x.to(dev), 2.0, alpha=0.5), x - 1.0)
+    assert_each(ops.mul(x.to(dev), -2.5), x * -2.5)
+    assert_each(ops.div(x.to(dev), 4.0), x / 4.0)
+    assert_each(ops.add(x.to(dev), torch.tensor(0.25)), x + 0.25)  # CPU 0-dim tensor is peeled to a scalar
     xb = x.bfloat16()
     y = xb.clone().to(dev)
     ops.mul_(y, 3.0)
-    assert_close(y, xb * 3.0)
+    assert_each(y, xb * 3.0)
     ops.add_(y, 1)
-    assert_close(y, xb * 3.0 + 1)
+    assert_each(y, xb * 3.0 + 1)
     f = torch.empty(7, 9, dtype=torch.float16, device=dev)
     ops.fill_(f, 2.5)
     assert_exact(f, torch.full((7, 9), 2.5, dtype=torch.float16))
@@ -116,21 +116,21 @@ def test_scalar_forms(ops, dev):
 def test_unary_ops(ops, dev, dtype):
     x = torch.randn(257, 130, generator=g(11)).to(dtype)
     d = x.to(dev)
-    assert_close(ops.silu(d), oracle.silu(x))
-    assert_close(ops.sigmoid(d), torch.sigmoid(x.float()).to(dtype))
-    assert_close(ops.neg(d), -x)
-    assert_close(ops.sin(d), torch.sin(x.float()).to(dtype))
-    assert_close(ops.cos(d), torch.cos(x.float()).to(dtype))
-    assert_close(ops.exp(d), torch.exp(x.float()).to(dtype))
+    assert_each(ops.silu(d), oracle.silu(x))
+    assert_each(ops.sigmoid(d), torch.sigmoid(x.float()).to(dtype))
+    assert_each(ops.neg(d), -x)
+    assert_each(ops.sin(d), torch.sin(x.float()).to(dtype))
+    assert_each(ops.cos(d), torch.cos(x.float()).to(dtype))
+    assert_each(ops.exp(d), torch.exp(x.float()).to(dtype))
     p = (x.abs() + 0.1)
-    assert_close(ops.rsqrt(p.to(dev)), torch.rsqrt(p.float()).to(dtype))
-    assert_close(ops.pow(d, 2), x.float().pow(2).to(dtype))
-    assert_close(ops.pow(p.to(dev), 1.7), p.float().pow(1.7).to(dtype))
+    assert_each(ops.rsqrt(p.to(dev)), torch.rsqrt(p.float()).to(dtype))
+    assert_each(ops.pow(d, 2), x.float().pow(2).to(dtype))
+    assert_each(ops.pow(p.to(dev), 1.7), p.float().pow(1.7).to(dtype))
     y = x.clone().to(dev)
     ops.silu_(y)
-    assert_close(y, oracle.silu(x))
+    assert_each(y, oracle.silu(x))
     u = torch.randn(257, 130, generator=g(12)).to(dtype)
-    assert_close(ops.silu_mul(d, u.to(dev)), (oracle.silu(x).float() * u.float()).to(dtype))
+    assert_each(ops.silu_mul(d, u.to(dev)), (oracle.silu(x).float() * u.float()).to(dtype))
 
 
 def test_known_answers_on_device(ops, dev):

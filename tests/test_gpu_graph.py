@@ -101,3 +101,35 @@ def test_decode_step_replays_from_a_hip_graph(ops, dev, pkg):
             torch.cuda.synchronize()
     del graph
     scope.close()
+
+
+def test_workspace_request_during_capture_is_served_from_the_cache_or_refused(ops, dev, pkg):
+    """While a stream is being captured a workspace request may not reach hipMalloc: a block cached for that stream is
+    handed out, anything else is an error that says what to do, raised before any HIP call is made."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    x = torch.randn(333, 777, device=dev).t()                                # strided input: softmax copies it densely
+    out = torch.empty(777, 333, device=dev)
+    big = torch.randn(2222, 3333, device=dev).t()                            # a size nothing has cached
+    big_out = torch.empty(3333, 2222, device=dev)
+    with torch.cuda.stream(side):
+        warm = ops.WorkspaceScope()
+        with warm:
+            ops.softmax(x, 1, out=out)
+        side.synchronize()
+        warm.close()                                                         # the block is now cached for `side`
+    mallocs = pkg.runtime.cachingStats()["num_device_malloc"]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        scope = ops.WorkspaceScope()
+        with scope:
+            ops.softmax(x, 1, out=out)                                       # served from the cache
+            with pytest.raises(pkg.diopi.DiopiError, match="captured into a graph"):
+                ops.softmax(big, 1, out=big_out)
+    assert pkg.runtime.cachingStats()["num_device_malloc"] == mallocs
+    out.zero_()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.allclose(out.cpu(), torch.softmax(x.cpu(), 1), atol=1e-6)
+    del graph
+    scope.close()

@@ -277,3 +277,54 @@ def test_expandable_segment_over_hip_virtual_memory(rt):
         seg.close()
     with pytest.raises(RuntimeError, match="granularity"):
         rt.ExpandableSegment(3000)
+
+
+def test_ops_emit_roctx_ranges_while_the_profiler_is_on(pkg, ops, dev):
+    """devapis::enableProfiler switches named ranges on around every op call, as the generated wrappers'
+    RecordBlockCreator does (dipu/scripts/autogen_diopi_wrapper/autogen_diopi_wrapper.py:1013-1016), and on a ROCm
+    machine they reach the ROCTX library (what rocprofv3 --marker-trace reads)."""
+    rt = pkg.runtime
+    a = torch.randn(64, 64, device=dev)
+    s0, e0, _ = rt.profilerCounts()
+    ops.add(a, a)
+    assert rt.profilerCounts()[:2] == (s0, e0)              # off: nothing recorded
+    rt.enableProfiler("")
+    try:
+        ops.add(a, a)
+        ops.softmax(a, -1)
+        with pytest.raises(pkg.diopi.DiopiError):
+            ops.mm(a, torch.randn(3, 3, device=dev), out=torch.empty(64, 3, device=dev))   # a failing op still ends its range
+        s1, e1, bound = rt.profilerCounts()
+        assert (s1 - s0, e1 - e0) == (3, 3)
+        assert bound, "no ROCTX library could be bound on a ROCm machine"
+    finally:
+        rt.disableProfiler()
+    ops.add(a, a)
+    assert rt.profilerCounts()[:2] == (s1, e1)
+    torch.cuda.synchronize()
+
+
+def test_allocator_metrics_through_the_caching_allocator(pkg, dev):
+    """dipu/tests/python/individual_scripts/test_metrics.py:41-68: 100 allocations of random size show up as 100 more
+    entries of allocator_size{type="caching", device, method="allocate"} and at least their bytes in its sum."""
+    import random
+    rt = pkg.runtime
+    rnd = random.Random(0)
+    d = str(rt.current_device())
+    key = lambda name, **kw: (name, frozenset({("type", "caching"), ("device", d)} | set(kw.items())))
+    p = rt.cachingMalloc(1000)                              # preheat
+    before = rt.metrics()
+    sizes = [rnd.randrange(1, 100000) for _ in range(100)]
+    ptrs = [rt.cachingMalloc(n) for n in sizes]
+    after = rt.metrics()
+    count = after[key("allocator_size_count", method="allocate")] - before[key("allocator_size_count", method="allocate")]
+    total = after[key("allocator_size_sum", method="allocate")] - before[key("allocator_size_sum", method="allocate")]
+    assert count == 100 and total >= sum(sizes)
+    for q in ptrs + [p]:
+        rt.cachingFree(q)
+    done = rt.metrics()
+    assert done[key("allocator_size_count", method="deallocate")] - before.get(key("allocator_size_count", method="deallocate"), 0) == 101
+    assert done[key("allocator_event_count", method="deallocate", event="unexpected")] == before[key("allocator_event_count", method="deallocate", event="unexpected")]
+    # the raw vendor calls underneath are counted under type "device"
+    dkey = ("allocator_size_count", frozenset({("type", "device"), ("device", d), ("method", "allocate")}))
+    assert done[dkey] >= 1

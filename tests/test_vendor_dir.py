@@ -1,0 +1,67 @@
+"""The vendor directory DIPU expects (deeplink.framework_amd/vendor/amd/): every link-required symbol is defined, and,
+where a DIPU tree and libtorch headers are at hand (this container, not the GPU box), the files that depend only on
+headers still compatible with the installed torch parse against DIPU's own declarations."""
+import os
+import re
+import shutil
+import subprocess
+import tempfile
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+VENDOR = os.path.join(ROOT, "deeplink.framework_amd", "vendor", "amd")
+DIPU = "/root/reference/dipu/torch_dipu"
+
+# dipu/torch_dipu/csrc_dipu/runtime/device/diclapis.h:17-82: the DIPU_API (non-weak) declarations
+DICL_REQUIRED = ["DICL_UNIQUE_ID_BYTES_SIZE", "diclGetCommAsyncError", "diclGetUniqueId", "diclCommInitRank", "diclCommDestroy",
+                 "diclAllReduce", "diclBroadcast", "diclAllGather", "diclReduce", "diclReduceScatter", "diclSend", "diclRecv"]
+
+
+def _text(name):
+    return open(os.path.join(VENDOR, name)).read()
+
+
+def test_vendor_directory_is_complete():
+    for f in ["vendorapi.h", "deviceimpl.cpp", "communicatorimpl.cpp", "AMDGeneratorImpl.cpp", "AMDCopyInplace.cpp",
+              "AMDExpandableSegment.cpp", "vendor_autocast.h", "CMakeLists.txt"]:
+        assert os.path.isfile(os.path.join(VENDOR, f)), f
+    comm = re.sub(r"//.*", "", _text("communicatorimpl.cpp"))
+    for sym in DICL_REQUIRED:
+        assert re.search(r"\b" + sym + r"\b\s*(\(|=)", comm), sym
+    assert comm.count("return DICL_ERR_UNDEF;") == 11
+    assert re.search(r"const at::Generator vendorMakeGenerator\(at::DeviceIndex", _text("AMDGeneratorImpl.cpp"))
+    assert "setDipuCopyInstance(&amd_copy_inplace)" in _text("AMDCopyInplace.cpp")
+    assert re.search(r"ExpandableSegment\* vendorCreateExpandableSegment\(int device, deviceStream_t stream, size_t size,\s*std::vector<int> peers\)",
+                     _text("AMDExpandableSegment.cpp"))
+    api = _text("vendorapi.h")
+    for name in ["deviceStream_t", "deviceEvent_t", "deviceDefaultStreamLiteral", "diclComm_t", "commUniqueId", "DIPU_CALLHIP"]:
+        assert name in api, name
+    cm = _text("CMakeLists.txt")
+    for var in ["VENDOR_INCLUDE_DIRS", "VENDOR_LIB_DIRS", "DIPU_VENDOR_LIB", "VENDOR_FILES"]:
+        assert re.search(r"set\(" + var + r"\b[^)]*PARENT_SCOPE\)", cm), var
+    # the device functions are the runtime library's own bodies, compiled against DIPU's declarations
+    assert '#include "runtime/deviceimpl.cpp"' in _text("deviceimpl.cpp")
+    assert os.path.isfile(os.path.join(VENDOR, "runtime", "deviceimpl.cpp"))
+
+
+@pytest.mark.skipif(not os.path.isdir(DIPU) or shutil.which("g++") is None, reason="needs a DIPU tree and g++")
+def test_vendor_files_parse_against_dipu_headers():
+    import torch
+    ti = os.path.join(os.path.dirname(torch.__file__), "include")
+    if not os.path.isdir(ti) or not os.path.isdir("/opt/rocm/include"):
+        pytest.skip("libtorch or HIP headers missing")
+    with tempfile.TemporaryDirectory() as tmp:
+        # DIPU's build copies the chosen vendor's vendorapi.h to csrc_dipu/vendor/vendorapi.h
+        os.makedirs(os.path.join(tmp, "csrc_dipu", "vendor"))
+        shutil.copy(os.path.join(VENDOR, "vendorapi.h"), os.path.join(tmp, "csrc_dipu", "vendor", "vendorapi.h"))
+        base = ["g++", "-std=c++17", "-fsyntax-only", "-D__HIP_PLATFORM_AMD__", "-DDIPU_TORCH_VERSION=20101", f"-I{tmp}", f"-I{DIPU}",
+                f"-I{os.path.join(ROOT, 'include')}", f"-I{ti}", f"-I{ti}/torch/csrc/api/include", "-I/opt/rocm/include", f"-I{VENDOR}",
+                f"-I{os.path.join(VENDOR, 'runtime')}"]
+        # AMDCopyInplace.cpp is left out: DIPUCopy.hpp pulls in DIPU's allocator headers, which no longer match the
+        # installed torch (c10::Allocator::allocate changed after 2.2)
+        files = ["deviceimpl.cpp", "communicatorimpl.cpp", "AMDGeneratorImpl.cpp", "AMDExpandableSegment.cpp"]
+        procs = [(f, subprocess.Popen(base + [os.path.join(VENDOR, f)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)) for f in files]
+        for f, p in procs:
+            out, _ = p.communicate(timeout=300)
+            assert p.returncode == 0, f + "\n" + out[-3000:]
