@@ -40,6 +40,7 @@
 // tiles, 4x4 outputs per lane, fp32 accumulate.
 #include <algorithm>
 #include <type_traits>
+#include <utility>
 
 #include "gemm.hpp"
 
@@ -317,6 +318,203 @@ __device__ __forceinline__ void loadToLds16(u32x4 rsrc, int voffset, int soffset
 // embedding on the leading rotCols columns (the q and k heads of a stacked QKV projection).
 enum PipeEpilogue { kEpiLinear = 0, kEpiSiluMul = 1, kEpiPartial = 2, kEpiRotary = 3 };
 
+template <int... Is, typename F>
+__device__ __forceinline__ void staticForImpl(std::integer_sequence<int, Is...>, F&& f) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+// f(std::integral_constant<int, 0>{}) ... f(std::integral_constant<int, N - 1>{}): a loop whose index is a constant
+// expression in the body (register names of inline assembly, array indices that must not become run-time).
+template <int N, typename F>
+__device__ __forceinline__ void staticFor(F&& f) {
+  staticForImpl(std::make_integer_sequence<int, N>{}, f);
+}
+
+// The vector epilogue of the 256 x 256 kernels: a wave's TM x TN fragments of 16 x 16 (v_mfma_f32_16x16x32 with the
+// weight fragment first, so lane (frow = l & 15, kq = l >> 4) holds columns 4 kq .. 4 kq + 3 of row frow of every
+// fragment) whose first row is row0 and first column colBase; accRow(ic, row) hands over the TN accumulators of
+// fragment row ic (a std::integral_constant), one fragment row at a time, so the accumulators may live anywhere.
+//
+// Straight from the accumulators: v_permlane16_swap between the two fragments of a 32-column pair leaves a lane
+// with 8 consecutive columns (lane group q gets the columns starting at 16 * (q & 1) + 8 * (q >> 1)),
+// so the addend is read and the result written as 16-byte pieces, 64 contiguous bytes per row and
+// instruction, without a trip through LDS. alpha / beta / bias are applied in fp32 after the swap.
+// Output and addend go through buffer descriptors (the host guarantees both span less than 2 GiB):
+// a piece outside the matrix gets an offset past the end, which the hardware drops (stores) or
+// answers with zeros (loads), so the instruction stream has no branches and the compiler can count
+// outstanding accesses exactly. Loads and stores share one in-order counter: a wait for an addend
+// piece also waits for every store before it, so the pieces of four fragment rows are requested
+// together before the first store of the four (one exposed round trip per four rows instead of one per
+// row), and without an addend there is no load (and no wait) in the stream.
+template <typename T, int EPI, int TM, int TN, typename AccRow>
+__device__ __forceinline__ void vectorEpilogue(const MfmaArgs& g, T* out, const T* cin, const T* bias, int row0, int colBase,
+                                               int frow, int kq, AccRow&& accRow) {
+  using Frag = typename MfmaOp<T>::Frag;
+  static_assert(TM % 4 == 0 && TN % 4 == 0, "rows are handled four at a time, columns in pairs of fragments");
+  const int cperm = (kq & 1) * 16 + (kq >> 1) * 8;
+  auto swapPair = [](f32x4& x0, f32x4& x1) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(x0[r]), __float_as_uint(x1[r]), false, false);
+      x0[r] = __uint_as_float(sw[0]);
+      x1[r] = __uint_as_float(sw[1]);
+    }
+  };
+  constexpr int kOutside = (int)0x80000000u;
+  constexpr int OW = EPI == kEpiSiluMul ? 2 : 1;  // input columns per output column
+  const int outCols = g.N / OW;
+  const __amdgpu_buffer_rsrc_t rsOut =
+      __builtin_amdgcn_make_buffer_rsrc(out, 0, (int)(((int64_t)(g.M - 1) * g.ldo + outCols) * sizeof(T)), 0x00020000);
+  const int col0 = colBase / OW + cperm;  // this lane's first output column
+  auto offsetOf = [&](int i, int jp, int64_t pitch) {
+    const int row = row0 + i * 16 + frow, col = col0 + jp * 32;
+    return row < g.M && col < outCols ? (int)(((int64_t)row * pitch + col) * sizeof(T)) : kOutside;
+  };
+  auto put = [&](int i, int jp, const Frag& o) {
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o), rsOut, offsetOf(i, jp, g.ldo), 0, 0);
+  };
+  if constexpr (EPI == kEpiSiluMul) {
+    // every 64 columns of a wave are one block: fragments 0, 1 are gate, 2, 3 the up values of the same 32 channels
+    staticFor<TM>([&](auto ic) {
+      constexpr int i = decltype(ic)::value;
+      f32x4 a[TN];
+      accRow(ic, a);
+#pragma unroll
+      for (int hb = 0; hb < TN / 4; ++hb) {
+        f32x4 x0, x1;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float g0 = a[4 * hb][r], g1 = a[4 * hb + 1][r];
+          x0[r] = g0 / (1.f + __expf(-g0)) * a[4 * hb + 2][r];
+          x1[r] = g1 / (1.f + __expf(-g1)) * a[4 * hb + 3][r];
+        }
+        swapPair(x0, x1);
+        Frag o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = static_cast<T>(x0[e]), o[4 + e] = static_cast<T>(x1[e]);
+        put(i, hb, o);
+      }
+    });
+  } else if constexpr (EPI == kEpiRotary) {
+    // A lane's 8 consecutive columns are 4 adjacent pairs of one head; their angles are 4 consecutive table
+    // entries of the lane's row. Pieces at or past rotCols (the v heads) pass through with cos = 1, sin = 0.
+    float bv[TN / 2][8];
+    int pair0[TN / 2];
+    bool rot[TN / 2];
+#pragma unroll
+    for (int jp = 0; jp < TN / 2; ++jp) {
+      const int col = min(col0 + jp * 32, g.N - 8);
+      Frag b8;
+      if (bias) b8 = *reinterpret_cast<const Frag*>(bias + col);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) bv[jp][e] = bias ? static_cast<float>(b8[e]) : 0.f;
+      rot[jp] = col < g.rotCols;
+      pair0[jp] = (col % g.rotHeadDim) >> 1;
+    }
+    const int half = g.rotHeadDim >> 1;
+    const int tsz = g.rotTableF32 ? 4 : (int)sizeof(T);
+    const __amdgpu_buffer_rsrc_t rsCos = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<void*>(g.rotCos), 0, (int)((int64_t)g.rotTableRows * half * tsz), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsSin = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<void*>(g.rotSin), 0, (int)((int64_t)g.rotTableRows * half * tsz), 0x00020000);
+    // Table entries are requested four fragment rows at a time,
+    // before any store of the batch: a request one row ahead would expose the L2 round trip once per row.
+    float cs[4][TN / 2][4], sn[4][TN / 2][4];
+    auto fetch = [&](int i) {
+      const int row = row0 + i * 16 + frow;
+#pragma unroll
+      for (int jp = 0; jp < TN / 2; ++jp) {
+        const int off = row < g.M ? ((row % g.rotTableRows) * half + pair0[jp]) * tsz : kOutside;
+        if (g.rotTableF32) {
+          const u32x4 c4 = __builtin_amdgcn_raw_buffer_load_b128(rsCos, off, 0, 0);
+          const u32x4 s4 = __builtin_amdgcn_raw_buffer_load_b128(rsSin, off, 0, 0);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) cs[i & 3][jp][e] = __uint_as_float(c4[e]), sn[i & 3][jp][e] = __uint_as_float(s4[e]);
+        } else {
+          typedef T T4 __attribute__((ext_vector_type(4)));
+          const T4 c4 = __builtin_bit_cast(T4, __builtin_amdgcn_raw_buffer_load_b64(rsCos, off, 0, 0));
+          const T4 s4 = __builtin_bit_cast(T4, __builtin_amdgcn_raw_buffer_load_b64(rsSin, off, 0, 0));
+#pragma unroll
+          for (int e = 0; e < 4; ++e) cs[i & 3][jp][e] = static_cast<float>(c4[e]), sn[i & 3][jp][e] = static_cast<float>(s4[e]);
+        }
+      }
+    };
+    staticFor<TM>([&](auto ic) {
+      constexpr int i = decltype(ic)::value;
+      if constexpr (i % 4 == 0) {
+#pragma unroll
+        for (int ii = i; ii < i + 4; ++ii) fetch(ii);
+      }
+      f32x4 a[TN];
+      accRow(ic, a);
+#pragma unroll
+      for (int jp = 0; jp < TN / 2; ++jp) {
+        f32x4 x0 = a[2 * jp], x1 = a[2 * jp + 1];
+        swapPair(x0, x1);
+        const float v[8] = {x0[0] + bv[jp][0], x0[1] + bv[jp][1], x0[2] + bv[jp][2], x0[3] + bv[jp][3],
+                            x1[0] + bv[jp][4], x1[1] + bv[jp][5], x1[2] + bv[jp][6], x1[3] + bv[jp][7]};
+        Frag o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float c = rot[jp] ? cs[i & 3][jp][e] : 1.f;
+          const float sv = rot[jp] ? sn[i & 3][jp][e] * g.rotSinSign : 0.f;
+          o[2 * e] = static_cast<T>(v[2 * e] * c - v[2 * e + 1] * sv);
+          o[2 * e + 1] = static_cast<T>(v[2 * e] * sv + v[2 * e + 1] * c);
+        }
+        put(i, jp, o);
+      }
+    });
+  } else {
+    float bv[TN / 2][8];
+#pragma unroll
+    for (int jp = 0; jp < TN / 2; ++jp) {
+      const int col = min(col0 + jp * 32, g.N - 8);  // N % 8 == 0 here; a clamped piece is never stored
+      Frag b8;
+      if (bias) b8 = *reinterpret_cast<const Frag*>(bias + col);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) bv[jp][e] = bias ? static_cast<float>(b8[e]) : 0.f;
+    }
+    auto store = [&](auto withAddend) {
+      constexpr bool kAddend = decltype(withAddend)::value;
+      const __amdgpu_buffer_rsrc_t rsC = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<T*>(kAddend ? cin : out), 0, (int)(((int64_t)(g.M - 1) * g.sCm + g.N) * sizeof(T)), 0x00020000);
+      u32x4 cv[4][TN / 2];
+      auto fetch = [&](int i) {
+#pragma unroll
+        for (int jp = 0; jp < TN / 2; ++jp) cv[i & 3][jp] = __builtin_amdgcn_raw_buffer_load_b128(rsC, offsetOf(i, jp, g.sCm), 0, 0);
+      };
+      staticFor<TM>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        if constexpr (kAddend && i % 4 == 0) {
+#pragma unroll
+          for (int ii = i; ii < i + 4; ++ii) fetch(ii);
+        }
+        f32x4 a[TN];
+        accRow(ic, a);
+#pragma unroll
+        for (int jp = 0; jp < TN / 2; ++jp) {
+          f32x4 x0 = a[2 * jp], x1 = a[2 * jp + 1];
+          swapPair(x0, x1);
+          const float v[8] = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+          Frag o, c8;
+          if constexpr (kAddend) c8 = __builtin_bit_cast(Frag, cv[i & 3][jp]);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            float x = v[e] * g.alpha + bv[jp][e];
+            if constexpr (kAddend) x += g.beta * static_cast<float>(c8[e]);
+            o[e] = static_cast<T>(x);
+          }
+          put(i, jp, o);
+        }
+      });
+    };
+    if (cin)
+      store(std::true_type{});
+    else
+      store(std::false_type{});
+  }
+}
+
+
 template <typename T, int EPI>
 __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs g) {
   using Frag = typename MfmaOp<T>::Frag;
@@ -522,175 +720,10 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
   const T* cin = g.Cin ? reinterpret_cast<const T*>(g.Cin) + (int64_t)batch * g.sCb : nullptr;
   const T* bias = reinterpret_cast<const T*>(g.bias);
   if (g.vecEpilogue) {
-    // Straight from the accumulators. A lane holds 4 consecutive columns of one row in each 16-column
-    // fragment; v_permlane16_swap between the two fragments of a 32-column pair leaves it with 8
-    // consecutive columns instead (lane group q gets the columns starting at 16 * (q & 1) + 8 * (q >> 1)),
-    // so the addend is read and the result written as 16-byte pieces, 64 contiguous bytes per row and
-    // instruction, without a trip through LDS. alpha / beta / bias are applied in fp32 after the swap.
-    // Output and addend go through buffer descriptors (the host guarantees both span less than 2 GiB):
-    // a piece outside the matrix gets an offset past the end, which the hardware drops (stores) or
-    // answers with zeros (loads), so the instruction stream has no branches and the compiler can count
-    // outstanding accesses exactly. Loads and stores share one in-order counter: a wait for an addend
-    // piece also waits for every store before it, so the pieces of four fragment rows are requested
-    // together before the first store of the four (one exposed round trip per four rows instead of one per
-    // row), and without an addend there is no load (and no wait) in the stream.
-    const int cperm = (kq & 1) * 16 + (kq >> 1) * 8;
-    auto swapPair = [](f32x4& x0, f32x4& x1) {
+    vectorEpilogue<T, EPI, TM, TN>(g, out, cin, bias, tm * BM + wm * WM, tn * BN + wn * WN, frow, kq, [&](auto ic, f32x4(&row)[TN]) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(x0[r]), __float_as_uint(x1[r]), false, false);
-        x0[r] = __uint_as_float(sw[0]);
-        x1[r] = __uint_as_float(sw[1]);
-      }
-    };
-    constexpr int kOutside = (int)0x80000000u;
-    constexpr int OW = EPI == kEpiSiluMul ? 2 : 1;  // input columns per output column
-    const int outCols = g.N / OW;
-    const __amdgpu_buffer_rsrc_t rsOut =
-        __builtin_amdgcn_make_buffer_rsrc(out, 0, (int)(((int64_t)(g.M - 1) * g.ldo + outCols) * sizeof(T)), 0x00020000);
-    const int col0 = (tn * BN + wn * WN) / OW + cperm;  // this lane's first output column
-    auto offsetOf = [&](int i, int jp, int64_t pitch) {
-      const int row = tm * BM + wm * WM + i * 16 + frow, col = col0 + jp * 32;
-      return row < g.M && col < outCols ? (int)(((int64_t)row * pitch + col) * sizeof(T)) : kOutside;
-    };
-    auto put = [&](int i, int jp, const Frag& o) {
-      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o), rsOut, offsetOf(i, jp, g.ldo), 0, 0);
-    };
-    if constexpr (EPI == kEpiSiluMul) {
-      // fragments 0, 1 of a wave are gate, 2, 3 the up values of the same 32 channels
-      static_assert(WN == 64, "a wave's columns are one 32 + 32 gate / up block");
-#pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        f32x4 x0, x1;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float g0 = acc[i][0][r], g1 = acc[i][1][r];
-          x0[r] = g0 / (1.f + __expf(-g0)) * acc[i][2][r];
-          x1[r] = g1 / (1.f + __expf(-g1)) * acc[i][3][r];
-        }
-        swapPair(x0, x1);
-        Frag o;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = static_cast<T>(x0[e]), o[4 + e] = static_cast<T>(x1[e]);
-        put(i, 0, o);
-      }
-    } else if constexpr (EPI == kEpiRotary) {
-      // A lane's 8 consecutive columns are 4 adjacent pairs of one head; their angles are 4 consecutive table
-      // entries of the lane's row. Pieces at or past rotCols (the v heads) pass through with cos = 1, sin = 0.
-      float bv[TN / 2][8];
-      int pair0[TN / 2];
-      bool rot[TN / 2];
-#pragma unroll
-      for (int jp = 0; jp < TN / 2; ++jp) {
-        const int col = min(col0 + jp * 32, g.N - 8);
-        Frag b8;
-        if (bias) b8 = *reinterpret_cast<const Frag*>(bias + col);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) bv[jp][e] = bias ? static_cast<float>(b8[e]) : 0.f;
-        rot[jp] = col < g.rotCols;
-        pair0[jp] = (col % g.rotHeadDim) >> 1;
-      }
-      const int half = g.rotHeadDim >> 1;
-      const int tsz = g.rotTableF32 ? 4 : (int)sizeof(T);
-      const __amdgpu_buffer_rsrc_t rsCos = __builtin_amdgcn_make_buffer_rsrc(
-          const_cast<void*>(g.rotCos), 0, (int)((int64_t)g.rotTableRows * half * tsz), 0x00020000);
-      const __amdgpu_buffer_rsrc_t rsSin = __builtin_amdgcn_make_buffer_rsrc(
-          const_cast<void*>(g.rotSin), 0, (int)((int64_t)g.rotTableRows * half * tsz), 0x00020000);
-      // Table entries are requested four fragment rows at a time,
-      // before any store of the batch: a request one row ahead would expose the L2 round trip once per row.
-      float cs[TM][TN / 2][4], sn[TM][TN / 2][4];
-      auto fetch = [&](int i) {
-        const int row = tm * BM + wm * WM + i * 16 + frow;
-#pragma unroll
-        for (int jp = 0; jp < TN / 2; ++jp) {
-          const int off = row < g.M ? ((row % g.rotTableRows) * half + pair0[jp]) * tsz : kOutside;
-          if (g.rotTableF32) {
-            const u32x4 c4 = __builtin_amdgcn_raw_buffer_load_b128(rsCos, off, 0, 0);
-            const u32x4 s4 = __builtin_amdgcn_raw_buffer_load_b128(rsSin, off, 0, 0);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) cs[i][jp][e] = __uint_as_float(c4[e]), sn[i][jp][e] = __uint_as_float(s4[e]);
-          } else {
-            typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
-            typedef T T4 __attribute__((ext_vector_type(4)));
-            const T4 c4 = __builtin_bit_cast(T4, __builtin_amdgcn_raw_buffer_load_b64(rsCos, off, 0, 0));
-            const T4 s4 = __builtin_bit_cast(T4, __builtin_amdgcn_raw_buffer_load_b64(rsSin, off, 0, 0));
-#pragma unroll
-            for (int e = 0; e < 4; ++e) cs[i][jp][e] = static_cast<float>(c4[e]), sn[i][jp][e] = static_cast<float>(s4[e]);
-          }
-        }
-      };
-#pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        if (i % 4 == 0) {
-#pragma unroll
-          for (int ii = i; ii < i + 4; ++ii) fetch(ii);
-        }
-#pragma unroll
-        for (int jp = 0; jp < TN / 2; ++jp) {
-          f32x4 x0 = acc[i][2 * jp], x1 = acc[i][2 * jp + 1];
-          swapPair(x0, x1);
-          const float v[8] = {x0[0] + bv[jp][0], x0[1] + bv[jp][1], x0[2] + bv[jp][2], x0[3] + bv[jp][3],
-                              x1[0] + bv[jp][4], x1[1] + bv[jp][5], x1[2] + bv[jp][6], x1[3] + bv[jp][7]};
-          Frag o;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float c = rot[jp] ? cs[i][jp][e] : 1.f;
-            const float sv = rot[jp] ? sn[i][jp][e] * g.rotSinSign : 0.f;
-            o[2 * e] = static_cast<T>(v[2 * e] * c - v[2 * e + 1] * sv);
-            o[2 * e + 1] = static_cast<T>(v[2 * e] * sv + v[2 * e + 1] * c);
-          }
-          put(i, jp, o);
-        }
-      }
-    } else {
-      float bv[TN / 2][8];
-#pragma unroll
-      for (int jp = 0; jp < TN / 2; ++jp) {
-        const int col = min(col0 + jp * 32, g.N - 8);  // N % 8 == 0 here; a clamped piece is never stored
-        Frag b8;
-        if (bias) b8 = *reinterpret_cast<const Frag*>(bias + col);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) bv[jp][e] = bias ? static_cast<float>(b8[e]) : 0.f;
-      }
-      auto store = [&](auto withAddend) {
-        constexpr bool kAddend = decltype(withAddend)::value;
-        const __amdgpu_buffer_rsrc_t rsC = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<T*>(kAddend ? cin : out), 0, (int)(((int64_t)(g.M - 1) * g.sCm + g.N) * sizeof(T)), 0x00020000);
-        u32x4 cv[TM][TN / 2];
-        auto fetch = [&](int i) {
-#pragma unroll
-          for (int jp = 0; jp < TN / 2; ++jp)
-            cv[i][jp] = __builtin_amdgcn_raw_buffer_load_b128(rsC, offsetOf(i, jp, g.sCm), 0, 0);
-        };
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-          if constexpr (kAddend)
-            if (i % 4 == 0) {
-#pragma unroll
-              for (int ii = i; ii < i + 4; ++ii) fetch(ii);
-            }
-#pragma unroll
-          for (int jp = 0; jp < TN / 2; ++jp) {
-            f32x4 x0 = acc[i][2 * jp], x1 = acc[i][2 * jp + 1];
-            swapPair(x0, x1);
-            const float v[8] = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
-            Frag o, c8;
-            if constexpr (kAddend) c8 = __builtin_bit_cast(Frag, cv[i][jp]);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-              float x = v[e] * g.alpha + bv[jp][e];
-              if constexpr (kAddend) x += g.beta * static_cast<float>(c8[e]);
-              o[e] = static_cast<T>(x);
-            }
-            put(i, jp, o);
-          }
-        }
-      };
-      if (cin)
-        store(std::true_type{});
-      else
-        store(std::false_type{});
-    }
+      for (int j = 0; j < TN; ++j) row[j] = acc[decltype(ic)::value][j];
+    });
     return;
   }
   // element-wise stores for outputs that do not allow 16-byte pieces; the addend of a fragment row is
@@ -729,6 +762,113 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
     storeScalar(std::true_type{});
   else
     storeScalar(std::false_type{});
+}
+
+
+// ------------------------------------------------------- 4 waves, hand-placed K loop ---
+// The same 256 x 256 x 64 macro tile with 4 waves (2 x 2, wave tile 128 x 128 = 8 x 8 tiles of
+// v_mfma_f32_16x16x32, 256 accumulators per lane in the accumulation registers): a third fewer LDS fragment reads per
+// MFMA than the 8-wave form (16 per 64 instead of 12 per 32), which is what the kernel pays for in clock at the power
+// limit. One wave per SIMD means that nothing hides a stall, so the K loop is generated text (gemm_loop_4wave.inc,
+// written by gen_gemm_loop_4wave.py, which documents the schedule): tile loads straight into a two-stage LDS ring,
+// fragment reads one k-step ahead into fixed registers, one barrier per K tile. Needs an even number of K tiles and
+// the vector epilogue; everything else stays with the 8-wave kernel.
+#include "gemm_loop_4wave.inc"
+
+template <int R>
+__device__ __forceinline__ float accRegister() {
+  float v;
+  asm volatile("v_accvgpr_read_b32 %0, a[%1:%1]" : "=v"(v) : "n"(R));
+  return v;
+}
+
+template <typename T, int EPI>
+__global__ __launch_bounds__(256) void gemmMfma4WaveKernel(MfmaArgs g) {
+  constexpr int BM = 256, BN = 256, WM = 128, WN = 128, TM = 8, TN = 8;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  int tm, tn;
+  {
+    const int total = g.tilesM * g.tilesN;
+    const int pid = blockIdx.x;
+    const int xcd = pid & 7, idx = pid >> 3;
+    const int q = total >> 3, r = total & 7;
+    const int logical = xcd * q + min(xcd, r) + idx;
+    constexpr int GROUP = 8;
+    const int width = GROUP * g.tilesN;
+    const int group = logical / width;
+    const int first = group * GROUP;
+    const int gsize = min(g.tilesM - first, GROUP);
+    const int in = logical - group * width;
+    tm = first + in % gsize;
+    tn = in / gsize;
+  }
+  const int batch = blockIdx.z;
+  const T* A = reinterpret_cast<const T*>(g.A) + (int64_t)batch * g.sAb;
+  const T* B = reinterpret_cast<const T*>(g.B) + (int64_t)batch * g.sBb;
+  // Rows past M / N and columns past K lie beyond the descriptors' extent and read as zeros.
+  auto descriptor = [](const T* base, int64_t bytes) {
+    const uint64_t p = reinterpret_cast<uint64_t>(base);
+    u32x4 d = {(uint32_t)p, (uint32_t)(p >> 32) & 0xffffu, (uint32_t)bytes, 0x00020000u};
+    return d;
+  };
+  const u32x4 rsA = descriptor(A, ((int64_t)(g.M - 1) * g.lda + g.K) * 2);
+  const u32x4 rsB = descriptor(B, ((int64_t)(g.N - 1) * g.ldb + g.K) * 2);
+  // lane l of a wave fills the l-th 16-byte slot of a 1 KiB block (8 rows of 128 bytes); the chunk swizzle
+  // c ^ ((row >> 1) & 7) is applied to the global address. A pass of the workgroup covers 32 rows.
+  const int srow = tid >> 3;
+  const int c8 = ((tid & 7) ^ ((srow >> 1) & 7)) * 8;
+  constexpr unsigned kFar = 0x80000000u;  // beyond every extent: the load returns zeros
+  unsigned voA[8], voB[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int ra = tm * BM + srow + 32 * i, rb = tn * BN + srow + 32 * i;
+    voA[i] = ra < g.M ? (unsigned)(((int64_t)ra * g.lda + c8) * 2) : kFar;
+    voB[i] = rb < g.N ? (unsigned)(((int64_t)rb * g.ldb + c8) * 2) : kFar;
+  }
+  const unsigned base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)smem;
+  const unsigned ldsWave = base + __builtin_amdgcn_readfirstlane(wave) * 1024u;
+  const int frow = lane & 15, kq = lane >> 4, swz = (frow >> 1) & 7;
+  const unsigned adA0 = base + ((wm * WM + frow) * kBK + ((kq ^ swz) << 3)) * 2;
+  const unsigned adA1 = base + ((wm * WM + frow) * kBK + (((4 + kq) ^ swz) << 3)) * 2;
+  const unsigned adB0 = base + 65536 + ((wn * WN + frow) * kBK + ((kq ^ swz) << 3)) * 2;
+  const unsigned adB1 = base + 65536 + ((wn * WN + frow) * kBK + (((4 + kq) ^ swz) << 3)) * 2;
+  const int pairs = g.K / (2 * kBK);
+  unsigned kcur = 0, m0s = 0;
+#define GEMM4W_OPERANDS                                                                                              \
+  : [kcur] "+s"(kcur), [m0s] "+s"(m0s)                                                                               \
+  : [voA0] "v"(voA[0]), [voA1] "v"(voA[1]), [voA2] "v"(voA[2]), [voA3] "v"(voA[3]), [voA4] "v"(voA[4]),              \
+    [voA5] "v"(voA[5]), [voA6] "v"(voA[6]), [voA7] "v"(voA[7]), [voB0] "v"(voB[0]), [voB1] "v"(voB[1]),              \
+    [voB2] "v"(voB[2]), [voB3] "v"(voB[3]), [voB4] "v"(voB[4]), [voB5] "v"(voB[5]), [voB6] "v"(voB[6]),              \
+    [voB7] "v"(voB[7]), [adA0] "v"(adA0), [adA1] "v"(adA1), [adB0] "v"(adB0), [adB1] "v"(adB1), [rsA] "s"(rsA),      \
+    [rsB] "s"(rsB), [lds] "s"(ldsWave)                                                                               \
+  : "memory", "scc", GEMM4W_CLOBBERS
+  if constexpr (std::is_same<T, bf16_t>::value) {
+    asm volatile(GEMM4W_PROLOGUE_BF16 GEMM4W_OPERANDS);
+    for (int p = 1; p < pairs; ++p) asm volatile(GEMM4W_BODY_BF16 GEMM4W_OPERANDS);
+    asm volatile(GEMM4W_TAIL_BF16 GEMM4W_OPERANDS);
+  } else {
+    asm volatile(GEMM4W_PROLOGUE_F16 GEMM4W_OPERANDS);
+    for (int p = 1; p < pairs; ++p) asm volatile(GEMM4W_BODY_F16 GEMM4W_OPERANDS);
+    asm volatile(GEMM4W_TAIL_F16 GEMM4W_OPERANDS);
+  }
+#undef GEMM4W_OPERANDS
+  T* out = reinterpret_cast<T*>(g.out) + (int64_t)batch * g.sOb;
+  const T* cin = g.Cin ? reinterpret_cast<const T*>(g.Cin) + (int64_t)batch * g.sCb : nullptr;
+  const T* bias = reinterpret_cast<const T*>(g.bias);
+  // one fragment row at a time out of the accumulation registers, which the compiler does not know to be live:
+  // the epilogue stays far below the 256 ordinary registers, so it never borrows them
+  vectorEpilogue<T, EPI, TM, TN>(g, out, cin, bias, tm * BM + wm * WM, tn * BN + wn * WN, frow, kq, [&](auto ic, f32x4(&row)[TN]) {
+    constexpr int i = decltype(ic)::value;
+    staticFor<TN>([&](auto jc) {
+      constexpr int j = decltype(jc)::value;
+      row[j][0] = accRegister<4 * (8 * i + j)>();
+      row[j][1] = accRegister<4 * (8 * i + j) + 1>();
+      row[j][2] = accRegister<4 * (8 * i + j) + 2>();
+      row[j][3] = accRegister<4 * (8 * i + j) + 3>();
+    });
+  });
 }
 
 // ------------------------------------------------------------ skinny M (decode) ---
@@ -1166,6 +1306,15 @@ static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p
   dim3 grid((unsigned)(g.tilesM * g.tilesN), (unsigned)splits, (unsigned)p.batch);
   if (EPI == kEpiSiluMul) AMD_CHECK(g.vecEpilogue, "gated linear: output rows must allow 16-byte stores");
   if (EPI == kEpiPartial) AMD_CHECK(g.vecEpilogue && p.batch == 1 && partial, "split-K: needs the vector epilogue and one batch");
+  if constexpr (EPI != kEpiPartial) {
+    // the 4-wave kernel: an even number of K tiles, 16-byte epilogue pieces, lane offsets that fit 31 bits
+    if (g.vecEpilogue && p.K % (2 * kBK) == 0 && p.M * p.sAm * 2 < (int64_t(1) << 31) && p.N * p.sBn * 2 < (int64_t(1) << 31)) {
+      AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmMfma4WaveKernel<T, EPI>), (int)lds));
+      hipLaunchKernelGGL((gemmMfma4WaveKernel<T, EPI>), grid, dim3(256), lds, stream, g);
+      AMD_LAUNCH_CHECK();
+      return diopiSuccess;
+    }
+  }
   hipLaunchKernelGGL((gemmMfmaPipelinedKernel<T, EPI>), grid, dim3(kPipeThreads), lds, stream, g);
   AMD_LAUNCH_CHECK();
   if (EPI == kEpiPartial) {
