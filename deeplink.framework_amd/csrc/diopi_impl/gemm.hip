@@ -775,11 +775,27 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
 // the vector epilogue; everything else stays with the 8-wave kernel.
 #include "gemm_loop_4wave.inc"
 
+// Sixteen consecutive accumulation registers a[R .. R + 15] as four fragments, in one statement: the reads issue back
+// to back, and what follows is ordinary code the compiler may schedule freely (one statement per register would pin
+// every read between its neighbours' dependent arithmetic, which a lone wave per SIMD cannot hide).
 template <int R>
-__device__ __forceinline__ float accRegister() {
-  float v;
-  asm volatile("v_accvgpr_read_b32 %0, a[%1:%1]" : "=v"(v) : "n"(R));
-  return v;
+__device__ __forceinline__ void accRegisters16(f32x4 (&f)[4]) {
+  float v[16];
+  asm volatile(
+      "v_accvgpr_read_b32 %0, a[%16:%16]\n\tv_accvgpr_read_b32 %1, a[%17:%17]\n\tv_accvgpr_read_b32 %2, a[%18:%18]\n\t"
+      "v_accvgpr_read_b32 %3, a[%19:%19]\n\tv_accvgpr_read_b32 %4, a[%20:%20]\n\tv_accvgpr_read_b32 %5, a[%21:%21]\n\t"
+      "v_accvgpr_read_b32 %6, a[%22:%22]\n\tv_accvgpr_read_b32 %7, a[%23:%23]\n\tv_accvgpr_read_b32 %8, a[%24:%24]\n\t"
+      "v_accvgpr_read_b32 %9, a[%25:%25]\n\tv_accvgpr_read_b32 %10, a[%26:%26]\n\tv_accvgpr_read_b32 %11, a[%27:%27]\n\t"
+      "v_accvgpr_read_b32 %12, a[%28:%28]\n\tv_accvgpr_read_b32 %13, a[%29:%29]\n\tv_accvgpr_read_b32 %14, a[%30:%30]\n\t"
+      "v_accvgpr_read_b32 %15, a[%31:%31]"
+      : "=v"(v[0]), "=v"(v[1]), "=v"(v[2]), "=v"(v[3]), "=v"(v[4]), "=v"(v[5]), "=v"(v[6]), "=v"(v[7]), "=v"(v[8]), "=v"(v[9]),
+        "=v"(v[10]), "=v"(v[11]), "=v"(v[12]), "=v"(v[13]), "=v"(v[14]), "=v"(v[15])
+      : "n"(R), "n"(R + 1), "n"(R + 2), "n"(R + 3), "n"(R + 4), "n"(R + 5), "n"(R + 6), "n"(R + 7), "n"(R + 8), "n"(R + 9),
+        "n"(R + 10), "n"(R + 11), "n"(R + 12), "n"(R + 13), "n"(R + 14), "n"(R + 15));
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) f[q][r] = v[4 * q + r];
 }
 
 template <typename T, int EPI>
@@ -861,13 +877,11 @@ __global__ __launch_bounds__(256) void gemmMfma4WaveKernel(MfmaArgs g) {
   // the epilogue stays far below the 256 ordinary registers, so it never borrows them
   vectorEpilogue<T, EPI, TM, TN>(g, out, cin, bias, tm * BM + wm * WM, tn * BN + wn * WN, frow, kq, [&](auto ic, f32x4(&row)[TN]) {
     constexpr int i = decltype(ic)::value;
-    staticFor<TN>([&](auto jc) {
-      constexpr int j = decltype(jc)::value;
-      row[j][0] = accRegister<4 * (8 * i + j)>();
-      row[j][1] = accRegister<4 * (8 * i + j) + 1>();
-      row[j][2] = accRegister<4 * (8 * i + j) + 2>();
-      row[j][3] = accRegister<4 * (8 * i + j) + 3>();
-    });
+    f32x4 lo[4], hi[4];
+    accRegisters16<32 * i>(lo);
+    accRegisters16<32 * i + 16>(hi);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) row[j] = lo[j], row[4 + j] = hi[j];
   });
 }
 

@@ -15,15 +15,22 @@ Operands of each block: %[voA0..7] %[voB0..7]  lane byte offsets of the 8 + 8 ti
                         %[rsA] %[rsB]  buffer descriptors, %[lds] LDS address of this wave's 1 KiB slot in stage 0 of A
                         %[kcur]  K byte offset of the tile whose loads are issued next, %[m0s]  the caller's M0
 
-One tile of the loop (stage s = tile & 1), 128 MFMAs:
-  k-step 0: 64 MFMAs out of fragment buffer 0 | the 16 fragment reads of k-step 1 (stage s) into buffer 1
-  s_waitcnt vmcnt(0) lgkmcnt(0); s_barrier    every wave is done reading stage s, tile t + 1 has landed in stage s ^ 1
-  k-step 1: 64 MFMAs out of buffer 1 | the 16 fragment reads of tile t + 1, k-step 0 into buffer 0
-                                     | the 16 loads of tile t + 2 into stage s, spread over the whole k-step
+One tile of the loop (stage s = tile & 1), 128 MFMAs, two barriers:
+  k-step 0, MFMAs 0-22    out of fragment buffer 0 | the 16 fragment reads of k-step 1 (stage s) into buffer 1, one per MFMA
+  s_waitcnt lgkmcnt(0); s_barrier (B1)    every wave is done reading stage s: it may be refilled
+  k-step 0, MFMAs 23-63   | the loads of tile t + 2 into stage s start here, one per five MFMAs, and run on into k-step 1
+  s_waitcnt vmcnt(loads of tile t + 2 issued so far); s_barrier (B2)    tile t + 1 has landed in stage s ^ 1
+  k-step 1, 64 MFMAs out of buffer 1 | the 16 fragment reads of tile t + 1, k-step 0 into buffer 0 | the rest of the loads
+A load is needed at B2 of the next tile, so the youngest has more than a whole tile (128 MFMAs, about 1.3 us) to
+arrive, at half the issue rate of a schedule that packs the loads between one barrier per tile and the next k-step
+boundary: 16.9 cycles per MFMA against 18.2 on 8192 x 4096 x 11008 (16.3 with no tile loads at all). The kernel runs at
+the power limit, where the cycles saved come back as a lower clock (1.59 against 1.65 GHz, the same time per launch); they
+count when the clock is not what limits it.
 Fragment reads are issued in the order the MFMAs need them (B0, A0..A7, B1..B7; the MFMAs run B-major) and LDS
 returns them in order, so the wait before an MFMA is a count of younger reads that may still be outstanding.
-Measured on 8192 x 4096 x 11008: issuing the loads later (half of them in the next k-step 0) or packed into the
-first half of k-step 1 is 5-10 % slower; every third MFMA slot for the reads against every second: no difference."""
+Measured and not used: K tiles of 32 in a four-stage ring (loads three tiles ahead) is 10 % slower, because a tile
+load then fetches 64-byte row pieces, twice the cache lines per byte; issuing the loads twice as densely (to gain
+slack) stalls the wave at issue."""
 import os
 import sys
 
@@ -62,44 +69,52 @@ def read_fragment(out, kind, idx, buf, stage, ks):
     out.append(f"ds_read_b128 {reg}, %[ad{kind}{ks}] offset:{idx * 2048 + stage * 32768}")
 
 
-def kstep(out, buf, prefetch, load_stage):
-    """64 MFMAs out of fragment buffer `buf`; prefetch = (stage, ks) read into the other buffer or None;
-    load_stage = stage that receives the 16 loads of the tile at %[kcur], or None."""
-    after = {m: [] for m in range(64)}
-    reads_before = [0] * 64
-    if prefetch:
-        slots = [1 + 3 * r for r in range(16)]
-        for r, slot in enumerate(slots):
-            after[slot].append(("read", r))
-        reads_before = [sum(1 for slot in slots if slot < m) for m in range(64)]
-    if load_stage is not None:
-        for d in range(16):
-            slot = 2 + (d * 60) // 16
-            after[slot].append(("m0", d))          # M0 is written one MFMA before the load that reads it
-            after[slot + 1].append(("load", d))
-    waited = -1
-    for j in range(8):
-        for i in range(8):
-            m = j * 8 + i
-            need = READ_ORDER.index(("A", 7)) if j == 0 else READ_ORDER.index(("B", j))
-            if need > waited:
-                out.append(f"s_waitcnt lgkmcnt({min(15 - need + reads_before[m], 15)})")
-                waited = need
-            out.append(f"MFMA {acc(i, j)}, {vb(buf, j)}, {va(buf, i)}, {acc(i, j)}")
-            for what, arg in after[m]:
-                if what == "read":
-                    read_fragment(out, READ_ORDER[arg][0], READ_ORDER[arg][1], 1 - buf, prefetch[0], prefetch[1])
-                elif what == "m0":
-                    load_m0(out, arg, load_stage)
-                else:
-                    load_issue(out, arg)
+B1_SLOT = 22       # B1 follows this MFMA of k-step 0
+LOAD_STEP = 5      # MFMAs between two tile loads
 
 
 def tile(out, s, loads, next_tile):
-    kstep(out, 0, (s, 1), None)
-    out.append("s_waitcnt vmcnt(0) lgkmcnt(0)")
-    out.append("s_barrier")
-    kstep(out, 1, (s ^ 1, 0) if next_tile else None, s if loads else None)
+    """128 MFMAs of one K tile in stage s; loads: issue the 16 loads of tile t + 2; next_tile: read tile t + 1's first
+    fragments during k-step 1."""
+    after = {m: [] for m in range(128)}
+    for r in range(16):                                    # this tile's k-step 1 fragments, right away
+        after[r].append(("read1", r))
+    after[B1_SLOT].append(("B1", None))
+    loads_before_b2 = 0
+    if loads:
+        for d in range(16):
+            slot = B1_SLOT + 1 + d * LOAD_STEP
+            if slot + 1 <= 63:
+                loads_before_b2 += 1
+            after[slot].append(("m0", d))                  # M0 is written one MFMA before the load that reads it
+            after[slot + 1].append(("load", d))
+    if next_tile:
+        for r in range(16):
+            after[65 + 3 * r].append(("read0", r))
+    for m in range(128):
+        ks, mm = divmod(m, 64)
+        j, i = divmod(mm, 8)
+        if m == 0:
+            out.append("s_waitcnt lgkmcnt(7)")             # B0, A0..A7 of buffer 0 (read during the previous k-step 1)
+        elif ks == 0 and i == 0 and j >= 1 and m <= B1_SLOT:
+            # B_j of buffer 0: 7 - j reads of its set are younger, and so are this tile's reads issued so far
+            out.append(f"s_waitcnt lgkmcnt({min(7 - j + min(m, 16), 15)})")
+        if m == 64:
+            out.append(f"s_waitcnt vmcnt({loads_before_b2}) lgkmcnt(0)")
+            out.append("s_barrier")
+        out.append(f"MFMA {acc(i, j)}, {vb(ks, j)}, {va(ks, i)}, {acc(i, j)}")
+        for what, arg in after[m]:
+            if what == "read1":
+                read_fragment(out, READ_ORDER[arg][0], READ_ORDER[arg][1], 1, s, 1)
+            elif what == "read0":
+                read_fragment(out, READ_ORDER[arg][0], READ_ORDER[arg][1], 0, s ^ 1, 0)
+            elif what == "B1":
+                out.append("s_waitcnt lgkmcnt(0)")
+                out.append("s_barrier")
+            elif what == "m0":
+                load_m0(out, arg, s)
+            else:
+                load_issue(out, arg)
 
 
 def prologue(out):

@@ -173,3 +173,13 @@ def test_allocator_metrics_labels_events_and_histogram(pkg):
     rt.metricsRecord(t, dev, 0x9000, 64)
     assert rt.metrics()[key("allocator_size_count", method="allocate")] == 4
     assert rt.metricsEnable(True) is True
+
+
+def test_generated_gemm_loop_is_current(tmp_path):
+    """The committed K loop of the 4-wave GEMM kernel is what its generator writes."""
+    import subprocess
+    import sys
+    d = os.path.join(ROOT, "deeplink.framework_amd", "csrc", "diopi_impl")
+    out = tmp_path / "loop.inc"
+    subprocess.run([sys.executable, os.path.join(d, "gen_gemm_loop_4wave.py"), str(out)], check=True)
+    assert out.read_text() == open(os.path.join(d, "gemm_loop_4wave.inc")).read()
