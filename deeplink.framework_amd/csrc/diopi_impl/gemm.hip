@@ -804,10 +804,11 @@ __global__ __launch_bounds__(256) void gemmMfma4WaveKernel(MfmaArgs g) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  int tm, tn;
-  {
-    const int total = g.tilesM * g.tilesN;
-    const int pid = blockIdx.x;
+  const int total = g.tilesM * g.tilesN;
+  // Persistent: the workgroup takes output tiles blockIdx.x, blockIdx.x + gridDim.x, ... (the grid is a multiple of
+  // 8 or covers every tile, so a workgroup's tiles all belong to the XCD it runs on, as in the one-tile-per-workgroup
+  // order). XCD x works on a contiguous band of tiles, walked in groups of 8 tile rows.
+  auto tileOf = [&](int pid, int& tm, int& tn) {
     const int xcd = pid & 7, idx = pid >> 3;
     const int q = total >> 3, r = total & 7;
     const int logical = xcd * q + min(xcd, r) + idx;
@@ -819,7 +820,7 @@ __global__ __launch_bounds__(256) void gemmMfma4WaveKernel(MfmaArgs g) {
     const int in = logical - group * width;
     tm = first + in % gsize;
     tn = in / gsize;
-  }
+  };
   const int batch = blockIdx.z;
   const T* A = reinterpret_cast<const T*>(g.A) + (int64_t)batch * g.sAb;
   const T* B = reinterpret_cast<const T*>(g.B) + (int64_t)batch * g.sBb;
@@ -837,12 +838,14 @@ __global__ __launch_bounds__(256) void gemmMfma4WaveKernel(MfmaArgs g) {
   const int c8 = ((tid & 7) ^ ((srow >> 1) & 7)) * 8;
   constexpr unsigned kFar = 0x80000000u;  // beyond every extent: the load returns zeros
   unsigned voA[8], voB[8];
+  auto laneOffsets = [&](int tm, int tn) {
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int ra = tm * BM + srow + 32 * i, rb = tn * BN + srow + 32 * i;
-    voA[i] = ra < g.M ? (unsigned)(((int64_t)ra * g.lda + c8) * 2) : kFar;
-    voB[i] = rb < g.N ? (unsigned)(((int64_t)rb * g.ldb + c8) * 2) : kFar;
-  }
+    for (int i = 0; i < 8; ++i) {
+      const int ra = tm * BM + srow + 32 * i, rb = tn * BN + srow + 32 * i;
+      voA[i] = ra < g.M ? (unsigned)(((int64_t)ra * g.lda + c8) * 2) : kFar;
+      voB[i] = rb < g.N ? (unsigned)(((int64_t)rb * g.ldb + c8) * 2) : kFar;
+    }
+  };
   const unsigned base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)smem;
   const unsigned ldsWave = base + __builtin_amdgcn_readfirstlane(wave) * 1024u;
   const int frow = lane & 15, kq = lane >> 4, swz = (frow >> 1) & 7;
@@ -852,6 +855,9 @@ __global__ __launch_bounds__(256) void gemmMfma4WaveKernel(MfmaArgs g) {
   const unsigned adB1 = base + 65536 + ((wn * WN + frow) * kBK + (((4 + kq) ^ swz) << 3)) * 2;
   const int pairs = g.K / (2 * kBK);
   unsigned kcur = 0, m0s = 0;
+  T* out = reinterpret_cast<T*>(g.out) + (int64_t)batch * g.sOb;
+  const T* cin = g.Cin ? reinterpret_cast<const T*>(g.Cin) + (int64_t)batch * g.sCb : nullptr;
+  const T* bias = reinterpret_cast<const T*>(g.bias);
 #define GEMM4W_OPERANDS                                                                                              \
   : [kcur] "+s"(kcur), [m0s] "+s"(m0s)                                                                               \
   : [voA0] "v"(voA[0]), [voA1] "v"(voA[1]), [voA2] "v"(voA[2]), [voA3] "v"(voA[3]), [voA4] "v"(voA[4]),              \
@@ -860,29 +866,48 @@ __global__ __launch_bounds__(256) void gemmMfma4WaveKernel(MfmaArgs g) {
     [voB7] "v"(voB[7]), [adA0] "v"(adA0), [adA1] "v"(adA1), [adB0] "v"(adB0), [adB1] "v"(adB1), [rsA] "s"(rsA),      \
     [rsB] "s"(rsB), [lds] "s"(ldsWave)                                                                               \
   : "memory", "scc", GEMM4W_CLOBBERS
-  if constexpr (std::is_same<T, bf16_t>::value) {
-    asm volatile(GEMM4W_PROLOGUE_BF16 GEMM4W_OPERANDS);
-    for (int p = 1; p < pairs; ++p) asm volatile(GEMM4W_BODY_BF16 GEMM4W_OPERANDS);
-    asm volatile(GEMM4W_TAIL_BF16 GEMM4W_OPERANDS);
-  } else {
-    asm volatile(GEMM4W_PROLOGUE_F16 GEMM4W_OPERANDS);
-    for (int p = 1; p < pairs; ++p) asm volatile(GEMM4W_BODY_F16 GEMM4W_OPERANDS);
-    asm volatile(GEMM4W_TAIL_F16 GEMM4W_OPERANDS);
-  }
-#undef GEMM4W_OPERANDS
-  T* out = reinterpret_cast<T*>(g.out) + (int64_t)batch * g.sOb;
-  const T* cin = g.Cin ? reinterpret_cast<const T*>(g.Cin) + (int64_t)batch * g.sCb : nullptr;
-  const T* bias = reinterpret_cast<const T*>(g.bias);
-  // one fragment row at a time out of the accumulation registers, which the compiler does not know to be live:
-  // the epilogue stays far below the 256 ordinary registers, so it never borrows them
-  vectorEpilogue<T, EPI, TM, TN>(g, out, cin, bias, tm * BM + wm * WM, tn * BN + wn * WN, frow, kq, [&](auto ic, f32x4(&row)[TN]) {
-    constexpr int i = decltype(ic)::value;
-    f32x4 lo[4], hi[4];
-    accRegisters16<32 * i>(lo);
-    accRegisters16<32 * i + 16>(hi);
+#define GEMM4W_RUN(NAME)                                                         \
+  do {                                                                           \
+    if constexpr (std::is_same<T, bf16_t>::value)                                \
+      asm volatile(GEMM4W_##NAME##_BF16 GEMM4W_OPERANDS);                        \
+    else                                                                         \
+      asm volatile(GEMM4W_##NAME##_F16 GEMM4W_OPERANDS);                         \
+  } while (0)
+  int pid = blockIdx.x, tm, tn;
+  tileOf(pid, tm, tn);
+  laneOffsets(tm, tn);
+  bool first = true;
+  while (true) {
+    if (first)
+      GEMM4W_RUN(PROLOGUE);
+    else
+      GEMM4W_RUN(PROLOGUE_LOADED);
+    for (int p = 1; p < pairs; ++p) GEMM4W_RUN(BODY);
+    const int next = pid + (int)gridDim.x;
+    int ntm = 0, ntn = 0;
+    if (next < total) {
+      // the last K tile also issues the first loads of the next output tile: they land while the epilogue runs
+      tileOf(next, ntm, ntn);
+      laneOffsets(ntm, ntn);
+      GEMM4W_RUN(TAIL_NEXT);
+    } else {
+      GEMM4W_RUN(TAIL);
+    }
+    // one fragment row at a time out of the accumulation registers, which the compiler does not know to be live:
+    // the epilogue stays far below the 256 ordinary registers, so it never borrows them
+    vectorEpilogue<T, EPI, TM, TN>(g, out, cin, bias, tm * BM + wm * WM, tn * BN + wn * WN, frow, kq, [&](auto ic, f32x4(&row)[TN]) {
+      constexpr int i = decltype(ic)::value;
+      f32x4 lo[4], hi[4];
+      accRegisters16<32 * i>(lo);
+      accRegisters16<32 * i + 16>(hi);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) row[j] = lo[j], row[4 + j] = hi[j];
-  });
+      for (int j = 0; j < 4; ++j) row[j] = lo[j], row[4 + j] = hi[j];
+    });
+    if (next >= total) break;
+    pid = next, tm = ntm, tn = ntn, first = false;
+  }
+#undef GEMM4W_RUN
+#undef GEMM4W_OPERANDS
 }
 
 // ------------------------------------------------------------ skinny M (decode) ---
@@ -1324,6 +1349,9 @@ static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p
     // the 4-wave kernel: an even number of K tiles, 16-byte epilogue pieces, lane offsets that fit 31 bits
     if (g.vecEpilogue && p.K % (2 * kBK) == 0 && p.M * p.sAm * 2 < (int64_t(1) << 31) && p.N * p.sBn * 2 < (int64_t(1) << 31)) {
       AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmMfma4WaveKernel<T, EPI>), (int)lds));
+      // one workgroup per CU (its LDS ring takes most of a CU's), each walking its share of the tiles
+      const int resident = computeUnits() / 8 * 8;
+      if (resident >= 8 && (int)grid.x > resident) grid.x = (unsigned)resident;
       hipLaunchKernelGGL((gemmMfma4WaveKernel<T, EPI>), grid, dim3(256), lds, stream, g);
       AMD_LAUNCH_CHECK();
       return diopiSuccess;

@@ -73,9 +73,11 @@ B1_SLOT = 22       # B1 follows this MFMA of k-step 0
 LOAD_STEP = 5      # MFMAs between two tile loads
 
 
-def tile(out, s, loads, next_tile):
+def tile(out, s, loads, next_tile, next_output=False):
     """128 MFMAs of one K tile in stage s; loads: issue the 16 loads of tile t + 2; next_tile: read tile t + 1's first
-    fragments during k-step 1."""
+    fragments during k-step 1; next_output (last K tile of an output tile only): once B1 has freed both stages, issue
+    the 32 loads of the first two K tiles of the workgroup's next output tile (the caller passes that tile's lane
+    offsets), so that they land while the epilogue runs."""
     after = {m: [] for m in range(128)}
     for r in range(16):                                    # this tile's k-step 1 fragments, right away
         after[r].append(("read1", r))
@@ -88,6 +90,12 @@ def tile(out, s, loads, next_tile):
                 loads_before_b2 += 1
             after[slot].append(("m0", d))                  # M0 is written one MFMA before the load that reads it
             after[slot + 1].append(("load", d))
+    if next_output:
+        after[B1_SLOT].append(("rewind", None))
+        for n in range(32):
+            slot = B1_SLOT + 1 + n * 3
+            after[slot].append(("m0n", n))
+            after[slot + 1].append(("load", n % 16))
     if next_tile:
         for r in range(16):
             after[65 + 3 * r].append(("read0", r))
@@ -99,7 +107,7 @@ def tile(out, s, loads, next_tile):
         elif ks == 0 and i == 0 and j >= 1 and m <= B1_SLOT:
             # B_j of buffer 0: 7 - j reads of its set are younger, and so are this tile's reads issued so far
             out.append(f"s_waitcnt lgkmcnt({min(7 - j + min(m, 16), 15)})")
-        if m == 64:
+        if m == 64 and next_tile:                          # B2; the last K tile has no successor to wait for
             out.append(f"s_waitcnt vmcnt({loads_before_b2}) lgkmcnt(0)")
             out.append("s_barrier")
         out.append(f"MFMA {acc(i, j)}, {vb(ks, j)}, {va(ks, i)}, {acc(i, j)}")
@@ -113,36 +121,47 @@ def tile(out, s, loads, next_tile):
                 out.append("s_barrier")
             elif what == "m0":
                 load_m0(out, arg, s)
+            elif what == "m0n":
+                load_m0(out, arg % 16, arg // 16)
+            elif what == "rewind":
+                out.append("s_mov_b32 %[kcur], 0")
             else:
                 load_issue(out, arg)
 
 
-def prologue(out):
+def prologue(out, issue_loads):
+    """issue_loads: issue the loads of K tiles 0 and 1 (otherwise the workgroup's previous output tile did, before its
+    epilogue). The wait that follows allows 16 operations to be outstanding. Loads return in order, so whatever else
+    is still counted (K tile 1's 16 loads, the previous epilogue's stores), K tile 0 has landed: if one of its
+    loads were pending, all 16 younger loads of K tile 1 would be too."""
     out.append("s_mov_b32 %[m0s], m0")
-    for stage in (0, 1):                            # tiles 0 and 1
-        for d in range(16):
-            load_m0(out, d, stage)
-            out.append("s_nop 0")
-            load_issue(out, d)
+    if issue_loads:
+        for stage in (0, 1):
+            for d in range(16):
+                load_m0(out, d, stage)
+                out.append("s_nop 0")
+                load_issue(out, d)
     for r in range(256):                            # while the loads are in flight
         out.append(f"v_accvgpr_write_b32 a{r}, 0")
-    out.append("s_waitcnt vmcnt(16)")               # tile 0 has landed
+    out.append("s_waitcnt vmcnt(16)")
     out.append("s_barrier")
     for kind, idx in READ_ORDER:
         read_fragment(out, kind, idx, 0, 0, 0)
 
 
 def main():
-    pro, body, tail = [], [], []
-    prologue(pro)
+    pro, proc, body, tail, tailn = [], [], [], [], []
+    prologue(pro, True)
+    prologue(proc, False)
     tile(body, 0, True, True)
     tile(body, 1, True, True)
-    tile(tail, 0, False, True)
-    tile(tail, 1, False, False)
-    tail += ["s_nop 15", "s_nop 15", "s_mov_b32 m0, %[m0s]"]   # the last MFMAs have written their accumulators
+    for t, nxt in ((tail, False), (tailn, True)):
+        tile(t, 0, False, True)
+        tile(t, 1, False, False, nxt)
+        t += ["s_nop 15", "s_nop 15", "s_mov_b32 m0, %[m0s]"]   # the last MFMAs have written their accumulators
     clobbers = ", ".join(f'"v{r}"' for r in range(VA0, VA0 + 128)) + ", " + ", ".join(f'"a{r}"' for r in range(256))
     text = ["// Generated by gen_gemm_loop_4wave.py (see there for the schedule); do not edit.\n"]
-    for name, lines in (("PROLOGUE", pro), ("BODY", body), ("TAIL", tail)):
+    for name, lines in (("PROLOGUE", pro), ("PROLOGUE_LOADED", proc), ("BODY", body), ("TAIL", tail), ("TAIL_NEXT", tailn)):
         for suffix, mnemonic in (("BF16", "v_mfma_f32_16x16x32_bf16"), ("F16", "v_mfma_f32_16x16x32_f16")):
             text.append(f"#define GEMM4W_{name}_{suffix} \\\n")
             text.append(" \\\n".join('  "' + l.replace("MFMA", mnemonic) + '\\n\\t"' for l in lines) + "\n\n")
