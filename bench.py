@@ -29,12 +29,12 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TF = 2500.0   # MI355X dense bf16, published
 # Bytes that leave L2 per GEMM launch (call-weighted mean of the layer's 4 GEMM launches), from two
 # rocprofv3 --pmc runs of `bench.py --only-layer` (FETCH_SIZE, then WRITE_SIZE), scaled by what the same
-# counters read for a 64 MiB device copy: (2 x 617 006 + 125 999) KiB. The summary is
+# counters read for a 64 MiB device copy: (2 x 618 560 + 127 720) KiB. The summary is
 # profiles/decoder_layer_hbm_traffic_counters.md;
 # a counter cannot be read from inside this process, so the figure is carried here as measured, with the commit
 # whose kernels the counters were taken on (it does not move when the kernel does; re-take it after a GEMM change).
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 1_393_000_000
-GEMM_TRAFFIC_MEASURED_AT = "11aac02"
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 1_398_000_000
+GEMM_TRAFFIC_MEASURED_AT = "a111839"
 
 
 def parse():
@@ -47,6 +47,8 @@ def parse():
     ap.add_argument("--only-layer", action="store_true", help="alias for --no-cpu --no-ops")
     ap.add_argument("--gemm", metavar="M,N,K", help="profiling aid: time only diopiLinear on bf16 [M,K] x [N,K]^T "
                     "(activations N(0,1), weights N(0,0.02)) for --steps launches and print one JSON line")
+    ap.add_argument("--vendor-library", action="store_true", help="with --gemm: time torch.nn.functional.linear (the vendor's GEMM "
+                    "library) on the same operands instead of diopiLinear, for side-by-side counter runs; never part of the measured path")
     ap.add_argument("--attention", action="store_true", help="profiling aid: time only the prefill attention of the "
                     "layer workload (batch 4 x seq 2048, 32 heads x 128, bf16) for --steps launches")
     return ap.parse_args()
@@ -427,8 +429,13 @@ def single_kernel(pkg, torch, dev, rt, stream, args):
         a = torch.randn(m, k, generator=g).bfloat16().to(dev)
         w = (torch.randn(n, k, generator=g) * 0.02).bfloat16().to(dev)
         out = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
-        call = Prepared(pkg, "diopiLinear", out, a, w, None)
-        work, unit, label = 2.0 * m * n * k / 1e12, "TFLOP/s", f"diopiLinear bf16 {m}x{n}x{k}"
+        if args.vendor_library:
+            call = lambda: torch.matmul(a, w.t(), out=out)
+            label = f"torch.matmul (vendor library) bf16 {m}x{n}x{k}"
+        else:
+            call = Prepared(pkg, "diopiLinear", out, a, w, None)
+            label = f"diopiLinear bf16 {m}x{n}x{k}"
+        work, unit = 2.0 * m * n * k / 1e12, "TFLOP/s"
     else:
         b, s, h, hd = 4, 2048, 32, 128
         g = torch.Generator().manual_seed(0)
@@ -567,7 +574,7 @@ def main():
     gemm_flops = sum(flops.values())
     achieved_tf = gemm_flops / (gemm_time_us * 1e-6) / 1e12
     breakdown = {l: round(sum(v) / args.steps, 1) for l, v in per_op.items()}      # us per step (labels used twice are summed)
-    roofline = {"bound": "mfma", "kernel": "gemmMfmaPipelinedKernel<bf16> 256x256x64 (4 launches per step: qkv with rotary, o + residual, gate+up with silu*mul, down + residual)",
+    roofline = {"bound": "mfma", "kernel": "gemmMfma4WaveKernel<bf16> 256x256x64 (4 launches per step: qkv with rotary, o + residual, gate+up with silu*mul, down + residual)",
                 "achieved": round(achieved_tf, 1), "peak": MFMA_BF16_PEAK_TF, "unit": "TFLOP/s",
                 "frac": round(achieved_tf / MFMA_BF16_PEAK_TF, 4), "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH,
                 "traffic_measured_at_commit": GEMM_TRAFFIC_MEASURED_AT,

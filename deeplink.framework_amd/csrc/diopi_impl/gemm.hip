@@ -419,7 +419,10 @@ __device__ __forceinline__ void vectorEpilogue(const MfmaArgs& g, T* out, const 
     // Table entries are requested four fragment rows at a time,
     // before any store of the batch: a request one row ahead would expose the L2 round trip once per row.
     float cs[4][TN / 2][4], sn[4][TN / 2][4];
+    // a wave whose columns all lie at or past rotCols (v heads) asks for no table entries at all
+    const bool anyRot = __builtin_amdgcn_readfirstlane(colBase) < g.rotCols;
     auto fetch = [&](int i) {
+      if (!anyRot) return;
       const int row = row0 + i * 16 + frow;
 #pragma unroll
       for (int jp = 0; jp < TN / 2; ++jp) {
