@@ -5,12 +5,16 @@
 // MFMA engine (bf16 / fp16 inputs, fp32 accumulate) -- C[M,N] = A[M,K] . B[N,K]^T with both
 // operands K-contiguous, which is exactly what the MFMA instructions want: every lane feeds 8
 // consecutive K elements (one 16-byte LDS read) of one row.
-//   * large problems (K a multiple of 64): 256x256x64 macro tile, workgroup = 512 threads = 8 waves
+//   * large problems with an even number of 64-wide K tiles: 256x256x64 macro tile, workgroup = 256 threads =
+//     4 waves in a 2x2 arrangement (wave tile 128x128 = 8x8 tiles of v_mfma_f32_16x16x32, 256 fp32 accumulators
+//     per lane in the accumulation registers), one persistent workgroup per CU, K loop placed instruction by
+//     instruction (gemm_loop_4wave.inc, generated); its counters match the vendor library's kernel;
+//   * large problems otherwise (K a multiple of 64): the same macro tile with 512 threads = 8 waves
 //     in a 2x4 arrangement (wave tile 128x64 = 8x4 tiles of v_mfma_f32_16x16x32, 128 fp32
 //     accumulators per lane, two waves per SIMD so one wave's LDS traffic hides behind the other's
 //     MFMAs). The 16x16x32 shape draws less power per flop than 32x32x16 (an MFMA-only loop holds
-//     ~2.02 GHz against ~1.86 GHz on random operands), and this kernel runs at the power limit;
-//   * its operand tiles go from memory straight into a two-stage LDS ring (buffer_load ... lds, no
+//     ~2.02 GHz against ~1.86 GHz on random operands), and these kernels run at the power limit;
+//   * operand tiles go from memory straight into a two-stage LDS ring (buffer_load ... lds, no
 //     registers and no ds_write in between): tile k+1 lands in the other stage while tile k is
 //     being multiplied, and the loads of tile k+2 start as soon as every wave is past the one
 //     barrier per K tile. Operand rows are addressed through buffer descriptors (32-bit lane offset
