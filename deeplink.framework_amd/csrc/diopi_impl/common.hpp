@@ -133,6 +133,26 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+// buffer_load_dwordx4 ... lds: lane l of the wave fetches 16 bytes at rsrc + voffset + soffset and the
+// data lands in LDS at ldsAddr + 16 * l without passing through registers. Issued as inline assembly so
+// that the compiler does not order it against fragment reads of the other stage; a kernel waits for
+// these loads itself (vmcnt) before the barrier that publishes a stage. The LDS address travels in M0,
+// which is read when the load issues; the previous M0 is put back so the statement has no side effect
+// on registers the compiler owns.
+__device__ __forceinline__ void loadToLds16(u32x4 rsrc, int voffset, int soffset, unsigned ldsAddr) {
+  unsigned savedM0;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\t"
+      "s_mov_b32 m0, %1\n\t"
+      "s_nop 0\n\t"
+      "buffer_load_dwordx4 %2, %3, %4 offen lds\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(savedM0)
+      : "s"(ldsAddr), "v"(voffset), "s"(rsrc), "s"(soffset)
+      : "memory");
+}
 
 template <typename T>
 struct Vec16 {  // 16 bytes of T

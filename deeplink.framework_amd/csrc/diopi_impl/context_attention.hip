@@ -14,15 +14,19 @@
 //   * The accumulator registers of S^T, converted to bf16, are already a valid B operand
 //     (P^T) for O^T += V^T . P^T: consecutive groups of 8 accumulator registers are the 8
 //     K-slots of a lane, for a fixed permutation of the 16 keys of the step. The A operand
-//     (V^T) is read from an LDS copy of V stored transposed [d][keys] with exactly that
-//     permutation: two 8-byte reads per operand.
-//   * K tile rows in LDS are XOR-swizzled per 16-byte chunk (measured conflict-free ds_read_b128);
-//     V is transposed on the way into LDS (4 keys x 8 d per lane, 8-byte stores).
+//     (V^T) comes from V kept row-major [keys][d] in LDS through the transposing LDS read
+//     (ds_read_b64_tr_b16): the addresses the lanes supply pick that same permutation, two
+//     8-byte reads per operand and no transposition work anywhere.
+//   * K and V tiles go from memory straight into LDS (buffer_load ... lds): no staging registers, no
+//     LDS stores. Rows are XOR-swizzled per 16-byte chunk on the global side of the copy: K for
+//     conflict-free ds_read_b128, V so that the 16 row pieces one transposing read touches spread
+//     evenly over the banks.
 //   * two workgroups per CU (<= 256 registers per lane) so one wave's softmax VALU work overlaps
 //     another's MFMAs; exp2 is the bare hardware instruction fed by one FMA; the O^T rescale is
 //     skipped while the running max does not move;
-//   * two LDS stages, register prefetch of the next tile through buffer descriptors (no per-row
-//     address arithmetic, rows past the sequence read as zero), one LDS-only barrier per tile;
+//   * two LDS stages; the copy of tile t + 1 is issued when tile t starts and waited for when it ends
+//     (buffer descriptors: no per-row address arithmetic, rows past the sequence read as zero), one
+//     barrier per tile;
 //   * causal work grows with the query block index: a workgroup processes the heaviest remaining
 //     block and then the lightest, so all workgroups stream the same number of key tiles; the
 //     one-dimensional grid is decoded so the workgroups of a head share one XCD (one L2).
@@ -82,7 +86,15 @@ __device__ __forceinline__ int kSwizzle(int key) {
   return D == 128 ? (key & 15) : ((key >> 1) & 7);
 }
 
-constexpr int kCaBQ = 128, kCaBKV = 64, kCaVtStride = 68;  // V^T rows padded to 68 keys (136 bytes)
+// XOR applied to the 16-byte chunk index of V row `key` in LDS (always even, so the 32 bytes a 16-lane
+// group takes from one row stay together). One transposing read touches 8 consecutive keys x 2 pieces of
+// 32 bytes; with these patterns every 32-byte bank group is hit exactly twice, the minimum for 512 bytes.
+template <int D>
+__device__ __forceinline__ int vSwizzle(int key) {
+  return D == 128 ? 2 * (key & 7) : 2 * ((key >> 1) & 3);
+}
+
+constexpr int kCaBQ = 128, kCaBKV = 64;
 
 // One 128-query block of one (sequence, head): the whole flash-attention pass over its key tiles.
 template <typename T, int D>
@@ -91,15 +103,15 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
   using Half = typename CaMfma<T>::Half;
   constexpr int KS = D / 16;        // MFMA k-steps over the head dim
   constexpr int DT = D / 32;        // 32-row tiles of O^T
-  constexpr int CPR = D / 8;        // 16-byte chunks per K row
-  constexpr int K_CH = kCaBKV * CPR / 256;  // K chunks per thread
-  constexpr int K_STAGE = kCaBKV * D;       // elements
-  constexpr int V_STAGE = D * kCaVtStride;
+  constexpr int CPR = D / 8;        // 16-byte chunks per row
+  constexpr int RPL = 64 / CPR;     // rows one wave-wide copy instruction covers (1 KiB)
+  constexpr int NLD = kCaBKV / RPL / 4;     // copy instructions per wave, per matrix, per tile
+  constexpr int STAGE = kCaBKV * D;         // elements
   extern __shared__ __attribute__((aligned(16))) char smem[];
   T* sK = reinterpret_cast<T*>(smem);   // [2][64][D] swizzled
-  T* sVt = sK + 2 * K_STAGE;            // [2][D][68]
+  T* sV = sK + 2 * STAGE;               // [2][64][D] swizzled
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l31 = lane & 31, half = lane >> 5;
   const int64_t start = ldIdxCA(a.bStart, b, a.start64);
   const int len = (int)ldIdxCA(a.bLen, b, a.len64);
@@ -120,53 +132,34 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
   const int ntiles = (min(len, q0 + kCaBQ) + kCaBKV - 1) / kCaBKV;
   const int waveMaxQ = min(q0 + wave * 32 + 31, len - 1);
 
-  // ---- staging roles. K and V rows come through buffer descriptors that end at the sequence's last
+  // ---- tile copies. K and V rows come through buffer descriptors that end at the sequence's last
   // row: a lane's offset is computed once (32 bits), the tile advances a scalar offset, and rows past
-  // the sequence read as zeros without any clamping arithmetic.
-  Frag kr[K_CH];
-  int kOff[K_CH], kVoff[K_CH];
-  const int cK = (tid % CPR) * 8;
+  // the sequence read as zeros without any clamping arithmetic. Copy instruction i of this wave fills
+  // the 1 KiB block (i * 4 + wave) of a stage: lane l owns physical slot (row l / CPR, chunk l % CPR) and
+  // fetches the logical chunk the swizzle puts there.
+  int kVoff[NLD], vVoff[NLD];
 #pragma unroll
-  for (int i = 0; i < K_CH; ++i) {
-    int chunk = tid + 256 * i;
-    int key = chunk / CPR, c = chunk % CPR;
-    kOff[i] = key * D + ((c ^ kSwizzle<D>(key)) << 3);
-    kVoff[i] = (key * (int)a.kTok + cK) * (int)sizeof(T);
+  for (int i = 0; i < NLD; ++i) {
+    const int key = (i * 4 + wave) * RPL + lane / CPR, pc = lane % CPR;
+    kVoff[i] = (key * (int)a.kTok + ((pc ^ kSwizzle<D>(key)) << 3)) * (int)sizeof(T);
+    vVoff[i] = (key * (int)a.vTok + ((pc ^ vSwizzle<D>(key)) << 3)) * (int)sizeof(T);
   }
-  const bool vActive = tid < 16 * (D / 8);
-  const int vKg = tid & 15, vDc = tid >> 4;
-  Frag vr[4];
-  int vVoff[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) vVoff[j] = ((vKg * 4 + j) * (int)a.vTok + vDc * 8) * (int)sizeof(T);
-  const __amdgpu_buffer_rsrc_t rsK = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<T*>(kg), 0, (int)(((int64_t)(len - 1) * a.kTok + D) * sizeof(T)), 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsV = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<T*>(vg), 0, (int)(((int64_t)(len - 1) * a.vTok + D) * sizeof(T)), 0x00020000);
-
-  auto gload = [&](int t) {
-    const int kS = t * kCaBKV * (int)a.kTok * (int)sizeof(T), vS = t * kCaBKV * (int)a.vTok * (int)sizeof(T);
-#pragma unroll
-    for (int i = 0; i < K_CH; ++i)
-      kr[i] = __builtin_bit_cast(Frag, __builtin_amdgcn_raw_buffer_load_b128(rsK, kVoff[i], kS, 0));
-    if (vActive) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        vr[j] = __builtin_bit_cast(Frag, __builtin_amdgcn_raw_buffer_load_b128(rsV, vVoff[j], vS, 0));
-    }
+  auto descriptor = [](const T* base, int64_t bytes) {
+    const uint64_t p = reinterpret_cast<uint64_t>(base);
+    u32x4 d = {(uint32_t)p, (uint32_t)(p >> 32) & 0xffffu, (uint32_t)bytes, 0x00020000u};
+    return d;
   };
-  auto swrite = [&](int stage) {
-    T* k = sK + stage * K_STAGE;
-    T* vt = sVt + stage * V_STAGE;
+  const u32x4 rsK = descriptor(kg, ((int64_t)(len - 1) * a.kTok + D) * sizeof(T));
+  const u32x4 rsV = descriptor(vg, ((int64_t)(len - 1) * a.vTok + D) * sizeof(T));
+  const unsigned ldsK = (unsigned)(uintptr_t)sK, ldsV = (unsigned)(uintptr_t)sV;
+
+  auto copyTile = [&](int t, int stage) {
+    const int kS = t * kCaBKV * (int)a.kTok * (int)sizeof(T), vS = t * kCaBKV * (int)a.vTok * (int)sizeof(T);
+    const unsigned to = (unsigned)(stage * STAGE * sizeof(T)) + (unsigned)wave * 1024u;
 #pragma unroll
-    for (int i = 0; i < K_CH; ++i) *reinterpret_cast<Frag*>(k + kOff[i]) = kr[i];
-    if (vActive) {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        Half p;
-        p[0] = vr[0][e], p[1] = vr[1][e], p[2] = vr[2][e], p[3] = vr[3][e];
-        *reinterpret_cast<Half*>(vt + (vDc * 8 + e) * kCaVtStride + vKg * 4) = p;
-      }
+    for (int i = 0; i < NLD; ++i) {
+      loadToLds16(rsK, kVoff[i], kS, ldsK + to + i * 4096u);
+      loadToLds16(rsV, vVoff[i], vS, ldsV + to + i * 4096u);
     }
   };
 
@@ -178,22 +171,22 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
   float m = -INFINITY, l = 0.f;
   const float scale2 = a.scale * kLog2eCA;
 
-  // barrier on LDS traffic only: the global loads of the tile after next stay in flight across it
-  auto ldsBarrier = []() {
-    __builtin_amdgcn_s_waitcnt(0xc07f);
+  // Everything this wave has in flight (its share of the next tile's copy, its LDS reads) is done, then
+  // the workgroup meets: past the barrier the next tile is complete in LDS and the stage just read is free.
+  auto tileBarrier = []() {
+    __builtin_amdgcn_s_waitcnt(0x0070);
     __builtin_amdgcn_s_barrier();
   };
-  gload(0);
-  swrite(0);
-  if (ntiles > 1) gload(1);
-  ldsBarrier();
+  copyTile(0, 0);
+  tileBarrier();
+  if (ntiles > 1) copyTile(1, 1);
 
   for (int t = 0; t < ntiles; ++t) {
     const int cur = t & 1;
     const int k0 = t * kCaBKV;
     if (k0 <= waveMaxQ) {
-      const T* k = sK + cur * K_STAGE;
-      const T* vt = sVt + cur * V_STAGE;
+      const T* k = sK + cur * STAGE;
+      const T* v = sV + cur * STAGE;
       f32x16 s[2];
 #pragma unroll
       for (int kt2 = 0; kt2 < 2; ++kt2)
@@ -252,14 +245,25 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
       // latency of a fragment is covered by the MFMAs in front of it.
       {
         constexpr int NPV = 4 * DT, kVAhead = 3;
+        // Transposing read: the 16 lanes of a group each supply the address of 4 consecutive d of one key,
+        // source lane j -> (key j >> 2, d 4 * (j & 3)), and lane i of the group receives d = i of those 4
+        // keys. Group G serves the half-wave G >> 1 and the d range 16 * (G & 1); read r of the two takes
+        // keys 8 r + 4 half + 0..3 of the step: the order the P^T operand holds them in.
+        const int trKey = half * 4 + ((lane & 15) >> 2);
+        const int trChunk = ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1), trIn = (lane & 1) * 4;
         auto vfrag = [&](int i) {
           const int g = i / DT, dt = i % DT;  // key group (kt2 * 2 + t2), d tile
-          const T* row = vt + (dt * 32 + l31) * kCaVtStride + g * 16 + half * 4;
-          Half lo = *reinterpret_cast<const Half*>(row);
-          Half hi = *reinterpret_cast<const Half*>(row + 8);
+          Half part[2];
+#pragma unroll
+          for (int r = 0; r < 2; ++r) {
+            const int key = g * 16 + r * 8 + trKey;
+            const T* p = v + key * D + (((dt * 4 + trChunk) ^ vSwizzle<D>(key)) << 3) + trIn;
+            part[r] = __builtin_bit_cast(Half, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                                   (__attribute__((address_space(3))) s16x4*)p));
+          }
           Frag vf;
-          vf[0] = lo[0], vf[1] = lo[1], vf[2] = lo[2], vf[3] = lo[3];
-          vf[4] = hi[0], vf[5] = hi[1], vf[6] = hi[2], vf[7] = hi[3];
+          vf[0] = part[0][0], vf[1] = part[0][1], vf[2] = part[0][2], vf[3] = part[0][3];
+          vf[4] = part[1][0], vf[5] = part[1][1], vf[6] = part[1][2], vf[7] = part[1][3];
           return vf;
         };
         Frag vfr[kVAhead + 1];
@@ -289,11 +293,8 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
         l += lsum[0];
       }
     }
-    if (t + 1 < ntiles) {
-      swrite(cur ^ 1);
-      if (t + 2 < ntiles) gload(t + 2);
-    }
-    ldsBarrier();
+    tileBarrier();
+    if (t + 2 < ntiles) copyTile(t + 2, cur);
   }
 
   // ---- epilogue: O^T (lane = query) -> LDS [query][d] -> coalesced 16-byte stores
@@ -402,7 +403,7 @@ __global__ __launch_bounds__(256) void contextAttnScalarKernel(CaArgs a, int max
 
 template <typename T, int D>
 static diopiError_t launchCaMfma(hipStream_t stream, const CaArgs& a, int maxLen, int64_t batch) {
-  constexpr size_t lds = 2 * (size_t)(kCaBKV * D + D * kCaVtStride) * sizeof(T);
+  constexpr size_t lds = 2 * (size_t)(2 * kCaBKV * D) * sizeof(T);
   static_assert(lds >= 4 * 32 * (D + 8) * sizeof(T), "epilogue staging must fit in the tile buffers");
   AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&contextAttnMfmaKernel<T, D>), (int)lds));
   const int numQBlocks = (int)ceilDiv(maxLen, kCaBQ);

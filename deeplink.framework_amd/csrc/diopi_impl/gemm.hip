@@ -295,25 +295,6 @@ struct MfmaOp16<half_t> {
   }
 };
 
-// buffer_load_dwordx4 ... lds: lane l of the wave fetches 16 bytes at rsrc + voffset + soffset and the
-// data lands in LDS at ldsAddr + 16 * l without passing through registers. Issued as inline assembly so
-// that the compiler does not order it against fragment reads of the other stage; the kernel waits for
-// these loads itself (vmcnt) before the barrier that publishes a stage. The LDS address travels in M0,
-// which is read when the load issues; the previous M0 is put back so the statement has no side effect
-// on registers the compiler owns.
-__device__ __forceinline__ void loadToLds16(u32x4 rsrc, int voffset, int soffset, unsigned ldsAddr) {
-  unsigned savedM0;
-  asm volatile(
-      "s_mov_b32 %0, m0\n\t"
-      "s_mov_b32 m0, %1\n\t"
-      "s_nop 0\n\t"
-      "buffer_load_dwordx4 %2, %3, %4 offen lds\n\t"
-      "s_mov_b32 m0, %0"
-      : "=&s"(savedM0)
-      : "s"(ldsAddr), "v"(voffset), "s"(rsrc), "s"(soffset)
-      : "memory");
-}
-
 // EPI selects the epilogue: kEpiLinear is alpha * acc + beta * C + bias; kEpiSiluMul treats every 64 consecutive
 // output columns as 32 gate columns followed by the 32 up columns of the same channels and stores
 // silu(gate) * up, half as wide (out has N / 2 columns); kEpiPartial is the split-K form: workgroup (tile, s)

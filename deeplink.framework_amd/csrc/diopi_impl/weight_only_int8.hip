@@ -75,21 +75,6 @@ __device__ __forceinline__ typename W8Mfma<T>::Frag cvt8(uint32_t lo, uint32_t h
   return r;
 }
 
-// buffer_load_dwordx4 ... lds: lane l fetches 16 bytes at rsrc + voffset + soffset and the data lands in LDS at
-// ldsAddr + 16 * l without passing through registers (the LDS address travels in M0, which is put back).
-__device__ __forceinline__ void loadToLds16(u32x4 rsrc, int voffset, int soffset, unsigned ldsAddr) {
-  unsigned savedM0;
-  asm volatile(
-      "s_mov_b32 %0, m0\n\t"
-      "s_mov_b32 m0, %1\n\t"
-      "s_nop 0\n\t"
-      "buffer_load_dwordx4 %2, %3, %4 offen lds\n\t"
-      "s_mov_b32 m0, %0"
-      : "=&s"(savedM0)
-      : "s"(ldsAddr), "v"(voffset), "s"(rsrc), "s"(soffset)
-      : "memory");
-}
-
 constexpr int kW8Block = 128;   // K elements one wave consumes per step (4 kgrps x 32)
 // One step (two 16-byte loads per lane) is in flight ahead of the one being multiplied, no more: measured,
 // a deeper queue is slower (9.7 us with four steps ahead, 10.4 with eight, 8.8 with one or two at M = 1).
