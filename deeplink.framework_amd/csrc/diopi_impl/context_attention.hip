@@ -86,12 +86,12 @@ __device__ __forceinline__ int kSwizzle(int key) {
   return D == 128 ? (key & 15) : ((key >> 1) & 7);
 }
 
-// XOR applied to the 16-byte chunk index of V row `key` in LDS (always even, so the 32 bytes a 16-lane
-// group takes from one row stay together). One transposing read touches 8 consecutive keys x 2 pieces of
-// 32 bytes; with these patterns every 32-byte bank group is hit exactly twice, the minimum for 512 bytes.
+// XOR applied to the 16-byte chunk index of V row `key` in LDS (a multiple of 4, so the 32 bytes a 16-lane
+// group takes from one row stay together). A transposing read is served half a wave at a time: 4
+// consecutive keys x 2 pieces of 32 bytes, which these patterns put on 8 different 32-byte bank groups.
 template <int D>
 __device__ __forceinline__ int vSwizzle(int key) {
-  return D == 128 ? 2 * (key & 7) : 2 * ((key >> 1) & 3);
+  return D == 128 ? 4 * (key & 3) : 4 * ((key >> 1) & 1);
 }
 
 constexpr int kCaBQ = 128, kCaBKV = 64;
@@ -153,14 +153,17 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
   const u32x4 rsV = descriptor(vg, ((int64_t)(len - 1) * a.vTok + D) * sizeof(T));
   const unsigned ldsK = (unsigned)(uintptr_t)sK, ldsV = (unsigned)(uintptr_t)sV;
 
-  auto copyTile = [&](int t, int stage) {
-    const int kS = t * kCaBKV * (int)a.kTok * (int)sizeof(T), vS = t * kCaBKV * (int)a.vTok * (int)sizeof(T);
-    const unsigned to = (unsigned)(stage * STAGE * sizeof(T)) + (unsigned)wave * 1024u;
+  auto copyK = [&](int t, int stage) {
+    const int kS = t * kCaBKV * (int)a.kTok * (int)sizeof(T);
+    const unsigned to = ldsK + (unsigned)(stage * STAGE * sizeof(T)) + (unsigned)wave * 1024u;
 #pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-      loadToLds16(rsK, kVoff[i], kS, ldsK + to + i * 4096u);
-      loadToLds16(rsV, vVoff[i], vS, ldsV + to + i * 4096u);
-    }
+    for (int i = 0; i < NLD; ++i) loadToLds16(rsK, kVoff[i], kS, to + i * 4096u);
+  };
+  auto copyV = [&](int t, int stage) {
+    const int vS = t * kCaBKV * (int)a.vTok * (int)sizeof(T);
+    const unsigned to = ldsV + (unsigned)(stage * STAGE * sizeof(T)) + (unsigned)wave * 1024u;
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) loadToLds16(rsV, vVoff[i], vS, to + i * 4096u);
   };
 
   f32x16 o[DT];
@@ -171,39 +174,55 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
   float m = -INFINITY, l = 0.f;
   const float scale2 = a.scale * kLog2eCA;
 
-  // Everything this wave has in flight (its share of the next tile's copy, its LDS reads) is done, then
-  // the workgroup meets: past the barrier the next tile is complete in LDS and the stage just read is free.
+  // Everything this wave has in flight (its share of the copies, its LDS reads) is done, then the
+  // workgroup meets: past the barrier the tiles those copies fill are complete in LDS.
   auto tileBarrier = []() {
     __builtin_amdgcn_s_waitcnt(0x0070);
     __builtin_amdgcn_s_barrier();
   };
-  copyTile(0, 0);
+  // K fragment i of a tile: key half i & 1 (32 keys), head-dim step i >> 1. A ring of them runs kKAhead
+  // MFMAs ahead of the score MFMAs, and the first kKAhead of the NEXT tile are read at the end of the
+  // P.V loop, so no score MFMA waits for LDS.
+  constexpr int NS = 2 * KS, kKAhead = 4;
+  Frag kfr[kKAhead + 1];
+  auto kfrag = [&](const T* k, int i) {
+    const int key = (i & 1) * 32 + l31, chunk = (i >> 1) * 2 + half;
+    return *reinterpret_cast<const Frag*>(k + key * D + ((chunk ^ kSwizzle<D>(key)) << 3));
+  };
+  // The barrier of tile t sits between its softmax and its P.V: it publishes K of tile t + 1 and V of tile t,
+  // and it says that every wave is done with K of tile t and V of tile t - 1, whose stages the copies
+  // issued right after it (K of t + 2, V of t + 1) overwrite. Every copy has a whole tile to land.
+  copyK(0, 0);
+  copyV(0, 0);
   tileBarrier();
-  if (ntiles > 1) copyTile(1, 1);
+  if (ntiles > 1) copyK(1, 1);
+#pragma unroll
+  for (int i = 0; i < kKAhead; ++i) kfr[i] = kfrag(sK, i);
 
   for (int t = 0; t < ntiles; ++t) {
     const int cur = t & 1;
     const int k0 = t * kCaBKV;
-    if (k0 <= waveMaxQ) {
-      const T* k = sK + cur * STAGE;
-      const T* v = sV + cur * STAGE;
-      f32x16 s[2];
+    const bool live = k0 <= waveMaxQ;  // wave-uniform; once false it stays false
+    const T* k = sK + cur * STAGE;
+    const T* v = sV + cur * STAGE;
+    f32x16 s[2];
+    if (live) {
 #pragma unroll
       for (int kt2 = 0; kt2 < 2; ++kt2)
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[kt2][r] = 0.f;
+      // A wave in an MFMA phase outranks one in its softmax when both want to issue: the matrix pipe then never
+      // waits behind the other wave's exp2 and conversions (measured: 169 -> 161 us on 4 x 2048 x 32 x 128).
+      __builtin_amdgcn_s_setprio(1);
       // the two 32-key halves are independent accumulation chains: alternate them so that no MFMA
       // waits for the one issued just before it
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const int chunk = ks * 2 + half;
-#pragma unroll
-        for (int kt2 = 0; kt2 < 2; ++kt2) {
-          const int key = kt2 * 32 + l31;
-          Frag kf = *reinterpret_cast<const Frag*>(k + key * D + ((chunk ^ kSwizzle<D>(key)) << 3));
-          s[kt2] = CaMfma<T>::run(kf, qf[ks], s[kt2]);
-        }
+      for (int i = 0; i < NS; ++i) {
+        if (i + kKAhead < NS) kfr[(i + kKAhead) % (kKAhead + 1)] = kfrag(k, i + kKAhead);
+        s[i & 1] = CaMfma<T>::run(kfr[i % (kKAhead + 1)], qf[i >> 1], s[i & 1]);
+        __builtin_amdgcn_sched_barrier(0);
       }
+      __builtin_amdgcn_s_setprio(0);
       // ---- online softmax for this lane's query over the 64 keys of the tile
       // (m and mn are kept in the scaled log2 domain: score * scale * log2 e)
       const bool needMask = (k0 + kCaBKV - 1 > q0 + wave * 32) || (k0 + kCaBKV > len);
@@ -240,6 +259,12 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
           for (int r = 0; r < 16; ++r) o[dt][r] *= corr;
         m = mn;
       }
+    }
+    tileBarrier();
+    if (t + 2 < ntiles) copyK(t + 2, cur);
+    if (t + 1 < ntiles) copyV(t + 1, cur ^ 1);
+    if (live) {
+      __builtin_amdgcn_s_setprio(2);
       // ---- O^T += V^T . P^T: 4 key groups of 16 x DT row tiles. The V^T fragment of MFMA i + kVAhead is
       // read while MFMA i issues, and a scheduling fence after every MFMA keeps that order, so the LDS
       // latency of a fragment is covered by the MFMAs in front of it.
@@ -287,15 +312,17 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
             lsum = CaMfma<T>::run(ones, pf, lsum);
           }
           if (i + kVAhead < NPV) vfr[(i + kVAhead) % (kVAhead + 1)] = vfrag(i + kVAhead);
+          // the next tile's first K fragments (after the last tile: a harmless read of the other stage)
+          if (i >= NPV - kKAhead) kfr[i - (NPV - kKAhead)] = kfrag(sK + (cur ^ 1) * STAGE, i - (NPV - kKAhead));
           o[dt] = CaMfma<T>::run(vfr[i % (kVAhead + 1)], pf, o[dt]);
           __builtin_amdgcn_sched_barrier(0);
         }
         l += lsum[0];
       }
     }
-    tileBarrier();
-    if (t + 2 < ntiles) copyTile(t + 2, cur);
   }
+  __builtin_amdgcn_s_setprio(0);
+  __syncthreads();  // the output staging below aliases the stages other waves may still be reading
 
   // ---- epilogue: O^T (lane = query) -> LDS [query][d] -> coalesced 16-byte stores
   constexpr int OS = D + 8;  // padded row, elements
