@@ -240,7 +240,10 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
       for (int kt2 = 0; kt2 < 2; ++kt2)
 #pragma unroll
         for (int r = 0; r < 16; ++r) mt = fmaxf(mt, s[kt2][r]);
-      mt = fmaxf(mt, __shfl_xor(mt, 32, 64)) * scale2;  // scale2 > 0, so the max commutes with the scaling
+      {  // the other half-wave holds the other 16 scores of the query: one lane swap, no trip through LDS
+        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mt), __float_as_uint(mt), false, false);
+        mt = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1])) * scale2;  // scale2 > 0, so the max commutes with the scaling
+      }
       const float mn = fmaxf(m, mt);  // key 0 is visible to every query, so mn is finite from tile 0 on
 #pragma unroll
       for (int kt2 = 0; kt2 < 2; ++kt2)
