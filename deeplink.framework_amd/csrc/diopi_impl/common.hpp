@@ -154,6 +154,21 @@ __device__ __forceinline__ void loadToLds16(u32x4 rsrc, int voffset, int soffset
       : "memory");
 }
 
+// The same copy marked non-temporal: for data that is read once (a weight stream), so that it does not push
+// re-used lines (the activations every workgroup reads) out of L2.
+__device__ __forceinline__ void loadToLds16Stream(u32x4 rsrc, int voffset, int soffset, unsigned ldsAddr) {
+  unsigned savedM0;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\t"
+      "s_mov_b32 m0, %1\n\t"
+      "s_nop 0\n\t"
+      "buffer_load_dwordx4 %2, %3, %4 offen nt lds\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(savedM0)
+      : "s"(ldsAddr), "v"(voffset), "s"(rsrc), "s"(soffset)
+      : "memory");
+}
+
 template <typename T>
 struct Vec16 {  // 16 bytes of T
   static constexpr int N = 16 / sizeof(T);

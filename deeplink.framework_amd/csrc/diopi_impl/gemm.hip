@@ -1031,75 +1031,100 @@ __global__ __launch_bounds__(NTW * KS * 64) void gemmSkinnyKernel(SkinnyArgs a) 
 }
 
 // 33 to 64 rows against a wide weight (at least 512 column tiles): no K split over the grid, so no partial products
-// and no reduction pass. One workgroup owns NTW column tiles for the whole of K and walks it in chunks of 512: the
-// four waves of a tile each take one 128-column step of the chunk. The activations of chunk c + 1 travel through
-// registers into the second LDS buffer while chunk c is multiplied, the weights are fetched two chunks ahead, and
-// every load is an ordinary one at a clamped (always valid) address, so the compiler counts outstanding loads
-// exactly and nothing in the loop waits for more than it needs.
+// and no reduction pass. One workgroup owns NTW column tiles for the whole of K and walks it in chunks of 256: the
+// four waves of a tile each take 64 columns of the chunk.
+//   * The activations of a chunk (64 rows x 512 bytes) go from memory straight into one of four LDS buffers, three
+//     chunks ahead of the one being multiplied (16-byte pieces XOR-swizzled by row on the global side; rows past M
+//     lie past the end of the buffer descriptor and read as zeros). Nothing passes through registers, and the one
+//     barrier per chunk waits for loads that were issued three chunks earlier.
+//   * The weights are fetched kSkinnyWDepth chunks ahead into a ring of registers by ordinary loads at clamped
+//     (always valid) addresses. Loads return in order, and the compiler counts only its own when it waits for a
+//     ring slot, so the ring is deeper than the activation queue: the wait for chunk c then covers the activation
+//     copy of chunk c + 1 and leaves the newer ones in flight.
+constexpr int kSkinnyWChunk = 256, kSkinnyWBufs = 4, kSkinnyWDepth = 5;
+
 template <typename T, int NTW>
 __global__ __launch_bounds__(NTW * 4 * 64) void gemmSkinnyWideKernel(SkinnyArgs a) {
   using Frag = typename MfmaOp<T>::Frag;
-  constexpr int KS = 4, G = 4, THREADS = NTW * KS * 64, CHUNK = KS * kSkinnyStep, LDX = CHUNK + kSkinnyPad;
-  constexpr int PIECES = 16 * G * (CHUNK / 8), PER = (PIECES + THREADS - 1) / THREADS;  // 16-byte pieces of a chunk
+  constexpr int KS = 4, G = 4, NW = NTW * KS, CHUNK = kSkinnyWChunk, NBUF = kSkinnyWBufs, DEPTH = kSkinnyWDepth;
+  constexpr int SLOTS = DEPTH + 1, UNROLL = SLOTS * NBUF / (SLOTS % 2 == 0 ? 2 : 1);  // a common multiple of both rings
+  static_assert(UNROLL % SLOTS == 0 && UNROLL % NBUF == 0, "ring indices must be compile-time");
+  constexpr int BUF = 64 * CHUNK;       // elements of one activation buffer
+  constexpr int XPW = (32 + NW - 1) / NW;  // copy instructions (two rows each) per wave and chunk, at most
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  T* sx = reinterpret_cast<T*>(smem);  // two buffers of 64 rows x LDX
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  T* sx = reinterpret_cast<T*>(smem);  // NBUF buffers of 64 rows x CHUNK
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int tile = wave / KS, ks = wave % KS;
   const int r16 = lane & 15, kgrp = lane >> 4;
   const int n0 = (blockIdx.x * NTW + tile) * 16;
-  const T* wbase = reinterpret_cast<const T*>(a.B) + (int64_t)min(n0 + r16, a.N - 1) * a.ldb + kgrp * 32;
-  const T* xbase = reinterpret_cast<const T*>(a.A);
   const int kBegin = blockIdx.y * a.kPerWg, kEnd = min(a.K, kBegin + a.kPerWg);  // grid.y slices K (whole chunks)
   const int nChunks = (kEnd - kBegin + CHUNK - 1) / CHUNK;
+  // lane (n = lane % 16, kgrp = lane / 16) takes 16 consecutive weights of row n per chunk: two 16-byte loads,
+  // the K slots of two MFMAs. Columns past the end of K read the last valid ones instead and are not used.
+  const T* wbase = reinterpret_cast<const T*>(a.B) + (int64_t)min(n0 + r16, a.N - 1) * a.ldb + kgrp * 16;
+  auto loadW = [&](int c, Frag (&w)[2]) {
+    const T* src = wbase + min(kBegin + min(c, nChunks - 1) * CHUNK + ks * 64, kEnd - 64);
+    w[0] = *reinterpret_cast<const Frag*>(src);
+    w[1] = *reinterpret_cast<const Frag*>(src + 8);
+  };
+  const uint64_t xp = reinterpret_cast<uint64_t>(a.A);
+  const u32x4 rsX = {(uint32_t)xp, (uint32_t)(xp >> 32) & 0xffffu, (uint32_t)(((int64_t)(a.M - 1) * a.lda + a.K) * sizeof(T)),
+                     0x00020000u};
+  const unsigned ldsBase = (unsigned)(size_t)(__attribute__((address_space(3))) char*)smem;
+  // copy instruction j of a chunk fills rows 2 j and 2 j + 1 of the buffer (1 KiB): lane l owns physical 16-byte
+  // piece l % 32 of row 2 j + l / 32 and fetches the logical piece the swizzle puts there
+  int xoff[XPW];
+#pragma unroll
+  for (int i = 0; i < XPW; ++i) {
+    const int row = 2 * (wave + i * NW) + (lane >> 5);
+    xoff[i] = (int)(((int64_t)row * a.lda + (((lane & 31) ^ (row & 15)) << 3)) * sizeof(T));
+  }
+  // (a chunk past the end copies the last one again, into a buffer nobody reads any more: every wave then has
+  // the same number of copies in flight at every barrier, which is what the wait below counts on)
+  auto copyX = [&](int c, int buf) {
+    const int from = (kBegin + min(c, nChunks - 1) * CHUNK) * (int)sizeof(T);
+#pragma unroll
+    for (int i = 0; i < XPW; ++i)
+      if (wave + i * NW < 32) loadToLds16(rsX, xoff[i], from, ldsBase + (unsigned)((buf * BUF) * sizeof(T)) + (unsigned)(wave + i * NW) * 1024u);
+  };
   f32x4 acc[G];
 #pragma unroll
   for (int gi = 0; gi < G; ++gi) acc[gi] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // fragment rows: group gi, row r16; logical piece ks * 8 + kgrp * 2 + t sits at that index XOR r16
+  const T* xlane[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) xlane[t] = sx + r16 * CHUNK + (((ks * 8 + kgrp * 2 + t) ^ r16) << 3);
 
-  u32x4 xa[PER];
-  auto loadW = [&](int c, Frag (&w)[4]) {  // a step past the end of K reads the last step instead and is not used
-    const T* src = wbase + min(kBegin + min(c, nChunks - 1) * CHUNK + ks * kSkinnyStep, kEnd - kSkinnyStep);
+  Frag w[SLOTS][2];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) w[t] = *reinterpret_cast<const Frag*>(src + 8 * t);
-  };
-  auto loadX = [&](int c) {  // rows past M and columns past K repeat valid ones; nothing multiplies them
-    const int kc = kBegin + min(c, nChunks - 1) * CHUNK, len = min(CHUNK, kEnd - kc);
+  for (int c = 0; c < NBUF - 1; ++c) copyX(c, c);
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int p = threadIdx.x + i * THREADS, r = min(p >> 6, a.M - 1), q = min((p & 63) * 8, len - 8);
-      xa[i] = *reinterpret_cast<const u32x4*>(xbase + (int64_t)r * a.lda + kc + q);
+  for (int c = 0; c < DEPTH; ++c) loadW(c, w[c]);
+  for (int c0 = 0; c0 < nChunks; c0 += UNROLL) {
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u;
+      if (c < nChunks) {  // workgroup-uniform
+        // This wave's copies of chunk c have landed: loads return in order, and what it requested after them is
+        // the copies of NBUF - 2 chunks (at least 32 / NW instructions each) and the weights of NBUF - 1 (two
+        // loads each). Past the barrier the whole chunk is in LDS and every wave has left the buffer of chunk c - 1.
+        constexpr int kAfter = (NBUF - 2) * (32 / NW) + (NBUF - 1) * 2;
+        __builtin_amdgcn_s_waitcnt(0x0f70 | (kAfter & 15) | ((kAfter >> 4) << 14));
+        __builtin_amdgcn_s_barrier();
+        copyX(c + NBUF - 1, (u + NBUF - 1) % NBUF);
+        loadW(c + DEPTH, w[(u + DEPTH) % SLOTS]);
+        if (kBegin + c * CHUNK + ks * 64 < kEnd) {  // wave-uniform: this wave's columns of the chunk exist
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int gi = 0; gi < G; ++gi)
+              acc[gi] = MfmaOp16<T>::run(*reinterpret_cast<const Frag*>(xlane[t] + (u % NBUF) * BUF + gi * 16 * CHUNK), w[u % SLOTS][t], acc[gi]);
+        }
+      }
     }
-  };
-  auto storeX = [&](int buf) {
-    T* dst = sx + buf * (16 * G * LDX);
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int p = threadIdx.x + i * THREADS;
-      if (PIECES % THREADS == 0 || p < PIECES) *reinterpret_cast<u32x4*>(dst + (p >> 6) * LDX + (p & 63) * 8) = xa[i];
-    }
-  };
-
-  Frag wc[4], w0[4], w1[4];
-  loadW(0, w0);
-  loadW(1, w1);
-  loadX(0);
-  storeX(0);
-  __syncthreads();
-  for (int c = 0; c < nChunks; ++c) {
-#pragma unroll
-    for (int t = 0; t < 4; ++t) wc[t] = w0[t], w0[t] = w1[t];
-    loadX(c + 1);
-    loadW(c + 2, w1);
-    if (kBegin + c * CHUNK + ks * kSkinnyStep < kEnd) {  // wave-uniform: this wave's step of the chunk exists
-      const T* xs = sx + (c & 1) * (16 * G * LDX) + ks * kSkinnyStep + kgrp * 32;
-#pragma unroll
-      for (int t = 0; t < 4; ++t)
-#pragma unroll
-        for (int gi = 0; gi < G; ++gi)
-          acc[gi] = MfmaOp16<T>::run(*reinterpret_cast<const Frag*>(xs + min(gi * 16 + r16, a.M - 1) * LDX + 8 * t), wc[t], acc[gi]);
-    }
-    storeX((c + 1) & 1);  // the buffer chunk c - 1 was read from; every wave left it at the last barrier
-    __syncthreads();
   }
+  __builtin_amdgcn_s_waitcnt(0x0070);
+  __syncthreads();
   // the four K shares of a tile meet where the activations were
   float* red = reinterpret_cast<float*>(smem);  // [NTW * KS][G][4][64]
 #pragma unroll
@@ -1130,6 +1155,169 @@ __global__ __launch_bounds__(NTW * 4 * 64) void gemmSkinnyWideKernel(SkinnyArgs 
           out[(int64_t)row * a.ldo + col] = static_cast<T>(v);
         }
       }
+  }
+}
+
+// Up to 64 rows, both operands staged through LDS. Weight loads that deliver MFMA fragments straight into registers
+// touch 16 rows x 64 bytes per instruction, and that pattern streams at 3.3 - 4.8 TB/s where whole-row pieces stream
+// at 6.5 (measured on a [11008, 4096] bf16 matrix, cold). Here the copy instructions take 256 contiguous bytes of 4
+// rows each (two full cache lines per row), for the weights as for the activations, and land in LDS without passing
+// through registers; the MFMA fragments are then LDS reads (16-byte pieces XOR-swizzled by row on the global side of
+// the copy, so those reads are conflict-free).
+//   * a workgroup of eight waves owns 64 output columns for the whole of K (or a grid.y slice of it); wave w multiplies
+//     k-step w % 4 of every stage (32 of its 128 columns), all G row groups against column tiles 2 (w / 4) and
+//     2 (w / 4) + 1: six fragment reads for eight MFMAs at 64 rows. The four k-step shares meet in LDS at the end,
+//     where wave w finishes row group w % 4;
+//   * K moves in stages of 128 columns. Loads return to a wave in the order it issued them, so a wave that copied
+//     both operands could not keep the weights (from HBM: long latency, the traffic that matters) further ahead than the
+//     activations (from L2). The two are therefore copied by different waves: waves 0-3 keep WST - 1 weight stages
+//     (64 rows x 256 bytes) in flight, waves 4-7 keep XST - 1 activation stages (16 G rows x 256 bytes) in flight,
+//     each waits only for its own stage, and one barrier per stage publishes both. Rows past M and past N lie past
+//     the end of the buffer descriptors and read as zeros. The weight copies are marked non-temporal: read once,
+//     they would otherwise push the activations out of L2, and a weight stream larger than the 256 MiB memory-side
+//     cache gains nothing from passing through it (at one row, cold: 18.3 -> 16.4 us; a weight that does fit in that
+//     cache and is re-read at once loses 1 us);
+//   * workgroup b starts its walk over K at stage (13 b) mod stages and wraps around: with every workgroup on the same
+//     columns at the same time the requests fall on a fraction of the memory channels (measured at 16 rows, cold:
+//     20.0 us with a common start, 18.5 with this one, 26 when neighbours start 8 stages apart).
+constexpr int kSkinnyLdsBK = 128, kSkinnyLdsBN = 64, kSkinnyLdsStagger = 13;
+
+template <typename T, int G, int WST, int XST>
+__global__ __launch_bounds__(512) void gemmSkinnyLdsKernel(SkinnyArgs a) {
+  using Frag = typename MfmaOp<T>::Frag;
+  constexpr int BK = kSkinnyLdsBK, BN = kSkinnyLdsBN;
+  constexpr int WIPW = BN / 4 / 4, XIPW = G;      // copy instructions (4 rows x 256 bytes) per wave and stage: weights, activations
+  constexpr int WBUF = BN * BK, XBUF = G * 16 * BK;  // elements per stage buffer
+  constexpr int UNROLL = WST % XST == 0 ? WST : (XST % WST == 0 ? XST : WST * XST);
+  constexpr int IPW = WIPW > XIPW ? WIPW : XIPW;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  T* sw = reinterpret_cast<T*>(smem);   // WST weight buffers
+  T* sx = sw + WST * WBUF;              // XST activation buffers
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r16 = lane & 15, kgrp = lane >> 4;
+  const int ci = wave & 3;               // copy instruction slot of this wave (rows 4 ci + 16 i of a buffer)
+  const int kq = wave & 3, nb = wave >> 2;  // multiplies k-step kq of every stage against column tiles 2 nb, 2 nb + 1
+  const int n0 = blockIdx.x * BN;
+  const int kBegin = blockIdx.y * a.kPerWg, kEnd = min(a.K, kBegin + a.kPerWg);
+  const int nStages = (kEnd - kBegin) / BK;  // K and the slices are multiples of 128
+  const int kStart = (int)((blockIdx.x * (unsigned)kSkinnyLdsStagger) % (unsigned)nStages);
+  auto descriptor = [](const void* base, int64_t bytes) {
+    const uint64_t p = reinterpret_cast<uint64_t>(base);
+    u32x4 d = {(uint32_t)p, (uint32_t)(p >> 32) & 0xffffu, (uint32_t)bytes, 0x00020000u};
+    return d;
+  };
+  // waves 0-3 copy weights, waves 4-7 activations (wave-uniform): descriptor, row stride and first row differ
+  const bool copiesW = wave < 4;
+  const u32x4 rs = copiesW ? descriptor(a.B, ((int64_t)(a.N - 1) * a.ldb + a.K) * sizeof(T))
+                           : descriptor(a.A, ((int64_t)(a.M - 1) * a.lda + a.K) * sizeof(T));
+  const int ipw = copiesW ? WIPW : XIPW;
+  const unsigned ldsBase = (unsigned)(size_t)(__attribute__((address_space(3))) char*)(copiesW ? sw : sx);
+  const unsigned bufBytes = (unsigned)((copiesW ? WBUF : XBUF) * sizeof(T));
+  // copy instruction q = ci + 4 i of a stage fills rows 4 q .. 4 q + 3 of the buffer; lane l owns physical piece l % 16
+  // of row l / 16 and fetches the logical piece the swizzle puts there
+  unsigned voff[IPW];
+#pragma unroll
+  for (int i = 0; i < IPW; ++i) {
+    const int row = 4 * (ci + 4 * i) + (lane >> 4), piece = ((lane & 15) ^ (row & 15)) << 3;
+    voff[i] = copiesW ? (unsigned)(((int64_t)(n0 + row) * a.ldb + piece) * sizeof(T)) : (unsigned)(((int64_t)row * a.lda + piece) * sizeof(T));
+  }
+  // (a stage past the end copies the last one again, into a buffer nobody reads any more: a wave then has the
+  // same number of copies in flight at every barrier, which is what its wait counts on)
+  auto copyStage = [&](int c, int buf) {
+    int cc = min(c, nStages - 1) + kStart;
+    if (cc >= nStages) cc -= nStages;
+    const int from = (kBegin + cc * BK) * (int)sizeof(T);
+#pragma unroll
+    for (int i = 0; i < IPW; ++i)
+      if (i < ipw) {
+        const unsigned to = ldsBase + (unsigned)buf * bufBytes + (unsigned)(ci + 4 * i) * 1024u;
+        if (copiesW) loadToLds16Stream(rs, (int)voff[i], from, to);  // read once: must not push the activations out of L2
+        else loadToLds16(rs, (int)voff[i], from, to);
+      }
+  };
+  f32x4 acc[G][2];
+#pragma unroll
+  for (int gi = 0; gi < G; ++gi) acc[gi][0] = acc[gi][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // this wave's fragments: logical piece 4 kq + kgrp of row r16 (activations: + 16 gi rows; weights: + 32 nb + 16 j rows).
+  // Every staged byte is read by two waves (activations) or one (weights): LDS bandwidth is what bounds 64 rows.
+  const int off = ((4 * kq + kgrp) ^ r16) << 3;
+  const T* xlane = sx + r16 * BK + off;
+  const T* wlane = sw + (nb * 32 + r16) * BK + off;
+
+  if (copiesW) {
+#pragma unroll
+    for (int c = 0; c < WST - 1; ++c) copyStage(c, c);
+  } else {
+#pragma unroll
+    for (int c = 0; c < XST - 1; ++c) copyStage(c, c);
+  }
+  for (int c0 = 0; c0 < nStages; c0 += UNROLL) {
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u;
+      if (c < nStages) {  // workgroup-uniform
+        // this wave's copies of stage c have landed: loads return in order, and only the stages it requested after that
+        // one are still in flight. Past the barrier both operands of the stage are in LDS and every wave has left the
+        // buffers of stage c - 1, which the next copies overwrite.
+        if (copiesW) {
+          constexpr int n = (WST - 2) * WIPW;
+          __builtin_amdgcn_s_waitcnt(0x0f70 | (n & 15) | ((n >> 4) << 14));
+        } else {
+          constexpr int n = (XST - 2) * XIPW;
+          __builtin_amdgcn_s_waitcnt(0x0f70 | (n & 15) | ((n >> 4) << 14));
+        }
+        __builtin_amdgcn_s_barrier();
+        if (copiesW) copyStage(c + WST - 1, (u + WST - 1) % WST);
+        else copyStage(c + XST - 1, (u + XST - 1) % XST);
+        const T* xs = xlane + (u % XST) * XBUF;
+        const T* ws = wlane + (u % WST) * WBUF;
+        const Frag w0 = *reinterpret_cast<const Frag*>(ws), w1 = *reinterpret_cast<const Frag*>(ws + 16 * BK);
+#pragma unroll
+        for (int gi = 0; gi < G; ++gi) {
+          const Frag xf = *reinterpret_cast<const Frag*>(xs + gi * 16 * BK);
+          acc[gi][0] = MfmaOp16<T>::run(xf, w0, acc[gi][0]);
+          acc[gi][1] = MfmaOp16<T>::run(xf, w1, acc[gi][1]);
+        }
+      }
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0x0070);  // the repeated copies of the last stage: nothing may land after the workgroup has gone
+  __syncthreads();
+  // the four k-step shares of a column tile pair meet where the stages were; wave (nb, kq) then finishes row group kq
+  float* red = reinterpret_cast<float*>(smem);  // [8 waves][G][2][4][64]
+#pragma unroll
+  for (int gi = 0; gi < G; ++gi)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[(((wave * G + gi) * 2 + j) * 4 + r) * 64 + lane] = acc[gi][j][r];
+  __syncthreads();
+  const int gi = kq;
+  if (gi < G) {
+    T* out = reinterpret_cast<T*>(a.out);
+    const T* cin = reinterpret_cast<const T*>(a.Cin);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int col = n0 + nb * 32 + j * 16 + r16;
+      if (col >= a.N) continue;
+      const float bv = a.bias ? static_cast<float>(reinterpret_cast<const T*>(a.bias)[col]) : 0.f;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = gi * 16 + kgrp * 4 + r;
+        if (row < a.M) {
+          float v = 0.f;
+#pragma unroll
+          for (int k2 = 0; k2 < 4; ++k2) v += red[((((nb * 4 + k2) * G + gi) * 2 + j) * 4 + r) * 64 + lane];
+          if (a.partial) {  // this slice's sum; the reduction pass applies the epilogue
+            a.partial[((int64_t)blockIdx.y * a.M + row) * a.N + col] = v;
+            continue;
+          }
+          v = v * a.alpha + bv;
+          if (cin) v += a.beta * static_cast<float>(cin[(int64_t)row * a.sCm + (int64_t)col * a.sCn]);
+          out[(int64_t)row * a.ldo + col] = static_cast<T>(v);
+        }
+      }
+    }
   }
 }
 
@@ -1379,10 +1567,20 @@ static diopiError_t launchSkinny(hipStream_t stream, const SkinnyArgs& a) {
   return diopiSuccess;
 }
 
+template <typename T, int G, int WST, int XST>
+static diopiError_t launchSkinnyLds(hipStream_t stream, const SkinnyArgs& a) {
+  const int lds = (WST * kSkinnyLdsBN + XST * G * 16) * kSkinnyLdsBK * (int)sizeof(T);
+  AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmSkinnyLdsKernel<T, G, WST, XST>), lds));
+  const int splits = (a.K + a.kPerWg - 1) / a.kPerWg;
+  hipLaunchKernelGGL((gemmSkinnyLdsKernel<T, G, WST, XST>), dim3((unsigned)((a.N + kSkinnyLdsBN - 1) / kSkinnyLdsBN), (unsigned)splits), dim3(512), lds,
+                     stream, a);
+  AMD_LAUNCH_CHECK();
+  return diopiSuccess;
+}
+
 template <typename T, int NTW>
 static diopiError_t launchSkinnyWide(hipStream_t stream, const SkinnyArgs& a) {
-  constexpr int CHUNK = 4 * kSkinnyStep;
-  const int lds = std::max(2 * 64 * (CHUNK + kSkinnyPad) * (int)sizeof(T), NTW * 4 * 4 * 4 * 64 * (int)sizeof(float));
+  const int lds = std::max(kSkinnyWBufs * 64 * kSkinnyWChunk * (int)sizeof(T), NTW * 4 * 4 * 4 * 64 * (int)sizeof(float));
   AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmSkinnyWideKernel<T, NTW>), lds));
   const int tiles = (a.N + 15) / 16;
   const int splits = (a.K + a.kPerWg - 1) / a.kPerWg;
@@ -1413,6 +1611,19 @@ static diopiError_t launchSkinnyForShape(diopiContextHandle_t ctx, hipStream_t s
   a.alpha = p.alpha, a.beta = p.beta;
   a.partial = nullptr, a.kPerWg = a.K;
   const int tiles = (a.N + 15) / 16, cus = computeUnits(), perCu = (tiles + cus - 1) / cus;
+  // Wide weights (64-column blocks for at least half the CUs): both operands through LDS, see gemmSkinnyLdsKernel.
+  // Measured cold against the forms below on K = 4096 (us): N = 8192 16.6 -> 15.0 at one row, 18.0 -> 17.1 at 16,
+  // 22.5 -> 19.3 at 32, 27.3 -> 23.5 at 64; N = 12288 20.3 -> 18.4, 21.9 -> 19.4, 26.0 -> 21.2, 29.6 -> 25.2;
+  // N = 22016 38.2 -> 35.2, 46.0 -> 36.8, 52.9 -> 41.5, 55.7 -> 48.5. Narrower weights (N = 4096: 64 workgroups)
+  // lose to the K-split forms and stay with them.
+  if ((a.N + kSkinnyLdsBN - 1) / kSkinnyLdsBN >= cus / 2 &&
+      ((int64_t)(a.N - 1) * a.ldb + a.K) * (int64_t)sizeof(T) < ((int64_t)1 << 32) &&
+      ((int64_t)(a.M - 1) * a.lda + a.K) * (int64_t)sizeof(T) < ((int64_t)1 << 32)) {
+    if (a.M <= 16) return launchSkinnyLds<T, 1, 4, 4>(stream, a);
+    if (a.M <= 32) return launchSkinnyLds<T, 2, 4, 4>(stream, a);
+    if (a.M <= 48) return launchSkinnyLds<T, 3, 4, 4>(stream, a);
+    return launchSkinnyLds<T, 4, 4, 4>(stream, a);
+  }
   if (a.M <= 16) {
     // 16-column tiles per workgroup: about one workgroup per CU, the other waves of the 15 or 16 split K
     if (perCu >= 4) return launchSkinny<T, 4, 4, 1>(stream, a);

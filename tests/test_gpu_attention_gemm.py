@@ -145,7 +145,8 @@ def test_split_k_gemm(ops, dev, dtype, m, n, k):
                                    (40, 16 * 7 + 3, 384), (64, 16000, 128), (1, 16, 128), (64, 4096, 4096),
                                    (48, 12288, 1024 + 768), (33, 2056, 11008),
                                    (64, 12288, 4096), (33, 12296, 4096 + 128), (50, 16384, 4096 + 384), (64, 22016, 4096), (64, 9216, 4096),
-                                   (64, 4096, 8192), (40, 4104, 11008), (64, 6144, 4096 + 640)])
+                                   (64, 4096, 8192), (40, 4104, 11008), (64, 6144, 4096 + 640),
+                                   (20, 8200, 640), (1, 12288, 256), (32, 32000, 384), (7, 8192, 128)])
 def test_skinny_m_linear_and_addmm(ops, dev, dtype, m, n, k):
     """At most 64 rows against a K-contiguous weight with K a multiple of 128 select the weight-streaming kernel:
     one, two and four 16-column tiles per workgroup (N = 4096, 11008, 32000), K in one and in two staged chunks
@@ -156,7 +157,10 @@ def test_skinny_m_linear_and_addmm(ops, dev, dtype, m, n, k):
     column tiles, K from 4096) take the whole-K form with double-buffered activations: three and four tiles per
     workgroup, a last chunk of one and of three steps, a ragged last tile and a last workgroup with a tile past N;
     the three after them run it on K slices (four even slices, four with a short last one, two with a ragged
-    second) that meet in the reduction pass."""
+    second) that meet in the reduction pass. Weights at least 8192 columns wide take the form that stages both
+    operands through LDS (64-column workgroups walking K in stages of 128 from a staggered start): one to four row
+    groups, ragged N with a last workgroup partly and wholly past it, K of one, two, three and five stages (fewer
+    than the ring holds) up to 35."""
     x = torch.randn(m, k, generator=g(50)).to(dtype)
     w = (torch.randn(n, k, generator=g(51)) * 0.05).to(dtype)
     b = torch.randn(n, generator=g(52)).to(dtype)
