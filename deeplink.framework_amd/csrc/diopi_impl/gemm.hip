@@ -925,6 +925,7 @@ struct SkinnyArgs {
   float alpha, beta;
   float* partial;  // K split over grid.y: fp32 partial products [gridDim.y][M][N] for splitKReduceKernel, else null
   int kPerWg;      // K columns per grid.y slice (K when not split)
+  int colsPerWg;   // gemmSkinnyLdsKernel: output columns per workgroup
 };
 
 constexpr int kSkinnyStep = 128;    // K elements one wave consumes per step (4 kgrps x 32)
@@ -1164,14 +1165,15 @@ __global__ __launch_bounds__(NTW * 4 * 64) void gemmSkinnyWideKernel(SkinnyArgs 
 // rows each (two full cache lines per row), for the weights as for the activations, and land in LDS without passing
 // through registers; the MFMA fragments are then LDS reads (16-byte pieces XOR-swizzled by row on the global side of
 // the copy, so those reads are conflict-free).
-//   * a workgroup of eight waves owns 64 output columns for the whole of K (or a grid.y slice of it); wave w multiplies
-//     k-step w % 4 of every stage (32 of its 128 columns), all G row groups against column tiles 2 (w / 4) and
-//     2 (w / 4) + 1: six fragment reads for eight MFMAs at 64 rows. The four k-step shares meet in LDS at the end,
-//     where wave w finishes row group w % 4;
+//   * a workgroup of eight waves owns colsPerWg output columns (at most 32 NTP: 64 or 128) for the whole of K (or a
+//     grid.y slice of it); the host deals the columns evenly over the CUs, and weight rows past a workgroup's share
+//     are not fetched. Wave w multiplies k-step w % 4 of every stage (32 of its 128 columns), all G row groups
+//     against the NTP column tiles of its half: G + NTP fragment reads for G NTP MFMAs. The four k-step shares meet
+//     in LDS at the end, where wave w finishes row group w % 4;
 //   * K moves in stages of 128 columns. Loads return to a wave in the order it issued them, so a wave that copied
 //     both operands could not keep the weights (from HBM: long latency, the traffic that matters) further ahead than the
 //     activations (from L2). The two are therefore copied by different waves: waves 0-3 keep WST - 1 weight stages
-//     (64 rows x 256 bytes) in flight, waves 4-7 keep XST - 1 activation stages (16 G rows x 256 bytes) in flight,
+//     (32 NTP rows x 256 bytes) in flight, waves 4-7 keep XST - 1 activation stages (16 G rows x 256 bytes) in flight,
 //     each waits only for its own stage, and one barrier per stage publishes both. Rows past M and past N lie past
 //     the end of the buffer descriptors and read as zeros. The weight copies are marked non-temporal: read once,
 //     they would otherwise push the activations out of L2, and a weight stream larger than the 256 MiB memory-side
@@ -1179,13 +1181,17 @@ __global__ __launch_bounds__(NTW * 4 * 64) void gemmSkinnyWideKernel(SkinnyArgs 
 //     cache and is re-read at once loses 1 us);
 //   * workgroup b starts its walk over K at stage (13 b) mod stages and wraps around: with every workgroup on the same
 //     columns at the same time the requests fall on a fraction of the memory channels (measured at 16 rows, cold:
-//     20.0 us with a common start, 18.5 with this one, 26 when neighbours start 8 stages apart).
-constexpr int kSkinnyLdsBK = 128, kSkinnyLdsBN = 64, kSkinnyLdsStagger = 13;
+//     20.0 us with a common start, 18.5 with this one, 26 when neighbours start 8 stages apart);
+//   * more stages in flight are slower, here as in the other streaming kernels (weights 5 or 7 stages ahead instead
+//     of 3: 16.9 -> 18.8 and 18.0 us at one row), and so is leaving the copies to four extra waves that do nothing else.
+//     What bounds 64 rows is the bytes a CU takes in: every workgroup reads all the activations (from L2), as many
+//     bytes again as its share of the weights.
+constexpr int kSkinnyLdsBK = 128, kSkinnyLdsBN = 64, kSkinnyLdsStagger = 13;  // (64: the narrower of the two workgroup widths)
 
-template <typename T, int G, int WST, int XST>
+template <typename T, int G, int NTP, int WST, int XST>
 __global__ __launch_bounds__(512) void gemmSkinnyLdsKernel(SkinnyArgs a) {
   using Frag = typename MfmaOp<T>::Frag;
-  constexpr int BK = kSkinnyLdsBK, BN = kSkinnyLdsBN;
+  constexpr int BK = kSkinnyLdsBK, BN = 32 * NTP;  // NTP column tiles of 16 per wave, two waves side by side
   constexpr int WIPW = BN / 4 / 4, XIPW = G;      // copy instructions (4 rows x 256 bytes) per wave and stage: weights, activations
   constexpr int WBUF = BN * BK, XBUF = G * 16 * BK;  // elements per stage buffer
   constexpr int UNROLL = WST % XST == 0 ? WST : (XST % WST == 0 ? XST : WST * XST);
@@ -1196,8 +1202,8 @@ __global__ __launch_bounds__(512) void gemmSkinnyLdsKernel(SkinnyArgs a) {
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r16 = lane & 15, kgrp = lane >> 4;
   const int ci = wave & 3;               // copy instruction slot of this wave (rows 4 ci + 16 i of a buffer)
-  const int kq = wave & 3, nb = wave >> 2;  // multiplies k-step kq of every stage against column tiles 2 nb, 2 nb + 1
-  const int n0 = blockIdx.x * BN;
+  const int kq = wave & 3, nb = wave >> 2;  // multiplies k-step kq of every stage against column tiles NTP nb ... NTP nb + NTP - 1
+  const int n0 = blockIdx.x * a.colsPerWg, nCols = min(a.colsPerWg, a.N - n0);  // this workgroup's columns: at most BN
   const int kBegin = blockIdx.y * a.kPerWg, kEnd = min(a.K, kBegin + a.kPerWg);
   const int nStages = (kEnd - kBegin) / BK;  // K and the slices are multiples of 128
   const int kStart = (int)((blockIdx.x * (unsigned)kSkinnyLdsStagger) % (unsigned)nStages);
@@ -1219,7 +1225,9 @@ __global__ __launch_bounds__(512) void gemmSkinnyLdsKernel(SkinnyArgs a) {
 #pragma unroll
   for (int i = 0; i < IPW; ++i) {
     const int row = 4 * (ci + 4 * i) + (lane >> 4), piece = ((lane & 15) ^ (row & 15)) << 3;
-    voff[i] = copiesW ? (unsigned)(((int64_t)(n0 + row) * a.ldb + piece) * sizeof(T)) : (unsigned)(((int64_t)row * a.lda + piece) * sizeof(T));
+    // (weight rows past this workgroup's columns: an offset past the end of the descriptor, which reads zeros without traffic)
+    voff[i] = copiesW ? (row < nCols ? (unsigned)(((int64_t)(n0 + row) * a.ldb + piece) * sizeof(T)) : 0x80000000u)
+                      : (unsigned)(((int64_t)row * a.lda + piece) * sizeof(T));
   }
   // (a stage past the end copies the last one again, into a buffer nobody reads any more: a wave then has the
   // same number of copies in flight at every barrier, which is what its wait counts on)
@@ -1235,14 +1243,16 @@ __global__ __launch_bounds__(512) void gemmSkinnyLdsKernel(SkinnyArgs a) {
         else loadToLds16(rs, (int)voff[i], from, to);
       }
   };
-  f32x4 acc[G][2];
+  f32x4 acc[G][NTP];
 #pragma unroll
-  for (int gi = 0; gi < G; ++gi) acc[gi][0] = acc[gi][1] = f32x4{0.f, 0.f, 0.f, 0.f};
-  // this wave's fragments: logical piece 4 kq + kgrp of row r16 (activations: + 16 gi rows; weights: + 32 nb + 16 j rows).
+  for (int gi = 0; gi < G; ++gi)
+#pragma unroll
+    for (int j = 0; j < NTP; ++j) acc[gi][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // this wave's fragments: logical piece 4 kq + kgrp of row r16 (activations: + 16 gi rows; weights: + 16 (NTP nb + j) rows).
   // Every staged byte is read by two waves (activations) or one (weights): LDS bandwidth is what bounds 64 rows.
   const int off = ((4 * kq + kgrp) ^ r16) << 3;
   const T* xlane = sx + r16 * BK + off;
-  const T* wlane = sw + (nb * 32 + r16) * BK + off;
+  const T* wlane = sw + (nb * NTP * 16 + r16) * BK + off;
 
   if (copiesW) {
 #pragma unroll
@@ -1271,12 +1281,14 @@ __global__ __launch_bounds__(512) void gemmSkinnyLdsKernel(SkinnyArgs a) {
         else copyStage(c + XST - 1, (u + XST - 1) % XST);
         const T* xs = xlane + (u % XST) * XBUF;
         const T* ws = wlane + (u % WST) * WBUF;
-        const Frag w0 = *reinterpret_cast<const Frag*>(ws), w1 = *reinterpret_cast<const Frag*>(ws + 16 * BK);
+        Frag wf[NTP];
+#pragma unroll
+        for (int j = 0; j < NTP; ++j) wf[j] = *reinterpret_cast<const Frag*>(ws + j * 16 * BK);
 #pragma unroll
         for (int gi = 0; gi < G; ++gi) {
           const Frag xf = *reinterpret_cast<const Frag*>(xs + gi * 16 * BK);
-          acc[gi][0] = MfmaOp16<T>::run(xf, w0, acc[gi][0]);
-          acc[gi][1] = MfmaOp16<T>::run(xf, w1, acc[gi][1]);
+#pragma unroll
+          for (int j = 0; j < NTP; ++j) acc[gi][j] = MfmaOp16<T>::run(xf, wf[j], acc[gi][j]);
         }
       }
     }
@@ -1284,22 +1296,22 @@ __global__ __launch_bounds__(512) void gemmSkinnyLdsKernel(SkinnyArgs a) {
   __builtin_amdgcn_s_waitcnt(0x0070);  // the repeated copies of the last stage: nothing may land after the workgroup has gone
   __syncthreads();
   // the four k-step shares of a column tile pair meet where the stages were; wave (nb, kq) then finishes row group kq
-  float* red = reinterpret_cast<float*>(smem);  // [8 waves][G][2][4][64]
+  float* red = reinterpret_cast<float*>(smem);  // [8 waves][G][NTP][4][64]
 #pragma unroll
   for (int gi = 0; gi < G; ++gi)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < NTP; ++j)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) red[(((wave * G + gi) * 2 + j) * 4 + r) * 64 + lane] = acc[gi][j][r];
+      for (int r = 0; r < 4; ++r) red[(((wave * G + gi) * NTP + j) * 4 + r) * 64 + lane] = acc[gi][j][r];
   __syncthreads();
   const int gi = kq;
   if (gi < G) {
     T* out = reinterpret_cast<T*>(a.out);
     const T* cin = reinterpret_cast<const T*>(a.Cin);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int col = n0 + nb * 32 + j * 16 + r16;
-      if (col >= a.N) continue;
+    for (int j = 0; j < NTP; ++j) {
+      const int lc = (nb * NTP + j) * 16 + r16, col = n0 + lc;
+      if (lc >= nCols) continue;
       const float bv = a.bias ? static_cast<float>(reinterpret_cast<const T*>(a.bias)[col]) : 0.f;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
@@ -1307,7 +1319,7 @@ __global__ __launch_bounds__(512) void gemmSkinnyLdsKernel(SkinnyArgs a) {
         if (row < a.M) {
           float v = 0.f;
 #pragma unroll
-          for (int k2 = 0; k2 < 4; ++k2) v += red[((((nb * 4 + k2) * G + gi) * 2 + j) * 4 + r) * 64 + lane];
+          for (int k2 = 0; k2 < 4; ++k2) v += red[((((nb * 4 + k2) * G + gi) * NTP + j) * 4 + r) * 64 + lane];
           if (a.partial) {  // this slice's sum; the reduction pass applies the epilogue
             a.partial[((int64_t)blockIdx.y * a.M + row) * a.N + col] = v;
             continue;
@@ -1567,13 +1579,14 @@ static diopiError_t launchSkinny(hipStream_t stream, const SkinnyArgs& a) {
   return diopiSuccess;
 }
 
-template <typename T, int G, int WST, int XST>
+template <typename T, int G, int NTP, int WST, int XST>
 static diopiError_t launchSkinnyLds(hipStream_t stream, const SkinnyArgs& a) {
-  const int lds = (WST * kSkinnyLdsBN + XST * G * 16) * kSkinnyLdsBK * (int)sizeof(T);
-  AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmSkinnyLdsKernel<T, G, WST, XST>), lds));
+  constexpr int BN = 32 * NTP;
+  AMD_CHECK(a.colsPerWg >= 1 && a.colsPerWg <= BN, "skinny linear: %d columns per workgroup do not fit %d", a.colsPerWg, BN);
+  const int lds = std::max((WST * BN + XST * G * 16) * kSkinnyLdsBK * (int)sizeof(T), 8 * G * NTP * 4 * 64 * (int)sizeof(float));
+  AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmSkinnyLdsKernel<T, G, NTP, WST, XST>), lds));
   const int splits = (a.K + a.kPerWg - 1) / a.kPerWg;
-  hipLaunchKernelGGL((gemmSkinnyLdsKernel<T, G, WST, XST>), dim3((unsigned)((a.N + kSkinnyLdsBN - 1) / kSkinnyLdsBN), (unsigned)splits), dim3(512), lds,
-                     stream, a);
+  hipLaunchKernelGGL((gemmSkinnyLdsKernel<T, G, NTP, WST, XST>), dim3((unsigned)((a.N + a.colsPerWg - 1) / a.colsPerWg), (unsigned)splits), dim3(512), lds, stream, a);
   AMD_LAUNCH_CHECK();
   return diopiSuccess;
 }
@@ -1611,18 +1624,30 @@ static diopiError_t launchSkinnyForShape(diopiContextHandle_t ctx, hipStream_t s
   a.alpha = p.alpha, a.beta = p.beta;
   a.partial = nullptr, a.kPerWg = a.K;
   const int tiles = (a.N + 15) / 16, cus = computeUnits(), perCu = (tiles + cus - 1) / cus;
-  // Wide weights (64-column blocks for at least half the CUs): both operands through LDS, see gemmSkinnyLdsKernel.
-  // Measured cold against the forms below on K = 4096 (us): N = 8192 16.6 -> 15.0 at one row, 18.0 -> 17.1 at 16,
-  // 22.5 -> 19.3 at 32, 27.3 -> 23.5 at 64; N = 12288 20.3 -> 18.4, 21.9 -> 19.4, 26.0 -> 21.2, 29.6 -> 25.2;
-  // N = 22016 38.2 -> 35.2, 46.0 -> 36.8, 52.9 -> 41.5, 55.7 -> 48.5. Narrower weights (N = 4096: 64 workgroups)
-  // lose to the K-split forms and stay with them.
-  if ((a.N + kSkinnyLdsBN - 1) / kSkinnyLdsBN >= cus / 2 &&
-      ((int64_t)(a.N - 1) * a.ldb + a.K) * (int64_t)sizeof(T) < ((int64_t)1 << 32) &&
-      ((int64_t)(a.M - 1) * a.lda + a.K) * (int64_t)sizeof(T) < ((int64_t)1 << 32)) {
-    if (a.M <= 16) return launchSkinnyLds<T, 1, 4, 4>(stream, a);
-    if (a.M <= 32) return launchSkinnyLds<T, 2, 4, 4>(stream, a);
-    if (a.M <= 48) return launchSkinnyLds<T, 3, 4, 4>(stream, a);
-    return launchSkinnyLds<T, 4, 4, 4>(stream, a);
+  // Both operands through LDS, see gemmSkinnyLdsKernel. The columns are dealt evenly over as many workgroups as there
+  // are CUs (43 each at N = 11008, where 64-column blocks would leave a third of the CUs idle): a CU takes in about
+  // 45 GB/s from a cold stream whatever the software pipeline depth, so the count of CUs at work sets the rate.
+  // Measured cold against the forms below on K = 4096 (us, at 1 / 16 / 32 / 64 rows): N = 6144 13.7 -> 12.9,
+  // 15.2 -> 13.4, 24.5 -> 14.9, 25.0 -> 18.2; N = 8192 16.6 -> 13.3, 18.0 -> 14.5, 22.5 -> 16.4, 27.3 -> 19.5;
+  // N = 11008 18.5 -> 16.9, 20.4 -> 17.7, 33 -> 19.3, 30.4 -> 23.2; N = 22016 38.2 -> 30.1, 46.0 -> 31.9,
+  // 52.9 -> 33.6, 55.7 -> 36.0. At N = 4096 (16 columns per workgroup: the activations are four times the weight
+  // bytes on the way into a CU) only 17 to 32 rows gain (14.4 -> 12.7); one row loses (9.1 -> 11.0), and so does
+  // everything narrower.
+  if ((a.N >= 5120 || (a.N >= 4096 && a.M > 16 && a.M <= 32)) &&
+      ((int64_t)(a.N - 1) * a.ldb + a.K) * (int64_t)sizeof(T) < ((int64_t)1 << 31) &&
+      ((int64_t)(a.M - 1) * a.lda + a.K) * (int64_t)sizeof(T) < ((int64_t)1 << 31)) {
+    const int rounds = (a.N + 128 * cus - 1) / (128 * cus);
+    a.colsPerWg = (a.N + cus * rounds - 1) / (cus * rounds);
+    if (a.colsPerWg > 64) {
+      if (a.M <= 16) return launchSkinnyLds<T, 1, 4, 3, 3>(stream, a);
+      if (a.M <= 32) return launchSkinnyLds<T, 2, 4, 3, 3>(stream, a);
+      if (a.M <= 48) return launchSkinnyLds<T, 3, 4, 3, 3>(stream, a);
+      return launchSkinnyLds<T, 4, 4, 3, 3>(stream, a);
+    }
+    if (a.M <= 16) return launchSkinnyLds<T, 1, 2, 4, 4>(stream, a);
+    if (a.M <= 32) return launchSkinnyLds<T, 2, 2, 4, 4>(stream, a);
+    if (a.M <= 48) return launchSkinnyLds<T, 3, 2, 4, 4>(stream, a);
+    return launchSkinnyLds<T, 4, 2, 4, 4>(stream, a);
   }
   if (a.M <= 16) {
     // 16-column tiles per workgroup: about one workgroup per CU, the other waves of the 15 or 16 split K

@@ -157,10 +157,11 @@ def test_skinny_m_linear_and_addmm(ops, dev, dtype, m, n, k):
     column tiles, K from 4096) take the whole-K form with double-buffered activations: three and four tiles per
     workgroup, a last chunk of one and of three steps, a ragged last tile and a last workgroup with a tile past N;
     the three after them run it on K slices (four even slices, four with a short last one, two with a ragged
-    second) that meet in the reduction pass. Weights at least 8192 columns wide take the form that stages both
-    operands through LDS (64-column workgroups walking K in stages of 128 from a staggered start): one to four row
-    groups, ragged N with a last workgroup partly and wholly past it, K of one, two, three and five stages (fewer
-    than the ring holds) up to 35."""
+    second) that meet in the reduction pass. Weights at least 5120 columns wide (4096 at 17 to 32 rows) take the
+    form that stages both operands through LDS (columns dealt evenly over the CUs, up to 64 or 128 per workgroup,
+    walking K in stages of 128 from a staggered start): one to four row groups, column shares that are no multiple
+    of 16, a last workgroup with fewer columns, K of one, two, three and five stages (fewer than the ring holds)
+    up to 86."""
     x = torch.randn(m, k, generator=g(50)).to(dtype)
     w = (torch.randn(n, k, generator=g(51)) * 0.05).to(dtype)
     b = torch.randn(n, generator=g(52)).to(dtype)
