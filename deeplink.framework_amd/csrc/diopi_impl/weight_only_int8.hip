@@ -52,6 +52,7 @@ struct W8Args {
   int64_t ldx, ldw, ldo;
   int M, N, K;
   int scaleDtype, biasDtype;
+  int colsPerWg;  // w8LinearLdsKernel: output channels per workgroup
 };
 
 // The four int8 of one dword as floats: one SDWA conversion per byte (left to itself the compiler shifts
@@ -182,6 +183,205 @@ __global__ __launch_bounds__(NTW * kW8KSplit * 64) void w8LinearKernel(W8Args a)
   }
 }
 
+// Wide weights: both operands staged through LDS, the int8 counterpart of the bf16 decode kernel.
+//   * Weight loads that deliver MFMA fragments straight into registers touch 16 rows x 32 bytes per instruction, a pattern
+//     that streams far below what whole-row pieces reach. Here a copy instruction takes 256 contiguous bytes of 4 weight
+//     rows (or 512 bytes of 2 activation rows) and lands in LDS without passing through registers, 16-byte pieces
+//     XOR-swizzled by row on the global side so that the fragment reads are conflict-free. The weight copies are
+//     non-temporal (read once; they must not push the activations out of L2).
+//   * The host deals the output channels evenly over the CUs: a workgroup of eight waves owns colsPerWg of them (at most
+//     32 NTP) for the whole of K and at most 64 rows (grid.y walks further row groups). K moves in stages of BK = 256
+//     (stages of 512, deeper rings of either operand and two stages per barrier all measured slower): wave w
+//     takes columns 64 (w % 4) .. + 63 of every stage, lane (n, kgrp) 16 consecutive int8 of them (one 16-byte LDS read,
+//     converted in registers into the operands of two MFMAs), all G row groups against the NTP channel tiles of its half.
+//     The four shares meet in LDS at the end, where wave w finishes row group w % 4: per-channel scale on the fp32 sum,
+//     bias, one rounding.
+//   * Loads return to a wave in the order it issued them, so weights (HBM) and activations (L2) are copied by
+//     different waves, 0-3 and 4-7, each waiting only for its own stage; one barrier per stage publishes both.
+//     Workgroup b starts its walk over K at stage (13 b) mod stages, so that the requests of a moment spread over
+//     the memory channels.
+constexpr int kW8LdsStagger = 13;
+
+template <typename T, int G, int NTP, int BK, int WST, int XST>
+__global__ __launch_bounds__(512) void w8LinearLdsKernel(W8Args a) {
+  using Frag = typename W8Mfma<T>::Frag;
+  constexpr int BN = 32 * NTP;
+  constexpr int LW = BK / 16, LX = BK * (int)sizeof(T) / 16;   // 16-byte pieces (= lanes of a copy instruction) per weight / activation row
+  constexpr int RW = 64 / LW, RX = 64 / LX;                    // rows one copy instruction covers
+  constexpr int WIPW = BN / RW / 4, XIPW = G * 16 / RX / 4;    // copy instructions (1 KiB) per wave and stage: weights, activations
+  constexpr int WBUF = BN * BK, XBUF = G * 16 * BK * (int)sizeof(T);  // bytes per stage buffer
+  constexpr int UNROLL = WST % XST == 0 ? WST : (XST % WST == 0 ? XST : WST * XST);
+  constexpr int IPW = WIPW > XIPW ? WIPW : XIPW;
+  constexpr int PPW = BK / 64 / 4;   // 64-column pieces of a stage per wave
+  static_assert(PPW >= 1 && LX <= 64, "a stage is 256 or 512 columns");
+  extern __shared__ __attribute__((aligned(16))) char w8smem[];
+  char* sw = w8smem;                 // WST weight buffers: BN rows x BK bytes
+  char* sx = sw + WST * WBUF;        // XST activation buffers: 16 G rows x 2 BK bytes
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r16 = lane & 15, kgrp = lane >> 4;
+  const int ci = wave & 3, kq = wave & 3, nb = wave >> 2;
+  const int n0 = blockIdx.x * a.colsPerWg, nCols = min(a.colsPerWg, a.N - n0);
+  const int m0 = blockIdx.y * 16 * G, rows = min(16 * G, a.M - m0);
+  const int nStages = a.K / BK;  // the host sends only K that are multiples of BK here
+  const int kStart = (int)((blockIdx.x * (unsigned)kW8LdsStagger) % (unsigned)nStages);
+  auto descriptor = [](const void* base, int64_t bytes) {
+    const uint64_t p = reinterpret_cast<uint64_t>(base);
+    u32x4 d = {(uint32_t)p, (uint32_t)(p >> 32) & 0xffffu, (uint32_t)bytes, 0x00020000u};
+    return d;
+  };
+  const bool copiesW = wave < 4;
+  const u32x4 rs = copiesW ? descriptor(a.w, (int64_t)(a.N - 1) * a.ldw + a.K)
+                           : descriptor(reinterpret_cast<const T*>(a.x) + (int64_t)m0 * a.ldx, ((int64_t)(rows - 1) * a.ldx + a.K) * sizeof(T));
+  const int ipw = copiesW ? WIPW : XIPW;
+  const unsigned ldsBase = (unsigned)(size_t)(__attribute__((address_space(3))) char*)(copiesW ? sw : sx);
+  const unsigned bufBytes = copiesW ? WBUF : XBUF;
+  // copy instruction q = ci + 4 i fills 1 KiB of a buffer: RW weight rows (LW pieces each) or RX activation rows (LX
+  // pieces each); a lane owns one physical piece and fetches the logical piece the swizzle puts there.
+  // Weight rows past this workgroup's channels and activation rows past M get an offset past the end of the descriptor,
+  // which reads zeros without traffic.
+  unsigned voff[IPW];
+#pragma unroll
+  for (int i = 0; i < IPW; ++i) {
+    const int q = ci + 4 * i;
+    if (copiesW) {
+      const int row = RW * q + lane / LW, piece = (lane % LW) ^ (row & 15);
+      voff[i] = row < nCols ? (unsigned)((int64_t)(n0 + row) * a.ldw + piece * 16) : 0x80000000u;
+    } else {
+      const int row = RX * q + lane / LX, piece = (lane % LX) ^ (row & 15);
+      voff[i] = row < rows ? (unsigned)(((int64_t)row * a.ldx) * sizeof(T) + piece * 16) : 0x80000000u;
+    }
+  }
+  auto copyStage = [&](int c, int buf) {  // a stage past the end copies the last one again, into a buffer nobody reads any more
+    int cc = min(c, nStages - 1) + kStart;
+    if (cc >= nStages) cc -= nStages;
+    const int from = __builtin_amdgcn_readfirstlane(cc * BK * (copiesW ? 1 : (int)sizeof(T)));
+#pragma unroll
+    for (int i = 0; i < IPW; ++i)
+      if (i < ipw) {
+        const unsigned to = ldsBase + (unsigned)buf * bufBytes + (unsigned)(ci + 4 * i) * 1024u;
+        if (copiesW) loadToLds16Stream(rs, (int)voff[i], from, to);
+        else loadToLds16(rs, (int)voff[i], from, to);
+      }
+  };
+  // scale and bias of the channels this wave finishes: requested now, used at the end
+  float sc[NTP], bv[NTP];
+#pragma unroll
+  for (int j = 0; j < NTP; ++j) {
+    const int lc = (nb * NTP + j) * 16 + r16;
+    sc[j] = bv[j] = 0.f;
+    if (lc < nCols) {
+      sc[j] = loadAs<float>(a.scale, n0 + lc, a.scaleDtype);
+      if (a.bias) bv[j] = loadAs<float>(a.bias, n0 + lc, a.biasDtype);
+    }
+  }
+  f32x4 acc[G][NTP];
+#pragma unroll
+  for (int gi = 0; gi < G; ++gi)
+#pragma unroll
+    for (int j = 0; j < NTP; ++j) acc[gi][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // this wave's fragments of 64-column piece p = kq + 4 pp: weights 16-byte piece 4 p + kgrp of row r16 (+ 16 (NTP nb + j)
+  // rows): 16 int8, the K slots of two MFMAs; activations pieces 8 p + 2 kgrp + t of row r16 (+ 16 gi rows): the 8
+  // elements that meet the t-th half of those int8
+  const char* wlane[PPW];
+  const char* xlane[PPW][2];
+#pragma unroll
+  for (int pp = 0; pp < PPW; ++pp) {
+    const int p = kq + 4 * pp;
+    wlane[pp] = sw + (nb * NTP * 16 + r16) * BK + (((4 * p + kgrp) ^ r16) << 4);
+#pragma unroll
+    for (int t = 0; t < 2; ++t) xlane[pp][t] = sx + r16 * BK * (int)sizeof(T) + (((8 * p + 2 * kgrp + t) ^ r16) << 4);
+  }
+
+  if (copiesW) {
+#pragma unroll
+    for (int c = 0; c < WST - 1; ++c) copyStage(c, c);
+  } else {
+#pragma unroll
+    for (int c = 0; c < XST - 1; ++c) copyStage(c, c);
+  }
+  for (int c0 = 0; c0 < nStages; c0 += UNROLL) {
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u;
+      if (c < nStages) {  // workgroup-uniform
+        // this wave's copies of stage c have landed (loads return in order; only the stages requested after it are in
+        // flight); past the barrier both operands of the stage are in LDS and every wave has left the buffers of stage c - 1
+        if (copiesW) {
+          constexpr int n = (WST - 2) * WIPW;
+          __builtin_amdgcn_s_waitcnt(0x0f70 | (n & 15) | ((n >> 4) << 14));
+        } else {
+          constexpr int n = (XST - 2) * XIPW;
+          __builtin_amdgcn_s_waitcnt(0x0f70 | (n & 15) | ((n >> 4) << 14));
+        }
+        __builtin_amdgcn_s_barrier();
+        if (copiesW) copyStage(c + WST - 1, (u + WST - 1) % WST);
+        else copyStage(c + XST - 1, (u + XST - 1) % XST);
+#pragma unroll
+        for (int pp = 0; pp < PPW; ++pp) {
+          Frag x0[G], x1[G];
+#pragma unroll
+          for (int gi = 0; gi < G; ++gi) {
+            x0[gi] = *reinterpret_cast<const Frag*>(xlane[pp][0] + (u % XST) * XBUF + gi * 16 * BK * (int)sizeof(T));
+            x1[gi] = *reinterpret_cast<const Frag*>(xlane[pp][1] + (u % XST) * XBUF + gi * 16 * BK * (int)sizeof(T));
+          }
+#pragma unroll
+          for (int j = 0; j < NTP; ++j) {
+            const u32x4 w = *reinterpret_cast<const u32x4*>(wlane[pp] + (u % WST) * WBUF + j * 16 * BK);
+            const Frag f0 = cvt8<T>(w[0], w[1]), f1 = cvt8<T>(w[2], w[3]);
+#pragma unroll
+            for (int gi = 0; gi < G; ++gi) {
+              acc[gi][j] = W8Mfma<T>::run(x0[gi], f0, acc[gi][j]);
+              acc[gi][j] = W8Mfma<T>::run(x1[gi], f1, acc[gi][j]);
+            }
+          }
+        }
+      }
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0x0070);  // the repeated copies of the last stage: nothing may land after the workgroup has gone
+  __syncthreads();
+  // the four shares of a channel tile meet where the stages were; wave (nb, kq) then finishes row group kq
+  float* red = reinterpret_cast<float*>(w8smem);  // [8 waves][G][NTP][4][64]
+#pragma unroll
+  for (int gi = 0; gi < G; ++gi)
+#pragma unroll
+    for (int j = 0; j < NTP; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[(((wave * G + gi) * NTP + j) * 4 + r) * 64 + lane] = acc[gi][j][r];
+  __syncthreads();
+  const int gi = kq;
+  if (gi < G) {
+    T* out = reinterpret_cast<T*>(a.out);
+#pragma unroll
+    for (int j = 0; j < NTP; ++j) {
+      const int lc = (nb * NTP + j) * 16 + r16;
+      if (lc >= nCols) continue;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = gi * 16 + kgrp * 4 + r;
+        if (row < rows) {
+          float v = 0.f;
+#pragma unroll
+          for (int k2 = 0; k2 < 4; ++k2) v += red[((((nb * 4 + k2) * G + gi) * NTP + j) * 4 + r) * 64 + lane];
+          out[(int64_t)(m0 + row) * a.ldo + n0 + lc] = static_cast<T>(v * sc[j] + bv[j]);
+        }
+      }
+    }
+  }
+}
+
+template <typename T, int G, int NTP, int BK, int WST, int XST>
+static diopiError_t launchW8Lds(hipStream_t stream, const W8Args& a) {
+  constexpr int BN = 32 * NTP;
+  AMD_CHECK(a.colsPerWg >= 1 && a.colsPerWg <= BN, "int8 linear: %d channels per workgroup do not fit %d", a.colsPerWg, BN);
+  const int lds = std::max((WST * BN + XST * G * 16 * (int)sizeof(T)) * BK, 8 * G * NTP * 4 * 64 * (int)sizeof(float));
+  AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&w8LinearLdsKernel<T, G, NTP, BK, WST, XST>), lds));
+  dim3 grid((unsigned)((a.N + a.colsPerWg - 1) / a.colsPerWg), (unsigned)((a.M + 16 * G - 1) / (16 * G)));
+  hipLaunchKernelGGL((w8LinearLdsKernel<T, G, NTP, BK, WST, XST>), grid, dim3(512), lds, stream, a);
+  AMD_LAUNCH_CHECK();
+  return diopiSuccess;
+}
+
 template <typename T, int NTW, int G>
 static diopiError_t launchW8(hipStream_t stream, const W8Args& a) {
   constexpr int CHUNK = kW8RowsK / (16 * G);
@@ -210,7 +410,24 @@ static diopiError_t launchW8ForTiles(hipStream_t stream, const W8Args& a) {
 }
 
 template <typename T>
-static diopiError_t launchW8ForShape(hipStream_t stream, const W8Args& a) {
+static diopiError_t launchW8ForShape(hipStream_t stream, const W8Args& a0) {
+  W8Args a = a0;
+  // Wide weights go through w8LinearLdsKernel, the channels dealt evenly over the CUs. Measured cold against the form
+  // below at K = 4096 (us, 1 / 16 / 32 / 64 rows): N = 11008 11.0 -> 10.8, 12.9 -> 11.7, 17.0 -> 14.2, 23.1 -> 21.1;
+  // N = 22016 22.0 -> 19.2, 26.8 -> 20.2. Both forms have about 10 us of floor at these sizes, so narrower weights
+  // gain only with more than 16 rows (N = 6144: 14.7 -> 13.1 at 32 rows, 9.0 -> 10.4 at one).
+  if ((a.N >= 10240 || (a.N >= 6144 && a.M > 16)) && a.K % 256 == 0 && (int64_t)(a.N - 1) * a.ldw + a.K < ((int64_t)1 << 31)) {
+    const int cus = computeUnits(), rounds = (a.N + 128 * cus - 1) / (128 * cus);
+    a.colsPerWg = (a.N + cus * rounds - 1) / (cus * rounds);
+    if (a.colsPerWg > 64) {
+      if (a.M <= 16) return launchW8Lds<T, 1, 4, 256, 3, 3>(stream, a);
+      if (a.M <= 32) return launchW8Lds<T, 2, 4, 256, 3, 3>(stream, a);
+      return launchW8Lds<T, 4, 4, 256, 2, 2>(stream, a);
+    }
+    if (a.M <= 16) return launchW8Lds<T, 1, 2, 256, 4, 4>(stream, a);
+    if (a.M <= 32) return launchW8Lds<T, 2, 2, 256, 4, 3>(stream, a);
+    return launchW8Lds<T, 4, 2, 256, 4, 2>(stream, a);
+  }
   if (a.M <= 16) return launchW8ForTiles<T, 1>(stream, a);
   if (a.M <= 32) return launchW8ForTiles<T, 2>(stream, a);
   return launchW8ForTiles<T, 4>(stream, a);

@@ -397,10 +397,15 @@ def test_weight_only_int8_full_shape_exact_cases(ops, dev, pkg):
     assert_half(got, oracle.weight_only_int8_linear(w["x"], w["w"], w["scale"]))
 
 @pytest.mark.parametrize("m,k,n", [(1, 11008, 4096), (5, 8192 + 128, 100), (37, 4096, 16 * 7 + 3), (16, 4096, 22016),
-                                   (64, 4096, 4096), (100, 1024 + 256, 520), (29, 2048 + 128, 11008)])
+                                   (64, 4096, 4096), (100, 1024 + 256, 520), (29, 2048 + 128, 11008),
+                                   (40, 2048, 11008), (20, 1024, 6200), (100, 512, 12288), (33, 768, 22016 + 8),
+                                   (24, 256, 30000), (3, 256, 10240)])
 def test_weight_only_int8_linear_chunked_k_row_groups_and_tile_counts(ops, dev, pkg, m, k, n):
     """K beyond one staged activation chunk (4096 columns), more than 16 rows (row groups), channel counts that leave
-    partly filled workgroups, and an N large enough to use the widest workgroup."""
+    partly filled workgroups, and an N large enough to use the widest workgroup. Wide weights with K a multiple of
+    256 take the form that stages both operands through LDS (the last six cases, and N = 22016 above): one, two and four
+    row groups, channel shares of up to 64 and up to 128 per workgroup that are no multiple of 16, more than 64 rows
+    (a second workgroup row), K of one to eight stages."""
     w = pkg.workloads.int8_linear(seed=5, m=m, k=k, n=n)
     got = ops.weight_only_int8_linear(w["x"].to(dev), w["w"].to(dev), w["scale"].to(dev))
     assert_half(got, oracle.weight_only_int8_linear(w["x"], w["w"], w["scale"]))
