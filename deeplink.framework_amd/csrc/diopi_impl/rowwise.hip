@@ -66,10 +66,12 @@ __global__ __launch_bounds__(256) void rowWaveKernel(T* __restrict__ out, const 
 #pragma unroll
     for (int i = 0; i < NV; ++i) cur[i] = pre[i];
     if (row + nWaves < rows) {  // next row in flight while this one is reduced
+      // (ordinary loads here, non-temporal ones for a wave's first row: measured on [8192, 4096] bf16, cold, 22.4 us
+      // against 24.0 with both non-temporal and 24.2 with both ordinary)
       const V* src = reinterpret_cast<const V*>(in + (row + nWaves) * inRowStride);
 #pragma unroll
       for (int i = 0; i < NV; ++i)
-        if (lane + 64 * i < nvec) pre[i] = __builtin_nontemporal_load(src + lane + 64 * i);
+        if (lane + 64 * i < nvec) pre[i] = src[lane + 64 * i];
     }
   }
 
