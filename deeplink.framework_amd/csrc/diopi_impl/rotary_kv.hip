@@ -48,8 +48,8 @@ __global__ __launch_bounds__(256) void rotaryVecKernel(T* __restrict__ out, cons
         oa[e] = static_cast<T>(x0 * c - x1 * s);
         ob[e] = static_cast<T>(x0 * s + x1 * c);
       }
-      *reinterpret_cast<V*>(outr + j * N) = oa;
-      *reinterpret_cast<V*>(outr + half + j * N) = ob;
+      __builtin_nontemporal_store(oa, reinterpret_cast<V*>(outr + j * N));
+      __builtin_nontemporal_store(ob, reinterpret_cast<V*>(outr + half + j * N));
     } else {
       V a = *reinterpret_cast<const V*>(xr + j * N);
       V o;
@@ -64,7 +64,7 @@ __global__ __launch_bounds__(256) void rotaryVecKernel(T* __restrict__ out, cons
         o[2 * e] = static_cast<T>(x0 * c - x1 * s);
         o[2 * e + 1] = static_cast<T>(x0 * s + x1 * c);
       }
-      *reinterpret_cast<V*>(outr + j * N) = o;
+      __builtin_nontemporal_store(o, reinterpret_cast<V*>(outr + j * N));
     }
   }
 }

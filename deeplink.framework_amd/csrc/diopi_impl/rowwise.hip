@@ -87,11 +87,11 @@ __global__ __launch_bounds__(256) void rowWaveKernel(T* __restrict__ out, const 
           m = fmaxf(m, f[i][j]);
         }
       }
-    if (row + nWaves < rows) {  // next row in flight while this one is reduced
+    if (row + nWaves < rows) {  // next row in flight while this one is reduced (ordinary loads, as for RMSNorm: 22.7 -> 21.1 us cold)
       const V* src = reinterpret_cast<const V*>(in + (row + nWaves) * inRowStride);
 #pragma unroll
       for (int i = 0; i < NV; ++i)
-        if (lane + 64 * i < nvec) pre[i] = __builtin_nontemporal_load(src + lane + 64 * i);
+        if (lane + 64 * i < nvec) pre[i] = src[lane + 64 * i];
     }
     m = waveMax(m);
     const float mScaled = (m == -INFINITY) ? 0.f : m * kLog2e;  // all -inf row -> nan like the CPU kernel
