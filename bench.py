@@ -40,8 +40,8 @@ GEMM_TRAFFIC_MEASURED_AT = "a111839"
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=40)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-ops", action="store_true", help="skip the per-op HBM microbenchmarks")
     ap.add_argument("--only-layer", action="store_true", help="alias for --no-cpu --no-ops")
