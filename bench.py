@@ -54,6 +54,48 @@ def parse():
     return ap.parse_args()
 
 
+def layer_graph_replay(pkg, torch, dev, x, p, cfg, want, steps):
+    """The same step recorded once into a HIP graph and replayed `steps` times between two synchronizations: what a
+    serving loop that replays a captured step would see. Reported beside `value`, which stays the figure of op-by-op
+    launches through the C ABI. `want` is the op-by-op output; every checked replay must equal it bit for bit (the
+    kernels of this step are deterministic and take no workspace, so recording allocates nothing)."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        plan, keep, _, out = layer_plan(pkg, torch, dev, x, p, cfg)   # contexts bound to the recording stream
+        for _, call in plan:
+            call()
+        side.synchronize()
+        before = pkg.runtime.cachingStats()["num_device_malloc"]
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for _, call in plan:
+                call()
+    torch.cuda.synchronize()
+    allocated = pkg.runtime.cachingStats()["num_device_malloc"] - before
+    same = True
+    for _ in range(3):   # replays with eager work and synchronizations between them, each checked
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        same = same and bool(torch.equal(out, want))
+    for _ in range(10):
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    same = same and bool(torch.equal(out, want))
+    del graph
+    for _, call in plan:
+        call.close()
+    tokens = x.shape[0] * x.shape[1]
+    return {"ms_per_step": round(ms, 4), "tokens_per_s": round(tokens / (ms * 1e-3), 1), "steps": steps,
+            "replay_equals_op_by_op": same, "device_mallocs_while_recording": allocated}
+
+
 class Prepared:
     """A DIOPI call with its arguments marshalled once: per launch it costs two C calls
     (the op and the release of the context's workspace), so short kernels are not host-bound."""
@@ -603,6 +645,7 @@ def main():
         "layer_breakdown_us": breakdown,
         "ms_per_step_with_events": round(elapsed_events / args.steps * 1e3, 4),
     }
+    result["graph_replay"] = layer_graph_replay(pkg, torch, dev, x, p, cfg, out.clone(), args.steps)
     if not args.no_ops:
         host_threads(torch)
         result["ops"] = op_microbench(pkg, torch, dev, rt, stream, with_cpu=not args.no_cpu)
