@@ -12,7 +12,9 @@
 // The fused kernel is HBM-bound: every K and V row of the sequence is read exactly once
 // (d * itemsize bytes each), nothing else of size is touched. Mapping:
 //   * a head row of d elements is covered by LPT = d*itemsize/16 lanes with one 16-byte
-//     load each, so one wave-wide load fetches 64/LPT tokens;
+//     load each, so one wave-wide load fetches 64/LPT head rows: consecutive heads of one token
+//     (one contiguous piece of the slot; the workgroup then owns 64/LPT heads) when the head count
+//     is a multiple of that, otherwise 64/LPT tokens of one head;
 //   * every lane group keeps its OWN running (max, sum, acc[8]) online-softmax state, so the
 //     inner loop needs no cross-group traffic: per token only the log2(LPT) butterfly steps
 //     of the dot product;
@@ -70,15 +72,17 @@ __device__ __forceinline__ void mergeState(float& m, float& l, float (&acc)[E], 
 }
 
 // T: bf16_t / half_t (8 per 16 B) or float (4 per 16 B). LPT lanes cover one head row.
-template <typename T, int LPT>
+template <typename T, int LPT, bool HIW>
 __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* __restrict__ out,
                                                                      float* __restrict__ partial) {
   using V = typename Vec16<T>::type;
   constexpr int N = Vec16<T>::N;
   constexpr int TPW = 64 / LPT;  // tokens per wave-wide load
-  const int h = blockIdx.x, split = blockIdx.y, b = blockIdx.z;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int sub = lane % LPT, grp = lane / LPT;
+  // HIW: the lane groups of a wave take TPW consecutive heads of the same token (a wave load is TPW head rows, contiguous
+  // in a slot) instead of TPW tokens of one head
+  const int h = HIW ? blockIdx.x * TPW + grp : blockIdx.x, split = blockIdx.y, b = blockIdx.z;
   const int len = min(max((int)ldIndex(a.bLen, b, a.len64), 0), a.maxLen);  // a length beyond the table's width is cut to it
   const int begin = split * a.chunk;
   if (begin >= len && !(split == 0)) return;  // nothing to do; split 0 still writes zeros for len == 0
@@ -99,17 +103,18 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
 #pragma unroll
   for (int e = 0; e < N; ++e) acc[e] = 0.f;
 
-  constexpr int STEP = kTaWaves * kTaUnroll * TPW;  // tokens per workgroup iteration
+  constexpr int TPI = HIW ? 1 : TPW;  // tokens per wave-wide load
+  constexpr int STEP = kTaWaves * kTaUnroll * TPI;  // tokens per workgroup iteration
   // Two-deep software pipeline: while the rows of iteration i are being reduced, the K/V rows
   // of iteration i+1 and the slot indices of iteration i+2 are already in flight.
   int64_t slot[kTaUnroll];
   V kr[kTaUnroll], vr[kTaUnroll], kn[kTaUnroll], vn[kTaUnroll];
   bool ok[kTaUnroll], okn[kTaUnroll];
   auto loadSlots = [&](int it) {
-    int t0 = it + wave * kTaUnroll * TPW + grp;
+    int t0 = it + wave * kTaUnroll * TPI + (HIW ? 0 : grp);
 #pragma unroll
     for (int u = 0; u < kTaUnroll; ++u) {
-      int t = t0 + u * TPW;
+      int t = t0 + u * TPI;
       slot[u] = t < end ? ldIndex(a.bLoc, locBase + t, a.loc64) : -1;
     }
   };
@@ -162,7 +167,8 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
     for (int u = 0; u < kTaUnroll; ++u) kr[u] = kn[u], vr[u] = vn[u], ok[u] = okn[u];
   }
 
-  // merge the TPW lane groups of the wave
+  // merge the TPW lane groups of the wave (each holds other tokens of the same head)
+  if (!HIW)
 #pragma unroll
   for (int off = LPT; off < 64; off <<= 1) {
     float m2 = __shfl_xor(m, off, 64), l2 = __shfl_xor(l, off, 64), acc2[N];
@@ -171,20 +177,22 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
     mergeState<N>(m, l, acc, m2, l2, acc2);
   }
   // merge the waves through LDS: [wave][2 + LPT*N]
-  __shared__ float red[kTaWaves][2 + LPT * N];
-  if (grp == 0) {
-    if (sub == 0) red[wave][0] = m, red[wave][1] = l;
+  constexpr int RG = HIW ? TPW : 1;  // lane groups with a state of their own
+  const int rg = HIW ? grp : 0;
+  __shared__ float red[kTaWaves][RG][2 + LPT * N];
+  if (HIW || grp == 0) {
+    if (sub == 0) red[wave][rg][0] = m, red[wave][rg][1] = l;
 #pragma unroll
-    for (int e = 0; e < N; ++e) red[wave][2 + sub * N + e] = acc[e];
+    for (int e = 0; e < N; ++e) red[wave][rg][2 + sub * N + e] = acc[e];
   }
   __syncthreads();
-  if (wave == 0 && grp == 0) {
+  if (wave == 0 && (HIW || grp == 0)) {
 #pragma unroll
     for (int w = 1; w < kTaWaves; ++w) {
       float acc2[N];
 #pragma unroll
-      for (int e = 0; e < N; ++e) acc2[e] = red[w][2 + sub * N + e];
-      mergeState<N>(m, l, acc, red[w][0], red[w][1], acc2);
+      for (int e = 0; e < N; ++e) acc2[e] = red[w][rg][2 + sub * N + e];
+      mergeState<N>(m, l, acc, red[w][rg][0], red[w][rg][1], acc2);
     }
     if (a.nsplit == 1) {
       float inv = l > 0.f ? 1.f / l : 0.f;
@@ -556,10 +564,16 @@ static diopiError_t decodeAttention(diopiContextHandle_t ctx, diopiTensorHandle_
       partial = static_cast<float*>(ws);
     }
   }
-  dim3 grid(a.heads, a.nsplit, (unsigned)batch), block(kTaWaves * 64);
   const int64_t bytes = t.q.shape[2] * t.q.itemsize;
-#define DECODE_CALL(T, LPT) \
-  hipLaunchKernelGGL((decodeSplitKernel<T, LPT>), grid, block, 0, stream, a, out.ptr<T>(), partial)
+  // The lane groups of a wave take consecutive heads of one token when the head count allows it: a wave load is then
+  // one contiguous piece of a slot (1 KiB) instead of head rows of four different slots (431 -> 421 us at batch 64,
+  // 32 heads x 128, 156 043 cached tokens).
+  const int tpw = (int)(64 / std::max<int64_t>(1, bytes / 16));
+  const bool hiw = (bytes == 128 || bytes == 256 || bytes == 512) && a.heads % tpw == 0;
+  dim3 grid(hiw ? a.heads / tpw : a.heads, a.nsplit, (unsigned)batch), block(kTaWaves * 64);
+#define DECODE_CALL(T, LPT)                                                                                               \
+  if (hiw) hipLaunchKernelGGL((decodeSplitKernel<T, LPT, true>), grid, block, 0, stream, a, out.ptr<T>(), partial);       \
+  else hipLaunchKernelGGL((decodeSplitKernel<T, LPT, false>), grid, block, 0, stream, a, out.ptr<T>(), partial)
   TA_DISPATCH(t.q.dtype, bytes, DECODE_CALL);
 #undef DECODE_CALL
   AMD_LAUNCH_CHECK();

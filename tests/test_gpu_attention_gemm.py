@@ -348,8 +348,11 @@ def test_token_attention_fused_and_two_call(ops, dev, pkg, dtype, d, idt):
     chk(out2, want)
 
 
-def test_token_attention_len_one_and_gqa(ops, dev):
-    slots, heads, kvh, d = 64, 8, 2, 128
+@pytest.mark.parametrize("heads,kvh", [(8, 2), (6, 3)])
+def test_token_attention_len_one_and_gqa(ops, dev, heads, kvh):
+    """Grouped-query decode: 8 heads (a wave's lane groups take four consecutive heads of one token) and 6 heads (not a
+    multiple of four: the lane groups take four tokens of one head)."""
+    slots, d = 64, 128
     kp = torch.randn(slots, kvh, d, generator=g(30)).bfloat16()
     vp = torch.randn(slots, kvh, d, generator=g(31)).bfloat16()
     q = torch.randn(3, heads, d, generator=g(32)).bfloat16()
@@ -363,8 +366,8 @@ def test_token_attention_len_one_and_gqa(ops, dev):
     want = oracle.token_attention(q.float(), kp.float(), vp.float(), b_loc, lens, 5)
     assert_half(got, want)
     # a single cached token: the output is that token's V row for the mapped kv head
-    assert_exact(got[0].cpu(), vp[17].repeat_interleave(4, dim=0))
-    assert_exact(got[2].cpu(), vp[63].repeat_interleave(4, dim=0))
+    assert_exact(got[0].cpu(), vp[17].repeat_interleave(heads // kvh, dim=0))
+    assert_exact(got[2].cpu(), vp[63].repeat_interleave(heads // kvh, dim=0))
 
 
 # ------------------------------------------------------------------ int8 weight-only linear
