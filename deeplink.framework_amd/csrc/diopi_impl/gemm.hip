@@ -926,6 +926,7 @@ struct SkinnyArgs {
   float* partial;  // K split over grid.y: fp32 partial products [gridDim.y][M][N] for splitKReduceKernel, else null
   int kPerWg;      // K columns per grid.y slice (K when not split)
   int colsPerWg;   // gemmSkinnyLdsKernel: output columns per workgroup
+  bool siluMul;    // gemmSkinnyLdsKernel: every 64 columns are 32 gate and 32 up columns; out (N / 2 wide) = silu(gate) * up
 };
 
 constexpr int kSkinnyStep = 128;    // K elements one wave consumes per step (4 kgrps x 32)
@@ -1306,6 +1307,35 @@ __global__ __launch_bounds__(512) void gemmSkinnyLdsKernel(SkinnyArgs a) {
       for (int r = 0; r < 4; ++r) red[(((wave * G + gi) * NTP + j) * 4 + r) * 64 + lane] = acc[gi][j][r];
   __syncthreads();
   const int gi = kq;
+  if (a.siluMul) {
+    // A workgroup's columns are whole blocks of 64: 32 gate columns, then the up columns of the same 32 channels.
+    // Output tile t of 16 channels takes its gate values from column tile 4 (t / 2) + t % 2 and its up values from the
+    // tile two further on; both sit at this lane's place in the partial sums, whichever waves produced them.
+    constexpr int OTW = BN / 64;  // output tiles per wave half
+    if (gi < G) {
+      T* out = reinterpret_cast<T*>(a.out);
+#pragma unroll
+      for (int tt = 0; tt < OTW; ++tt) {
+        const int t = nb * OTW + tt, tg = 4 * (t >> 1) + (t & 1), tu = tg + 2;
+        if (tg * 16 >= nCols) continue;
+        const int oc = n0 / 2 + (t >> 1) * 32 + (t & 1) * 16 + r16;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int row = gi * 16 + kgrp * 4 + r;
+          if (row < a.M) {
+            float gsum = 0.f, usum = 0.f;
+#pragma unroll
+            for (int k2 = 0; k2 < 4; ++k2) {
+              gsum += red[(((((tg / NTP) * 4 + k2) * G + gi) * NTP + tg % NTP) * 4 + r) * 64 + lane];
+              usum += red[(((((tu / NTP) * 4 + k2) * G + gi) * NTP + tu % NTP) * 4 + r) * 64 + lane];
+            }
+            out[(int64_t)row * a.ldo + oc] = static_cast<T>(gsum / (1.f + __expf(-gsum)) * usum);
+          }
+        }
+      }
+    }
+    return;
+  }
   if (gi < G) {
     T* out = reinterpret_cast<T*>(a.out);
     const T* cin = reinterpret_cast<const T*>(a.Cin);
@@ -1624,6 +1654,7 @@ static diopiError_t launchSkinnyForShape(diopiContextHandle_t ctx, hipStream_t s
   a.M = (int)p.M, a.N = (int)p.N, a.K = (int)p.K;
   a.alpha = p.alpha, a.beta = p.beta;
   a.partial = nullptr, a.kPerWg = a.K;
+  a.siluMul = false;
   const int tiles = (a.N + 15) / 16, cus = computeUnits(), perCu = (tiles + cus - 1) / cus;
   // Both operands through LDS, see gemmSkinnyLdsKernel. The columns are dealt evenly over as many workgroups as there
   // are CUs (43 each at N = 11008, where 64-column blocks would leave a third of the CUs idle): a CU takes in about
@@ -1823,6 +1854,32 @@ static diopiError_t runGatedSiluGemm(diopiContextHandle_t ctx, hipStream_t strea
   if (direct) {
     return p.dtype == diopi_dtype_bfloat16 ? launchMfmaPipelined<bf16_t, kEpiSiluMul>(stream, p)
                                            : launchMfmaPipelined<half_t, kEpiSiluMul>(stream, p);
+  }
+  // decode-sized: the weight-streaming kernel that stages both operands through LDS applies the gate to its sums
+  if (half && p.batch == 1 && p.M <= kSkinnyMaxM && p.K % kSkinnyLdsBK == 0 && p.N % 64 == 0 && p.N >= 4096 && p.sAk == 1 &&
+      mult8(p.sAm) && ptr16(p.A) && p.sBk == 1 && mult8(p.sBn) && ptr16(p.B) && p.Cin == nullptr && p.bias == nullptr &&
+      p.alpha == 1.f && ((p.M - 1) * p.sAm + p.K) * 2 < (int64_t(1) << 31) && ((p.N - 1) * p.sBn + p.K) * 2 < (int64_t(1) << 31)) {
+    SkinnyArgs a;
+    a.A = p.A, a.B = p.B, a.Cin = nullptr, a.bias = nullptr, a.out = p.out;
+    a.lda = p.sAm, a.ldb = p.sBn, a.ldo = p.sOm, a.sCm = 0, a.sCn = 0;
+    a.M = (int)p.M, a.N = (int)p.N, a.K = (int)p.K;
+    a.alpha = 1.f, a.beta = 0.f, a.partial = nullptr, a.kPerWg = a.K, a.siluMul = true;
+    // whole blocks of 64 columns per workgroup: 128 while that still gives half the CUs a workgroup
+    a.colsPerWg = p.N / 128 >= computeUnits() / 2 ? 128 : 64;
+    const bool bf = p.dtype == diopi_dtype_bfloat16;
+#define SKINNY_SILU(G, NTP, WST, XST) \
+  return bf ? launchSkinnyLds<bf16_t, G, NTP, WST, XST>(stream, a) : launchSkinnyLds<half_t, G, NTP, WST, XST>(stream, a)
+    if (a.colsPerWg == 128) {
+      if (a.M <= 16) SKINNY_SILU(1, 4, 3, 3);
+      if (a.M <= 32) SKINNY_SILU(2, 4, 3, 3);
+      if (a.M <= 48) SKINNY_SILU(3, 4, 3, 3);
+      SKINNY_SILU(4, 4, 3, 3);
+    }
+    if (a.M <= 16) SKINNY_SILU(1, 2, 4, 4);
+    if (a.M <= 32) SKINNY_SILU(2, 2, 4, 4);
+    if (a.M <= 48) SKINNY_SILU(3, 2, 4, 4);
+    SKINNY_SILU(4, 2, 4, 4);
+#undef SKINNY_SILU
   }
   // two passes: the full-width projection into workspace, then the gate
   void* ws = nullptr;

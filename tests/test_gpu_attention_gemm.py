@@ -180,10 +180,14 @@ def test_skinny_m_linear_and_addmm(ops, dev, dtype, m, n, k):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
-@pytest.mark.parametrize("m,f,k", [(4096, 3584, 256), (3700, 4000 - 32, 192), (96, 64, 80), (1, 32, 8)])
+@pytest.mark.parametrize("m,f,k", [(4096, 3584, 256), (3700, 4000 - 32, 192), (96, 64, 80), (1, 32, 8),
+                                   (5, 2048, 256), (33, 5536, 384), (48, 16384, 128), (64, 11008, 640), (20, 8224, 256)])
 def test_linear_silu_mul(ops, dev, dtype, m, f, k):
     """silu(x Wg^T) * (x Wu^T) from the interleaved weight: the single-launch path (at least 144 tiles, K a
-    multiple of 64, 16-bit dtypes) and the two-pass path, against the reference's four-op form in fp32."""
+    multiple of 64, 16-bit dtypes) and the two-pass path, against the reference's four-op form in fp32. The last five
+    cases (at most 64 rows, K a multiple of 128, at least 4096 stacked columns, 16-bit dtypes) take the decode-sized
+    kernel with the gate applied to its sums: one to four row groups, workgroups of 64 and of 128 columns, a last
+    workgroup with a single block of 64, K of one to five stages."""
     x = torch.randn(m, k, generator=g(60)).to(dtype)
     wg = (torch.randn(f, k, generator=g(61)) * 0.08).to(dtype)
     wu = (torch.randn(f, k, generator=g(62)) * 0.08).to(dtype)
