@@ -927,6 +927,13 @@ struct SkinnyArgs {
   int kPerWg;      // K columns per grid.y slice (K when not split)
   int colsPerWg;   // gemmSkinnyLdsKernel: output columns per workgroup
   bool siluMul;    // gemmSkinnyLdsKernel: every 64 columns are 32 gate and 32 up columns; out (N / 2 wide) = silu(gate) * up
+  // gemmSkinnyLdsKernel: the interleaved rotary embedding on the leading rotCols columns (heads of rotHeadDim), tables
+  // [rotTableRows, rotHeadDim / 2] of T or fp32, row m uses table row m % rotTableRows; rotCols = 0: none
+  const void* rotCos;
+  const void* rotSin;
+  int rotCols, rotHeadDim, rotTableRows;
+  bool rotTableF32;
+  float rotSinSign;
 };
 
 constexpr int kSkinnyStep = 128;    // K elements one wave consumes per step (4 kgrps x 32)
@@ -1357,6 +1364,17 @@ __global__ __launch_bounds__(512) void gemmSkinnyLdsKernel(SkinnyArgs a) {
           }
           v = v * a.alpha + bv;
           if (cin) v += a.beta * static_cast<float>(cin[(int64_t)row * a.sCm + (int64_t)col * a.sCn]);
+          if (a.rotCols > 0) {
+            // adjacent columns are a pair and sit in adjacent lanes (the column shares are even): every lane takes part
+            // in the exchange, columns at or past rotCols keep their value
+            const float other = __shfl_xor(v, 1, 64);
+            if (col < a.rotCols) {
+              const int64_t ti = (int64_t)(row % a.rotTableRows) * (a.rotHeadDim >> 1) + ((col % a.rotHeadDim) >> 1);
+              const float c = a.rotTableF32 ? reinterpret_cast<const float*>(a.rotCos)[ti] : static_cast<float>(reinterpret_cast<const T*>(a.rotCos)[ti]);
+              const float sn = (a.rotTableF32 ? reinterpret_cast<const float*>(a.rotSin)[ti] : static_cast<float>(reinterpret_cast<const T*>(a.rotSin)[ti])) * a.rotSinSign;
+              v = (col & 1) ? other * sn + v * c : v * c - other * sn;
+            }
+          }
           out[(int64_t)row * a.ldo + col] = static_cast<T>(v);
         }
       }
@@ -1647,14 +1665,20 @@ static bool mult8(int64_t v) { return (v & 7) == 0; }
 static bool ptr16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 template <typename T>
-static diopiError_t launchSkinnyForShape(diopiContextHandle_t ctx, hipStream_t stream, const GemmProblem& p) {
+// With `rot` (a rotary epilogue) only the LDS-staged form qualifies: *handled tells the caller whether it ran.
+static diopiError_t launchSkinnyForShape(diopiContextHandle_t ctx, hipStream_t stream, const GemmProblem& p,
+                                         const RotaryEpilogue* rot = nullptr, bool* handled = nullptr) {
   SkinnyArgs a;
   a.A = p.A, a.B = p.B, a.Cin = p.Cin, a.bias = p.bias, a.out = p.out;
   a.lda = p.sAm, a.ldb = p.sBn, a.ldo = p.sOm, a.sCm = p.sCm, a.sCn = p.sCn;
   a.M = (int)p.M, a.N = (int)p.N, a.K = (int)p.K;
   a.alpha = p.alpha, a.beta = p.beta;
   a.partial = nullptr, a.kPerWg = a.K;
-  a.siluMul = false;
+  a.siluMul = false, a.rotCols = 0;
+  if (rot != nullptr) {
+    a.rotCos = rot->cosT, a.rotSin = rot->sinT, a.rotCols = rot->cols, a.rotHeadDim = rot->headDim, a.rotTableRows = rot->tableRows;
+    a.rotTableF32 = rot->tableF32, a.rotSinSign = rot->sinSign;
+  }
   const int tiles = (a.N + 15) / 16, cus = computeUnits(), perCu = (tiles + cus - 1) / cus;
   // Both operands through LDS, see gemmSkinnyLdsKernel. The columns are dealt evenly over as many workgroups as there
   // are CUs (43 each at N = 11008, where 64-column blocks would leave a third of the CUs idle): a CU takes in about
@@ -1670,6 +1694,8 @@ static diopiError_t launchSkinnyForShape(diopiContextHandle_t ctx, hipStream_t s
       ((int64_t)(a.M - 1) * a.lda + a.K) * (int64_t)sizeof(T) < ((int64_t)1 << 31)) {
     const int rounds = (a.N + 128 * cus - 1) / (128 * cus);
     a.colsPerWg = (a.N + cus * rounds - 1) / (cus * rounds);
+    if (rot != nullptr) a.colsPerWg = (a.colsPerWg + 1) & ~1;  // even: the two columns of a rotary pair stay together
+    if (handled) *handled = true;
     if (a.colsPerWg > 64) {
       if (a.M <= 16) return launchSkinnyLds<T, 1, 4, 3, 3>(stream, a);
       if (a.M <= 32) return launchSkinnyLds<T, 2, 4, 3, 3>(stream, a);
@@ -1680,6 +1706,10 @@ static diopiError_t launchSkinnyForShape(diopiContextHandle_t ctx, hipStream_t s
     if (a.M <= 32) return launchSkinnyLds<T, 2, 2, 4, 4>(stream, a);
     if (a.M <= 48) return launchSkinnyLds<T, 3, 2, 4, 4>(stream, a);
     return launchSkinnyLds<T, 4, 2, 4, 4>(stream, a);
+  }
+  if (rot != nullptr) {
+    if (handled) *handled = false;
+    return diopiSuccess;
   }
   if (a.M <= 16) {
     // 16-column tiles per workgroup: about one workgroup per CU, the other waves of the 15 or 16 split K
@@ -1863,7 +1893,7 @@ static diopiError_t runGatedSiluGemm(diopiContextHandle_t ctx, hipStream_t strea
     a.A = p.A, a.B = p.B, a.Cin = nullptr, a.bias = nullptr, a.out = p.out;
     a.lda = p.sAm, a.ldb = p.sBn, a.ldo = p.sOm, a.sCm = 0, a.sCn = 0;
     a.M = (int)p.M, a.N = (int)p.N, a.K = (int)p.K;
-    a.alpha = 1.f, a.beta = 0.f, a.partial = nullptr, a.kPerWg = a.K, a.siluMul = true;
+    a.alpha = 1.f, a.beta = 0.f, a.partial = nullptr, a.kPerWg = a.K, a.siluMul = true, a.rotCols = 0;
     // whole blocks of 64 columns per workgroup: 128 while that still gives half the CUs a workgroup
     a.colsPerWg = p.N / 128 >= computeUnits() / 2 ? 128 : 64;
     const bool bf = p.dtype == diopi_dtype_bfloat16;
@@ -2274,8 +2304,18 @@ GEMM_EXPORT diopiError_t diopiLinearRotary(diopiContextHandle_t ctx, diopiTensor
     AMD_TRY(p.dtype == diopi_dtype_bfloat16 ? (launchMfmaPipelined<bf16_t, kEpiRotary>(stream, p, nullptr, 1, 0, &r))
                                             : (launchMfmaPipelined<half_t, kEpiRotary>(stream, p, nullptr, 1, 0, &r)));
   } else {
-    AMD_TRY(runGemm(ctx, stream, p));
-    if (rotaryCols > 0) {
+    // decode-sized: the weight-streaming kernel that stages both operands through LDS rotates its sums
+    bool fused = false;
+    if (interleaved && rotaryCols > 0 && halfT && tableOk && p.M <= kSkinnyMaxM && k % kSkinnyLdsBK == 0 && ptr16(p.A) && ptr16(p.B) &&
+        (p.M - 1) * k * 2 + k * 2 < (int64_t(1) << 31)) {
+      RotaryEpilogue r;
+      r.cosT = cc.data, r.sinT = cs.data, r.cols = (int)rotaryCols, r.headDim = (int)headDim, r.tableRows = (int)tableRows;
+      r.tableF32 = cc.dtype == diopi_dtype_float32, r.sinSign = conj ? -1.f : 1.f;
+      AMD_TRY(p.dtype == diopi_dtype_bfloat16 ? launchSkinnyForShape<bf16_t>(ctx, stream, p, &r, &fused)
+                                              : launchSkinnyForShape<half_t>(ctx, stream, p, &r, &fused));
+    }
+    if (!fused) AMD_TRY(runGemm(ctx, stream, p));
+    if (!fused && rotaryCols > 0) {
       TensorView v;
       v.data = cout.data, v.ndim = 3, v.dtype = out.dtype, v.itemsize = out.itemsize;
       v.shape[0] = rows, v.shape[1] = rotaryCols / headDim, v.shape[2] = headDim;

@@ -212,6 +212,9 @@ def test_linear_silu_mul(ops, dev, dtype, m, f, k):
     (2400, 57, 64, 0, 192, True, True, True),         # ragged rows and columns, all columns rotated, negative angle, bias
     (2304, 16, 128, 2048, 256, False, False, False),  # half-split pairs: projection + rotary kernel
     (40, 4, 64, 128, 128, True, False, True),         # small: projection + rotary kernel
+    (64, 64, 128, 4096, 256, True, False, False),     # decode-sized, 12288 columns: the LDS-staged kernel rotates its sums (48 columns per workgroup)
+    (7, 45, 128, 640, 384, True, True, True),         # one row group, 25 columns per workgroup made 26, negative angle, bias
+    (33, 96, 64, 22016 - 6144, 128, True, False, True),  # 22016 columns: workgroups of 86 columns, three row groups
 ])
 def test_linear_rotary(ops, dev, dtype, table_dtype, m, heads, hd, vcols, k, interleaved, conj, bias):
     """The stacked projection with the rotary embedding in its epilogue against the oracle's projection followed by
