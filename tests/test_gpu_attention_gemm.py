@@ -203,6 +203,11 @@ def test_linear_silu_mul(ops, dev, dtype, m, f, k):
         ops.linear_silu_mul(x3.to(dev), w, out=dst[..., :f])
         (assert_fp32 if dtype == torch.float32 else assert_half)(dst[..., :f], want[:96].reshape(2, 48, f))
         assert_exact(dst[..., f:], torch.zeros(2, 48, f, dtype=dtype))
+    elif f >= 2048:  # the decode-sized kernel into a strided destination
+        dst = torch.zeros(m, 2 * f, dtype=dtype, device=dev)
+        ops.linear_silu_mul(x.to(dev), w, out=dst[:, :f])
+        assert_exact(dst[:, :f], got.cpu())
+        assert_exact(dst[:, f:], torch.zeros(m, f, dtype=dtype))
 
 
 # ------------------------------------------------------------------ prefill attention
