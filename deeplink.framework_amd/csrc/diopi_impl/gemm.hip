@@ -1195,7 +1195,7 @@ __global__ __launch_bounds__(NTW * 4 * 64) void gemmSkinnyWideKernel(SkinnyArgs 
 //     What bounds 64 rows is the bytes a CU takes in: every workgroup reads all the activations (from L2), as many
 //     bytes again as its share of the weights. Splitting K over grid.y (each workgroup then takes in half or a quarter
 //     of the activations) loses more to the fp32 slices and their reduction pass: 23.5 -> 26.1 us two ways, 35.8 four ways.
-constexpr int kSkinnyLdsBK = 128, kSkinnyLdsBN = 64, kSkinnyLdsStagger = 13;  // (64: the narrower of the two workgroup widths)
+constexpr int kSkinnyLdsBK = 128, kSkinnyLdsStagger = 13;
 
 template <typename T, int G, int NTP, int WST, int XST>
 __global__ __launch_bounds__(512) void gemmSkinnyLdsKernel(SkinnyArgs a) {

@@ -30,7 +30,12 @@ Fragment reads are issued in the order the MFMAs need them (B0, A0..A7, B1..B7; 
 returns them in order, so the wait before an MFMA is a count of younger reads that may still be outstanding.
 Measured and not used: K tiles of 32 in a four-stage ring (loads three tiles ahead) is 10 % slower, because a tile
 load then fetches 64-byte row pieces, twice the cache lines per byte; issuing the loads twice as densely (to gain
-slack) stalls the wave at issue."""
+slack) stalls the wave at issue. The same tile out of v_mfma_f32_32x32x16 (4 x 4 blocks per wave, four 16-wide k-steps,
+the same number of fragment reads) takes 1.5 % fewer cycles and 9 % more time (592 -> 646 us on 8192 x 4096 x 12288): that
+instruction reads and writes twice the accumulator registers per multiply-add, and at the power limit this is paid in
+clock. Register-only loops of either instruction over the whole chip (no memory traffic at all) sustain 2160 TFLOP/s at
+2.12 GHz (16x16x32, 16.4 cycles per instruction) against 1940 TFLOP/s at 1.87 GHz (32x32x16, 32.4 cycles): the first
+figure is the ceiling that the power limit leaves to any bf16 GEMM here, 0.86 of the nominal peak."""
 import os
 import sys
 
