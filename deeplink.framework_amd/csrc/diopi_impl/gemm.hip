@@ -382,6 +382,12 @@ __device__ __forceinline__ void vectorEpilogue(const MfmaArgs& g, T* out, const 
   } else if constexpr (EPI == kEpiRotary) {
     // A lane's 8 consecutive columns are 4 adjacent pairs of one head; their angles are 4 consecutive table
     // entries of the lane's row. Pieces at or past rotCols (the v heads) pass through with cos = 1, sin = 0.
+    // the two divisors are made opaque so that the set-up of the divisions by them is done here, per call, and not
+    // once per kernel with its results kept in registers across the K loop of a persistent caller
+    int headDim = g.rotHeadDim, tableRows = g.rotTableRows;
+    asm volatile("" : "+s"(headDim), "+s"(tableRows));
+    float zero = 0.f;  // produced here for the same reason: a zero kept from before the K loop came back from scratch
+    asm volatile("" : "+v"(zero));
     float bv[TN / 2][8];
     int pair0[TN / 2];
     bool rot[TN / 2];
@@ -391,46 +397,51 @@ __device__ __forceinline__ void vectorEpilogue(const MfmaArgs& g, T* out, const 
       Frag b8;
       if (bias) b8 = *reinterpret_cast<const Frag*>(bias + col);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) bv[jp][e] = bias ? static_cast<float>(b8[e]) : 0.f;
+      for (int e = 0; e < 8; ++e) bv[jp][e] = bias ? static_cast<float>(b8[e]) : zero;
       rot[jp] = col < g.rotCols;
-      pair0[jp] = (col % g.rotHeadDim) >> 1;
+      pair0[jp] = (col % headDim) >> 1;
     }
-    const int half = g.rotHeadDim >> 1;
+    const int half = headDim >> 1;
     const int tsz = g.rotTableF32 ? 4 : (int)sizeof(T);
     const __amdgpu_buffer_rsrc_t rsCos = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<void*>(g.rotCos), 0, (int)((int64_t)g.rotTableRows * half * tsz), 0x00020000);
+        const_cast<void*>(g.rotCos), 0, (int)((int64_t)tableRows * half * tsz), 0x00020000);
     const __amdgpu_buffer_rsrc_t rsSin = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<void*>(g.rotSin), 0, (int)((int64_t)g.rotTableRows * half * tsz), 0x00020000);
-    // Table entries are requested four fragment rows at a time,
-    // before any store of the batch: a request one row ahead would expose the L2 round trip once per row.
+        const_cast<void*>(g.rotSin), 0, (int)((int64_t)tableRows * half * tsz), 0x00020000);
+    // Table entries are requested four fragment rows at a time, before any store of the batch: loads and stores share
+    // one in-order counter, so a request one row ahead would expose the L2 round trip once per row. (Measured on the
+    // stacked QKV projection, 8192 x 4096 x 12288, same box: a ring of three rows requested two rows ahead 593.8 us,
+    // this form 588.7; the same ring for the addend of the linear form is 3 us slower than its batches of four.)
     float cs[4][TN / 2][4], sn[4][TN / 2][4];
     // a wave whose columns all lie at or past rotCols (v heads) asks for no table entries at all
     const bool anyRot = __builtin_amdgcn_readfirstlane(colBase) < g.rotCols;
-    auto fetch = [&](int i) {
+    auto fetch = [&](auto ic) {
+      constexpr int i = decltype(ic)::value;
       if (!anyRot) return;
       const int row = row0 + i * 16 + frow;
 #pragma unroll
       for (int jp = 0; jp < TN / 2; ++jp) {
-        const int off = row < g.M ? ((row % g.rotTableRows) * half + pair0[jp]) * tsz : kOutside;
+        const int off = row < g.M ? ((row % tableRows) * half + pair0[jp]) * tsz : kOutside;
         if (g.rotTableF32) {
           const u32x4 c4 = __builtin_amdgcn_raw_buffer_load_b128(rsCos, off, 0, 0);
           const u32x4 s4 = __builtin_amdgcn_raw_buffer_load_b128(rsSin, off, 0, 0);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) cs[i & 3][jp][e] = __uint_as_float(c4[e]), sn[i & 3][jp][e] = __uint_as_float(s4[e]);
+          for (int e = 0; e < 4; ++e) cs[i % 4][jp][e] = __uint_as_float(c4[e]), sn[i % 4][jp][e] = __uint_as_float(s4[e]);
         } else {
           typedef T T4 __attribute__((ext_vector_type(4)));
           const T4 c4 = __builtin_bit_cast(T4, __builtin_amdgcn_raw_buffer_load_b64(rsCos, off, 0, 0));
           const T4 s4 = __builtin_bit_cast(T4, __builtin_amdgcn_raw_buffer_load_b64(rsSin, off, 0, 0));
 #pragma unroll
-          for (int e = 0; e < 4; ++e) cs[i & 3][jp][e] = static_cast<float>(c4[e]), sn[i & 3][jp][e] = static_cast<float>(s4[e]);
+          for (int e = 0; e < 4; ++e) cs[i % 4][jp][e] = static_cast<float>(c4[e]), sn[i % 4][jp][e] = static_cast<float>(s4[e]);
         }
       }
     };
     staticFor<TM>([&](auto ic) {
       constexpr int i = decltype(ic)::value;
       if constexpr (i % 4 == 0) {
-#pragma unroll
-        for (int ii = i; ii < i + 4; ++ii) fetch(ii);
+        fetch(std::integral_constant<int, i>{});
+        fetch(std::integral_constant<int, i + 1>{});
+        fetch(std::integral_constant<int, i + 2>{});
+        fetch(std::integral_constant<int, i + 3>{});
       }
       f32x4 a[TN];
       accRow(ic, a);
@@ -443,8 +454,8 @@ __device__ __forceinline__ void vectorEpilogue(const MfmaArgs& g, T* out, const 
         Frag o;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const float c = rot[jp] ? cs[i & 3][jp][e] : 1.f;
-          const float sv = rot[jp] ? sn[i & 3][jp][e] * g.rotSinSign : 0.f;
+          const float c = rot[jp] ? cs[i % 4][jp][e] : 1.f;
+          const float sv = rot[jp] ? sn[i % 4][jp][e] * g.rotSinSign : 0.f;
           o[2 * e] = static_cast<T>(v[2 * e] * c - v[2 * e + 1] * sv);
           o[2 * e + 1] = static_cast<T>(v[2 * e] * sv + v[2 * e + 1] * c);
         }
@@ -708,7 +719,12 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
   const T* cin = g.Cin ? reinterpret_cast<const T*>(g.Cin) + (int64_t)batch * g.sCb : nullptr;
   const T* bias = reinterpret_cast<const T*>(g.bias);
   if (g.vecEpilogue) {
-    vectorEpilogue<T, EPI, TM, TN>(g, out, cin, bias, tm * BM + wm * WM, tn * BN + wn * WN, frow, kq, [&](auto ic, f32x4(&row)[TN]) {
+    // The lane's position is made opaque here: otherwise every lane-dependent value of the epilogue that does not depend
+    // on the tile is hoisted out of the persistent loop, has to stay live across the K loop, whose text owns v120-v247,
+    // and is spilled (13 registers in the rotary form, reloaded behind the K loop's tile loads).
+    int efrow = frow, ekq = kq;
+    asm volatile("" : "+v"(efrow), "+v"(ekq));
+    vectorEpilogue<T, EPI, TM, TN>(g, out, cin, bias, tm * BM + wm * WM, tn * BN + wn * WN, efrow, ekq, [&](auto ic, f32x4(&row)[TN]) {
 #pragma unroll
       for (int j = 0; j < TN; ++j) row[j] = acc[decltype(ic)::value][j];
     });
@@ -822,11 +838,23 @@ __global__ __launch_bounds__(256) void gemmMfma4WaveKernel(MfmaArgs g) {
   const u32x4 rsB = descriptor(B, ((int64_t)(g.N - 1) * g.ldb + g.K) * 2);
   // lane l of a wave fills the l-th 16-byte slot of a 1 KiB block (8 rows of 128 bytes); the chunk swizzle
   // c ^ ((row >> 1) & 7) is applied to the global address. A pass of the workgroup covers 32 rows.
-  const int srow = tid >> 3;
-  const int c8 = ((tid & 7) ^ ((srow >> 1) & 7)) * 8;
   constexpr unsigned kFar = 0x80000000u;  // beyond every extent: the load returns zeros
+  const int waveS = __builtin_amdgcn_readfirstlane(wave);
+  // this lane's number within the wave, asked of the hardware each time (volatile: neither hoisted nor shared)
+  auto laneNow = []() {
+    int l;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+    return l;
+  };
   unsigned voA[8], voB[8];
   auto laneOffsets = [&](int tm, int tn) {
+    // recomputed on every call from the lane number the hardware hands out: the eight row numbers and the chunk
+    // offset (or the thread index they come from) would otherwise be kept live across the K loop, whose text owns
+    // v120-v247, and spilled; a reload between two pieces of that text waits for every tile load in flight (loads
+    // return in order)
+    const int t = waveS * 64 + laneNow();
+    const int srow = t >> 3;
+    const int c8 = ((t & 7) ^ ((srow >> 1) & 7)) * 8;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int ra = tm * BM + srow + 32 * i, rb = tn * BN + srow + 32 * i;
@@ -883,7 +911,11 @@ __global__ __launch_bounds__(256) void gemmMfma4WaveKernel(MfmaArgs g) {
     }
     // one fragment row at a time out of the accumulation registers, which the compiler does not know to be live:
     // the epilogue stays far below the 256 ordinary registers, so it never borrows them
-    vectorEpilogue<T, EPI, TM, TN>(g, out, cin, bias, tm * BM + wm * WM, tn * BN + wn * WN, frow, kq, [&](auto ic, f32x4(&row)[TN]) {
+    // The lane's position is asked for again here: otherwise every lane-dependent value of the epilogue that does not
+    // depend on the tile is hoisted out of the persistent loop, has to stay live across the K loop, and is spilled
+    // (13 registers in the rotary form, reloaded behind the tile loads already issued for the next output tile).
+    const int elane = laneNow(), efrow = elane & 15, ekq = elane >> 4;
+    vectorEpilogue<T, EPI, TM, TN>(g, out, cin, bias, tm * BM + (waveS >> 1) * WM, tn * BN + (waveS & 1) * WN, efrow, ekq, [&](auto ic, f32x4(&row)[TN]) {
       constexpr int i = decltype(ic)::value;
       f32x4 lo[4], hi[4];
       accRegisters16<32 * i>(lo);
