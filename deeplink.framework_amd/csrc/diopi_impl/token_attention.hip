@@ -25,6 +25,10 @@
 //   * a workgroup = 4 waves owns a chunk of the sequence (split-KV, chunks of at least 512
 //     tokens and at most 64 per sequence); states are merged by wave butterflies, then through
 //     LDS, then across chunks by a small lane-parallel second kernel.
+//
+// Head rows of 128, 256 or 512 bytes at 16-byte aligned strides take the kernels above; any other head size or
+// alignment (up to 1024 elements) takes the generic kernels at the end: one workgroup per (sequence, head), 256 tokens
+// at a time, one token's dot product per thread and P.V with the threads over d. A correctness path.
 #include <algorithm>
 #include <mutex>
 
@@ -50,6 +54,7 @@ struct TaArgs {
   const void* bStart;
   const void* bLen;
   bool loc64, start64, len64;
+  bool generic;  // head rows the vector kernels do not take: the generic kernels run
   int64_t locRowStride;  // elements
   int64_t kSlotStride, kHeadStride, vSlotStride, vHeadStride;  // elements
   int64_t qBatchStride, qHeadStride;
@@ -399,6 +404,157 @@ __global__ __launch_bounds__(256) void softmaxReduceVKernel(TaArgs a, T* __restr
   }
 }
 
+// ------------------------------------------------ any head size: generic kernels --
+constexpr int kTaGenericMaxD = 1024;  // four elements of the head row per thread
+
+// max / sum of one value per thread over the workgroup of 256 (red: 4 floats of LDS; two barriers)
+__device__ __forceinline__ float blockMax256(float v, float* red) {
+  v = waveMax(v);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  v = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  return v;
+}
+__device__ __forceinline__ float blockSum256(float v, float* red) {
+  v = waveSum(v);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  v = red[0] + red[1] + red[2] + red[3];
+  __syncthreads();
+  return v;
+}
+
+// Fused decode attention, one workgroup per (sequence, head) (ext_ops.py:100-133). Tokens whose slot lies outside the
+// pool are skipped, as in the vector kernels; a sequence of length 0 gives zeros.
+template <typename T>
+__global__ __launch_bounds__(256) void decodeGenericKernel(TaArgs a, T* __restrict__ out) {
+  __shared__ float prob[256];
+  __shared__ int64_t slotOf[256];
+  __shared__ float red[4];
+  const int h = blockIdx.x, b = blockIdx.z, tid = threadIdx.x;
+  const int len = min(max((int)ldIndex(a.bLen, b, a.len64), 0), a.maxLen);
+  const int kvh = h / (a.heads / a.kvHeads);
+  const int64_t locBase = (int64_t)b * a.locRowStride + (a.maxLen - len);
+  const T* q = reinterpret_cast<const T*>(a.q) + b * a.qBatchStride + h * a.qHeadStride;
+  const T* kHead = reinterpret_cast<const T*>(a.k) + kvh * a.kHeadStride;
+  const T* vHead = reinterpret_cast<const T*>(a.v) + kvh * a.vHeadStride;
+  float m = -INFINITY, l = 0.f, acc[4] = {0.f, 0.f, 0.f, 0.f};  // acc[j]: element tid + 256 j of the output row
+  for (int t0 = 0; t0 < len; t0 += 256) {
+    const int t = t0 + tid;
+    int64_t slot = t < len ? ldIndex(a.bLoc, locBase + t, a.loc64) : -1;
+    if (slot >= a.slots) slot = -1;
+    float sc = -INFINITY;  // in the scaled log2 domain
+    if (slot >= 0) {
+      const T* k = kHead + slot * a.kSlotStride;
+      float d = 0.f;
+      for (int e = 0; e < a.d; ++e) d += static_cast<float>(q[e]) * static_cast<float>(k[e]);
+      sc = d * a.scaleLog2e;
+    }
+    const float mn = fmaxf(m, blockMax256(sc, red));
+    const float pr = sc == -INFINITY ? 0.f : exp2f(sc - mn);
+    prob[tid] = pr;
+    slotOf[tid] = slot;
+    const float bs = blockSum256(pr, red);  // its barriers also publish prob / slotOf
+    const float corr = m == -INFINITY ? 0.f : exp2f(m - mn);
+    l = l * corr + bs;
+    const int cnt = min(256, len - t0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int e = tid + 256 * j;
+      if (e < a.d) {
+        float x = acc[j] * corr;
+        for (int i = 0; i < cnt; ++i)
+          if (slotOf[i] >= 0) x += prob[i] * static_cast<float>(vHead[slotOf[i] * a.vSlotStride + e]);
+        acc[j] = x;
+      }
+    }
+    m = mn;
+    __syncthreads();  // prob / slotOf are rewritten by the next block of tokens
+  }
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int e = tid + 256 * j;
+    if (e < a.d) out[((int64_t)b * a.heads + h) * a.d + e] = static_cast<T>(acc[j] * inv);
+  }
+}
+
+// Two-call form, first half: att[h, start_b + t] = q[b,h,:] . k[slot_t,h,:] / sqrt(d); -inf for a slot outside the pool.
+template <typename T, typename OT>
+__global__ __launch_bounds__(256) void tokenLogitsGenericKernel(TaArgs a, OT* __restrict__ att, int64_t attHeadStride) {
+  const int h = blockIdx.x, b = blockIdx.z;
+  const int len = min(max((int)ldIndex(a.bLen, b, a.len64), 0), a.maxLen);
+  const int64_t start = ldIndex(a.bStart, b, a.start64);
+  const int begin = blockIdx.y * a.chunk, end = min(len, begin + a.chunk);
+  const int kvh = h / (a.heads / a.kvHeads);
+  const int64_t locBase = (int64_t)b * a.locRowStride + (a.maxLen - len);
+  const T* q = reinterpret_cast<const T*>(a.q) + b * a.qBatchStride + h * a.qHeadStride;
+  const T* kHead = reinterpret_cast<const T*>(a.k) + kvh * a.kHeadStride;
+  const float scale = a.scaleLog2e / kLog2eTA;
+  for (int t = begin + threadIdx.x; t < end; t += 256) {
+    const int64_t slot = ldIndex(a.bLoc, locBase + t, a.loc64);
+    float v = -INFINITY;
+    if (slot >= 0 && slot < a.slots) {
+      const T* k = kHead + slot * a.kSlotStride;
+      float d = 0.f;
+      for (int e = 0; e < a.d; ++e) d += static_cast<float>(q[e]) * static_cast<float>(k[e]);
+      v = d * scale;
+    }
+    att[h * attHeadStride + start + t] = static_cast<OT>(v);
+  }
+}
+
+// Two-call form, second half: out[b,h,:] = softmax(logics[h, start_b : start_b + len]) . v[slots].
+template <typename T, typename LT>
+__global__ __launch_bounds__(256) void softmaxReduceVGenericKernel(TaArgs a, T* __restrict__ out, const LT* __restrict__ logics,
+                                                                    int64_t logHeadStride) {
+  __shared__ float prob[256];
+  __shared__ int64_t slotOf[256];
+  __shared__ float red[4];
+  const int h = blockIdx.x, b = blockIdx.z, tid = threadIdx.x;
+  const int len = min(max((int)ldIndex(a.bLen, b, a.len64), 0), a.maxLen);
+  const int64_t start = ldIndex(a.bStart, b, a.start64);
+  const int kvh = h / (a.heads / a.kvHeads);
+  const int64_t locBase = (int64_t)b * a.locRowStride + (a.maxLen - len);
+  const LT* lg = logics + h * logHeadStride + start;
+  const T* vHead = reinterpret_cast<const T*>(a.v) + kvh * a.vHeadStride;
+  float m = -INFINITY;
+  for (int t = tid; t < len; t += 256) m = fmaxf(m, static_cast<float>(lg[t]));
+  m = blockMax256(m, red);
+  const float mS = m == -INFINITY ? 0.f : m * kLog2eTA;
+  float sum = 0.f;
+  for (int t = tid; t < len; t += 256) sum += exp2f(static_cast<float>(lg[t]) * kLog2eTA - mS);
+  sum = blockSum256(sum, red);
+  const float inv = sum > 0.f ? 1.f / sum : 0.f;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int t0 = 0; t0 < len; t0 += 256) {
+    const int t = t0 + tid;
+    int64_t slot = t < len ? ldIndex(a.bLoc, locBase + t, a.loc64) : -1;
+    if (slot >= a.slots) slot = -1;
+    prob[tid] = slot >= 0 ? exp2f(static_cast<float>(lg[t]) * kLog2eTA - mS) : 0.f;
+    slotOf[tid] = slot;
+    __syncthreads();
+    const int cnt = min(256, len - t0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int e = tid + 256 * j;
+      if (e < a.d) {
+        float x = acc[j];
+        for (int i = 0; i < cnt; ++i)
+          if (slotOf[i] >= 0) x += prob[i] * static_cast<float>(vHead[slotOf[i] * a.vSlotStride + e]);
+        acc[j] = x;
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int e = tid + 256 * j;
+    if (e < a.d) out[((int64_t)b * a.heads + h) * a.d + e] = static_cast<T>(acc[j] * inv);
+  }
+}
+
 // ---------------------------------------------------------------- host side --
 struct TaViews {
   TensorView q, k, v, loc, start, len;
@@ -440,15 +596,16 @@ static diopiError_t fillArgs(const TaViews& t, bool needK, bool needV, int maxLe
             (long)t.loc.shape[1], maxLen);
   AMD_CHECK(t.start.numel == batch && t.len.numel == batch, "token attention: b_start_loc/b_seq_len must have %ld entries",
             (long)batch);
+  AMD_CHECK(q.dtype == diopi_dtype_bfloat16 || q.dtype == diopi_dtype_float16 || q.dtype == diopi_dtype_float32,
+            "token attention: unsupported dtype %s", dtypeName(q.dtype));
   const int64_t bytes = q.shape[2] * q.itemsize;
-  AMD_CHECK(bytes == 128 || bytes == 256 || bytes == 512,
-            "token attention: head rows of %ld bytes are not supported (128, 256 or 512)", (long)bytes);
-  AMD_CHECK(q.aligned16() && kv.aligned16() && (kv.stride[0] * kv.itemsize) % 16 == 0 && (kv.stride[1] * kv.itemsize) % 16 == 0 &&
-                (q.stride[0] * q.itemsize) % 16 == 0 && (q.stride[1] * q.itemsize) % 16 == 0,
-            "token attention: q/k/v rows must be 16-byte aligned");
+  bool vector = (bytes == 128 || bytes == 256 || bytes == 512) && q.aligned16() && kv.aligned16() &&
+                (kv.stride[0] * kv.itemsize) % 16 == 0 && (kv.stride[1] * kv.itemsize) % 16 == 0 &&
+                (q.stride[0] * q.itemsize) % 16 == 0 && (q.stride[1] * q.itemsize) % 16 == 0;
   if (needK && needV)
-    AMD_CHECK(t.v.aligned16() && (t.v.stride[0] * q.itemsize) % 16 == 0 && (t.v.stride[1] * q.itemsize) % 16 == 0,
-              "token attention: v rows must be 16-byte aligned");
+    vector = vector && t.v.aligned16() && (t.v.stride[0] * q.itemsize) % 16 == 0 && (t.v.stride[1] * q.itemsize) % 16 == 0;
+  a->generic = !vector;
+  AMD_CHECK(vector || q.shape[2] <= kTaGenericMaxD, "token attention: head_dim %ld exceeds %d", (long)q.shape[2], kTaGenericMaxD);
   a->q = q.data;
   a->k = needK ? t.k.data : nullptr;
   a->v = needV ? t.v.data : nullptr;
@@ -490,6 +647,13 @@ static diopiError_t fillArgs(const TaViews& t, bool needK, bool needV, int maxLe
       setLastError("token attention: unsupported dtype %s", dtypeName(DTYPE));                 \
       return diopiErrorOccurred;                                                               \
     }                                                                                          \
+  } while (0)
+
+#define TA_GENERIC_DISPATCH(DTYPE, CALL)                                \
+  do {                                                                  \
+    if (DTYPE == diopi_dtype_bfloat16) { CALL(bf16_t); }                \
+    else if (DTYPE == diopi_dtype_float16) { CALL(half_t); }            \
+    else { CALL(float); }                                               \
   } while (0)
 
 // Split-KV partial results for the entry point that allocates nothing. Every device the library's code object is
@@ -544,6 +708,15 @@ static diopiError_t decodeAttention(diopiContextHandle_t ctx, diopiTensorHandle_
             "token attention: out must be a dense tensor shaped like q");
   const int64_t batch = t.q.shape[0];
   if (batch == 0 || t.q.numel == 0) return diopiSuccess;
+  if (a.generic) {
+    AMD_CHECK(batch <= 65535, "token attention: batch %ld exceeds the grid limits", (long)batch);
+    dim3 grid(a.heads, 1, (unsigned)batch);
+#define GENERIC_CALL(T) hipLaunchKernelGGL((decodeGenericKernel<T>), grid, dim3(256), 0, stream, a, out.ptr<T>())
+    TA_GENERIC_DISPATCH(t.q.dtype, GENERIC_CALL);
+#undef GENERIC_CALL
+    AMD_LAUNCH_CHECK();
+    return diopiSuccess;
+  }
   a.nsplit = (int)std::max<int64_t>(1, ceilDiv(maxInputLen, a.chunk));
   AMD_CHECK(batch <= 65535 && a.nsplit <= 65535, "token attention: batch %ld / splits %d exceed the grid limits", (long)batch,
             a.nsplit);
@@ -631,6 +804,20 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiTokenAttenti
   AMD_CHECK(batch <= 65535 && nchunk <= 65535, "token attention: grid limits exceeded");
   dim3 grid(a.heads, nchunk, (unsigned)batch), block(256);
   const int64_t bytes = t.q.shape[2] * t.q.itemsize;
+  if (a.generic) {
+    if (att.dtype == diopi_dtype_float32) {
+#define GENERIC_CALL(T) \
+  hipLaunchKernelGGL((tokenLogitsGenericKernel<T, float>), grid, block, 0, stream, a, att.ptr<float>(), att.stride[0])
+      TA_GENERIC_DISPATCH(t.q.dtype, GENERIC_CALL);
+#undef GENERIC_CALL
+    } else {
+#define GENERIC_CALL(T) hipLaunchKernelGGL((tokenLogitsGenericKernel<T, T>), grid, block, 0, stream, a, att.ptr<T>(), att.stride[0])
+      TA_GENERIC_DISPATCH(t.q.dtype, GENERIC_CALL);
+#undef GENERIC_CALL
+    }
+    AMD_LAUNCH_CHECK();
+    return diopiSuccess;
+  }
   if (att.dtype == diopi_dtype_float32) {
 #define LOGIT_CALL(T, LPT) \
   hipLaunchKernelGGL((tokenLogitsKernel<T, LPT, float>), grid, block, 0, stream, a, att.ptr<float>(), att.stride[0])
@@ -673,6 +860,21 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiTokenSoftmax
   AMD_CHECK(batch <= 65535, "token attention: grid limits exceeded");
   dim3 grid(a.heads, 1, (unsigned)batch), block(256);
   const int64_t bytes = out.shape[2] * out.itemsize;
+  if (a.generic) {
+    if (lg.dtype == diopi_dtype_float32) {
+#define GENERIC_CALL(T) \
+  hipLaunchKernelGGL((softmaxReduceVGenericKernel<T, float>), grid, block, 0, stream, a, out.ptr<T>(), lg.ptr<float>(), lg.stride[0])
+      TA_GENERIC_DISPATCH(out.dtype, GENERIC_CALL);
+#undef GENERIC_CALL
+    } else {
+#define GENERIC_CALL(T) \
+  hipLaunchKernelGGL((softmaxReduceVGenericKernel<T, T>), grid, block, 0, stream, a, out.ptr<T>(), lg.ptr<T>(), lg.stride[0])
+      TA_GENERIC_DISPATCH(out.dtype, GENERIC_CALL);
+#undef GENERIC_CALL
+    }
+    AMD_LAUNCH_CHECK();
+    return diopiSuccess;
+  }
   if (lg.dtype == diopi_dtype_float32) {
 #define RV_CALL(T, LPT) \
   hipLaunchKernelGGL((softmaxReduceVKernel<T, LPT, float>), grid, block, 0, stream, a, out.ptr<T>(), lg.ptr<float>(), lg.stride[0])

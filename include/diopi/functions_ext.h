@@ -47,7 +47,9 @@ DIOPI_API diopiError_t diopiDestIndexCopyKV(diopiContextHandle_t ctx, diopiTenso
  * for t in [0, b_seq_len[b]), slot = b_loc[b, max_input_len - b_seq_len[b] + t] (right-aligned slot table).
  * q [batch, heads, d]; k [slots, kv_heads, d]; attention_out [heads, total_tokens] (fp32 or q dtype).
  * In all three decode entry points a b_seq_len[b] outside [0, max_input_len] is cut to that range (the table row
- * holds no more), and slots outside the pool are skipped, never dereferenced.
+ * holds no more), and slots outside the pool are skipped, never dereferenced. q, k, v are float32, float16 or
+ * bfloat16 with a contiguous head dimension; head rows of 128, 256 or 512 bytes at 16-byte aligned strides take the
+ * streaming kernels, any other head size up to 1024 elements a plain kernel (one workgroup per sequence and head).
  * Semantics: the q.K^T/sqrt(d) step of ext_ops.py:100-133. */
 DIOPI_API diopiError_t diopiTokenAttentionInference(diopiContextHandle_t ctx, diopiTensorHandle_t attention_out,
                                                     diopiConstTensorHandle_t q, diopiConstTensorHandle_t k,

@@ -360,6 +360,35 @@ def test_token_attention_fused_and_two_call(ops, dev, pkg, dtype, d, idt):
     chk(out2, want)
 
 
+@pytest.mark.parametrize("dtype,d,kvh,rep", [(torch.bfloat16, 80, 4, 2), (torch.float16, 32, 2, 1), (torch.float32, 96, 1, 4),
+                                             (torch.bfloat16, 40, 8, 1), (torch.float32, 300, 2, 1)])
+def test_token_attention_any_head_size(ops, dev, pkg, dtype, d, kvh, rep):
+    """Head rows that are not 128, 256 or 512 bytes long (or not 16-byte aligned: d = 40 in bf16 is 80 bytes) take
+    the generic kernels: the fused form, the entry point that allocates nothing and the two-call form against the
+    oracle (ext_ops.py:100-133), with a sequence of one token and one longer than a block of 256."""
+    heads = kvh * rep
+    w = pkg.workloads.paged_decode(seed=11, batch=5, heads=kvh, head_dim=d, min_len=1, max_len=700, pool_slots=4096, dtype=dtype)
+    w["b_seq_len"][0] = 1                                    # b_loc is right-aligned: the last column is the token
+    gq = torch.Generator().manual_seed(12)
+    q = torch.randn(5, heads, d, generator=gq).to(dtype)
+    want = oracle.token_attention(q.float(), w["k_pool"].float(), w["v_pool"].float(), w["b_loc"], w["b_seq_len"], w["max_input_len"])
+    dk, dv = w["k_pool"].to(dev), w["v_pool"].to(dev)
+    args = (w["b_loc"].to(dev), w["b_start_loc"].to(dev), w["b_seq_len"].to(dev), w["max_input_len"])
+    chk = assert_fp32 if dtype == torch.float32 else assert_half
+    got = ops.token_decode_attention(q.to(dev), dk, dv, *args)
+    chk(got, want)
+    assert_exact(ops.token_decode_attention(q.to(dev), dk, dv, *args, no_alloc=True), got.cpu())
+    att = torch.zeros(heads, w["total_tokens"], dtype=torch.float32, device=dev)
+    ops.token_attention(q.to(dev), dk, att, *args)
+    want_att = oracle.token_logits(q, w["k_pool"], w["b_loc"], w["b_start_loc"], w["b_seq_len"], w["max_input_len"], w["total_tokens"])
+    for b in range(5):                                       # only the columns of live tokens are defined
+        s0, n = int(w["b_start_loc"][b]), int(w["b_seq_len"][b])
+        assert_fp32(att[:, s0:s0 + n], want_att[:, s0:s0 + n], rel=1e-5)
+    out2 = torch.empty_like(got)
+    ops.token_softmax_reducev(att, dv, out2, *args)
+    chk(out2, want)
+
+
 @pytest.mark.parametrize("heads,kvh", [(8, 2), (6, 3)])
 def test_token_attention_len_one_and_gqa(ops, dev, heads, kvh):
     """Grouped-query decode: 8 heads (a wave's lane groups take four consecutive heads of one token) and 6 heads (not a
