@@ -323,7 +323,7 @@ def copy_(self, src):
 def cat(tensors, dim=0, *, out=None):
     tensors = list(tensors)
     if out is None:
-        ref = next(t for t in tensors if not (t.dim() == 1 and t.numel() == 0))
+        ref = next((t for t in tensors if not (t.dim() == 1 and t.numel() == 0)), tensors[0])  # all legacy-empty: the result is empty
         d = dim % ref.dim()
         shape = list(ref.shape)
         shape[d] = sum(t.shape[d] for t in tensors if not (t.dim() == 1 and t.numel() == 0))

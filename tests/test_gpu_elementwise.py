@@ -162,6 +162,9 @@ def test_copy_cast_cat_mean(ops, dev):
     a, b = torch.randn(3, 4, 5, generator=g(15)), torch.randn(3, 2, 5, generator=g(16))
     assert_exact(ops.cat([a.to(dev), b.to(dev)], dim=1), torch.cat([a, b], 1))
     assert_exact(ops.cat([a.to(dev), a.to(dev)], dim=-1), torch.cat([a, a], -1))
+    e = torch.empty(0)                                # 1-D empties are skipped; all of them empty: an empty result
+    assert_exact(ops.cat([e.to(dev), a.to(dev), e.to(dev)], dim=2), torch.cat([e, a, e], 2))
+    assert_exact(ops.cat([e.to(dev), e.to(dev)], dim=0), torch.cat([e, e], 0))
     m = torch.randn(6, 7, 64, generator=g(17))
     assert_fp32(ops.mean(m.to(dev), -1, keepdim=True), m.mean(-1, keepdim=True))
     assert_fp32(ops.mean(m.to(dev), [0, 2]), m.mean([0, 2]))
