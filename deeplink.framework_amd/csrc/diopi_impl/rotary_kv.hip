@@ -173,6 +173,23 @@ struct IndexTables {  // passed by value as a kernel argument
   int64_t strides[kMaxDims];
 };
 
+// *addr += v for a 16-bit float: compare-and-swap on the aligned 32-bit word that holds it (the sum is rounded to
+// the element type after every addition, as a 16-bit accumulate does).
+template <typename T>
+__device__ __forceinline__ void atomicAdd16(T* addr, float v) {
+  const uintptr_t a = reinterpret_cast<uintptr_t>(addr);
+  unsigned* word = reinterpret_cast<unsigned*>(a & ~uintptr_t(3));
+  const int shift = (int)(a & 2) * 8;
+  unsigned old = *word, assumed;
+  do {
+    assumed = old;
+    const unsigned short curBits = (unsigned short)(assumed >> shift);
+    const T next = static_cast<T>(static_cast<float>(__builtin_bit_cast(T, curBits)) + v);
+    const unsigned repl = (assumed & ~(0xffffu << shift)) | ((unsigned)__builtin_bit_cast(unsigned short, next) << shift);
+    old = atomicCAS(word, assumed, repl);
+  } while (old != assumed);
+}
+
 template <typename IDX>
 __global__ __launch_bounds__(256) void indexPutKernel(void* input, const void* values, int dtIn, int dtVal,
                                                        IndexTables tab, int nIdx, int64_t rows, int64_t inner,
@@ -203,6 +220,10 @@ __global__ __launch_bounds__(256) void indexPutKernel(void* input, const void* v
                   (unsigned long long)loadAs<int64_t>(values, r * valRowStride + c, dtVal));
       } else if (dtIn == diopi_dtype_float64) {
         atomicAdd(reinterpret_cast<double*>(input) + off, loadAs<double>(values, r * valRowStride + c, dtVal));
+      } else if (dtIn == diopi_dtype_bfloat16) {
+        atomicAdd16(reinterpret_cast<bf16_t*>(input) + off, loadAs<float>(values, r * valRowStride + c, dtVal));
+      } else if (dtIn == diopi_dtype_float16) {
+        atomicAdd16(reinterpret_cast<half_t*>(input) + off, loadAs<float>(values, r * valRowStride + c, dtVal));
       }
     }
   }
@@ -349,8 +370,9 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiIndexPutInp(
   AMD_CHECK(in.isContiguous(), "diopiIndexPutInp: input must be dense");
   if (accumulate)
     AMD_CHECK(in.dtype == diopi_dtype_float32 || in.dtype == diopi_dtype_float64 || in.dtype == diopi_dtype_int32 ||
-                  in.dtype == diopi_dtype_int64,
-              "diopiIndexPutInp: accumulate supports float32/float64/int32/int64 inputs, got %s", dtypeName(in.dtype));
+                  in.dtype == diopi_dtype_int64 || in.dtype == diopi_dtype_bfloat16 || in.dtype == diopi_dtype_float16,
+              "diopiIndexPutInp: accumulate supports float16/bfloat16/float32/float64/int32/int64 inputs, got %s",
+              dtypeName(in.dtype));
   TensorView idx[kMaxDims];
   int64_t rows = -1;
   diopiDtype_t idt = diopi_dtype_int64;

@@ -315,6 +315,16 @@ def test_index_put(ops, dev):
             got = inp.clone().to(dev)
             ops.index_put_(got, [i.to(dev) for i in ind], vals.to(dev), accumulate=True)
             assert_fp32(got, want, rel=1e-4)   # assertRtolEqual's 1e-4 (common_utils.py:266-269)
+    # accumulate into 16-bit floats, odd and even element offsets, a repeated row (three additions into one element)
+    for dt in (torch.bfloat16, torch.float16):
+        base = torch.randn(9, 7, generator=g(42)).to(dt)
+        vals = torch.randn(4, 7, generator=g(43)).to(dt)
+        loc = torch.tensor([8, 2, 2, 2])
+        want = base.float().index_put((loc,), vals.float(), accumulate=True)
+        got = base.clone().to(dev)
+        ops.index_put_(got, [loc.to(dev)], vals.to(dev), accumulate=True)
+        assert_half(got, want)
+        assert_exact(got[[0, 1, 3, 4, 5, 6, 7]], base[[0, 1, 3, 4, 5, 6, 7]])
     # row scatter without accumulate: the KV-cache form
     pool = torch.zeros(20, 4, 8).bfloat16()
     rows = torch.randn(5, 4, 8, generator=g(41)).bfloat16()
