@@ -428,3 +428,158 @@ def test_sweep_rotary_index_and_batched(ops, dev, seed, n):
         except RuntimeError as e:   # nothing in these ranges may be refused
             failed.append(desc + ": refused: " + str(e)[:300])
     _report(failed, n)
+
+
+@pytest.mark.parametrize("seed,n", [(1, 400), (2, 400)])
+def test_sweep_strided_operands_and_argument_forms(ops, dev, pkg, seed, n):
+    """q / k / v as views of one packed projection and a strided destination for prefill attention, K and V as the halves
+    of one packed pool for decode, RMSNorm with bias / inv_rms on n-d input, rotary in place on a packed view, softmax on
+    transposed input, div rounding modes, comparisons with scalars, masked_fill with a value tensor, fill on hollow views,
+    broadcast copies with a cast into a transposed destination, in-place ops on hollow views."""
+    rng = random.Random(seed)
+    failed = []
+    for case in range(n):
+        g = torch.Generator().manual_seed(seed * 32452843 + case)
+        kind = rng.choice(["prefill_packed", "decode_strided", "rms_forms", "rotary_strided", "softmax_strided", "div_modes", "cmp_scalar", "masked_fill_tensor", "fill", "copy_bcast", "silu_mul", "sub_scalar", "linear_out_strided3d", "where_scalar", "inplace_strided"])
+        desc = f"case {case} {kind}"
+        try:
+            if kind == "prefill_packed":
+                dt = rng.choice(FLOATS); d = rng.choice([64, 128, 80]); kvh = rng.choice([1, 2, 4]); heads = kvh * rng.choice([1, 2, 4])
+                lens = [rng.randint(1, 300 if dt != torch.float32 and d != 80 else 150) for _ in range(rng.choice([1, 2, 4]))]
+                toks = sum(lens); starts = [sum(lens[:i]) for i in range(len(lens))]
+                desc += f" {dt} heads={heads}/{kvh} d={d} lens={lens}"
+                qkv = torch.randn(toks, (heads + 2 * kvh) * d, generator=g).to(dt)
+                q, k, v = qkv[:, :heads * d].view(toks, heads, d), qkv[:, heads * d:(heads + kvh) * d].view(toks, kvh, d), qkv[:, (heads + kvh) * d:].view(toks, kvh, d)
+                st, ln = torch.tensor(starts, dtype=torch.int32), torch.tensor(lens, dtype=torch.int32)
+                want = oracle.context_attention(q.contiguous(), k.contiguous(), v.contiguous(), st, ln)
+                dq = qkv.to(dev)
+                Q, K, V = dq[:, :heads * d].view(toks, heads, d), dq[:, heads * d:(heads + kvh) * d].view(toks, kvh, d), dq[:, (heads + kvh) * d:].view(toks, kvh, d)
+                big = torch.zeros(toks, heads * d + 16, dtype=dt, device=dev)
+                out = big[:, :heads * d].view(toks, heads, d)
+                ops.context_attention(Q, K, V, st.to(dev), ln.to(dev), max(lens), out=out)
+                (assert_fp32 if dt == torch.float32 else assert_half)(out, want)
+                assert float(big[:, heads * d:].abs().sum()) == 0.0
+            elif kind == "decode_strided":
+                dt = rng.choice(FLOATS); d = rng.choice([64, 128, 48]); kvh = rng.choice([1, 2, 8]); heads = kvh * rng.choice([1, 4])
+                batch = rng.choice([1, 3, 9]); maxl = rng.choice([1, 70, 600, 1100])
+                desc += f" {dt} heads={heads}/{kvh} d={d} batch={batch} maxlen={maxl}"
+                w = pkg.workloads.paged_decode(seed=seed * 13 + case, batch=batch, heads=kvh, head_dim=d, min_len=1, max_len=maxl, pool_slots=max(1024, batch * (maxl + 2)), dtype=dt)
+                q = torch.randn(batch, heads, d, generator=g).to(dt)
+                want = oracle.token_attention(q.float(), w["k_pool"].float(), w["v_pool"].float(), w["b_loc"], w["b_seq_len"], w["max_input_len"])
+                # K and V as the two halves of one packed pool [slots, 2, kv_heads, d]; b_loc wider than max_input_len is not allowed, so keep it
+                kv = torch.stack([w["k_pool"], w["v_pool"]], 1).to(dev)
+                args = (w["b_loc"].to(dev), w["b_start_loc"].to(dev), w["b_seq_len"].to(dev), w["max_input_len"])
+                qq = torch.zeros(batch, heads, d + 8, dtype=dt, device=dev); qq[..., :d] = q.to(dev)
+                got = ops.token_decode_attention(qq[..., :d] if d % 8 == 0 else q.to(dev), kv[:, 0], kv[:, 1], *args)
+                (assert_fp32 if dt == torch.float32 else assert_half)(got, want.to(dt))
+            elif kind == "rms_forms":
+                dt = rng.choice(FLOATS); shape = rng.choice([(3, 5, 64), (2, 2, 2, 100), (7, 4096), (1, 8), (300, 1000)])
+                bias = rng.random() < 0.4; inv = rng.random() < 0.5
+                desc += f" {dt} {shape} bias={bias} inv_rms={inv}"
+                x = torch.randn(shape, generator=g).to(dt); wt = (torch.randn(shape[-1], generator=g) * 0.1 + 1).to(dt)
+                b = torch.randn(shape[-1], generator=g).to(dt) if bias else None
+                want = oracle.rms_norm(x, wt, 1e-6)
+                if bias:   # one rounding, after the bias: the norm in fp32 (rms_norm_fp32 follows model.py:34-39)
+                    xf = x.float()
+                    want = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-6) * wt.float() + b.float()).to(dt)
+                ir = torch.empty(shape[:-1], dtype=torch.float32, device=dev) if inv else None
+                got = ops.rms_norm(x.to(dev), wt.to(dev), 1e-6, bias=b.to(dev) if bias else None, inv_rms=ir)
+                assert_close(got, want)
+                if inv: assert_fp32(ir, torch.rsqrt(x.float().pow(2).mean(-1) + 1e-6), rel=1e-5)
+            elif kind == "rotary_strided":
+                dt = rng.choice(FLOATS); toks, heads, d = rng.choice([1, 33, 200]), rng.choice([2, 8]), rng.choice([64, 128, 32])
+                inter = rng.random() < 0.5
+                desc += f" {dt} [{toks},{heads},{d}] interleaved={inter} packed qkv view, in place"
+                qkv = torch.randn(toks, 3 * heads * d, generator=g).to(dt)
+                cos, sin = oracle.precompute_freqs(d, toks); cos, sin = cos.to(dt), sin.to(dt)
+                want = qkv.clone()
+                wq = (oracle.rotary_emb_interleaved if inter else oracle.rotary_emb)(qkv[:, :heads * d].reshape(toks, heads, d), cos.float(), sin.float())
+                want[:, :heads * d] = wq.reshape(toks, heads * d).to(dt)
+                dq = qkv.to(dev); view = dq[:, :heads * d].view(toks, heads, d)
+                ops.rotary_emb(view, cos.to(dev), sin.to(dev), interleaved=inter, out=view)
+                assert_close(dq[:, :heads * d], want[:, :heads * d]); assert_exact(dq[:, heads * d:], want[:, heads * d:])
+            elif kind == "softmax_strided":
+                dt = rng.choice(FLOATS); shape = rng.choice([(4, 8, 33), (2, 3, 5, 7), (64, 300), (5, 70000)]); dim = rng.randrange(-len(shape), len(shape))
+                desc += f" {dt} {shape} dim={dim} transposed input"
+                x = torch.randn(shape, generator=g).to(dt)
+                X = x.to(dev).transpose(0, -1).contiguous().transpose(0, -1)
+                assert_close(ops.softmax(X, dim), oracle.softmax(x, dim))
+            elif kind == "div_modes":
+                dt = rng.choice(FLOATS + [torch.int32, torch.int64]); mode = rng.choice([None, "floor", "trunc"]); shape = rng.choice([(7,), (3, 50), (2, 1, 9)])
+                desc += f" {dt} {shape} mode={mode}"
+                a = (torch.randn(shape, generator=g) * 20).to(dt); b = (torch.randn(shape[-1:], generator=g) * 5).to(dt)
+                b = torch.where(b == 0, torch.ones_like(b) * 3, b)
+                if dt.is_floating_point and mode is not None: a, b = a.round(), b.round().masked_fill(b.round() == 0, 2)
+                want = torch.div(a.float(), b.float(), rounding_mode=mode).to(dt) if dt == torch.float16 else torch.div(a, b, rounding_mode=mode)
+                got = ops.div(a.to(dev), b.to(dev), rounding_mode=mode)
+                assert got.dtype == want.dtype, (got.dtype, want.dtype)
+                assert_each(got, want)
+            elif kind == "cmp_scalar":
+                dt = rng.choice(FLOATS + [torch.int32]); op = rng.choice(["eq", "ne", "lt", "le", "gt", "ge"]); sc = rng.choice([0, 1, -2, 0.5])
+                desc += f" {op} {dt} scalar={sc}"
+                a = torch.randint(-3, 4, (5, 40), generator=g).to(dt)
+                assert_exact(getattr(ops, op)(a.to(dev), sc), getattr(torch, op)(a, sc))
+            elif kind == "masked_fill_tensor":
+                dt = rng.choice(FLOATS + [torch.int64]); shape = (rng.choice([1, 6]), rng.choice([1, 33]))
+                desc += f" {dt} {shape} value tensor (cpu / device), in place"
+                x = (torch.randn(shape, generator=g) * 5).to(dt); m = torch.rand(shape, generator=g) > 0.5
+                val = torch.tensor(3, dtype=dt)
+                want = x.masked_fill(m, val)
+                dx = x.to(dev); ops.masked_fill_(dx, m.to(dev), val if rng.random() < 0.5 else val.to(dev))
+                assert_exact(dx, want)
+            elif kind == "fill":
+                dt = rng.choice(FLOATS + [torch.int32, torch.int64, torch.bool, torch.uint8]); shape = rng.choice([(), (1,), (1000,), (3, 4, 5)])
+                v = rng.choice([0, 1, 7]) if not dt.is_floating_point else rng.choice([0.0, -2.5, 1e4])
+                if dt == torch.bool: v = bool(v)
+                desc += f" {dt} {shape} value={v}"
+                x = torch.zeros(shape, dtype=dt, device=dev)
+                big = torch.zeros((6, 10), dtype=dt, device=dev)
+                ops.fill_(x, v); ops.fill_(big[::2, 1::3], v)
+                assert_exact(x, torch.full(shape, v, dtype=dt))
+                wb = torch.zeros((6, 10), dtype=dt); wb[::2, 1::3] = v
+                assert_exact(big, wb)
+            elif kind == "copy_bcast":
+                da, db = rng.choice(FLOATS + [torch.int32]), rng.choice(FLOATS + [torch.int64])
+                desc += f" {da}->{db} broadcast + transposed destination"
+                src = torch.randint(-20, 20, (1, 7), generator=g).to(da)
+                dst = torch.zeros(7, 5, dtype=db, device=dev).t()
+                ops.copy_(dst, src.to(dev).expand(5, 7)); assert_exact(dst.contiguous(), src.to(db).expand(5, 7).contiguous())
+            elif kind == "silu_mul":
+                dt = rng.choice(FLOATS); shape = rng.choice([(1, 8), (33, 1000), (4, 3, 64)])
+                desc += f" {dt} {shape}"
+                a, b = torch.randn(shape, generator=g).to(dt), torch.randn(shape, generator=g).to(dt)
+                want = (torch.nn.functional.silu(a.float()) * b.float()).to(dt)
+                assert_close(ops.silu_mul(a.to(dev), b.to(dev)), want)
+            elif kind == "sub_scalar":
+                dt = rng.choice(FLOATS + [torch.int64]); sc, al = rng.choice([1, 2.5, -3]), rng.choice([1, 2])
+                if not dt.is_floating_point: sc = int(sc)
+                desc += f" {dt} scalar={sc} alpha={al}"
+                a = torch.randint(-9, 9, (4, 9), generator=g).to(dt)
+                want = torch.sub(a, sc, alpha=al); got = ops.sub(a.to(dev), sc, alpha=al)
+                assert got.dtype == want.dtype; assert_each(got, want)
+            elif kind == "linear_out_strided3d":
+                dt = rng.choice(FLOATS); b0, s0, k, nn = rng.choice([1, 3]), rng.choice([1, 40]), rng.choice([64, 200]), rng.choice([8, 136])
+                desc += f" {dt} [{b0},{s0},{k}] -> {nn} into a strided 3-D destination"
+                x = torch.randn(b0, s0, k, generator=g).to(dt); wt = (torch.randn(nn, k, generator=g) * 0.1).to(dt)
+                big = torch.zeros(b0, s0, nn + 8, dtype=dt, device=dev)
+                ops.linear(x.to(dev), wt.to(dev), out=big[..., :nn])
+                want = torch.nn.functional.linear(x.float(), wt.float())
+                (assert_fp32 if dt == torch.float32 else assert_half)(big[..., :nn], want); assert float(big[..., nn:].abs().sum()) == 0
+            elif kind == "where_scalar":
+                dt = rng.choice(FLOATS + [torch.int64]); shape = (rng.choice([1, 5]), rng.choice([1, 40]))
+                desc += f" {dt} {shape}"
+                c = torch.rand(shape, generator=g) > 0.5; a = torch.randint(-5, 5, shape, generator=g).to(dt)
+                assert_exact(ops.where(c.to(dev), a.to(dev), 0), torch.where(c, a, torch.zeros((), dtype=dt)))
+                assert_exact(ops.where(c.to(dev), 1, a.to(dev)), torch.where(c, torch.ones((), dtype=dt), a))
+            else:
+                dt = rng.choice(FLOATS + [torch.int32]); 
+                desc += f" {dt} add_/mul_ on a hollow view"
+                base = torch.randint(-9, 9, (8, 12), generator=g).to(dt); other = torch.randint(-4, 4, (4, 4), generator=g).to(dt)
+                want = base.clone(); want[::2, 1:9:2] += 2 * other; want[::2, 1:9:2] *= other
+                db = base.to(dev); ops.add_(db[::2, 1:9:2], other.to(dev), alpha=2); ops.mul_(db[::2, 1:9:2], other.to(dev))
+                assert_each(db, want)
+        except AssertionError as e:
+            failed.append(desc + ": " + str(e)[:300])
+        except (RuntimeError, TypeError) as e:
+            failed.append(desc + ": refused: " + type(e).__name__ + " " + str(e)[:300])
+    _report(failed, n)
