@@ -1223,7 +1223,9 @@ __global__ __launch_bounds__(NTW * 4 * 64) void gemmSkinnyWideKernel(SkinnyArgs 
 //     columns at the same time the requests fall on a fraction of the memory channels (measured at 16 rows, cold:
 //     20.0 us with a common start, 18.5 with this one, 26 when neighbours start 8 stages apart);
 //   * more stages in flight are slower, here as in the other streaming kernels (weights 5 or 7 stages ahead instead
-//     of 3: 16.9 -> 18.8 and 18.0 us at one row), and so is leaving the copies to four extra waves that do nothing else.
+//     of 3: 16.9 -> 18.8 and 18.0 us at one row; at 64 rows rings of 5 + 5, 6 + 3, 6 + 4, 5 + 3 and 5 + 4 stages all read
+//     23.4-23.6 us against 23.1 with 4 + 4, and two activation stages 31.8), and so is leaving the copies to four extra
+//     waves that do nothing else.
 //     What bounds 64 rows is the bytes a CU takes in: every workgroup reads all the activations (from L2), as many
 //     bytes again as its share of the weights. Splitting K over grid.y (each workgroup then takes in half or a quarter
 //     of the activations) loses more to the fp32 slices and their reduction pass: 23.5 -> 26.1 us two ways, 35.8 four ways.
