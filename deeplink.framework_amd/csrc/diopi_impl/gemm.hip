@@ -1225,7 +1225,8 @@ __global__ __launch_bounds__(NTW * 4 * 64) void gemmSkinnyWideKernel(SkinnyArgs 
 //   * more stages in flight are slower, here as in the other streaming kernels (weights 5 or 7 stages ahead instead
 //     of 3: 16.9 -> 18.8 and 18.0 us at one row; at 64 rows rings of 5 + 5, 6 + 3, 6 + 4, 5 + 3 and 5 + 4 stages all read
 //     23.4-23.6 us against 23.1 with 4 + 4, and two activation stages 31.8), and so is leaving the copies to four extra
-//     waves that do nothing else.
+//     waves that do nothing else, or to eight of sixteen (a workgroup of 1024 with the roles apart: 22.5 -> 23.8 us at 64
+//     rows, 15.8 -> 16.9 at one).
 //     What bounds 64 rows is the bytes a CU takes in: every workgroup reads all the activations (from L2), as many
 //     bytes again as its share of the weights. Splitting K over grid.y (each workgroup then takes in half or a quarter
 //     of the activations) loses more to the fp32 slices and their reduction pass: 23.5 -> 26.1 us two ways, 35.8 four ways.
