@@ -7,6 +7,9 @@
 //     workgroups. This is the HBM-bound path the workloads hit; it is fastest with the fewest
 //     loads in flight per lane (add on [8192,4096] bf16: 29.5 us with one vector per lane and
 //     128 threads, 31.2 with two, 31.9 with four, 33.6 with eight).
+//   * rows-of-8 path - floating operands whose dtypes may differ, two dims after merging, every operand either
+//     dense along the row or broadcast along it (and free to be broadcast across rows): bias rows, per-row
+//     scales, mixed-precision adds, copies with a cast. A lane takes 8 consecutive columns of one row.
 //   * generic path - any strides (including broadcast stride 0), any rank <= 8, mixed
 //     dtypes, integer tensors; one element per lane with run-time dtype load/store.
 // Semantics follow the reference's CPU path: out = self + alpha*other with type promotion
@@ -294,6 +297,112 @@ static void coalesceDims(StridedArgs* s) {
   s->ndim = w;
 }
 
+// ------------------------------------------------------------ rows of 8
+struct Rows8Operand {
+  const void* p;      // nullptr: the op does not take this operand
+  int dtype;          // bfloat16, float16 or float32
+  int inner;          // 1: dense along the row, 0: one value per row
+  int64_t rowStride;  // elements; 0: the same row for every output row
+};
+
+__device__ __forceinline__ void rows8Load(const Rows8Operand& o, int64_t r, int64_t c, float (&f)[8]) {
+  if (o.p == nullptr) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f[j] = 0.f;
+    return;
+  }
+  const int64_t off = r * o.rowStride + (o.inner ? c : 0);
+  if (!o.inner) {
+    const float v = loadAs<float>(o.p, off, o.dtype);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f[j] = v;
+  } else if (o.dtype == diopi_dtype_float32) {
+    const f32x4 lo = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(o.p) + off);
+    const f32x4 hi = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(o.p) + off + 4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) f[j] = lo[j], f[4 + j] = hi[j];
+  } else if (o.dtype == diopi_dtype_bfloat16) {
+    const bf16x8 v = *reinterpret_cast<const bf16x8*>(reinterpret_cast<const bf16_t*>(o.p) + off);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f[j] = static_cast<float>(v[j]);
+  } else {
+    const f16x8 v = *reinterpret_cast<const f16x8*>(reinterpret_cast<const half_t*>(o.p) + off);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f[j] = static_cast<float>(v[j]);
+  }
+}
+
+template <int OP>
+__global__ __launch_bounds__(256) void ewRows8Kernel(void* out, int dto, int64_t outRowStride, Rows8Operand a, Rows8Operand b,
+                                                     int64_t nvec, int rowVecs, float p0) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= nvec) return;
+  const int64_t r = i / rowVecs, c = (i - r * rowVecs) * 8;
+  float fa[8], fb[8], fo[8];
+  rows8Load(a, r, c, fa);
+  rows8Load(b, r, c, fb);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) fo[j] = ewApply<OP, float>(fa[j], fb[j], p0);
+  const int64_t off = r * outRowStride + c;
+  if (dto == diopi_dtype_float32) {
+    float* o = reinterpret_cast<float*>(out) + off;
+    *reinterpret_cast<f32x4*>(o) = f32x4{fo[0], fo[1], fo[2], fo[3]};
+    *reinterpret_cast<f32x4*>(o + 4) = f32x4{fo[4], fo[5], fo[6], fo[7]};
+  } else if (dto == diopi_dtype_bfloat16) {
+    bf16x8 v;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = static_cast<bf16_t>(fo[j]);
+    *reinterpret_cast<bf16x8*>(reinterpret_cast<bf16_t*>(out) + off) = v;
+  } else {
+    f16x8 v;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = static_cast<half_t>(fo[j]);
+    *reinterpret_cast<f16x8*>(reinterpret_cast<half_t*>(out) + off) = v;
+  }
+}
+
+static bool rows8Dtype(diopiDtype_t d) {
+  return d == diopi_dtype_bfloat16 || d == diopi_dtype_float16 || d == diopi_dtype_float32;
+}
+
+// Launches ewRows8Kernel when the (merged) problem has its form; *launched says whether it did.
+template <int OP>
+diopiError_t tryRows8(hipStream_t stream, const TensorView& out, const TensorView* a, const TensorView* b, double p0,
+                      bool* launched) {
+  *launched = false;
+  if (!rows8Dtype(out.dtype) || (a && !rows8Dtype(a->dtype)) || (b && !rows8Dtype(b->dtype))) return diopiSuccess;
+  StridedArgs s;
+  s.ndim = out.ndim;
+  for (int d = 0; d < kMaxDims; ++d) s.shape[d] = 1, s.so[d] = s.sa[d] = s.sb[d] = 0;
+  for (int d = 0; d < out.ndim; ++d) {
+    s.shape[d] = out.shape[d];
+    s.so[d] = out.shape[d] == 1 ? 0 : out.stride[d];
+  }
+  if (a) AMD_TRY(broadcastStrides(out, *a, s.sa, "input"));
+  if (b) AMD_TRY(broadcastStrides(out, *b, s.sb, "other"));
+  coalesceDims(&s);
+  if (s.ndim > 2) return diopiSuccess;
+  const int64_t rows = s.ndim == 2 ? s.shape[0] : 1, cols = s.shape[s.ndim - 1];
+  const int last = s.ndim - 1;
+  if (cols % 8 != 0 || cols / 8 >= ((int64_t)1 << 31) || s.so[last] != 1) return diopiSuccess;
+  auto rowStrideOf = [&](const int64_t* st) { return s.ndim == 2 ? st[0] : 0; };
+  auto operandOk = [&](const TensorView* t, const int64_t* st) {
+    if (!t) return true;
+    if (st[last] == 0) return true;                      // one value per row: any address
+    return st[last] == 1 && t->aligned16() && rowStrideOf(st) % 8 == 0;
+  };
+  if (!out.aligned16() || rowStrideOf(s.so) % 8 != 0 || !operandOk(a, s.sa) || !operandOk(b, s.sb)) return diopiSuccess;
+  Rows8Operand oa{a ? a->data : nullptr, a ? (int)a->dtype : 0, a ? (int)s.sa[last] : 0, a ? rowStrideOf(s.sa) : 0};
+  Rows8Operand ob{b ? b->data : nullptr, b ? (int)b->dtype : 0, b ? (int)s.sb[last] : 0, b ? rowStrideOf(s.sb) : 0};
+  const int64_t nvec = rows * (cols / 8), blocks = ceilDiv(nvec, 256);
+  AMD_CHECK(blocks <= 0x7fffffff, "elementwise: %ld vectors exceed the grid limit", (long)nvec);
+  hipLaunchKernelGGL((ewRows8Kernel<OP>), dim3((unsigned)blocks), dim3(256), 0, stream, out.data, (int)out.dtype,
+                     rowStrideOf(s.so), oa, ob, nvec, (int)(cols / 8), (float)p0);
+  AMD_LAUNCH_CHECK();
+  *launched = true;
+  return diopiSuccess;
+}
+
 template <int OP>
 diopiError_t launchGeneric(hipStream_t stream, const TensorView& out, const TensorView* a, const TensorView* b,
                            double p0f, int64_t p0i, bool p0IsFloat) {
@@ -426,6 +535,9 @@ diopiError_t runEw(diopiContextHandle_t ctx, diopiTensorHandle_t outH, diopiCons
       default: return launchVecRows<OP, float>(stream, out.data, da, db, rows, cols, so, sa, sb, p);
     }
   }
+  bool launched = false;
+  AMD_TRY(tryRows8<OP>(stream, out, pa, pb, p0IsFloat ? p0f : (double)p0i, &launched));
+  if (launched) return diopiSuccess;
   return launchGeneric<OP>(stream, out, pa, pb, p0f, p0i, p0IsFloat);
 }
 
@@ -445,6 +557,9 @@ diopiError_t stridedCopy(hipStream_t stream, const TensorView& src, const Tensor
       default: return launchVecRows<kCopy, float>(stream, dst.data, src.data, nullptr, rows, cols, so, sa, sb, 0.0);
     }
   }
+  bool launched = false;
+  AMD_TRY(tryRows8<kCopy>(stream, dst, &src, nullptr, 0.0, &launched));
+  if (launched) return diopiSuccess;
   return launchGeneric<kCopy>(stream, dst, &src, nullptr, 0.0, 0, true);
 }
 
