@@ -1816,6 +1816,15 @@ static diopiError_t launchTranspose(hipStream_t stream, void* dst, const void* s
   return diopiSuccess;
 }
 
+diopiError_t transposeCopy(hipStream_t stream, void* dst, const void* src, int itemsize, int64_t batch, int64_t rows,
+                           int64_t cols, int64_t sRow, int64_t sCol, int64_t sBatch) {
+  AMD_CHECK(itemsize == 2 || itemsize == 4, "transpose: %d-byte elements are not supported", itemsize);
+  AMD_CHECK(batch <= 65535 && ceilDiv(rows, 64) <= 65535, "transpose: %ld batches x %ld rows exceed the grid limits", (long)batch,
+            (long)rows);
+  if (itemsize == 2) return launchTranspose<uint16_t>(stream, dst, src, batch, rows, cols, sRow, sCol, sBatch);
+  return launchTranspose<uint32_t>(stream, dst, src, batch, rows, cols, sRow, sCol, sBatch);
+}
+
 diopiError_t runGemm(diopiContextHandle_t ctx, hipStream_t stream, GemmProblem p) {
   if (p.batch == 0 || p.M == 0 || p.N == 0) return diopiSuccess;
   AMD_CHECK(p.batch <= 65535, "gemm: batch %ld exceeds the grid limit", (long)p.batch);

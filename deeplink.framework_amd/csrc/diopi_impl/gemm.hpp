@@ -31,4 +31,9 @@ diopiError_t runGemm(diopiContextHandle_t ctx, hipStream_t stream, GemmProblem p
 diopiError_t runRotary(diopiContextHandle_t ctx, hipStream_t stream, const TensorView& out, const TensorView& x,
                        const TensorView& cosT, const TensorView& sinT, bool conj, bool interleaved);
 
+// dst[b, c, r] = src[b, r, c] for 2-byte or 4-byte elements (64 x 64 tiles through LDS): src is [rows, cols] with the
+// element strides given, dst dense [cols, rows] per batch.
+diopiError_t transposeCopy(hipStream_t stream, void* dst, const void* src, int itemsize, int64_t batch, int64_t rows,
+                           int64_t cols, int64_t sRow, int64_t sCol, int64_t sBatch);
+
 }  // namespace amd

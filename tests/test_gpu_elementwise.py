@@ -179,6 +179,29 @@ def test_softmax(ops, dev, dtype):
         assert_close(ops.softmax(x.to(dev), dim), oracle.softmax(x, dim))
     xt = torch.randn(96, 80, generator=g(19)).to(dtype)
     assert_close(ops.softmax(xt.to(dev).t(), -1), oracle.softmax(xt.t(), -1))   # non-contiguous input
+    # long columns (the tiled form): ragged column blocks, masked entries, a fully masked column (NaN on both sides)
+    for shape, dim in [((4100, 70), 0), ((3, 1000, 33), 1), ((128, 16), 0)]:
+        x = (torch.randn(shape, generator=g(118)) * 4).to(dtype)
+        x[torch.rand(shape, generator=g(119)) < 0.1] = float("-inf")
+        x.select(dim, 0).fill_(1.0)                  # at least one finite entry everywhere ...
+        x.movedim(dim, -1).reshape(-1, shape[dim])[5].fill_(float("-inf"))   # ... except in one column
+        # (4 100 terms: stock ATen's fp32 result is itself 1.1e-5 from the float64 one here, the device's 3e-7, so the
+        # fp32 case is held against the float64 computation)
+        got, want = ops.softmax(x.to(dev), dim).cpu(), oracle.softmax(x.double() if dtype == torch.float32 else x, dim).to(dtype)
+        assert torch.equal(got.isnan(), want.isnan())
+        assert_close(got.nan_to_num(0.0), want.nan_to_num(0.0))
+
+
+def test_copy_from_a_transposed_view(ops, dev):
+    """Dense destinations filled from transposed sources go through 64 x 64 tiles: ragged edges, a batch dim, 2- and
+    4-byte elements, and a source whose rows are further apart than their length."""
+    for shape, dt in [((130, 70), torch.bfloat16), ((64, 64), torch.float32), ((3, 100, 257), torch.float16),
+                      ((1000, 33), torch.int32)]:
+        src = (torch.randn(*shape[:-2], shape[-1], shape[-2] + 8, generator=g(120)) * 50).to(dt)
+        view = src[..., : shape[-2]].transpose(-1, -2)          # [.., rows, cols], unit stride along rows
+        dst = torch.zeros(shape, dtype=dt, device=dev)
+        ops.copy_(dst, src.to(dev)[..., : shape[-2]].transpose(-1, -2))
+        assert_exact(dst, view.contiguous())
 
 
 def test_softmax_rows_sum_to_one_at_full_size(ops, dev):
