@@ -235,14 +235,30 @@ template <int OP, typename C>
 __global__ __launch_bounds__(256) void ewGenericKernel(void* out, const void* a, const void* b, int dto, int dta,
                                                        int dtb, StridedArgs s, int64_t n, C p0) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
-    int64_t rem = i, oo = 0, oa = 0, ob = 0;
-    for (int d = s.ndim - 1; d >= 0; --d) {
-      int64_t q = rem / s.shape[d];
-      int64_t r = rem - q * s.shape[d];
-      rem = q;
-      oo += r * s.so[d];
-      oa += r * s.sa[d];
-      ob += r * s.sb[d];
+    int64_t oo = 0, oa = 0, ob = 0;
+    if (s.ndim == 1) {  // everything merged into one run: no division
+      oo = i * s.so[0], oa = i * s.sa[0], ob = i * s.sb[0];
+    } else if (i < ((int64_t)1 << 31)) {  // 32-bit divisions: every quotient and remainder of such an index fits
+      unsigned rem = (unsigned)i;
+      for (int d = s.ndim - 1; d >= 0 && rem != 0; --d) {
+        const unsigned extent = s.shape[d] >= ((int64_t)1 << 31) ? 0x80000000u : (unsigned)s.shape[d];
+        const unsigned q = rem / extent;
+        const int64_t r = rem - q * extent;
+        rem = q;
+        oo += r * s.so[d];
+        oa += r * s.sa[d];
+        ob += r * s.sb[d];
+      }
+    } else {
+      int64_t rem = i;
+      for (int d = s.ndim - 1; d >= 0; --d) {
+        int64_t q = rem / s.shape[d];
+        int64_t r = rem - q * s.shape[d];
+        rem = q;
+        oo += r * s.so[d];
+        oa += r * s.sa[d];
+        ob += r * s.sb[d];
+      }
     }
     C va = opHasA(OP) ? loadAs<C>(a, oa, dta) : C(0);
     C vb = opHasB(OP) ? loadAs<C>(b, ob, dtb) : C(0);
