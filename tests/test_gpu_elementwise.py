@@ -192,6 +192,34 @@ def test_softmax(ops, dev, dtype):
         assert_close(got.nan_to_num(0.0), want.nan_to_num(0.0))
 
 
+def test_broadcast_rows_groups_and_mixed_dtypes(ops, dev):
+    """The 8-columns-per-lane path: a bias row, a per-row scale, a table shared by every head ([b, 1, s, d] against
+    [b, h, s, d]), operands of different floating dtypes, an in-place form, and a column slice as destination."""
+    gq = g(130)
+    x = torch.randn(2, 6, 40, 64, generator=gq).bfloat16()
+    row, colv = torch.randn(64, generator=gq).bfloat16(), torch.randn(2, 6, 40, 1, generator=gq).bfloat16()
+    tab = torch.randn(2, 1, 40, 64, generator=gq).bfloat16()
+    f32 = torch.randn(2, 6, 40, 64, generator=gq)
+    assert_each(ops.add(x.to(dev), row.to(dev), alpha=2), torch.add(x, row, alpha=2))
+    assert_each(ops.mul(x.to(dev), colv.to(dev)), x * colv)
+    assert_each(ops.mul(x.to(dev), tab.to(dev)), x * tab)
+    assert_each(ops.sub(tab.to(dev), x.to(dev)), tab - x)                   # the broadcast operand first
+    mixed = ops.add(x.to(dev), f32.to(dev))
+    assert mixed.dtype == torch.float32
+    assert_each(mixed, x + f32)
+    assert_each(ops.div(f32.to(dev), x.half().to(dev)), f32 / x.half())
+    inp = f32.clone().to(dev)
+    ops.add_(inp, tab.to(dev))
+    assert_each(inp, f32 + tab)
+    wide = torch.zeros(2, 6, 40, 128, device=dev)
+    ops.mul(f32.to(dev), row.to(dev), out=wide[..., 64:])
+    assert_each(wide[..., 64:], f32 * row)
+    assert float(wide[..., :64].abs().sum()) == 0.0
+    half = torch.empty(2, 6, 40, 64, dtype=torch.float16, device=dev)
+    ops.copy_(half, tab.to(dev).expand(2, 6, 40, 64))                        # broadcast copy with a cast
+    assert_exact(half, tab.expand(2, 6, 40, 64).half())
+
+
 def test_copy_from_a_transposed_view(ops, dev):
     """Dense destinations filled from transposed sources go through 64 x 64 tiles: ragged edges, a batch dim, 2- and
     4-byte elements, and a source whose rows are further apart than their length."""
