@@ -305,7 +305,21 @@ __global__ __launch_bounds__(256) void rowMeanKernel(T* out, const T* in, int64_
   if (row >= rows) return;
   const T* src = in + row * cols;
   float s = 0.f;
-  for (int64_t c = lane; c < cols; c += 64) s += static_cast<float>(src[c]);
+  // 16-byte loads where the row allows (a lane reading one 2-byte element per step keeps a wave at 128 bytes per load:
+  // [8192, 4096] bf16 took 22.8 us, as long as the fp32 tensor of twice the bytes)
+  using V = typename Vec16<T>::type;
+  constexpr int N = Vec16<T>::N;
+  int64_t done = 0;
+  if ((reinterpret_cast<uintptr_t>(src) & 15) == 0) {
+    const int64_t nvec = cols / N;
+    for (int64_t v = lane; v < nvec; v += 64) {
+      const V x = reinterpret_cast<const V*>(src)[v];
+#pragma unroll
+      for (int j = 0; j < N; ++j) s += static_cast<float>(x[j]);
+    }
+    done = nvec * N;
+  }
+  for (int64_t c = done + lane; c < cols; c += 64) s += static_cast<float>(src[c]);
   s = waveSum(s);
   if (lane == 0) out[row] = static_cast<T>(s / (float)cols);
 }

@@ -109,6 +109,36 @@ __global__ __launch_bounds__(kSelThreads) void selectKernel(void* out, const voi
 
 enum CmpOp : int { kEq = 0, kNe, kLt, kLe, kGt, kGe };
 
+__device__ __forceinline__ bool compareOne(float x, float y, int cmp) {
+  switch (cmp) {
+    case kEq: return x == y;
+    case kNe: return x != y;
+    case kLt: return x < y;
+    case kLe: return x <= y;
+    case kGt: return x > y;
+    default: return x >= y;
+  }
+}
+
+// out = a CMP b on dense operands of one floating dtype (b may be the scalar sb, already rounded to that dtype) into a
+// dense 1-byte output: 8 elements per lane.
+template <typename T>
+__global__ __launch_bounds__(kSelThreads) void compareVecKernel(uint8_t* __restrict__ out, const T* __restrict__ a,
+                                                                const T* __restrict__ b, int64_t nvec, int cmp, float sb) {
+  typedef T T8 __attribute__((ext_vector_type(8)));
+  typedef uint8_t C8 __attribute__((ext_vector_type(8)));
+  const int64_t i = (int64_t)blockIdx.x * kSelThreads + threadIdx.x;
+  if (i >= nvec) return;
+  const T8 va = reinterpret_cast<const T8*>(a)[i];
+  T8 vb;
+  if (b != nullptr) vb = reinterpret_cast<const T8*>(b)[i];
+  C8 r;
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+    r[j] = compareOne(static_cast<float>(va[j]), b != nullptr ? static_cast<float>(vb[j]) : sb, cmp) ? 1 : 0;
+  reinterpret_cast<C8*>(out)[i] = r;
+}
+
 // out = a CMP b; `b` is the scalar `sb` when bScalar.
 template <typename C>
 __global__ __launch_bounds__(kSelThreads) void compareKernel(void* out, const void* a, const void* b, int dto, int dta,
@@ -146,6 +176,31 @@ __global__ __launch_bounds__(kSelThreads) void triangleKernel(void* out, const v
   }
 }
 
+// tril / triu on dense [..., rows, cols] of one 2-byte or 4-byte dtype, cols a multiple of 8: 8 elements per lane as bits.
+template <typename E>
+__global__ __launch_bounds__(kSelThreads) void triangleVecKernel(E* __restrict__ out, const E* __restrict__ x, int64_t nvec,
+                                                                 int rowVecs, int64_t rows, int64_t diag, bool lower) {
+  typedef E E8 __attribute__((ext_vector_type(8)));
+  const int64_t i = (int64_t)blockIdx.x * kSelThreads + threadIdx.x;
+  if (i >= nvec) return;
+  const int64_t rowAll = i / rowVecs, c0 = (i - rowAll * rowVecs) * 8, r = rowAll % rows;
+  // the whole piece on the zero side: no load
+  const bool allZero = lower ? (c0 - r > diag) : (c0 + 7 - r < diag);
+  E8 v;
+  if (allZero) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = 0;
+  } else {
+    v = reinterpret_cast<const E8*>(x)[i];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int64_t d = c0 + j - r;
+      if (!(lower ? d <= diag : d >= diag)) v[j] = 0;
+    }
+  }
+  reinterpret_cast<E8*>(out)[i] = v;
+}
+
 template <typename C>
 __global__ __launch_bounds__(kSelThreads) void arangeKernel(void* out, int dto, int64_t stride, int64_t n, C start,
                                                             C step) {
@@ -167,6 +222,21 @@ __global__ __launch_bounds__(kSelThreads) void gatherKernel(void* out, const voi
     if (j >= 0 && j < dimSize) v = loadAs<C>(src, o.o[1] + j * dimStride, dts);
     storeAs<C>(out, o.o[0], dto, v);
   }
+}
+
+// index_select of dense blocks: out[o, i, :] = src[o, index[i], :] with `inner` contiguous 16-byte vectors per block
+// (an embedding lookup is outer = 1, inner = the hidden size). One workgroup per output block; an index outside the
+// source writes zeros, as the one-element kernel does.
+template <typename IDX>
+__global__ __launch_bounds__(256) void selectRowsKernel(u32x4* __restrict__ out, const u32x4* __restrict__ src,
+                                                        const IDX* __restrict__ index, int64_t indexStride, int64_t nIndex,
+                                                        int64_t dimSize, int64_t innerVecs) {
+  const int64_t blk = blockIdx.x, o = blk / nIndex, i = blk - o * nIndex;
+  const int64_t j = static_cast<int64_t>(index[i * indexStride]);
+  const bool ok = j >= 0 && j < dimSize;
+  const u32x4* s = src + (o * dimSize + (ok ? j : 0)) * innerVecs;
+  u32x4* d = out + blk * innerVecs;
+  for (int64_t v = threadIdx.x; v < innerVecs; v += 256) d[v] = ok ? s[v] : u32x4{0, 0, 0, 0};
 }
 
 // --------------------------------------------------------------------- host
@@ -336,10 +406,45 @@ static diopiError_t runCompare(diopiContextHandle_t ctx, diopiTensorHandle_t out
   // compare as floating point as soon as either side is; integers compare exactly as int64
   const bool asFloat = isFloatDtype(a.dtype) || (bScalar ? scalarIsFloat(bScalar) : isFloatDtype(b.dtype));
   const int dtb = bScalar ? (int)a.dtype : (int)b.dtype;
+  // A scalar compared with a floating tensor is first rounded to the tensor's dtype, as ATen's type promotion has it
+  // (a bfloat16 tensor holding bfloat16(0.1) is equal to the scalar 0.1).
+  double sbFloat = scalarToDouble(bScalar, 0.0);
+  if (bScalar) {
+    if (a.dtype == diopi_dtype_bfloat16) sbFloat = static_cast<float>(static_cast<bf16_t>(static_cast<float>(sbFloat)));
+    else if (a.dtype == diopi_dtype_float16) sbFloat = static_cast<float>(static_cast<half_t>(static_cast<float>(sbFloat)));
+    else if (a.dtype == diopi_dtype_float32) sbFloat = static_cast<float>(sbFloat);
+  }
+  // dense, one floating dtype on the input side, a 1-byte output: 8 elements per lane
+  {
+    auto dense = [&](const TensorView& t) {
+      if (!t.isContiguous() || t.ndim != out.ndim) return false;
+      for (int d = 0; d < out.ndim; ++d)
+        if (t.shape[d] != out.shape[d]) return false;
+      return true;
+    };
+    const bool vecType = a.dtype == diopi_dtype_bfloat16 || a.dtype == diopi_dtype_float16 || a.dtype == diopi_dtype_float32;
+    if (vecType && out.itemsize == 1 && out.numel % 8 == 0 && out.isContiguous() && (reinterpret_cast<uintptr_t>(out.data) & 7) == 0 &&
+        dense(a) && a.aligned16() && (bScalar || (dense(b) && b.dtype == a.dtype && b.aligned16()))) {
+      const int64_t nvec = out.numel / 8, blocks = ceilDiv(nvec, kSelThreads);
+      AMD_CHECK(blocks <= 0x7fffffff, "%s: %ld elements exceed the grid limit", name, (long)out.numel);
+      const dim3 grid((unsigned)blocks), block(kSelThreads);
+      if (a.dtype == diopi_dtype_bfloat16)
+        hipLaunchKernelGGL((compareVecKernel<bf16_t>), grid, block, 0, stream, out.ptr<uint8_t>(), a.ptr<bf16_t>(),
+                           bScalar ? nullptr : b.ptr<bf16_t>(), nvec, cmp, (float)sbFloat);
+      else if (a.dtype == diopi_dtype_float16)
+        hipLaunchKernelGGL((compareVecKernel<half_t>), grid, block, 0, stream, out.ptr<uint8_t>(), a.ptr<half_t>(),
+                           bScalar ? nullptr : b.ptr<half_t>(), nvec, cmp, (float)sbFloat);
+      else
+        hipLaunchKernelGGL((compareVecKernel<float>), grid, block, 0, stream, out.ptr<uint8_t>(), a.ptr<float>(),
+                           bScalar ? nullptr : b.ptr<float>(), nvec, cmp, (float)sbFloat);
+      AMD_LAUNCH_CHECK();
+      return diopiSuccess;
+    }
+  }
   if (asFloat) {
     hipLaunchKernelGGL((compareKernel<double>), dim3(gridFor(out.numel)), dim3(kSelThreads), 0, stream, out.data,
                        a.data, bScalar ? nullptr : b.data, (int)out.dtype, (int)a.dtype, dtb, s, out.numel, cmp,
-                       scalarToDouble(bScalar, 0.0), bScalar != nullptr);
+                       sbFloat, bScalar != nullptr);
   } else {
     hipLaunchKernelGGL((compareKernel<int64_t>), dim3(gridFor(out.numel)), dim3(kSelThreads), 0, stream, out.data,
                        a.data, bScalar ? nullptr : b.data, (int)out.dtype, (int)a.dtype, dtb, s, out.numel, cmp,
@@ -368,6 +473,22 @@ static diopiError_t runTriangle(diopiContextHandle_t ctx, diopiTensorHandle_t ou
   clearStrided(&s, out);
   for (int d = 0; d < x.ndim; ++d) s.st[1][d] = x.shape[d] == 1 ? 0 : x.stride[d];
   coalesce(&s, 2);
+  {
+    const int64_t cols = out.shape[out.ndim - 1], rows = out.shape[out.ndim - 2];
+    if (x.dtype == out.dtype && (out.itemsize == 2 || out.itemsize == 4) && out.isContiguous() && x.isContiguous() && out.aligned16() &&
+        x.aligned16() && cols % 8 == 0 && cols / 8 < ((int64_t)1 << 31)) {
+      const int64_t nvec = out.numel / 8, blocks = ceilDiv(nvec, kSelThreads);
+      AMD_CHECK(blocks <= 0x7fffffff, "%s: %ld elements exceed the grid limit", name, (long)out.numel);
+      if (out.itemsize == 2)
+        hipLaunchKernelGGL((triangleVecKernel<uint16_t>), dim3((unsigned)blocks), dim3(kSelThreads), 0, stream, out.ptr<uint16_t>(),
+                           x.ptr<uint16_t>(), nvec, (int)(cols / 8), rows, diagonal, lower);
+      else
+        hipLaunchKernelGGL((triangleVecKernel<uint32_t>), dim3((unsigned)blocks), dim3(kSelThreads), 0, stream, out.ptr<uint32_t>(),
+                           x.ptr<uint32_t>(), nvec, (int)(cols / 8), rows, diagonal, lower);
+      AMD_LAUNCH_CHECK();
+      return diopiSuccess;
+    }
+  }
   if (isFloatDtype(out.dtype))
     hipLaunchKernelGGL((triangleKernel<double>), dim3(gridFor(out.numel)), dim3(kSelThreads), 0, stream, out.data,
                        x.data, (int)out.dtype, (int)x.dtype, s, out.numel, diagonal, lower);
@@ -424,6 +545,26 @@ static diopiError_t runGather(diopiContextHandle_t ctx, diopiTensorHandle_t outH
   }
   if (out.numel == 0) return diopiSuccess;
   const int64_t dimStride = s1.stride[dim], dimSize = s1.shape[dim];
+  // index_select on dense tensors of one dtype whose blocks behind `dim` are whole 16-byte vectors: block copies
+  // ([32000, 4096] bf16, 8192 indices: 122 us one element per lane)
+  if (select && src.dtype == out.dtype && src.isContiguous() && out.isContiguous() && src.aligned16() && out.aligned16() &&
+      src.ndim == out.ndim) {
+    int64_t outer = 1, inner = 1;
+    for (int d = 0; d < (int)dim; ++d) outer *= s1.shape[d];
+    for (int d = (int)dim + 1; d < rank; ++d) inner *= s1.shape[d];
+    const int64_t blockBytes = inner * src.itemsize, blocks = outer * index.numel;
+    if (blockBytes % 16 == 0 && blockBytes >= 256 && blocks < ((int64_t)1 << 31)) {
+      const int64_t istr = index.ndim == 1 ? index.stride[0] : 0;
+      if (index.dtype == diopi_dtype_int64)
+        hipLaunchKernelGGL((selectRowsKernel<int64_t>), dim3((unsigned)blocks), dim3(256), 0, stream, out.ptr<u32x4>(),
+                           src.ptr<u32x4>(), index.ptr<int64_t>(), istr, index.numel, dimSize, blockBytes / 16);
+      else
+        hipLaunchKernelGGL((selectRowsKernel<int32_t>), dim3((unsigned)blocks), dim3(256), 0, stream, out.ptr<u32x4>(),
+                           src.ptr<u32x4>(), index.ptr<int32_t>(), istr, index.numel, dimSize, blockBytes / 16);
+      AMD_LAUNCH_CHECK();
+      return diopiSuccess;
+    }
+  }
   // no coalescing: `dim` has to stay a dim of its own for both operand tables
   if (isFloatDtype(out.dtype))
     hipLaunchKernelGGL((gatherKernel<double>), dim3(gridFor(out.numel)), dim3(kSelThreads), 0, stream, out.data,

@@ -170,3 +170,41 @@ def test_causal_mask_from_primitives_matches_fused_attention(ops, dev):
     assert_fp32(out, want)
     fused = ops.context_attention(q.to(dev), k.to(dev), v.to(dev), start.to(dev), lens.to(dev), S)
     assert_fp32(fused, want)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_comparison_with_a_scalar_uses_the_tensor_dtype(ops, dev, dtype):
+    """ATen rounds the scalar to the floating tensor's dtype before comparing: a tensor holding dtype(0.1) equals the
+    scalar 0.1 (which it does not in double precision). Dense operands in multiples of 8 take the 8-per-lane kernel,
+    the 13-element tail case the one-element kernel: both must agree with ATen."""
+    for n in (4096, 13):
+        x = torch.linspace(-1, 1, n).to(dtype)
+        x[::3] = torch.tensor(0.1).to(dtype)
+        y = x.clone()
+        y[::5] += 1
+        for name in ("eq", "ne", "lt", "le", "gt", "ge"):
+            assert_exact(getattr(ops, name)(x.to(dev), 0.1), getattr(torch, name)(x, 0.1))
+            assert_exact(getattr(ops, name)(x.to(dev), y.to(dev)), getattr(torch, name)(x, y))
+    ints = torch.arange(-4, 5, dtype=torch.int32)
+    assert_exact(ops.lt(ints.to(dev), 2.5), ints < 2.5)
+    assert_exact(ops.eq(ints.to(dev), 3), ints == 3)
+
+
+def test_index_select_blocks_and_triangles_vector_paths(ops, dev):
+    """index_select whose blocks behind `dim` are whole 16-byte vectors (embedding rows; a middle dim with an outer
+    one) and tril / triu with rows that are multiples of 8: the block-copy and 8-per-lane kernels, bit-exact."""
+    emb = torch.randn(300, 256, generator=g(60)).bfloat16()
+    idx = torch.randint(0, 300, (77,), generator=g(61))
+    assert_exact(ops.index_select(emb.to(dev), 0, idx.to(dev)), emb.index_select(0, idx))
+    assert_exact(ops.index_select(emb.to(dev), 0, idx.int().to(dev)), emb.index_select(0, idx))
+    x3 = torch.randn(5, 40, 128, generator=g(62))
+    i3 = torch.randint(0, 40, (9,), generator=g(63))
+    assert_exact(ops.index_select(x3.to(dev), 1, i3.to(dev)), x3.index_select(1, i3))
+    for dt in (torch.bfloat16, torch.float32, torch.int32):
+        m = (torch.randn(2, 3, 70, 72, generator=g(64)) * 9).to(dt)
+        for diag in (0, 1, -1, 9, -70, 100):
+            assert_exact(ops.tril(m.to(dev), diag), torch.tril(m, diag))
+            assert_exact(ops.triu(m.to(dev), diag), torch.triu(m, diag))
+        inp = m.clone().to(dev)
+        ops.triu_(inp, 1)
+        assert_exact(inp, torch.triu(m, 1))
