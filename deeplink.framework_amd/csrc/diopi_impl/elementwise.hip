@@ -7,7 +7,7 @@
 //     workgroups. This is the HBM-bound path the workloads hit; it is fastest with the fewest
 //     loads in flight per lane (add on [8192,4096] bf16: 29.5 us with one vector per lane and
 //     128 threads, 31.2 with two, 31.9 with four, 33.6 with eight).
-//   * rows-of-8 path - floating operands whose dtypes may differ, at most three dims after merging, every operand either
+//   * rows-of-8 path - floating operands whose dtypes may differ, at most four dims after merging, every operand either
 //     dense along the row or broadcast along it (and free to be broadcast across rows or groups of rows): bias rows,
 //     per-row scales, tables shared by all heads, mixed-precision adds, copies with a cast. A lane takes 8 consecutive columns of one row.
 //   * generic path - any strides (including broadcast stride 0), any rank <= 8, mixed
@@ -320,16 +320,17 @@ struct Rows8Operand {
   int dtype;          // bfloat16, float16 or float32
   int inner;          // 1: dense along the row, 0: one value per row
   int64_t rowStride;  // elements, between rows of one group; 0: the same row for every output row
-  int64_t groupStride;  // elements, between groups of rows (the outermost of three merged dims); 0: broadcast
+  int64_t groupStride;  // elements, between groups of rows; 0: broadcast
+  int64_t superStride;  // elements, between groups of groups (the outermost of four merged dims); 0: broadcast
 };
 
-__device__ __forceinline__ void rows8Load(const Rows8Operand& o, int64_t grp, int64_t r, int64_t c, float (&f)[8]) {
+__device__ __forceinline__ void rows8Load(const Rows8Operand& o, int64_t sup, int64_t grp, int64_t r, int64_t c, float (&f)[8]) {
   if (o.p == nullptr) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) f[j] = 0.f;
     return;
   }
-  const int64_t off = grp * o.groupStride + r * o.rowStride + (o.inner ? c : 0);
+  const int64_t off = sup * o.superStride + grp * o.groupStride + r * o.rowStride + (o.inner ? c : 0);
   if (!o.inner) {
     const float v = loadAs<float>(o.p, off, o.dtype);
 #pragma unroll
@@ -352,18 +353,20 @@ __device__ __forceinline__ void rows8Load(const Rows8Operand& o, int64_t grp, in
 
 template <int OP>
 __global__ __launch_bounds__(256) void ewRows8Kernel(void* out, int dto, int64_t outRowStride, int64_t outGroupStride,
-                                                     Rows8Operand a, Rows8Operand b, int64_t nvec, int rowVecs, int64_t rowsPerGroup,
-                                                     float p0) {
+                                                     int64_t outSuperStride, Rows8Operand a, Rows8Operand b, int64_t nvec, int rowVecs,
+                                                     unsigned rowsPerGroup, unsigned groupsPerSuper, float p0) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= nvec) return;
-  const int64_t row = i / rowVecs, c = (i - row * rowVecs) * 8;
-  const int64_t grp = row / rowsPerGroup, r = row - grp * rowsPerGroup;
+  const int64_t rowAll = i / rowVecs, c = (i - rowAll * rowVecs) * 8;
+  // the host keeps the row count below 2^31: 32-bit divisions
+  const unsigned row = (unsigned)rowAll, grpAll = row / rowsPerGroup, r = row - grpAll * rowsPerGroup;
+  const unsigned sup = grpAll / groupsPerSuper, grp = grpAll - sup * groupsPerSuper;
   float fa[8], fb[8], fo[8];
-  rows8Load(a, grp, r, c, fa);
-  rows8Load(b, grp, r, c, fb);
+  rows8Load(a, sup, grp, r, c, fa);
+  rows8Load(b, sup, grp, r, c, fb);
 #pragma unroll
   for (int j = 0; j < 8; ++j) fo[j] = ewApply<OP, float>(fa[j], fb[j], p0);
-  const int64_t off = grp * outGroupStride + r * outRowStride + c;
+  const int64_t off = sup * outSuperStride + grp * outGroupStride + r * outRowStride + c;
   if (dto == diopi_dtype_float32) {
     float* o = reinterpret_cast<float*>(out) + off;
     *reinterpret_cast<f32x4*>(o) = f32x4{fo[0], fo[1], fo[2], fo[3]};
@@ -401,28 +404,33 @@ diopiError_t tryRows8(hipStream_t stream, const TensorView& out, const TensorVie
   if (a) AMD_TRY(broadcastStrides(out, *a, s.sa, "input"));
   if (b) AMD_TRY(broadcastStrides(out, *b, s.sb, "other"));
   coalesceDims(&s);
-  if (s.ndim > 3) return diopiSuccess;
-  // up to three merged dims: groups x rows x columns (e.g. [batch, heads, seq * d] against [batch, 1, seq * d])
+  if (s.ndim > 4) return diopiSuccess;
+  // up to four merged dims: supers x groups x rows x columns (e.g. [batch, heads, seq * d] against [batch, 1, seq * d];
+  // [batch, seq, heads, d / 2] slices against a [1, seq, 1, d / 2] table; a permuted source with dense inner rows)
   const int last = s.ndim - 1;
-  const int64_t cols = s.shape[last], rowsPerGroup = s.ndim >= 2 ? s.shape[last - 1] : 1, groups = s.ndim == 3 ? s.shape[0] : 1;
-  if (cols % 8 != 0 || cols / 8 >= ((int64_t)1 << 31) || s.so[last] != 1) return diopiSuccess;
+  const int64_t cols = s.shape[last], rowsPerGroup = s.ndim >= 2 ? s.shape[last - 1] : 1;
+  const int64_t groupsPerSuper = s.ndim >= 3 ? s.shape[last - 2] : 1, supers = s.ndim == 4 ? s.shape[0] : 1;
+  if (cols % 8 != 0 || cols / 8 >= ((int64_t)1 << 31) || s.so[last] != 1 || supers * groupsPerSuper * rowsPerGroup >= ((int64_t)1 << 31))
+    return diopiSuccess;
   auto rowStrideOf = [&](const int64_t* st) { return s.ndim >= 2 ? st[last - 1] : 0; };
-  auto groupStrideOf = [&](const int64_t* st) { return s.ndim == 3 ? st[0] : 0; };
+  auto groupStrideOf = [&](const int64_t* st) { return s.ndim >= 3 ? st[last - 2] : 0; };
+  auto superStrideOf = [&](const int64_t* st) { return s.ndim == 4 ? st[0] : 0; };
+  auto stridesOk = [&](const int64_t* st) { return rowStrideOf(st) % 8 == 0 && groupStrideOf(st) % 8 == 0 && superStrideOf(st) % 8 == 0; };
   auto operandOk = [&](const TensorView* t, const int64_t* st) {
     if (!t) return true;
     if (st[last] == 0) return true;                      // one value per row: any address
-    return st[last] == 1 && t->aligned16() && rowStrideOf(st) % 8 == 0 && groupStrideOf(st) % 8 == 0;
+    return st[last] == 1 && t->aligned16() && stridesOk(st);
   };
-  if (!out.aligned16() || rowStrideOf(s.so) % 8 != 0 || groupStrideOf(s.so) % 8 != 0 || !operandOk(a, s.sa) || !operandOk(b, s.sb))
-    return diopiSuccess;
+  if (!out.aligned16() || !stridesOk(s.so) || !operandOk(a, s.sa) || !operandOk(b, s.sb)) return diopiSuccess;
   Rows8Operand oa{a ? a->data : nullptr, a ? (int)a->dtype : 0, a ? (int)s.sa[last] : 0, a ? rowStrideOf(s.sa) : 0,
-                  a ? groupStrideOf(s.sa) : 0};
+                  a ? groupStrideOf(s.sa) : 0, a ? superStrideOf(s.sa) : 0};
   Rows8Operand ob{b ? b->data : nullptr, b ? (int)b->dtype : 0, b ? (int)s.sb[last] : 0, b ? rowStrideOf(s.sb) : 0,
-                  b ? groupStrideOf(s.sb) : 0};
-  const int64_t nvec = groups * rowsPerGroup * (cols / 8), blocks = ceilDiv(nvec, 256);
+                  b ? groupStrideOf(s.sb) : 0, b ? superStrideOf(s.sb) : 0};
+  const int64_t nvec = supers * groupsPerSuper * rowsPerGroup * (cols / 8), blocks = ceilDiv(nvec, 256);
   AMD_CHECK(blocks <= 0x7fffffff, "elementwise: %ld vectors exceed the grid limit", (long)nvec);
   hipLaunchKernelGGL((ewRows8Kernel<OP>), dim3((unsigned)blocks), dim3(256), 0, stream, out.data, (int)out.dtype,
-                     rowStrideOf(s.so), groupStrideOf(s.so), oa, ob, nvec, (int)(cols / 8), rowsPerGroup, (float)p0);
+                     rowStrideOf(s.so), groupStrideOf(s.so), superStrideOf(s.so), oa, ob, nvec, (int)(cols / 8), (unsigned)rowsPerGroup,
+                     (unsigned)groupsPerSuper, (float)p0);
   AMD_LAUNCH_CHECK();
   *launched = true;
   return diopiSuccess;

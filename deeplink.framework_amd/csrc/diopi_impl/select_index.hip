@@ -70,12 +70,13 @@ __device__ __forceinline__ Offsets4 offsetsOf(const Strided4& s, int64_t i) {
 template <typename E>
 __global__ __launch_bounds__(kSelThreads) void selectVecKernel(E* __restrict__ out, const uint8_t* __restrict__ cond,
                                                                const E* __restrict__ a, const E* __restrict__ b, int64_t nvec,
-                                                               E aBits) {
+                                                               int64_t condVecs, E aBits) {
   typedef E E8 __attribute__((ext_vector_type(8)));
   typedef uint8_t C8 __attribute__((ext_vector_type(8)));
   const int64_t i = (int64_t)blockIdx.x * kSelThreads + threadIdx.x;
   if (i >= nvec) return;
-  const C8 c = reinterpret_cast<const C8*>(cond)[i];
+  // a condition that covers the trailing dims only repeats every condVecs vectors (a [s, s] mask on [b, h, s, s] scores)
+  const C8 c = reinterpret_cast<const C8*>(cond)[condVecs == nvec ? i : i % condVecs];
   const E8 vb = reinterpret_cast<const E8*>(b)[i];
   E8 va;
   if (a != nullptr) {
@@ -338,9 +339,29 @@ static diopiError_t runSelect(diopiContextHandle_t ctx, diopiTensorHandle_t outH
         if (t.shape[d] != out.shape[d]) return false;
       return true;
     };
+    // the condition: dense like the output, or dense over the trailing dims and broadcast over all the leading ones
+    auto trailing = [&](const TensorView& t) {
+      if (!t.isContiguous() || t.ndim > out.ndim || t.numel % 8 != 0 || t.numel == 0) return false;
+      int64_t covered = 1;
+      bool lead = false;  // once a dim is broadcast, every dim before it must be too
+      for (int d = out.ndim - 1; d >= 0; --d) {
+        const int td = d - (out.ndim - t.ndim);
+        const int64_t e = td >= 0 ? t.shape[td] : 1;
+        if (lead) {
+          if (e != 1) return false;
+        } else if (e == out.shape[d]) {
+          covered *= e;
+        } else if (e == 1) {
+          lead = true;
+        } else {
+          return false;
+        }
+      }
+      return covered == t.numel;
+    };
     const bool floatScalarIntoInt = aScalar && scalarIsFloat(aScalar) && !isFloatDtype(out.dtype);
-    if ((out.itemsize == 2 || out.itemsize == 4) && out.numel % 8 == 0 && out.isContiguous() && out.aligned16() && dense(cond) &&
-        cond.itemsize == 1 && (reinterpret_cast<uintptr_t>(cond.data) & 7) == 0 && dense(b) && b.dtype == out.dtype && b.aligned16() &&
+    if ((out.itemsize == 2 || out.itemsize == 4) && out.numel % 8 == 0 && out.isContiguous() && out.aligned16() &&
+        (dense(cond) || trailing(cond)) && cond.itemsize == 1 && (reinterpret_cast<uintptr_t>(cond.data) & 7) == 0 && dense(b) && b.dtype == out.dtype && b.aligned16() &&
         (aScalar ? !floatScalarIntoInt : (dense(a) && a.dtype == out.dtype && a.aligned16()))) {
       // the scalar in the output dtype's bits, through the same conversion the one-element path applies
       uint32_t bits = 0;
@@ -357,14 +378,15 @@ static diopiError_t runSelect(diopiContextHandle_t ctx, diopiTensorHandle_t outH
           bits = (uint32_t)scalarToInt(aScalar, 0);
         }
       }
-      const int64_t nvec = out.numel / 8, blocks = ceilDiv(nvec, kSelThreads);
+      const int64_t nvec = out.numel / 8, blocks = ceilDiv(nvec, kSelThreads), condVecs = cond.numel / 8;
       AMD_CHECK(blocks <= 0x7fffffff, "%s: %ld elements exceed the grid limit", name, (long)out.numel);
       if (out.itemsize == 2)
         hipLaunchKernelGGL((selectVecKernel<uint16_t>), dim3((unsigned)blocks), dim3(kSelThreads), 0, stream, out.ptr<uint16_t>(),
-                           cond.ptr<uint8_t>(), aScalar ? nullptr : a.ptr<uint16_t>(), b.ptr<uint16_t>(), nvec, (uint16_t)bits);
+                           cond.ptr<uint8_t>(), aScalar ? nullptr : a.ptr<uint16_t>(), b.ptr<uint16_t>(), nvec, condVecs,
+                           (uint16_t)bits);
       else
         hipLaunchKernelGGL((selectVecKernel<uint32_t>), dim3((unsigned)blocks), dim3(kSelThreads), 0, stream, out.ptr<uint32_t>(),
-                           cond.ptr<uint8_t>(), aScalar ? nullptr : a.ptr<uint32_t>(), b.ptr<uint32_t>(), nvec, bits);
+                           cond.ptr<uint8_t>(), aScalar ? nullptr : a.ptr<uint32_t>(), b.ptr<uint32_t>(), nvec, condVecs, bits);
       AMD_LAUNCH_CHECK();
       return diopiSuccess;
     }

@@ -215,6 +215,16 @@ def test_broadcast_rows_groups_and_mixed_dtypes(ops, dev):
     ops.mul(f32.to(dev), row.to(dev), out=wide[..., 64:])
     assert_each(wide[..., 64:], f32 * row)
     assert float(wide[..., :64].abs().sum()) == 0.0
+    # four dims that do not merge: the two halves of packed heads against a table shared by batch and heads
+    # ([b, s, h, d / 2] slices of a [b, s, 3 h d] projection times [1, s, 1, d / 2]), and a permuted copy with dense rows
+    qkv = torch.randn(2, 40, 3 * 6 * 64, generator=gq).bfloat16()
+    q = qkv[..., : 6 * 64].reshape(2, 40, 6, 64)
+    cosT = torch.randn(1, 40, 1, 32, generator=gq).bfloat16()
+    dq = qkv.to(dev)[..., : 6 * 64].reshape(2, 40, 6, 64)
+    assert_each(ops.mul(dq[..., 32:], cosT.to(dev)), q[..., 32:] * cosT)
+    perm = torch.empty(2, 6, 40, 64, dtype=torch.bfloat16, device=dev)
+    ops.copy_(perm, dq.permute(0, 2, 1, 3))
+    assert_exact(perm, q.permute(0, 2, 1, 3).contiguous())
     half = torch.empty(2, 6, 40, 64, dtype=torch.float16, device=dev)
     ops.copy_(half, tab.to(dev).expand(2, 6, 40, 64))                        # broadcast copy with a cast
     assert_exact(half, tab.expand(2, 6, 40, 64).half())

@@ -208,3 +208,13 @@ def test_index_select_blocks_and_triangles_vector_paths(ops, dev):
         inp = m.clone().to(dev)
         ops.triu_(inp, 1)
         assert_exact(inp, torch.triu(m, 1))
+
+
+def test_masked_fill_with_a_mask_over_the_trailing_dims(ops, dev):
+    """A [s, s] (or [1, 1, s, s]) mask on [b, h, s, s] scores: the condition repeats over the leading dims (the
+    8-per-lane kernel indexes it modulo its length); a mask that is broadcast in the middle takes the general kernel."""
+    sc = torch.randn(3, 4, 24, 40, generator=g(70)).bfloat16()
+    for mshape in [(24, 40), (1, 1, 24, 40), (4, 24, 40), (3, 1, 24, 40), (40,)]:
+        m = torch.rand(mshape, generator=g(71)) > 0.5
+        assert_exact(ops.masked_fill(sc.to(dev), m.to(dev), float("-inf")), sc.masked_fill(m, float("-inf")))
+        assert_exact(ops.where(m.to(dev), sc.to(dev), sc.neg().to(dev)), torch.where(m, sc, sc.neg()))
