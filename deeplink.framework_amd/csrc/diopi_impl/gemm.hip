@@ -1448,6 +1448,274 @@ __global__ __launch_bounds__(256) void transposeKernel(U* __restrict__ dst, cons
 }
 
 // ---------------------------------------------------------------- FMA engine --
+// ------------------------------------------------------------ fp32 on MFMA ---
+// Epilogue of the fp32 MFMA kernels: register 4 g + r of a block is output row l32, column 8 g + 4 half + r.
+template <int WT>
+__device__ __forceinline__ void gemmF32StoreTile(const GemmProblem& p, const f32x16 (&acc)[WT][WT], int64_t m0, int64_t n0, int64_t batch,
+                                                 int wm, int wn, int l32, int half) {
+  float* out = reinterpret_cast<float*>(p.out) + batch * p.sOb;
+  const float* cin = p.Cin ? reinterpret_cast<const float*>(p.Cin) + batch * p.sCb : nullptr;
+  const float* bias = reinterpret_cast<const float*>(p.bias);
+  const bool vec = (p.N & 3) == 0 && (p.sOm & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+#pragma unroll
+  for (int bm = 0; bm < WT; ++bm) {
+    const int64_t row = m0 + (wm * WT + bm) * 32 + l32;
+    if (row >= p.M) continue;
+#pragma unroll
+    for (int bn = 0; bn < WT; ++bn)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int64_t col = n0 + (wn * WT + bn) * 32 + 8 * g + 4 * half;
+        if (col >= p.N) continue;
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          v[r] = acc[bm][bn][4 * g + r] * p.alpha;
+          if (col + r < p.N) {
+            if (bias) v[r] += bias[col + r];
+            if (cin) v[r] += p.beta * cin[row * p.sCm + (col + r) * p.sCn];
+          }
+        }
+        if (vec) {
+          *reinterpret_cast<f32x4*>(out + row * p.sOm + col) = f32x4{v[0], v[1], v[2], v[3]};
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (col + r < p.N) out[row * p.sOm + col + r] = v[r];
+        }
+      }
+  }
+}
+
+// fp32 operands through v_mfma_f32_32x32x2f32 (true fp32 products and sums; 157 TFLOP/s peak against 79 for the vector
+// unit): 4 waves in 2 x 2, a wave owns WT x WT blocks of 32 x 32, K in stages of BK through two LDS buffers filled
+// from registers (the loads of stage t + 1 are issued before the MFMAs of stage t). The instruction takes one k per
+// lane half; which two k meet in one instruction does not matter as long as both operands agree, so lane half h
+// takes k = 8 q + 4 h + j at step (q, j): its four steps of a half-stage are one 16-byte LDS read per fragment.
+// LDS rows are BK + 4 floats apart: 16 consecutive rows then start on 16 different 16-byte bank groups.
+// Either operand may be K-contiguous ([rows, K]) or row-contiguous ([K, rows], e.g. the second operand of mm);
+// the weight fragment goes first, so a lane ends up with four consecutive columns of one output row per register
+// quad (16-byte stores). With the tiles staged through registers the MFMA pipe is busy 79 % of the time
+// (123 TFLOP/s at 8192 x 4096 x 4096); without the global loads 135, without loads and LDS writes 148: the kernel
+// below, which has neither, takes the layout that allows it.
+template <int WT, int BK, bool A_BY_K, bool B_BY_K>
+__global__ __launch_bounds__(256) void gemmMfmaF32Kernel(GemmProblem p) {
+  constexpr int BM = 64 * WT, BN = 64 * WT, PAD = BK + 4;
+  constexpr int LPT = BM * BK / 4 / 256;  // 16-byte loads per thread, stage and operand
+  __shared__ __attribute__((aligned(16))) float sA[2][BM * PAD];
+  __shared__ __attribute__((aligned(16))) float sB[2][BN * PAD];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, half = lane >> 5;
+  const int64_t m0 = (int64_t)blockIdx.y * BM, n0 = (int64_t)blockIdx.x * BN, batch = blockIdx.z;
+  const float* A = reinterpret_cast<const float*>(p.A) + batch * p.sAb;
+  const float* B = reinterpret_cast<const float*>(p.B) + batch * p.sBb;
+  f32x4 ra[LPT], rb[LPT];
+  // 16 bytes of an operand tile: along K when the operand is K-contiguous, along the rows otherwise. Every thread
+  // keeps one running pointer per load; rows past the end are clamped to the last ones (their products land in
+  // output rows or columns that are never stored), so only the last stage of a ragged K needs a predicate.
+  const float* pa[LPT];
+  const float* pb[LPT];
+  int ka[LPT], kb[LPT];  // k of the load within its stage
+  int wa[LPT], wb[LPT];  // where it goes in the LDS tile
+  auto aim = [&](const float* base, auto byK, int64_t rowStride, int64_t kStride, int64_t row0, int64_t rows, const float* (&ptr)[LPT],
+                 int (&kk)[LPT], int (&ww)[LPT]) {
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) {
+      const int f = tid + 256 * i;
+      constexpr int RV = BM / 4, KV = BK / 4;  // 4-row vectors per k, 4-k vectors per row
+      const int r = byK ? f / KV : (f % RV) * 4;
+      kk[i] = byK ? (f % KV) * 4 : f / RV;
+      ww[i] = r * PAD + kk[i];
+      ptr[i] = base + min(row0 + r, rows - (byK ? 1 : 4)) * rowStride + kk[i] * kStride;
+    }
+  };
+  aim(A, std::integral_constant<bool, A_BY_K>{}, p.sAm, p.sAk, m0, p.M, pa, ka, wa);
+  aim(B, std::integral_constant<bool, B_BY_K>{}, p.sBn, p.sBk, n0, p.N, pb, kb, wb);
+  const int64_t stepA = BK * p.sAk, stepB = BK * p.sBk;
+  auto fetch = [&](int64_t k0, bool ragged) {
+    if (!ragged) {
+#pragma unroll
+      for (int i = 0; i < LPT; ++i) {
+        ra[i] = *reinterpret_cast<const f32x4*>(pa[i]);
+        rb[i] = *reinterpret_cast<const f32x4*>(pb[i]);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < LPT; ++i) {
+        ra[i] = rb[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (k0 + ka[i] < p.K) ra[i] = *reinterpret_cast<const f32x4*>(pa[i]);
+        if (k0 + kb[i] < p.K) rb[i] = *reinterpret_cast<const f32x4*>(pb[i]);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) {
+      pa[i] += stepA;
+      pb[i] += stepB;
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) {
+      if (A_BY_K) {
+        *reinterpret_cast<f32x4*>(sA[buf] + wa[i]) = ra[i];
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sA[buf][wa[i] + j * PAD] = ra[i][j];
+      }
+      if (B_BY_K) {
+        *reinterpret_cast<f32x4*>(sB[buf] + wb[i]) = rb[i];
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sB[buf][wb[i] + j * PAD] = rb[i][j];
+      }
+    }
+  };
+  f32x16 acc[WT][WT];
+#pragma unroll
+  for (int i = 0; i < WT; ++i)
+#pragma unroll
+    for (int j = 0; j < WT; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  const int stages = (int)((p.K + BK - 1) / BK);
+  const bool raggedK = (p.K % BK) != 0;  // then the last stage is partial
+  fetch(0, raggedK && stages == 1);
+  stash(0);
+  __syncthreads();
+  for (int t = 0; t < stages; ++t) {
+    const int cur = t & 1;
+    if (t + 1 < stages) fetch((int64_t)(t + 1) * BK, raggedK && t + 2 == stages);
+    const float* ta = sA[cur] + (wm * 32 * WT + l32) * PAD + 4 * half;
+    const float* tb = sB[cur] + (wn * 32 * WT + l32) * PAD + 4 * half;
+#pragma unroll
+    for (int q = 0; q < BK / 8; ++q) {
+      f32x4 fa[WT], fb[WT];
+#pragma unroll
+      for (int i = 0; i < WT; ++i) {
+        fa[i] = *reinterpret_cast<const f32x4*>(ta + i * 32 * PAD + 8 * q);
+        fb[i] = *reinterpret_cast<const f32x4*>(tb + i * 32 * PAD + 8 * q);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int bm = 0; bm < WT; ++bm)
+#pragma unroll
+          for (int bn = 0; bn < WT; ++bn)
+            acc[bm][bn] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[bn][j], fa[bm][j], acc[bm][bn], 0, 0, 0);
+    }
+    if (t + 1 < stages) stash(cur ^ 1);
+    __syncthreads();
+  }
+  gemmF32StoreTile<WT>(p, acc, m0, n0, batch, wm, wn, l32, half);
+}
+
+// The same product for the layout of linear (both operands K-contiguous, K a multiple of 32): the tiles go from
+// global memory straight into LDS (global_load_lds_dwordx4: lane i of a wave fills bytes 16 i .. 16 i + 15 of a 1 KiB
+// piece), so no staging registers, no LDS writes by the waves and no wait between a load's return and its use other
+// than the barrier. Rows are 32 floats (8 pieces of 16 bytes) without padding; piece c of row r sits at position
+// c ^ swz(r), swz(r) = (r ^ (r >> 3)) & 7, chosen by the loading lane through the global address it reads, which makes
+// the 16-byte fragment reads of 16 consecutive rows hit 16 different bank groups (no bank conflict is counted).
+// 138 TFLOP/s at 8192 x 4096 x 4096 and at 2048 x 4096 x 4096 (88 % of the MFMA rate a register-only loop of the same
+// instruction sustains, 156); what is left is the barrier and the wait for the stage's loads once per 64 MFMAs with
+// two waves per SIMD. A third LDS buffer would leave room for one workgroup per compute unit only.
+__device__ __forceinline__ int f32Swz(int row) { return (row ^ (row >> 3)) & 7; }
+
+template <int WT>
+__global__ __launch_bounds__(256) void gemmMfmaF32DirectKernel(GemmProblem p) {
+  constexpr int BM = 64 * WT, BN = 64 * WT, BK = 32;
+  constexpr int LPT = BM * BK / 4 / 256;  // 16-byte pieces per thread, stage and operand
+  __shared__ __attribute__((aligned(1024))) float sA[2][BM * BK];
+  __shared__ __attribute__((aligned(1024))) float sB[2][BN * BK];
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, half = lane >> 5;
+  const int64_t m0 = (int64_t)blockIdx.y * BM, n0 = (int64_t)blockIdx.x * BN, batch = blockIdx.z;
+  const float* A = reinterpret_cast<const float*>(p.A) + batch * p.sAb;
+  const float* B = reinterpret_cast<const float*>(p.B) + batch * p.sBb;
+  // piece i * 256 + tid of a tile: row (i * 256 + tid) / 8 at position tid % 8, holding chunk position ^ swz(row);
+  // rows past the end are clamped (their products land in rows or columns that are never stored)
+  const float* pa[LPT];
+  const float* pb[LPT];
+#pragma unroll
+  for (int i = 0; i < LPT; ++i) {
+    const int row = (i * 256 + tid) >> 3, chunk = (tid & 7) ^ f32Swz(row);
+    pa[i] = A + min(m0 + row, p.M - 1) * p.sAm + chunk * 4;
+    pb[i] = B + min(n0 + row, p.N - 1) * p.sBn + chunk * 4;
+  }
+  typedef __attribute__((address_space(3))) void* LdsPtr;
+  auto fetch = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) {
+      // as assembly: the compiler would wait for a load into LDS before the next LDS read of any buffer
+      const uint32_t la = (uint32_t)(uintptr_t)(LdsPtr)(sA[buf] + (i * 256 + wave * 64) * 4);
+      const uint32_t lb = (uint32_t)(uintptr_t)(LdsPtr)(sB[buf] + (i * 256 + wave * 64) * 4);
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(la), "v"(pa[i]) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lb), "v"(pb[i]) : "memory", "m0");
+      pa[i] += BK;
+      pb[i] += BK;
+    }
+  };
+  // fragment of block row i at step q: row R = wave rows + 32 i + l32, chunk 2 q + half
+  int offA[WT], offB[WT], swA[WT], swB[WT];
+#pragma unroll
+  for (int i = 0; i < WT; ++i) {
+    const int ra = (wm * WT + i) * 32 + l32, rb = (wn * WT + i) * 32 + l32;
+    offA[i] = ra * BK, offB[i] = rb * BK;
+    swA[i] = f32Swz(ra) ^ half, swB[i] = f32Swz(rb) ^ half;
+  }
+  f32x16 acc[WT][WT];
+#pragma unroll
+  for (int i = 0; i < WT; ++i)
+#pragma unroll
+    for (int j = 0; j < WT; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  const int stages = (int)(p.K / BK);
+  fetch(0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  for (int t = 0; t < stages; ++t) {
+    const int cur = t & 1;
+    if (t + 1 < stages) fetch(cur ^ 1);
+    f32x4 fa[2][WT], fb[2][WT];
+    auto frags = [&](int q) {
+#pragma unroll
+      for (int i = 0; i < WT; ++i) {
+        fa[q & 1][i] = *reinterpret_cast<const f32x4*>(sA[cur] + offA[i] + (((2 * q) ^ swA[i]) << 2));
+        fb[q & 1][i] = *reinterpret_cast<const f32x4*>(sB[cur] + offB[i] + (((2 * q) ^ swB[i]) << 2));
+      }
+    };
+    frags(0);
+#pragma unroll
+    for (int q = 0; q < BK / 8; ++q) {
+      if (q + 1 < BK / 8) frags(q + 1);  // under the MFMAs of step q
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int bm = 0; bm < WT; ++bm)
+#pragma unroll
+          for (int bn = 0; bn < WT; ++bn)
+            acc[bm][bn] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[q & 1][bn][j], fa[q & 1][bm][j], acc[bm][bn], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
+  gemmF32StoreTile<WT>(p, acc, m0, n0, batch, wm, wn, l32, half);
+}
+
+// Whether gemmMfmaF32Kernel can take the problem: each operand contiguous along K or along its rows, 16-byte pieces
+// whole and aligned.
+constexpr int kF32BKBig = 32;  // stage depth of the 128 x 128 tile
+static bool f32MfmaEligible(const GemmProblem& p) {
+  auto operand = [&](const void* base, int64_t rowStride, int64_t kStride, int64_t batchStride, int64_t rows) {
+    if ((reinterpret_cast<uintptr_t>(base) & 15) != 0 || (batchStride & 3) != 0) return false;
+    if (kStride == 1) return (p.K & 3) == 0 && (rowStride & 3) == 0;
+    return rowStride == 1 && (rows & 3) == 0 && (kStride & 3) == 0;
+  };
+  return p.K > 0 && operand(p.A, p.sAm, p.sAk, p.sAb, p.M) && operand(p.B, p.sBn, p.sBk, p.sBb, p.N) &&
+         ceilDiv(p.M, 64) <= 65535;
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void gemmFmaKernel(GemmProblem p) {
   __shared__ float sA[16][64 + 4];
@@ -1885,6 +2153,33 @@ diopiError_t runGemm(diopiContextHandle_t ctx, hipStream_t stream, GemmProblem p
     dim3 grid((unsigned)ceilDiv(p.N, 256), (unsigned)p.M, (unsigned)p.batch);
     AMD_CHECK(p.M <= 65535, "gemm(float64): M exceeds the grid limit");
     hipLaunchKernelGGL(gemmFmaKernelF64, grid, dim3(256), 0, stream, p);
+    AMD_LAUNCH_CHECK();
+    return diopiSuccess;
+  }
+  if (p.dtype == diopi_dtype_float32 && p.M >= 32 && p.N >= 32 && f32MfmaEligible(p)) {
+    // 128 x 128 tiles (less LDS traffic per product: 138 against 121 TFLOP/s at 2048 x 4096 x 4096) when their count
+    // fills whole rounds of one workgroup per compute unit to at least 90 %; 64 x 64 tiles, whose rounds are four
+    // times finer, otherwise (384 big tiles: 103 against 119 TFLOP/s)
+    const int64_t tiles128 = ceilDiv(p.M, 128) * ceilDiv(p.N, 128) * p.batch, cus = computeUnits();
+    const bool big = tiles128 >= cus && 10 * tiles128 >= 9 * ceilDiv(tiles128, cus) * cus;
+    const int tile = big ? 128 : 64;
+    dim3 grid((unsigned)ceilDiv(p.N, tile), (unsigned)ceilDiv(p.M, tile), (unsigned)p.batch);
+    if (p.sAk == 1 && p.sBk == 1 && p.K % 32 == 0) {  // tiles straight into LDS
+      if (big) hipLaunchKernelGGL(gemmMfmaF32DirectKernel<2>, grid, dim3(256), 0, stream, p);
+      else hipLaunchKernelGGL(gemmMfmaF32DirectKernel<1>, grid, dim3(256), 0, stream, p);
+      AMD_LAUNCH_CHECK();
+      return diopiSuccess;
+    }
+    auto launch = [&](auto aByK, auto bByK) {
+      if (big)
+        hipLaunchKernelGGL((gemmMfmaF32Kernel<2, kF32BKBig, decltype(aByK)::value, decltype(bByK)::value>), grid, dim3(256), 0, stream, p);
+      else
+        hipLaunchKernelGGL((gemmMfmaF32Kernel<1, 16, decltype(aByK)::value, decltype(bByK)::value>), grid, dim3(256), 0, stream, p);
+    };
+    if (p.sAk == 1 && p.sBk == 1) launch(std::true_type{}, std::true_type{});
+    else if (p.sAk == 1) launch(std::true_type{}, std::false_type{});
+    else if (p.sBk == 1) launch(std::false_type{}, std::true_type{});
+    else launch(std::false_type{}, std::false_type{});
     AMD_LAUNCH_CHECK();
     return diopiSuccess;
   }

@@ -86,6 +86,64 @@ def test_sweep_gemm(ops, dev, seed, n):
     _report(failed, n)
 
 
+@pytest.mark.parametrize("seed,n", [(1, 80), (2, 80)])
+def test_sweep_gemm_fp32(ops, dev, seed, n):
+    """fp32 products (linear with and without bias, into a strided destination, addmm, mm with either operand layout,
+    bmm) over shapes on both sides of what the matrix-core kernel takes (multiples of 4 along the contiguous
+    dims, at least 32 rows and columns) and its two tile sizes, against the product in float64: true fp32
+    multiplies and adds, so the error is that of the summation order, a few 1e-7 of the scale of the terms."""
+    rng = random.Random(seed)
+    pick = rng.choice
+    Ms = [1, 4, 31, 32, 33, 36, 63, 64, 65, 100, 128, 132, 200, 256, 300, 512, 700, 1024, 2048]
+    Ks = [4, 8, 12, 16, 20, 30, 64, 72, 100, 128, 250, 256, 512, 1000, 1024, 2048, 4096]
+    Ns = [8, 32, 36, 40, 64, 100, 128, 130, 136, 256, 512, 1000, 1024, 2048, 4096, 4100]
+    failed = []
+    for case in range(n):
+        kind = pick(["linear", "linear_bias", "linear_strided", "addmm", "mm", "mm_at", "bmm"])
+        m, k, nn = pick(Ms), pick(Ks), pick(Ns)
+        if m * k * nn > 3e9: m = max(1, int(3e9 / (k * nn)))
+        g = torch.Generator().manual_seed(seed * 7919 + case)
+        desc = f"case {case} {kind} m={m} k={k} n={nn}"
+        try:
+            if kind == "bmm":
+                bt = pick([1, 3, 8])
+                m, nn, k = min(m, 256), min(nn, 256), min(k, 512)
+                a, b = torch.randn(bt, m, k, generator=g), torch.randn(bt, k, nn, generator=g)
+                want = torch.bmm(a.double(), b.double())
+                got = ops.bmm(a.to(dev), b.to(dev))
+            else:
+                x, w = torch.randn(m, k, generator=g), torch.randn(nn, k, generator=g)
+                want = x.double() @ w.double().t()
+                if kind == "linear":
+                    got = ops.linear(x.to(dev), w.to(dev))
+                elif kind == "linear_bias":
+                    b = torch.randn(nn, generator=g)
+                    want = want + b.double()
+                    got = ops.linear(x.to(dev), w.to(dev), b.to(dev))
+                elif kind == "linear_strided":
+                    pad = pick([4, 8, 3])
+                    xs = torch.randn(m, k + pad, generator=g)
+                    dst = torch.zeros(m, nn + pad, device=dev)
+                    want = xs[:, :k].double() @ w.double().t()
+                    ops.linear(xs.to(dev)[:, :k], w.to(dev), out=dst[:, :nn])
+                    got = dst[:, :nn]
+                    assert float(dst[:, nn:].abs().max()) == 0.0, "wrote past the destination view"
+                elif kind == "addmm":
+                    c = torch.randn(m, nn, generator=g)
+                    beta, alpha = pick([1, 0.5, 2]), pick([1, 0.25])
+                    want = beta * c.double() + alpha * want
+                    got = ops.addmm(c.to(dev), x.to(dev), w.to(dev).t(), beta=beta, alpha=alpha)
+                elif kind == "mm":
+                    got = ops.mm(x.to(dev), w.t().contiguous().to(dev))           # [k, n] row-major second operand
+                else:
+                    got = ops.mm(x.t().contiguous().to(dev).t(), w.to(dev).t())   # column-major first operand
+            # terms of magnitude ~1, sums of magnitude ~sqrt(k): 1e-5 of the largest sum
+            assert_fp32(got, want, rel=1e-5)
+        except AssertionError as e:
+            failed.append(desc + ": " + str(e)[:200])
+    _report(failed, n)
+
+
 @pytest.mark.parametrize("seed,n", [(1, 150), (2, 150)])
 def test_sweep_attention(ops, dev, pkg, seed, n):
     """Prefill over ragged packed sequences (gaps between them, empty ones) and decode over a paged pool (fused, without
