@@ -1609,7 +1609,7 @@ __global__ __launch_bounds__(256) void gemmMfmaF32Kernel(GemmProblem p) {
   gemmF32StoreTile<WT>(p, acc, m0, n0, batch, wm, wn, l32, half);
 }
 
-// The same product for the layout of linear (both operands K-contiguous, K a multiple of 32): the tiles go from
+// The same product for a K-contiguous first operand and K a multiple of 32 (linear, mm, bmm): the tiles go from
 // global memory straight into LDS (global_load_lds_dwordx4: lane i of a wave fills bytes 16 i .. 16 i + 15 of a 1 KiB
 // piece), so no staging registers, no LDS writes by the waves and no wait between a load's return and its use other
 // than the barrier. Rows are 32 floats (8 pieces of 16 bytes) without padding; piece c of row r sits at position
@@ -1620,7 +1620,10 @@ __global__ __launch_bounds__(256) void gemmMfmaF32Kernel(GemmProblem p) {
 // two waves per SIMD. A third LDS buffer would leave room for one workgroup per compute unit only.
 __device__ __forceinline__ int f32Swz(int row) { return (row ^ (row >> 3)) & 7; }
 
-template <int WT>
+// With B_BY_K false the second operand is [K, N] row-major (mm, bmm, matmul): its tile sits in LDS as it sits in memory,
+// 32 rows of k by BN columns, and a lane reads its operand of every MFMA step on its own (4-byte reads along n:
+// consecutive lanes, consecutive banks).
+template <int WT, bool B_BY_K>
 __global__ __launch_bounds__(256) void gemmMfmaF32DirectKernel(GemmProblem p) {
   constexpr int BM = 64 * WT, BN = 64 * WT, BK = 32;
   constexpr int LPT = BM * BK / 4 / 256;  // 16-byte pieces per thread, stage and operand
@@ -1639,8 +1642,14 @@ __global__ __launch_bounds__(256) void gemmMfmaF32DirectKernel(GemmProblem p) {
   for (int i = 0; i < LPT; ++i) {
     const int row = (i * 256 + tid) >> 3, chunk = (tid & 7) ^ f32Swz(row);
     pa[i] = A + min(m0 + row, p.M - 1) * p.sAm + chunk * 4;
-    pb[i] = B + min(n0 + row, p.N - 1) * p.sBn + chunk * 4;
+    if (B_BY_K) {
+      pb[i] = B + min(n0 + row, p.N - 1) * p.sBn + chunk * 4;
+    } else {  // piece: k = piece / (BN / 4), columns 4 (piece % (BN / 4)) .. + 3, clamped to the last four
+      const int piece = i * 256 + tid;
+      pb[i] = B + (piece / (BN / 4)) * p.sBk + min(n0 + (piece % (BN / 4)) * 4, p.N - 4);
+    }
   }
+  const int64_t stepB = B_BY_K ? BK : BK * p.sBk;
   typedef __attribute__((address_space(3))) void* LdsPtr;
   auto fetch = [&](int buf) {
 #pragma unroll
@@ -1651,7 +1660,7 @@ __global__ __launch_bounds__(256) void gemmMfmaF32DirectKernel(GemmProblem p) {
       asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(la), "v"(pa[i]) : "memory", "m0");
       asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lb), "v"(pb[i]) : "memory", "m0");
       pa[i] += BK;
-      pb[i] += BK;
+      pb[i] += stepB;
     }
   };
   // fragment of block row i at step q: row R = wave rows + 32 i + l32, chunk 2 q + half
@@ -1659,7 +1668,7 @@ __global__ __launch_bounds__(256) void gemmMfmaF32DirectKernel(GemmProblem p) {
 #pragma unroll
   for (int i = 0; i < WT; ++i) {
     const int ra = (wm * WT + i) * 32 + l32, rb = (wn * WT + i) * 32 + l32;
-    offA[i] = ra * BK, offB[i] = rb * BK;
+    offA[i] = ra * BK, offB[i] = B_BY_K ? rb * BK : 4 * half * BN + rb;
     swA[i] = f32Swz(ra) ^ half, swB[i] = f32Swz(rb) ^ half;
   }
   f32x16 acc[WT][WT];
@@ -1681,7 +1690,12 @@ __global__ __launch_bounds__(256) void gemmMfmaF32DirectKernel(GemmProblem p) {
 #pragma unroll
       for (int i = 0; i < WT; ++i) {
         fa[q & 1][i] = *reinterpret_cast<const f32x4*>(sA[cur] + offA[i] + (((2 * q) ^ swA[i]) << 2));
-        fb[q & 1][i] = *reinterpret_cast<const f32x4*>(sB[cur] + offB[i] + (((2 * q) ^ swB[i]) << 2));
+        if (B_BY_K) {
+          fb[q & 1][i] = *reinterpret_cast<const f32x4*>(sB[cur] + offB[i] + (((2 * q) ^ swB[i]) << 2));
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) fb[q & 1][i][j] = sB[cur][offB[i] + (8 * q + j) * BN];
+        }
       }
     };
     frags(0);
@@ -2164,9 +2178,14 @@ diopiError_t runGemm(diopiContextHandle_t ctx, hipStream_t stream, GemmProblem p
     const bool big = tiles128 >= cus && 10 * tiles128 >= 9 * ceilDiv(tiles128, cus) * cus;
     const int tile = big ? 128 : 64;
     dim3 grid((unsigned)ceilDiv(p.N, tile), (unsigned)ceilDiv(p.M, tile), (unsigned)p.batch);
-    if (p.sAk == 1 && p.sBk == 1 && p.K % 32 == 0) {  // tiles straight into LDS
-      if (big) hipLaunchKernelGGL(gemmMfmaF32DirectKernel<2>, grid, dim3(256), 0, stream, p);
-      else hipLaunchKernelGGL(gemmMfmaF32DirectKernel<1>, grid, dim3(256), 0, stream, p);
+    if (p.sAk == 1 && p.K % 32 == 0) {  // tiles straight into LDS
+      if (p.sBk == 1) {
+        if (big) hipLaunchKernelGGL((gemmMfmaF32DirectKernel<2, true>), grid, dim3(256), 0, stream, p);
+        else hipLaunchKernelGGL((gemmMfmaF32DirectKernel<1, true>), grid, dim3(256), 0, stream, p);
+      } else {
+        if (big) hipLaunchKernelGGL((gemmMfmaF32DirectKernel<2, false>), grid, dim3(256), 0, stream, p);
+        else hipLaunchKernelGGL((gemmMfmaF32DirectKernel<1, false>), grid, dim3(256), 0, stream, p);
+      }
       AMD_LAUNCH_CHECK();
       return diopiSuccess;
     }
