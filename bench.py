@@ -45,8 +45,9 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-ops", action="store_true", help="skip the per-op HBM microbenchmarks")
     ap.add_argument("--only-layer", action="store_true", help="alias for --no-cpu --no-ops")
-    ap.add_argument("--gemm", metavar="M,N,K", help="profiling aid: time only diopiLinear on bf16 [M,K] x [N,K]^T "
+    ap.add_argument("--gemm", metavar="M,N,K", help="profiling aid: time only diopiLinear on [M,K] x [N,K]^T (bf16 unless --gemm-dtype says otherwise) "
                     "(activations N(0,1), weights N(0,0.02)) for --steps launches and print one JSON line")
+    ap.add_argument("--gemm-dtype", choices=["bf16", "fp16", "fp32"], default="bf16", help="with --gemm: the operand dtype")
     ap.add_argument("--vendor-library", action="store_true", help="with --gemm: time torch.nn.functional.linear (the vendor's GEMM "
                     "library) on the same operands instead of diopiLinear, for side-by-side counter runs; never part of the measured path")
     ap.add_argument("--attention", action="store_true", help="profiling aid: time only the prefill attention of the "
@@ -468,15 +469,16 @@ def single_kernel(pkg, torch, dev, rt, stream, args):
     if args.gemm:
         m, n, k = (int(v) for v in args.gemm.split(","))
         g = torch.Generator().manual_seed(0)
-        a = torch.randn(m, k, generator=g).bfloat16().to(dev)
-        w = (torch.randn(n, k, generator=g) * 0.02).bfloat16().to(dev)
-        out = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+        dt = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[args.gemm_dtype]
+        a = torch.randn(m, k, generator=g).to(dt).to(dev)
+        w = (torch.randn(n, k, generator=g) * 0.02).to(dt).to(dev)
+        out = torch.empty(m, n, dtype=dt, device=dev)
         if args.vendor_library:
             call = lambda: torch.matmul(a, w.t(), out=out)
-            label = f"torch.matmul (vendor library) bf16 {m}x{n}x{k}"
+            label = f"torch.matmul (vendor library) {args.gemm_dtype} {m}x{n}x{k}"
         else:
             call = Prepared(pkg, "diopiLinear", out, a, w, None)
-            label = f"diopiLinear bf16 {m}x{n}x{k}"
+            label = f"diopiLinear {args.gemm_dtype} {m}x{n}x{k}"
         work, unit = 2.0 * m * n * k / 1e12, "TFLOP/s"
     else:
         b, s, h, hd = 4, 2048, 32, 128
