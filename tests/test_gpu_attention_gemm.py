@@ -73,6 +73,47 @@ def test_mm_bmm_matmul_addmm_baddbmm(ops, dev, dtype):
     chk(ops.baddbmm(c3[:, :1].to(dev), ba.to(dev), bb.to(dev)), c3[:, :1].float() + torch.bmm(ba.float(), bb.float()))
 
 
+@pytest.mark.parametrize("m,n,k,form", [
+    (2048, 2048, 64, "linear"),      # 256 tiles of 128 x 128, operands straight into LDS
+    (2048, 2048, 64, "mm"),          # the same with a row-major [K, N] second operand
+    (200, 328, 96, "linear"),        # 64 x 64 tiles, ragged rows and columns
+    (200, 328, 96, "mm"),
+    (1100, 2100, 32, "addmm"),       # one stage; alpha, beta and a matrix addend in the epilogue
+    (130, 200, 72, "linear"),        # K no multiple of 32: tiles staged through registers
+    (130, 200, 72, "mm"),
+    (136, 200, 36, "mm_at"),         # transposed first operand (row-contiguous along M)
+    (2304, 2048, 40, "mm"),          # staged, 128 x 128 tiles, ragged last stage
+    (64, 64, 4100, "bmm"),           # long K, batch 3
+    (33, 40, 8, "linear"),           # one partial tile
+    (31, 64, 64, "linear"),          # fewer than 32 rows: the FMA engine
+])
+def test_fp32_gemm_on_the_matrix_cores(ops, dev, m, n, k, form):
+    """fp32 operands through the fp32 MFMA kernels (both tile sizes, operands straight into LDS or staged through
+    registers, either layout of the second operand) against the product in float64: true fp32 products and sums, so
+    only the summation order differs (1e-5 of the largest sum)."""
+    x, w = torch.randn(m, k, generator=g(40)), torch.randn(n, k, generator=g(41))
+    want = x.double() @ w.double().t()
+    if form == "linear":
+        b = torch.randn(n, generator=g(42))
+        assert_fp32(ops.linear(x.to(dev), w.to(dev)), want)
+        assert_fp32(ops.linear(x.to(dev), w.to(dev), b.to(dev)), want + b.double())
+    elif form == "mm":
+        assert_fp32(ops.mm(x.to(dev), w.t().contiguous().to(dev)), want)
+    elif form == "mm_at":
+        assert_fp32(ops.mm(x.t().contiguous().to(dev).t(), w.t().contiguous().to(dev)), want)
+    elif form == "addmm":
+        c = torch.randn(m, n, generator=g(43))
+        assert_fp32(ops.addmm(c.to(dev), x.to(dev), w.to(dev).t(), beta=0.5, alpha=2), 0.5 * c.double() + 2 * want)
+    else:
+        xb, wb = torch.randn(3, m, k, generator=g(44)), torch.randn(3, k, n, generator=g(45))
+        assert_fp32(ops.bmm(xb.to(dev), wb.to(dev)), torch.bmm(xb.double(), wb.double()))
+    # a one-hot row picks one weight column exactly, whatever the tiling
+    if form == "linear":
+        onehot = torch.zeros(m, k)
+        onehot[torch.arange(m), torch.arange(m) % k] = 1.0
+        assert_exact(ops.linear(onehot.to(dev), w.to(dev)), w.t()[torch.arange(m) % k])
+
+
 def test_gemm_linearity_at_7b_shapes(ops, dev):
     # size-independent property at the full prefill shape: f(x1 + x2) = f(x1) + f(x2), and a
     # one-hot row selects a weight column exactly
