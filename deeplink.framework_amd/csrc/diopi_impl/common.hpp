@@ -154,6 +154,21 @@ __device__ __forceinline__ void loadToLds16(u32x4 rsrc, int voffset, int soffset
       : "memory");
 }
 
+// The same copy from a flat global address per lane (global_load_lds_dwordx4), for kernels that address their operands
+// with 64-bit pointers instead of a buffer descriptor.
+__device__ __forceinline__ void globalLoadToLds16(const void* lanePtr, unsigned ldsAddr) {
+  unsigned savedM0;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\t"
+      "s_mov_b32 m0, %1\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %2, off\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(savedM0)
+      : "s"(ldsAddr), "v"(lanePtr)
+      : "memory");
+}
+
 // The same copy marked non-temporal: for data that is read once (a weight stream), so that it does not push
 // re-used lines (the activations every workgroup reads) out of L2.
 __device__ __forceinline__ void loadToLds16Stream(u32x4 rsrc, int voffset, int soffset, unsigned ldsAddr) {

@@ -1678,10 +1678,8 @@ __global__ __launch_bounds__(256) void gemmMfmaF32DirectKernel(GemmProblem p) {
 #pragma unroll
     for (int i = 0; i < LPT; ++i) {
       // as assembly: the compiler would wait for a load into LDS before the next LDS read of any buffer
-      const uint32_t la = (uint32_t)(uintptr_t)(LdsPtr)(sA[buf] + (i * 256 + wave * 64) * 4);
-      const uint32_t lb = (uint32_t)(uintptr_t)(LdsPtr)(sB[buf] + (i * 256 + wave * 64) * 4);
-      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(la), "v"(pa[i]) : "memory", "m0");
-      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lb), "v"(pb[i]) : "memory", "m0");
+      globalLoadToLds16(pa[i], (uint32_t)(uintptr_t)(LdsPtr)(sA[buf] + (i * 256 + wave * 64) * 4));
+      globalLoadToLds16(pb[i], (uint32_t)(uintptr_t)(LdsPtr)(sB[buf] + (i * 256 + wave * 64) * 4));
       pa[i] += BK;
       pb[i] += stepB;
     }
