@@ -777,6 +777,14 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
 // written by gen_gemm_loop_4wave.py, which documents the schedule): tile loads straight into a two-stage LDS ring,
 // fragment reads one k-step ahead into fixed registers, one barrier per K tile. Needs an even number of K tiles and
 // the vector epilogue; everything else stays with the 8-wave kernel.
+//
+// Invariant the compiler does not check: between the PROLOGUE, BODY and TAIL statements, and from the TAIL to the last
+// accRegisters16 read of the epilogue, a0-a255 (the accumulators) and v120-v247 (operand fragments read ahead) are
+// live, but to the compiler they are only clobbers of each statement. The code in between (tile arithmetic, lane
+// offsets, the epilogue's conversions and address arithmetic) must therefore fit the other 128 ordinary registers
+// and touch no accumulation register, and nothing may spill: a reload would also stall behind the tile loads in
+// flight. build.py compiles this file with the resource-usage remark and fails when any instantiation reports
+// scratch or spills; tests/test_gpu_attention_gemm.py runs every instantiation by name on exact inputs.
 #include "gemm_loop_4wave.inc"
 
 // Sixteen consecutive accumulation registers a[R .. R + 15] as four fragments, in one statement: the reads issue back

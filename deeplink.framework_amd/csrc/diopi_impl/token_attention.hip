@@ -707,6 +707,11 @@ static diopiError_t decodeAttention(diopiContextHandle_t ctx, diopiTensorHandle_
   AMD_CHECK(out.defined() && out.dtype == t.q.dtype && out.numel == t.q.numel && out.isContiguous(),
             "token attention: out must be a dense tensor shaped like q");
   const int64_t batch = t.q.shape[0];
+  // The device address of the library's own array is looked up by the first call of either entry point on a device,
+  // so that a caller who records the allocation-free one into a graph only has to have run decode attention once,
+  // eagerly, on that device before: the lookup itself is then never made while a stream is being captured.
+  float* ownScratch = nullptr;
+  AMD_TRY(decodeScratch(&ownScratch));
   if (batch == 0 || t.q.numel == 0) return diopiSuccess;
   if (a.generic) {
     AMD_CHECK(batch <= 65535, "token attention: batch %ld exceeds the grid limits", (long)batch);
@@ -730,7 +735,7 @@ static diopiError_t decodeAttention(diopiContextHandle_t ctx, diopiTensorHandle_
                 (long)batch, a.heads, a.nsplit, a.chunk, (long)need, (long)kDecodeScratchBytes);
       // Nothing has to start at zero: the split kernel writes every (max, sum, acc) row the merge kernel uses, and
       // rows of splits that hold no tokens are read but discarded by a select.
-      AMD_TRY(decodeScratch(&partial));
+      partial = ownScratch;
     } else {
       void* ws = nullptr;
       AMD_TRY(requireWorkspace(ctx, need, &ws));

@@ -63,7 +63,7 @@ void fillStats(const DeviceStats& s, dipuAmdMemoryStats* o) {
 // Host-memory stand-in for the device: capacity-limited malloc, events that complete
 // only when the test says so.
 struct SimBackend {
-  uint64_t capacity = 0, inUse = 0, segments = 0;
+  uint64_t capacity = 0, inUse = 0, segments = 0, eventQueries = 0;
   uintptr_t nextAddr = uintptr_t(1) << 44;
   std::map<void*, size_t> live;
   struct SimEvent {
@@ -156,7 +156,10 @@ RawBackend makeSimBackend(SimBackend* sb) {
     ev->stream = s;
     ev->ready = false;
   };
-  b.eventReady = [](EventHandle e) { return static_cast<SimBackend::SimEvent*>(e)->ready; };
+  b.eventReady = [sb](EventHandle e) {
+    ++sb->eventQueries;
+    return static_cast<SimBackend::SimEvent*>(e)->ready;
+  };
   b.syncDevice = [sb]() {
     for (auto* e : sb->events) e->ready = true;
   };
@@ -368,6 +371,12 @@ int dipuAmdSimAllocatorDestroy(void* handle) {
 }
 int dipuAmdSimAllocatorMalloc(void* handle, void** p, size_t n, void* stream) {
   return guarded([&] { *p = static_cast<SimAllocator*>(handle)->alloc->malloc(n, stream); });
+}
+int dipuAmdSimAllocatorMallocFromCache(void* handle, void** p, size_t n, void* stream) {
+  return guarded([&] { *p = static_cast<SimAllocator*>(handle)->alloc->mallocFromCache(n, stream); });
+}
+int dipuAmdSimAllocatorEventQueries(void* handle, uint64_t* queries) {
+  return guarded([&] { *queries = static_cast<SimAllocator*>(handle)->backend.eventQueries; });
 }
 int dipuAmdSimAllocatorFree(void* handle, void* p) {
   return guarded([&] { static_cast<SimAllocator*>(handle)->alloc->free(p); });

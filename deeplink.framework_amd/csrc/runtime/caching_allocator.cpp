@@ -291,7 +291,9 @@ void* DeviceCachingAllocator::mallocFromCache(size_t size, StreamHandle stream) 
 void* DeviceCachingAllocator::malloc(size_t origSize, StreamHandle stream) {
   if (origSize == 0) return nullptr;
   std::lock_guard<std::recursive_mutex> lock(mutex_);
-  processEvents();
+  // A cache-only request comes from inside a stream capture, where an event query may be refused:
+  // blocks whose events are still pending stay parked until the next ordinary malloc.
+  if (!cacheOnly_) processEvents();
   size_t size = roundSize(origSize, config_);
   BlockPool& pool = size <= kSmallSize ? small_ : large_;
   size_t allocSize = allocationSize(size, config_);

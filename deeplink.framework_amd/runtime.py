@@ -294,6 +294,16 @@ class SimAllocator:
         _check(_rt().dipuAmdSimAllocatorMalloc(self.h, byref(p), c_size_t(n), c_void_p(stream)))
         return p.value or 0
 
+    def malloc_from_cache(self, n, stream=0):
+        p = c_void_p()
+        _check(_rt().dipuAmdSimAllocatorMallocFromCache(self.h, byref(p), c_size_t(n), c_void_p(stream)))
+        return p.value or 0
+
+    def event_queries(self):
+        n = c_uint64()
+        _check(_rt().dipuAmdSimAllocatorEventQueries(self.h, byref(n)))
+        return n.value
+
     def free(self, p):
         _check(_rt().dipuAmdSimAllocatorFree(self.h, c_void_p(p)))
 

@@ -94,7 +94,11 @@ DIOPI_API diopiError_t diopiTokenDecodeAttentionInference(diopiContextHandle_t c
  * the call makes no hipMalloc, hipFree or workspace request. It has no counterpart in the reference. Fails with a
  * clear error when batch x heads x splits x (2 + head_dim) x 4 bytes exceeds 32 MiB (splits = ceil(max_input_len /
  * 512), at most 64; batch 64 x 32 heads x head_dim 128 fits up to max_input_len 15872). Every call on a device
- * shares that device's array: calls that overlap on one device (two streams, two threads) race. */
+ * shares that device's array: calls that overlap on one device (two streams, two threads) race, and so do replays of
+ * graphs that hold this call when they run at the same time on different streams (every graph recorded on a device
+ * points at the same array). The array's device address is looked up by the first call of this function or of
+ * diopiTokenDecodeAttentionInference on a device: make that first call eagerly, outside stream capture, before
+ * recording this one into a graph. */
 DIOPI_API diopiError_t diopiTokenDecodeAttentionInferenceNoAlloc(diopiContextHandle_t ctx, diopiTensorHandle_t out,
                                                                  diopiConstTensorHandle_t q, diopiConstTensorHandle_t k,
                                                                  diopiConstTensorHandle_t v, diopiConstTensorHandle_t b_loc,

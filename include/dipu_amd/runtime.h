@@ -133,6 +133,11 @@ DIPU_AMD_API int dipuAmdSimAllocatorCreateBS(void** handle, uint64_t capacity_by
                                              int power_of_two);
 DIPU_AMD_API int dipuAmdSimAllocatorDestroy(void* handle);
 DIPU_AMD_API int dipuAmdSimAllocatorMalloc(void* handle, void** p, size_t nbytes, void* stream);
+/* The request a workspace allocation makes while its stream is being captured: served from cached blocks only
+ * (NULL when none fits), without querying any event. */
+DIPU_AMD_API int dipuAmdSimAllocatorMallocFromCache(void* handle, void** p, size_t nbytes, void* stream);
+/* How many times the allocator has asked the simulated device whether an event has completed. */
+DIPU_AMD_API int dipuAmdSimAllocatorEventQueries(void* handle, uint64_t* queries);
 DIPU_AMD_API int dipuAmdSimAllocatorFree(void* handle, void* p);
 DIPU_AMD_API int dipuAmdSimAllocatorRecordStream(void* handle, void* p, void* stream);
 DIPU_AMD_API int dipuAmdSimAllocatorEmptyCache(void* handle);

@@ -141,6 +141,25 @@ def test_record_stream_defers_reuse_until_event_completes(sim):
     assert r == p
 
 
+def test_cache_only_request_queries_no_event(sim):
+    # what a workspace request does while its stream is being captured: cached blocks only, no event query
+    a = sim()
+    s1, s2 = 0x1000, 0x2000
+    p = a.malloc(8192, s1)
+    a.record_stream(p, s2)
+    a.free(p)                                   # parked behind an event on s2 that has not completed
+    spare = a.malloc(4096, s1)
+    a.free(spare)
+    before = a.event_queries()
+    assert a.malloc_from_cache(4096, s1) == spare   # a cache hit
+    assert a.malloc_from_cache(64 * MiB, s1) == 0   # nothing cached fits: refused, nothing allocated
+    assert a.event_queries() == before
+    assert a.stats()["active_bytes"] == 8192 + 4096  # p is still held by its event
+    a.complete_events(s2)
+    q = a.malloc(8192, s1)                      # the next ordinary request sees the event and reuses p
+    assert q == p
+
+
 def test_oom_ladder_releases_cache_then_raises(pkg, sim):
     a = sim(capacity=64 * MiB)
     p = a.malloc(40 * MiB)

@@ -64,3 +64,34 @@ def test_no_alloc_decode_attention_requests_no_workspace_and_rejects_oversize(op
     # the allocating entry point takes the same call
     ops.token_decode_attention(q, pool, pool, big_loc, lens, lens, 40000)
     torch.cuda.synchronize()
+
+
+def test_no_alloc_decode_attention_recorded_into_a_graph_and_replayed(ops, dev, pkg):
+    """What the entry point is for: after one eager call on the device (the address lookup), the call is recorded into a
+    HIP graph with no workspace scope at all and replayed; every replay, with eager work and synchronizations between
+    them, equals the eager result bit for bit, also after the inputs changed in place."""
+    w, d = _case(pkg, dev, 15, 7, 8, 4000)
+    args = (d["q"], d["k_pool"], d["v_pool"], d["b_loc"], d["b_start_loc"], d["b_seq_len"], w["max_input_len"])
+    want = ops.token_decode_attention(*args)                    # eager: also warms the address lookup
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    out = torch.full_like(want, float("nan"))
+    mallocs = pkg.runtime.cachingStats()["num_device_malloc"]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        ops.token_decode_attention(*args, out=out, no_alloc=True)
+    assert pkg.runtime.cachingStats()["num_device_malloc"] == mallocs
+    for i in range(3):
+        out.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_exact(out, want)
+        # eager work of the same kind between replays (it uses the same device array)
+        ops.token_decode_attention(*args, out=torch.empty_like(want), no_alloc=True)
+        torch.cuda.synchronize()
+    d["q"].mul_(0.5)                                            # same buffers, new values
+    want2 = ops.token_decode_attention(*args)
+    graph.replay()
+    torch.cuda.synchronize()
+    assert_exact(out, want2)
+    del graph
