@@ -378,8 +378,7 @@ def decode_layer_step(pkg, torch, dev, rt, stream, g):
         P = lambda name, *a: Prepared(pkg, name, *a, hold=hold)
         return [P("diopiRMSNorm", h1, None, x, d.size([hidden]), n1, None, 1e-5),
                 P("diopiLinearRotary", qkv, h1, wqkv, None, cos, sin, 2 * hidden, hd, False, True),
-                P("diopiDestIndexCopyKV", g["k_pool"], k, g["dest_loc"]),
-                P("diopiDestIndexCopyKV", g["v_pool"], v, g["dest_loc"]),
+                P("diopiDestIndexCopyKVPair", g["k_pool"], k, g["v_pool"], v, g["dest_loc"]),
                 P("diopiTokenDecodeAttentionInference", att, q, g["k_pool"], g["v_pool"], g["b_loc"], g["b_start_loc"],
                   g["b_seq_len"], int(g["max_input_len"])),
                 P("diopiAddmm", x1, x, att.view(B, hidden), wo.t(), one, one),
@@ -422,7 +421,7 @@ def decode_layer_step(pkg, torch, dev, rt, stream, g):
     del graph
     for c in recorded:
         c.close()
-    return {"op": "decode layer step, 9 DIOPI calls", "workload": "7B-shaped layer, batch 64, paged KV as above",
+    return {"op": "decode layer step, 8 DIOPI calls", "workload": "7B-shaped layer, batch 64, paged KV as above",
             "us_eager_launches": round(t_eager, 2), "us_hip_graph_replay": round(t_graph, 2),
             "tokens_per_s_graph": round(B / (t_graph * 1e-6), 1), "replay_equals_eager": same}
 
@@ -488,6 +487,7 @@ def op_microbench(pkg, torch, dev, rt, stream, with_cpu=True):
     scat_bytes = 2 * 64 * 8192 * 2 + 2 * 64 * idx_b
     ck = Prepared(pkg, "diopiDestIndexCopyKV", g["k_pool"], g["k_new"], g["dest_loc"])
     cv = Prepared(pkg, "diopiDestIndexCopyKV", g["v_pool"], g["v_new"], g["dest_loc"])
+    ckv = Prepared(pkg, "diopiDestIndexCopyKVPair", g["k_pool"], g["k_new"], g["v_pool"], g["v_new"], g["dest_loc"])
     at = Prepared(pkg, "diopiTokenDecodeAttentionInference", out, g["q"], g["k_pool"], g["v_pool"], g["b_loc"],
                   g["b_start_loc"], g["b_seq_len"], int(g["max_input_len"]))
 
@@ -496,12 +496,12 @@ def op_microbench(pkg, torch, dev, rt, stream, with_cpu=True):
         cv()
 
     def step():
-        ck()
-        cv()
+        ckv()
         at()
-    p_sc, p_at, p_step = time_ops_stats(rt, stream, [scatter, at, step], 30, 6)
+    p_sc, p_pair, p_at, p_step = time_ops_stats(rt, stream, [scatter, ckv, at, step], 30, 6)
     t_step = p_step[0]
-    res.append(hbm_row("diopiDestIndexCopyKV(K)+(V)", "64 tokens into a 262144-slot pool", scat_bytes, None, p_sc))
+    res.append(hbm_row("diopiDestIndexCopyKV(K)+(V)", "64 tokens into a 262144-slot pool, two calls", scat_bytes, None, p_sc))
+    res.append(hbm_row("diopiDestIndexCopyKVPair", "64 tokens into a 262144-slot pool, K and V in one launch", scat_bytes, None, p_pair))
     res.append(hbm_row("diopiTokenDecodeAttentionInference", f"batch 64, 32x128, sum(len)={L}", attn_bytes, None, p_at))
     res.append({"op": "decode step (scatter + attention)", "workload": "batch 64", "us_cold": round(t_step, 2),
                 "us_cold_min": round(p_step[1], 2), "tokens_per_s": round(64 / (t_step * 1e-6), 1)})
@@ -510,7 +510,7 @@ def op_microbench(pkg, torch, dev, rt, stream, with_cpu=True):
         # (dipu/torch_dipu/csrc_dipu/aten/ops/CustomFallbackFunctions.hpp:78-91); one run each, no warm-up, they take seconds.
         def scatter_cpu(kp, vp, kn, vn, loc):
             return oracle.dest_index_copy_kv(kp, kn, loc), oracle.dest_index_copy_kv(vp, vn, loc)
-        res[-3]["cpu"] = cpu_op(torch, dev, scatter_cpu, (g["k_pool"], g["v_pool"], g["k_new"], g["v_new"], g["dest_loc"]), warm=1, runs=3)
+        res[-4]["cpu"] = cpu_op(torch, dev, scatter_cpu, (g["k_pool"], g["v_pool"], g["k_new"], g["v_new"], g["dest_loc"]), warm=1, runs=3)
         mil = int(pd["max_input_len"])
         res[-2]["cpu"] = cpu_op(torch, dev, lambda q, kp, vp, loc, ln: oracle.token_attention(q, kp, vp, loc, ln, mil),
                                 (g["q"], g["k_pool"], g["v_pool"], g["b_loc"], g["b_seq_len"]), warm=1, runs=3)

@@ -179,32 +179,46 @@ static diopiError_t launchRotary(hipStream_t stream, const TensorView& out, cons
 }
 
 // ---------------------------------------------------------------- KV scatter --
+// One workgroup per (token, pool): grid.y walks the pools of a call, so the K and the V row of a new token go out in
+// one launch (the op is all launch latency: 64 rows of 8 KiB).
+struct KvScatterPool {
+  void* out;
+  const void* src;
+  int64_t outRowStrideVecs, srcRowStrideVecs, slots;
+};
+struct KvScatterArgs {
+  KvScatterPool pool[2];
+  const void* destLoc;
+  int64_t tokens, rowVecs;
+};
+
 template <typename VEC, typename IDX>
-__global__ __launch_bounds__(256) void destIndexCopyKernel(VEC* __restrict__ out, const VEC* __restrict__ src,
-                                                            const IDX* __restrict__ destLoc, int64_t tokens,
-                                                            int64_t rowVecs, int64_t outRowStrideVecs,
-                                                            int64_t srcRowStrideVecs, int64_t slots) {
+__global__ __launch_bounds__(256) void destIndexCopyKernel(KvScatterArgs a) {
   const int64_t t = blockIdx.x;
-  if (t >= tokens) return;
-  int64_t slot = static_cast<int64_t>(destLoc[t]);
-  if (slot < 0) slot += slots;             // python-style negative index
-  if (slot < 0 || slot >= slots) return;   // an out-of-range slot is dropped, never written
-  const VEC* s = src + t * srcRowStrideVecs;
-  VEC* o = out + slot * outRowStrideVecs;
-  for (int64_t i = threadIdx.x; i < rowVecs; i += blockDim.x) o[i] = s[i];
+  if (t >= a.tokens) return;
+  const KvScatterPool& p = a.pool[blockIdx.y];
+  int64_t slot = static_cast<int64_t>(static_cast<const IDX*>(a.destLoc)[t]);
+  if (slot < 0) slot += p.slots;             // python-style negative index
+  if (slot < 0 || slot >= p.slots) return;   // an out-of-range slot is dropped, never written
+  const VEC* s = static_cast<const VEC*>(p.src) + t * p.srcRowStrideVecs;
+  VEC* o = static_cast<VEC*>(p.out) + slot * p.outRowStrideVecs;
+  for (int64_t i = threadIdx.x; i < a.rowVecs; i += blockDim.x) o[i] = s[i];
 }
 
+// Strides in `a` arrive in bytes and are scaled here to the widest vector every pointer, row length and stride allows.
 template <typename IDX>
-static diopiError_t launchDestCopy(hipStream_t stream, void* out, const void* src, const void* loc, int64_t tokens,
-                                   int64_t rowBytes, int64_t outRowStrideBytes, int64_t srcRowStrideBytes,
-                                   int64_t slots) {
-  uintptr_t bits = reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(src) | (uintptr_t)rowBytes |
-                   (uintptr_t)outRowStrideBytes | (uintptr_t)srcRowStrideBytes;
-  int threads = 256;
-#define KV_LAUNCH(VEC)                                                                                              \
-  hipLaunchKernelGGL((destIndexCopyKernel<VEC, IDX>), dim3((unsigned)tokens), dim3(threads), 0, stream, (VEC*)out,  \
-                     (const VEC*)src, (const IDX*)loc, tokens, rowBytes / (int64_t)sizeof(VEC),                     \
-                     outRowStrideBytes / (int64_t)sizeof(VEC), srcRowStrideBytes / (int64_t)sizeof(VEC), slots)
+static diopiError_t launchDestCopy(hipStream_t stream, KvScatterArgs a, int pools, int64_t rowBytes) {
+  uintptr_t bits = (uintptr_t)rowBytes;
+  for (int i = 0; i < pools; ++i)
+    bits |= reinterpret_cast<uintptr_t>(a.pool[i].out) | reinterpret_cast<uintptr_t>(a.pool[i].src) |
+            (uintptr_t)a.pool[i].outRowStrideVecs | (uintptr_t)a.pool[i].srcRowStrideVecs;
+#define KV_LAUNCH(VEC)                                                                                                   \
+  do {                                                                                                                   \
+    a.rowVecs = rowBytes / (int64_t)sizeof(VEC);                                                                         \
+    for (int i = 0; i < pools; ++i)                                                                                      \
+      a.pool[i].outRowStrideVecs /= (int64_t)sizeof(VEC), a.pool[i].srcRowStrideVecs /= (int64_t)sizeof(VEC);            \
+    hipLaunchKernelGGL((destIndexCopyKernel<VEC, IDX>), dim3((unsigned)a.tokens, (unsigned)pools), dim3(256), 0, stream, a); \
+  } while (0)
   if ((bits & 15) == 0) KV_LAUNCH(u32x4);
   else if ((bits & 7) == 0) KV_LAUNCH(u32x2);
   else if ((bits & 3) == 0) KV_LAUNCH(uint32_t);
@@ -365,6 +379,33 @@ diopiError_t amd::runRotary(diopiContextHandle_t ctx, hipStream_t stream, const 
   return diopiSuccess;
 }
 
+// Checks one (pool, new rows) pair of the scatter and fills its part of the launch arguments (strides in bytes).
+static diopiError_t kvScatterPool(diopiContextHandle_t ctx, hipStream_t stream, const char* what, const TensorView& out, const TensorView& k,
+                                  int64_t tokens, KvScatterPool* pool, int64_t* rowBytes) {
+  AMD_CHECK(out.defined() && k.defined(), "%s: null tensor", what);
+  AMD_CHECK(out.dtype == k.dtype, "%s: out dtype %s differs from k dtype %s", what, dtypeName(out.dtype), dtypeName(k.dtype));
+  AMD_CHECK(out.ndim == k.ndim && k.ndim >= 1, "%s: rank mismatch", what);
+  for (int d = 1; d < k.ndim; ++d) AMD_CHECK(out.shape[d] == k.shape[d], "%s: trailing extent mismatch at dim %d", what, d);
+  AMD_CHECK(k.shape[0] == tokens, "%s: dest_loc has %ld entries for %ld tokens", what, (long)tokens, (long)k.shape[0]);
+  if (tokens == 0 || k.numel == 0) {
+    *rowBytes = 0;
+    return diopiSuccess;
+  }
+  AMD_CHECK(out.shape[0] > 0, "%s: empty destination pool", what);
+  // rows (everything after dim 0) must be dense in both tensors; dim 0 may be strided
+  TensorView rowK = k, rowO = out;
+  rowK.shape[0] = rowO.shape[0] = 1;
+  TensorView ck = k;
+  if (!rowK.isContiguous()) AMD_TRY(makeContiguous(ctx, stream, k, &ck));
+  AMD_CHECK(rowO.isContiguous(), "%s: rows of the destination pool must be dense", what);
+  const int64_t rowElems = k.numel / tokens;
+  *rowBytes = rowElems * k.itemsize;
+  pool->out = out.data, pool->src = ck.data, pool->slots = out.shape[0];
+  pool->srcRowStrideVecs = (tokens > 1 ? ck.stride[0] : rowElems) * k.itemsize;
+  pool->outRowStrideVecs = (out.shape[0] > 1 ? out.stride[0] : rowElems) * out.itemsize;
+  return diopiSuccess;
+}
+
 extern "C" __attribute__((visibility("default"))) diopiError_t diopiDestIndexCopyKV(diopiContextHandle_t ctx,
                                                                                     diopiTensorHandle_t outH,
                                                                                     diopiConstTensorHandle_t kH,
@@ -375,36 +416,55 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiDestIndexCop
   AMD_TRY(getView(outH, &out, "out"));
   AMD_TRY(getView(kH, &k, "k"));
   AMD_TRY(getView(locH, &loc, "dest_loc"));
-  AMD_CHECK(out.defined() && k.defined() && loc.defined(), "diopiDestIndexCopyKV: null tensor");
-  AMD_CHECK(out.dtype == k.dtype, "diopiDestIndexCopyKV: out dtype %s differs from k dtype %s", dtypeName(out.dtype),
-            dtypeName(k.dtype));
-  AMD_CHECK(out.ndim == k.ndim && k.ndim >= 1, "diopiDestIndexCopyKV: rank mismatch");
-  for (int d = 1; d < k.ndim; ++d)
-    AMD_CHECK(out.shape[d] == k.shape[d], "diopiDestIndexCopyKV: trailing extent mismatch at dim %d", d);
+  AMD_CHECK(loc.defined(), "diopiDestIndexCopyKV: null tensor");
   AMD_CHECK(loc.dtype == diopi_dtype_int32 || loc.dtype == diopi_dtype_int64,
             "diopiDestIndexCopyKV: dest_loc must be int32 or int64, got %s", dtypeName(loc.dtype));
-  const int64_t tokens = k.shape[0];
-  AMD_CHECK(loc.numel == tokens, "diopiDestIndexCopyKV: dest_loc has %ld entries for %ld tokens", (long)loc.numel,
-            (long)tokens);
-  if (tokens == 0 || k.numel == 0) return diopiSuccess;
-  AMD_CHECK(out.shape[0] > 0, "diopiDestIndexCopyKV: empty destination pool");
-  // rows (everything after dim 0) must be dense in both tensors; dim 0 may be strided
-  TensorView rowK = k, rowO = out;
-  rowK.shape[0] = rowO.shape[0] = 1;
-  TensorView ck = k;
-  if (!rowK.isContiguous()) AMD_TRY(makeContiguous(ctx, stream, k, &ck));
-  AMD_CHECK(rowO.isContiguous(), "diopiDestIndexCopyKV: rows of the destination pool must be dense");
+  KvScatterArgs a;
+  int64_t rowBytes = 0;
+  a.tokens = loc.numel;
+  AMD_TRY(kvScatterPool(ctx, stream, "diopiDestIndexCopyKV", out, k, a.tokens, &a.pool[0], &rowBytes));
+  if (rowBytes == 0) return diopiSuccess;
+  a.pool[1] = a.pool[0];
   TensorView cloc;
   AMD_TRY(makeContiguous(ctx, stream, loc, &cloc));
-  const int64_t rowElems = k.numel / tokens;
-  const int64_t rowBytes = rowElems * k.itemsize;
-  const int64_t srcStride = (tokens > 1 ? ck.stride[0] : rowElems) * k.itemsize;
-  const int64_t outStride = (out.shape[0] > 1 ? out.stride[0] : rowElems) * out.itemsize;
-  if (loc.dtype == diopi_dtype_int32)
-    return launchDestCopy<int32_t>(stream, out.data, ck.data, cloc.data, tokens, rowBytes, outStride, srcStride,
-                                   out.shape[0]);
-  return launchDestCopy<int64_t>(stream, out.data, ck.data, cloc.data, tokens, rowBytes, outStride, srcStride,
-                                 out.shape[0]);
+  a.destLoc = cloc.data;
+  return loc.dtype == diopi_dtype_int32 ? launchDestCopy<int32_t>(stream, a, 1, rowBytes) : launchDestCopy<int64_t>(stream, a, 1, rowBytes);
+}
+
+// The K and the V rows of the new tokens into their two pools in one launch (see functions_ext.h): the same result as two
+// diopiDestIndexCopyKV calls with the same dest_loc.
+extern "C" __attribute__((visibility("default"))) diopiError_t diopiDestIndexCopyKVPair(diopiContextHandle_t ctx, diopiTensorHandle_t outKH,
+                                                                                        diopiConstTensorHandle_t kH, diopiTensorHandle_t outVH,
+                                                                                        diopiConstTensorHandle_t vH, diopiConstTensorHandle_t locH) {
+  hipStream_t stream;
+  AMD_TRY(getStream(ctx, &stream));
+  TensorView outK, k, outV, v, loc;
+  AMD_TRY(getView(outKH, &outK, "out_k"));
+  AMD_TRY(getView(kH, &k, "k"));
+  AMD_TRY(getView(outVH, &outV, "out_v"));
+  AMD_TRY(getView(vH, &v, "v"));
+  AMD_TRY(getView(locH, &loc, "dest_loc"));
+  AMD_CHECK(loc.defined(), "diopiDestIndexCopyKVPair: null tensor");
+  AMD_CHECK(loc.dtype == diopi_dtype_int32 || loc.dtype == diopi_dtype_int64,
+            "diopiDestIndexCopyKVPair: dest_loc must be int32 or int64, got %s", dtypeName(loc.dtype));
+  KvScatterArgs a;
+  int64_t rowBytesK = 0, rowBytesV = 0;
+  a.tokens = loc.numel;
+  AMD_TRY(kvScatterPool(ctx, stream, "diopiDestIndexCopyKVPair (k)", outK, k, a.tokens, &a.pool[0], &rowBytesK));
+  AMD_TRY(kvScatterPool(ctx, stream, "diopiDestIndexCopyKVPair (v)", outV, v, a.tokens, &a.pool[1], &rowBytesV));
+  if (rowBytesK == 0 && rowBytesV == 0) return diopiSuccess;
+  TensorView cloc;
+  AMD_TRY(makeContiguous(ctx, stream, loc, &cloc));
+  a.destLoc = cloc.data;
+  const bool i32 = loc.dtype == diopi_dtype_int32;
+  if (rowBytesK != rowBytesV) {  // rows of different length (or one side empty): one launch each
+    KvScatterArgs one = a;
+    if (rowBytesK) AMD_TRY(i32 ? launchDestCopy<int32_t>(stream, one, 1, rowBytesK) : launchDestCopy<int64_t>(stream, one, 1, rowBytesK));
+    one.pool[0] = a.pool[1];
+    if (rowBytesV) AMD_TRY(i32 ? launchDestCopy<int32_t>(stream, one, 1, rowBytesV) : launchDestCopy<int64_t>(stream, one, 1, rowBytesV));
+    return diopiSuccess;
+  }
+  return i32 ? launchDestCopy<int32_t>(stream, a, 2, rowBytesK) : launchDestCopy<int64_t>(stream, a, 2, rowBytesK);
 }
 
 extern "C" __attribute__((visibility("default"))) diopiError_t diopiIndexPutInp(

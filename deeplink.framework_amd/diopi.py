@@ -277,6 +277,7 @@ SIGNATURES = {
     "diopiRMSNorm": [_T, _T, _T, _SZ, _T, _T, c_double],
     "diopiRotaryEmbedding": [_T, _T, _T, _T, c_bool, c_bool],
     "diopiDestIndexCopyKV": [_T, _T, _T],
+    "diopiDestIndexCopyKVPair": [_T, _T, _T, _T, _T],
     "diopiTokenAttentionInference": [_T, _T, _T, _T, _T, _T, c_int],
     "diopiTokenSoftmaxReduceVInference": [_T, _T, _T, _T, _T, _T, c_int, c_int],
     "diopiContextAttentionInference": [_T, _T, _T, _T, _T, _T, c_int],

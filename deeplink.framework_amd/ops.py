@@ -624,6 +624,17 @@ def dest_index_copy_kv(k, dest_loc, out):
     return out
 
 
+def dest_index_copy_kv_pair(k, v, dest_loc, out_k, out_v):
+    """out_k[dest_loc[i]] = k[i] and out_v[dest_loc[i]] = v[i] in one launch (backend extension, functions_ext.h)."""
+    hok, pok = handle(out_k)
+    hk, pk = handle(k)
+    hov, pov = handle(out_v)
+    hv, pv = handle(v)
+    hl, pl = handle(dest_loc)
+    _call("diopiDestIndexCopyKVPair", pok, pk, pov, pv, pl)
+    return out_k, out_v
+
+
 def token_attention(q, k, attention_out, b_loc, b_start_loc, b_seq_len, max_input_len):
     ho, po = handle(attention_out)
     hq, pq = handle(q)

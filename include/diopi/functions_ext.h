@@ -88,6 +88,14 @@ DIOPI_API diopiError_t diopiTokenDecodeAttentionInference(diopiContextHandle_t c
                                                           diopiConstTensorHandle_t b_start_loc,
                                                           diopiConstTensorHandle_t b_seq_len, int max_input_len);
 
+/* The K row and the V row of every new token into their two pools in one launch: the same result, bit for bit, as
+ * diopiDestIndexCopyKV(out_k, k, dest_loc) followed by diopiDestIndexCopyKV(out_v, v, dest_loc). The scatter of a
+ * decode step moves a few hundred KiB and costs one launch latency per call; this halves it. The reference runs the two
+ * calls (lightllm's destindex_copy_kv for K and for V). */
+DIOPI_API diopiError_t diopiDestIndexCopyKVPair(diopiContextHandle_t ctx, diopiTensorHandle_t out_k,
+                                                diopiConstTensorHandle_t k, diopiTensorHandle_t out_v,
+                                                diopiConstTensorHandle_t v, diopiConstTensorHandle_t dest_loc);
+
 /* diopiTokenDecodeAttentionInference for callers that cannot allocate (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc): same arguments, same kernels, same result bit for bit, but the split-KV
  * partial results live in a 32 MiB device array inside the library instead of workspace from diopiRequireBuffer, and

@@ -347,6 +347,48 @@ def test_dest_index_copy_kv_bit_exact(ops, dev, dtype, idt):
     assert_exact(got, want)
 
 
+@pytest.mark.parametrize("idt", [torch.int32, torch.int64])
+def test_dest_index_copy_kv_pair_equals_two_calls(ops, dev, idt):
+    """K and V rows scattered in one launch: bit-identical pools to the two single calls and to the oracle, with
+    a strided source (slices of a stacked projection), a dropped out-of-range slot, rows of different length in the two
+    pools (two launches inside) and an empty batch."""
+    g0 = torch.Generator().manual_seed(5)
+    qkv = torch.randn(37, 3 * 4 * 64, generator=g0).bfloat16()
+    k, v = qkv[:, 256:512].view(37, 4, 64), qkv[:, 512:].view(37, 4, 64)
+    loc = torch.randperm(500, generator=g0)[:37].to(idt)
+    loc[5] = 700                                                   # outside the pool: dropped
+    pk, pv = torch.randn(500, 4, 64, generator=g0).bfloat16(), torch.randn(500, 4, 64, generator=g0).bfloat16()
+    keep = loc != 700
+    wk, wv = pk.clone(), pv.clone()
+    oracle.dest_index_copy_kv(wk, k[keep], loc[keep])
+    oracle.dest_index_copy_kv(wv, v[keep], loc[keep])
+    qd = qkv.to(dev)
+    kd, vd = qd[:, 256:512].view(37, 4, 64), qd[:, 512:].view(37, 4, 64)
+    gk, gv = pk.to(dev), pv.to(dev)
+    ops.dest_index_copy_kv_pair(kd, vd, loc.to(dev), gk, gv)
+    assert_exact(gk, wk)
+    assert_exact(gv, wv)
+    sk, sv = pk.to(dev), pv.to(dev)
+    ops.dest_index_copy_kv(kd, loc.to(dev), sk)
+    ops.dest_index_copy_kv(vd, loc.to(dev), sv)
+    assert_exact(gk, sk.cpu())
+    assert_exact(gv, sv.cpu())
+    # V rows half as long as K rows
+    v2, pv2 = torch.randn(37, 4, 32, generator=g0).bfloat16(), torch.zeros(500, 4, 32, dtype=torch.bfloat16)
+    gk, gv2 = pk.to(dev), pv2.to(dev)
+    ops.dest_index_copy_kv_pair(kd, v2.to(dev), loc.to(dev), gk, gv2)
+    wv2 = pv2.clone()
+    oracle.dest_index_copy_kv(wv2, v2[keep], loc[keep])
+    assert_exact(gk, wk)
+    assert_exact(gv2, wv2)
+    # no tokens: nothing happens
+    ops.dest_index_copy_kv_pair(torch.empty(0, 4, 64, dtype=torch.bfloat16, device=dev), torch.empty(0, 4, 64, dtype=torch.bfloat16, device=dev),
+                                torch.empty(0, dtype=idt, device=dev), gk, gv)
+    assert_exact(gk, wk)
+    with pytest.raises(Exception, match="dest_loc has"):
+        ops.dest_index_copy_kv_pair(kd, vd[:5], loc.to(dev), gk, gv)
+
+
 def test_dest_index_copy_kv_full_pool_round_trip(ops, dev, pkg):
     w = pkg.workloads.paged_decode(seed=0, fill_pool=False)
     pool = torch.zeros_like(w["k_pool"]).to(dev)
