@@ -10,6 +10,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <utility>
+
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -182,6 +184,17 @@ __device__ __forceinline__ void loadToLds16Stream(u32x4 rsrc, int voffset, int s
       : "=&s"(savedM0)
       : "s"(ldsAddr), "v"(voffset), "s"(rsrc), "s"(soffset)
       : "memory");
+}
+
+template <int... Is, typename F>
+__device__ __forceinline__ void staticForImpl(std::integer_sequence<int, Is...>, F&& f) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+// f(std::integral_constant<int, 0>{}) ... f(std::integral_constant<int, N - 1>{}): a loop whose index is a constant
+// expression in the body (register names of inline assembly, array indices that must not become run-time).
+template <int N, typename F>
+__device__ __forceinline__ void staticFor(F&& f) {
+  staticForImpl(std::make_integer_sequence<int, N>{}, f);
 }
 
 template <typename T>

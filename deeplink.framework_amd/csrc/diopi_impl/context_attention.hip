@@ -95,6 +95,11 @@ __device__ __forceinline__ int vSwizzle(int key) {
 }
 
 constexpr int kCaBQ = 128, kCaBKV = 64;
+// A new row maximum replaces the running one only when it exceeds it by more than this (log2 domain). Until then the
+// probabilities of a tile are taken against the stale maximum (at most 2^8: harmless in the fp32 sums and in bf16 / fp16
+// operands) and the softmax is the same; the rescale of O^T, which otherwise runs in most tiles (one of a wave's 32
+// queries nearly always sees a new maximum), becomes rare.
+constexpr float kCaRescaleStep = 8.0f;
 
 // One 128-query block of one (sequence, head): the whole flash-attention pass over its key tiles.
 template <typename T, int D>
@@ -183,12 +188,23 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
   // K fragment i of a tile: key half i & 1 (32 keys), head-dim step i >> 1. A ring of them runs kKAhead
   // MFMAs ahead of the score MFMAs, and the first kKAhead of the NEXT tile are read at the end of the
   // P.V loop, so no score MFMA waits for LDS.
-  constexpr int NS = 2 * KS, kKAhead = 4;
+  // Addresses: the XOR swizzles touch only bits that the rest of a fragment's address leaves zero, so the LDS byte
+  // address is (lane constant + stage) ^ (step constant) plus an immediate: one register per matrix, made opaque per
+  // tile so that the derived addresses are recomputed (one XOR each) rather than kept or re-derived with several adds.
+  constexpr int NS = 2 * KS, kKAhead = 4, ROWB = D * (int)sizeof(T);
+  constexpr unsigned kStageBytes = STAGE * sizeof(T);
   Frag kfr[kKAhead + 1];
-  auto kfrag = [&](const T* k, int i) {
-    const int key = (i & 1) * 32 + l31, chunk = (i >> 1) * 2 + half;
-    return *reinterpret_cast<const Frag*>(k + key * D + ((chunk ^ kSwizzle<D>(key)) << 3));
+  const int kswz = kSwizzle<D>(l31);
+  const unsigned kLane = (unsigned)(l31 * ROWB + ((half ^ (kswz & 1)) << 4) + ((kswz >> 1) << 5));
+  typedef __attribute__((address_space(3))) const Frag* LdsFrag;
+  auto kfragAt = [&](unsigned kBase, int i) {  // kBase = kLane + LDS byte address of the stage
+    return *(LdsFrag)(uintptr_t)((kBase ^ (unsigned)((i >> 1) << 5)) + (unsigned)((i & 1) * 32 * ROWB));
   };
+  auto opaque = [](unsigned x) {
+    asm volatile("" : "+v"(x));
+    return x;
+  };
+  const unsigned ldsK0 = (unsigned)(uintptr_t)sK, ldsV0 = (unsigned)(uintptr_t)sV;
   // The barrier of tile t sits between its softmax and its P.V: it publishes K of tile t + 1 and V of tile t,
   // and it says that every wave is done with K of tile t and V of tile t - 1, whose stages the copies
   // issued right after it (K of t + 2, V of t + 1) overwrite. Every copy has a whole tile to land.
@@ -197,14 +213,13 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
   tileBarrier();
   if (ntiles > 1) copyK(1, 1);
 #pragma unroll
-  for (int i = 0; i < kKAhead; ++i) kfr[i] = kfrag(sK, i);
+  for (int i = 0; i < kKAhead; ++i) kfr[i] = kfragAt(kLane + ldsK0, i);
 
   for (int t = 0; t < ntiles; ++t) {
     const int cur = t & 1;
     const int k0 = t * kCaBKV;
     const bool live = k0 <= waveMaxQ;  // wave-uniform; once false it stays false
-    const T* k = sK + cur * STAGE;
-    const T* v = sV + cur * STAGE;
+    const unsigned kCur = opaque(kLane + ldsK0 + cur * kStageBytes), kOther = opaque(kLane + ldsK0 + (cur ^ 1) * kStageBytes);
     f32x16 s[2];
     if (live) {
 #pragma unroll
@@ -218,7 +233,7 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
       // waits for the one issued just before it
 #pragma unroll
       for (int i = 0; i < NS; ++i) {
-        if (i + kKAhead < NS) kfr[(i + kKAhead) % (kKAhead + 1)] = kfrag(k, i + kKAhead);
+        if (i + kKAhead < NS) kfr[(i + kKAhead) % (kKAhead + 1)] = kfragAt(kCur, i + kKAhead);
         s[i & 1] = CaMfma<T>::run(kfr[i % (kKAhead + 1)], qf[i >> 1], s[i & 1]);
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -244,7 +259,8 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
         const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mt), __float_as_uint(mt), false, false);
         mt = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1])) * scale2;  // scale2 > 0, so the max commutes with the scaling
       }
-      const float mn = fmaxf(m, mt);  // key 0 is visible to every query, so mn is finite from tile 0 on
+      // key 0 is visible to every query, so mn is finite from tile 0 on (m = -inf there: the difference is +inf)
+      const float mn = mt - m > kCaRescaleStep ? mt : m;
 #pragma unroll
       for (int kt2 = 0; kt2 < 2; ++kt2)
 #pragma unroll
@@ -279,16 +295,16 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
         // keys 8 r + 4 half + 0..3 of the step: the order the P^T operand holds them in.
         const int trKey = half * 4 + ((lane & 15) >> 2);
         const int trChunk = ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1), trIn = (lane & 1) * 4;
+        const int vsw = D == 128 ? (trKey & 3) : ((trKey >> 1) & 1);  // vSwizzle<D>(key) / 4: the low bits of the d tile
+        const unsigned vCur = opaque((unsigned)(trKey * ROWB + (trChunk << 4) + trIn * 2 + (vsw << 6)) + ldsV0 + cur * kStageBytes);
+        typedef __attribute__((address_space(3))) s16x4* LdsTr;
         auto vfrag = [&](int i) {
           const int g = i / DT, dt = i % DT;  // key group (kt2 * 2 + t2), d tile
           Half part[2];
 #pragma unroll
-          for (int r = 0; r < 2; ++r) {
-            const int key = g * 16 + r * 8 + trKey;
-            const T* p = v + key * D + (((dt * 4 + trChunk) ^ vSwizzle<D>(key)) << 3) + trIn;
+          for (int r = 0; r < 2; ++r)
             part[r] = __builtin_bit_cast(Half, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                                                   (__attribute__((address_space(3))) s16x4*)p));
-          }
+                                                   (LdsTr)(uintptr_t)((vCur ^ (unsigned)(dt << 6)) + (unsigned)((g * 16 + r * 8) * ROWB))));
           Frag vf;
           vf[0] = part[0][0], vf[1] = part[0][1], vf[2] = part[0][2], vf[3] = part[0][3];
           vf[4] = part[1][0], vf[5] = part[1][1], vf[6] = part[1][2], vf[7] = part[1][3];
@@ -316,7 +332,7 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
           }
           if (i + kVAhead < NPV) vfr[(i + kVAhead) % (kVAhead + 1)] = vfrag(i + kVAhead);
           // the next tile's first K fragments (after the last tile: a harmless read of the other stage)
-          if (i >= NPV - kKAhead) kfr[i - (NPV - kKAhead)] = kfrag(sK + (cur ^ 1) * STAGE, i - (NPV - kKAhead));
+          if (i >= NPV - kKAhead) kfr[i - (NPV - kKAhead)] = kfragAt(kOther, i - (NPV - kKAhead));
           o[dt] = CaMfma<T>::run(vfr[i % (kVAhead + 1)], pf, o[dt]);
           __builtin_amdgcn_sched_barrier(0);
         }

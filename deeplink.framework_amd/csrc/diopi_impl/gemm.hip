@@ -303,17 +303,6 @@ struct MfmaOp16<half_t> {
 // embedding on the leading rotCols columns (the q and k heads of a stacked QKV projection).
 enum PipeEpilogue { kEpiLinear = 0, kEpiSiluMul = 1, kEpiPartial = 2, kEpiRotary = 3 };
 
-template <int... Is, typename F>
-__device__ __forceinline__ void staticForImpl(std::integer_sequence<int, Is...>, F&& f) {
-  (f(std::integral_constant<int, Is>{}), ...);
-}
-// f(std::integral_constant<int, 0>{}) ... f(std::integral_constant<int, N - 1>{}): a loop whose index is a constant
-// expression in the body (register names of inline assembly, array indices that must not become run-time).
-template <int N, typename F>
-__device__ __forceinline__ void staticFor(F&& f) {
-  staticForImpl(std::make_integer_sequence<int, N>{}, f);
-}
-
 // The vector epilogue of the 256 x 256 kernels: a wave's TM x TN fragments of 16 x 16 (v_mfma_f32_16x16x32 with the
 // weight fragment first, so lane (frow = l & 15, kq = l >> 4) holds columns 4 kq .. 4 kq + 3 of row frow of every
 // fragment) whose first row is row0 and first column colBase; accRow(ic, row) hands over the TN accumulators of
