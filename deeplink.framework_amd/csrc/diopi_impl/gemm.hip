@@ -503,19 +503,23 @@ __device__ __forceinline__ void vectorEpilogue(const MfmaArgs& g, T* out, const 
 }
 
 
-template <typename T, int EPI>
-__global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs g) {
+// TILE is the edge of the square macro tile: 256 (8 waves, 2 x 4, wave tile 128 x 64) or 128 (4 waves, 2 x 2, wave
+// tile 64 x 64, 64 KiB of LDS, two workgroups per CU) for problems with too few 256 x 256 tiles to fill the chip:
+// the same pipeline with half as many A fragments per phase.
+template <typename T, int EPI, int TILE = 256>
+__global__ __launch_bounds__(TILE == 256 ? kPipeThreads : 256, TILE == 256 ? 1 : 2) void gemmMfmaPipelinedKernel(MfmaArgs g) {
   using Frag = typename MfmaOp<T>::Frag;
-  constexpr int BM = 256, BN = 256, WM = BM / kPipeWavesM, WN = BN / kPipeWavesN, TM = WM / 16, TN = WN / 16;
-  constexpr int HM = TM / 2;               // A fragments of one phase (half of the wave's rows)
-  constexpr int CH = 2048 / kPipeThreads;  // 16-byte chunks per thread per operand tile
-  constexpr int RS = kPipeThreads / 8;     // rows covered by one pass of the workgroup
-  static_assert(HM == 4 && TN == 4 && CH == 4, "the phase schedule below is written for 4 x 4 fragments");
+  constexpr int kWavesN = TILE == 256 ? kPipeWavesN : 2, kThreads = TILE == 256 ? kPipeThreads : 256;
+  constexpr int BM = TILE, BN = TILE, WM = BM / kPipeWavesM, WN = BN / kWavesN, TM = WM / 16, TN = WN / 16;
+  constexpr int HM = TM / 2;                 // A fragments of one phase (half of the wave's rows)
+  constexpr int CH = BM * 8 / kThreads;      // 16-byte chunks per thread per operand tile
+  constexpr int RS = kThreads / 8;           // rows covered by one pass of the workgroup
+  static_assert((HM == 4 || HM == 2) && TN == 4 && CH == 4, "the phase schedule below is written for 4 (or 2) x 4 fragments");
   extern __shared__ __attribute__((aligned(16))) char smem[];
   T* sA = reinterpret_cast<T*>(smem);  // [2][BM][64]
   T* sB = sA + 2 * BM * kBK;           // [2][BN][64]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave / kPipeWavesN, wn = wave % kPipeWavesN;
+  const int wm = wave / kWavesN, wn = wave % kWavesN;
   int tm, tn;
   {
     const int total = g.tilesM * g.tilesN;
@@ -637,7 +641,7 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
     // ---- phase 0: k-step 0, rows 0-63 | A fragments of phase 1 | B half of the next tile
     phase(0, 0,
           [&](int j) {
-            if (j < 2) {
+            if (j < HM / 2) {
               loadA(cur, 0, 1, 1, 2 * j);
               loadA(cur, 0, 1, 1, 2 * j + 1);
             }
@@ -648,7 +652,7 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
     // ---- phase 1: k-step 0, rows 64-127 | A of phase 2, B of k-step 1
     phase(1, 1,
           [&](int j) {
-            if (j < 2) {
+            if (j < HM / 2) {
               loadA(cur, 1, 0, 0, 2 * j);
               loadA(cur, 1, 0, 0, 2 * j + 1);
             }
@@ -657,7 +661,7 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
     // ---- phase 2: k-step 1, rows 0-63 | A of phase 3
     phase(0, 0,
           [&](int j) {
-            if (j < 2) {
+            if (j < HM / 2) {
               loadA(cur, 1, 1, 1, 2 * j);
               loadA(cur, 1, 1, 1, 2 * j + 1);
             }
@@ -670,7 +674,7 @@ __global__ __launch_bounds__(kPipeThreads) void gemmMfmaPipelinedKernel(MfmaArgs
           [&](int j) {
             if constexpr (kNext2) dmaA(cur, kt + 2, j);
             if constexpr (kNext) {
-              if (j < 2) {
+              if (j < HM / 2) {
                 loadA(cur ^ 1, 0, 0, 0, 2 * j);
                 loadA(cur ^ 1, 0, 0, 0, 2 * j + 1);
               }
@@ -1868,12 +1872,12 @@ __global__ __launch_bounds__(256) void splitKReduceKernel(MfmaArgs g, int splits
   *reinterpret_cast<Frag*>(reinterpret_cast<T*>(g.out) + (int64_t)row * g.ldo + col) = o;
 }
 
-// How many ways to split K so that a problem with few 256 x 256 tiles still fills the chip: tiles * splits close
-// to the CU count, at least four K tiles per split, at most 16 splits. 1 = do not split.
+// How many ways to split K so that a problem with few 128 x 128 tiles still fills the chip (two workgroups per CU):
+// tiles * splits close to twice the CU count, at least four K tiles per split, at most 16 splits. 1 = do not split.
 // *perSplit receives the K tiles per split; the last split has the remainder, never fewer than two (the kernel's
 // pipeline needs two).
 static int splitKWays(int64_t tiles, int64_t kTiles, int* perSplit) {
-  const int64_t byChip = computeUnits() / std::max<int64_t>(tiles, 1), byK = kTiles / 4;
+  const int64_t byChip = 2 * computeUnits() / std::max<int64_t>(tiles, 1), byK = kTiles / 4;
   int64_t splits = std::max<int64_t>(1, std::min<int64_t>(16, std::min(byChip, byK)));
   int64_t per = ceilDiv(kTiles, splits);
   while (per < kTiles && kTiles % per == 1) ++per;
@@ -1930,6 +1934,40 @@ static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p
     }
   }
   hipLaunchKernelGGL((gemmMfmaPipelinedKernel<T, EPI>), grid, dim3(kPipeThreads), lds, stream, g);
+  AMD_LAUNCH_CHECK();
+  if (EPI == kEpiPartial) {
+    const int64_t items = p.M * (p.N / 8);
+    hipLaunchKernelGGL(splitKReduceKernel<T>, dim3((unsigned)ceilDiv(items, 256)), dim3(256), 0, stream, g, splits);
+    AMD_LAUNCH_CHECK();
+  }
+  return diopiSuccess;
+}
+
+// The 128 x 128 form of the pipelined kernel (4 waves, two workgroups per CU): linear epilogue, or fp32 partial
+// products of a K split followed by the reduction pass.
+template <typename T, int EPI = kEpiLinear>
+static diopiError_t launchMfmaPipelined128(hipStream_t stream, const GemmProblem& p, float* partial = nullptr, int splits = 1,
+                                           int kTilesPerSplit = 0) {
+  static_assert(EPI == kEpiLinear || EPI == kEpiPartial, "the 128 x 128 form has the linear and the split-K epilogues");
+  MfmaArgs g;
+  g.A = p.A, g.B = p.B, g.out = p.out, g.Cin = p.Cin, g.bias = p.bias;
+  g.sAb = p.sAb, g.lda = p.sAm, g.sBb = p.sBb, g.ldb = p.sBn, g.sOb = p.sOb, g.ldo = p.sOm;
+  g.sCb = p.sCb, g.sCm = p.sCm, g.sCn = p.sCn;
+  g.M = (int)p.M, g.N = (int)p.N, g.K = (int)p.K;
+  g.tilesM = (int)ceilDiv(p.M, 128), g.tilesN = (int)ceilDiv(p.N, 128);
+  g.alpha = p.alpha, g.beta = p.beta;
+  auto al16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+  const bool span32 = ((p.M - 1) * p.sOm + p.N) * (int64_t)sizeof(T) < (int64_t(1) << 31) &&
+                      (!p.Cin || ((p.M - 1) * p.sCm + p.N) * (int64_t)sizeof(T) < (int64_t(1) << 31));
+  g.vecEpilogue = p.N % 8 == 0 && p.sOm % 8 == 0 && p.sOb % 8 == 0 && al16(p.out) && span32 &&
+                  (!p.Cin || (p.sCn == 1 && p.sCm % 8 == 0 && p.sCb % 8 == 0 && al16(p.Cin))) && (!p.bias || al16(p.bias));
+  g.partial = partial;
+  g.kTilesPerSplit = kTilesPerSplit;
+  if (EPI == kEpiPartial) AMD_CHECK(g.vecEpilogue && p.batch == 1 && partial, "split-K: needs the vector epilogue and one batch");
+  constexpr size_t lds = 2 * (size_t)(128 + 128) * kBK * sizeof(T);
+  AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmMfmaPipelinedKernel<T, EPI, 128>), (int)lds));
+  dim3 grid((unsigned)(g.tilesM * g.tilesN), (unsigned)splits, (unsigned)p.batch);
+  hipLaunchKernelGGL((gemmMfmaPipelinedKernel<T, EPI, 128>), grid, dim3(256), lds, stream, g);
   AMD_LAUNCH_CHECK();
   if (EPI == kEpiPartial) {
     const int64_t items = p.M * (p.N / 8);
@@ -2163,18 +2201,24 @@ diopiError_t runGemm(diopiContextHandle_t ctx, hipStream_t stream, GemmProblem p
     }
     // In between (too few 256 x 256 tiles for the chip, too many rows for the weight-streaming kernel): the same
     // large-tile kernel with K split over grid.y, fp32 partial products in workspace and a reduction pass.
-    if (!big && p.batch == 1 && p.K % kBK == 0 && fits2g && p.N % 8 == 0 && p.sOm % 8 == 0 && ptr16(p.out) &&
-        (!p.Cin || (p.sCn == 1 && p.sCm % 8 == 0 && ptr16(p.Cin))) && (!p.bias || ptr16(p.bias)) &&
-        p.M * p.N * 4 < (int64_t(1) << 31)) {
+    // In between (too few 256 x 256 tiles for the chip, too many rows for the weight-streaming kernels): the 128 x 128
+    // form of the pipelined kernel, two workgroups per CU, and when even its tiles are fewer than the 2 x CUs the chip
+    // holds, K split over grid.y with fp32 partial products in workspace and a reduction pass. Measured against
+    // the 256 x 256 tiles split over K that this replaces (rows x 4096 x 4096, us): 128 rows 23.6 -> 21.5, 256 33.5 -> 22.3,
+    // 512 37.4 -> 27.9, 1024 48.0 -> 41.7, 2048 71.3 -> 58.0; x 22016 x 4096: 128 rows 51.0 -> 38.8; K = 11008: 256 rows 45.0 -> 35.9.
+    if (!big && p.K % kBK == 0 && p.K >= 2 * kBK && fits2g) {
+      const int64_t tiles128 = ceilDiv(p.M, 128) * ceilDiv(p.N, 128) * p.batch;
+      const bool vecOk = p.N % 8 == 0 && p.sOm % 8 == 0 && ptr16(p.out) && (!p.Cin || (p.sCn == 1 && p.sCm % 8 == 0 && ptr16(p.Cin))) &&
+                         (!p.bias || ptr16(p.bias)) && p.M * p.N * 4 < (int64_t(1) << 31);
       int per = 0;
-      const int splits = splitKWays(ceilDiv(p.M, 256) * ceilDiv(p.N, 256), p.K / kBK, &per);
+      const int splits = p.batch == 1 && vecOk ? splitKWays(tiles128, p.K / kBK, &per) : 1;
       if (splits >= 2) {
         void* ws = nullptr;
         AMD_TRY(requireWorkspace(ctx, (int64_t)splits * p.M * p.N * 4, &ws));
-        return p.dtype == diopi_dtype_bfloat16
-                   ? launchMfmaPipelined<bf16_t, kEpiPartial>(stream, p, static_cast<float*>(ws), splits, per)
-                   : launchMfmaPipelined<half_t, kEpiPartial>(stream, p, static_cast<float*>(ws), splits, per);
+        return p.dtype == diopi_dtype_bfloat16 ? launchMfmaPipelined128<bf16_t, kEpiPartial>(stream, p, static_cast<float*>(ws), splits, per)
+                                               : launchMfmaPipelined128<half_t, kEpiPartial>(stream, p, static_cast<float*>(ws), splits, per);
       }
+      return p.dtype == diopi_dtype_bfloat16 ? launchMfmaPipelined128<bf16_t>(stream, p) : launchMfmaPipelined128<half_t>(stream, p);
     }
     if (p.dtype == diopi_dtype_bfloat16) {
       return big ? launchMfma<bf16_t, 256, 256>(stream, p) : launchMfma<bf16_t, 128, 128>(stream, p);
