@@ -159,6 +159,36 @@ def test_large_tile_gemm_batched_and_row_strided_operands(ops, dev):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("batch,m,k,n", [(1, 4096, 512, 4096),      # 256 x 256 tiles
+                                         (1, 1024, 4096, 4096),     # 128 x 128 tiles
+                                         (1, 200, 1024, 520),       # 128 x 128 tiles, K split, ragged edges
+                                         (3, 700, 128, 136),        # batched, two K tiles, a narrow matrix
+                                         (16, 2048, 2048, 128),     # the P . V product of decomposed attention
+                                         (2, 2304, 192, 2048)])     # batched 256 x 256 tiles, three K tiles
+def test_second_operand_read_in_place_as_k_by_n(ops, dev, dtype, batch, m, k, n):
+    """mm / bmm / matmul with the right-hand side as the caller holds it, [K, N] row-major: the tile kernels read it in
+    place. Checked against the fp32 product, and exactly: one-hot rows on the left select rows of the right."""
+    g0 = g(91)
+    a = torch.randn(batch, m, k, generator=g0).to(dtype)
+    b = (torch.randn(batch, k, n, generator=g0) * 0.05).to(dtype)
+    want = a.float() @ b.float()
+    got = ops.bmm(a.to(dev), b.to(dev)) if batch > 1 else ops.mm(a[0].to(dev), b[0].to(dev)).unsqueeze(0)
+    assert_half(got, want)
+    rows = torch.randint(0, k, (batch, m), generator=g0)
+    onehot = torch.zeros(batch, m, k, dtype=dtype)
+    onehot.scatter_(2, rows.unsqueeze(-1), 1)
+    sel = torch.gather(b, 1, rows.unsqueeze(-1).expand(batch, m, n))
+    got = ops.bmm(onehot.to(dev), b.to(dev)) if batch > 1 else ops.mm(onehot[0].to(dev), b[0].to(dev)).unsqueeze(0)
+    assert_exact(got, sel)
+    if batch == 1:
+        # a column slice of a wider matrix as the right-hand side (row stride above N), through matmul with a broadcast left side
+        wide = (torch.randn(k, n + 64, generator=g0) * 0.05).to(dtype)
+        a3 = torch.randn(2, m, k, generator=g0).to(dtype)
+        got = ops.matmul(a3.to(dev), wide.to(dev)[:, 8:8 + n])
+        assert_half(got, a3.float() @ wide[:, 8:8 + n].float())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("epilogue", ["linear", "bias", "addend", "rotary", "silu_mul"])
 def test_four_wave_gemm_every_instantiation_exact(ops, dev, dtype, epilogue):
     """Every instantiation of the 4-wave large-tile kernel (two dtypes x plain, bias, addend, rotary and gated
