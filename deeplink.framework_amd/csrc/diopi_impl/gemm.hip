@@ -2068,6 +2068,15 @@ static diopiError_t launchSkinnyLds(hipStream_t stream, const SkinnyArgs& a) {
   const int splits = (a.K + a.kPerWg - 1) / a.kPerWg;
   hipLaunchKernelGGL((gemmSkinnyLdsKernel<T, G, NTP, WST, XST>), dim3((unsigned)((a.N + a.colsPerWg - 1) / a.colsPerWg), (unsigned)splits), dim3(512), lds, stream, a);
   AMD_LAUNCH_CHECK();
+  if (a.partial) {
+    MfmaArgs g;
+    g.out = a.out, g.Cin = a.Cin, g.bias = a.bias, g.partial = a.partial;
+    g.ldo = a.ldo, g.sCm = a.sCm, g.sCn = a.sCn;
+    g.M = a.M, g.N = a.N, g.K = a.K, g.alpha = a.alpha, g.beta = a.beta;
+    hipLaunchKernelGGL(splitKReduceKernel<T>, dim3((unsigned)ceilDiv((int64_t)a.M * (a.N / 8), 256)), dim3(256), 0, stream, g,
+                       splits);
+    AMD_LAUNCH_CHECK();
+  }
   return diopiSuccess;
 }
 
@@ -2120,11 +2129,25 @@ static diopiError_t launchSkinnyForShape(diopiContextHandle_t ctx, hipStream_t s
   // 52.9 -> 33.6, 55.7 -> 36.0. At N = 4096 (16 columns per workgroup: the activations are four times the weight
   // bytes on the way into a CU) only 17 to 32 rows gain (14.4 -> 12.7); one row loses (9.1 -> 11.0), and so does
   // everything narrower.
-  if ((a.N >= 5120 || (a.N >= 4096 && a.M > 16 && a.M <= 32)) &&
+  // A 4096-wide weight with a long K at 33 to 64 rows (the down projection of a decode step) takes this form too, K
+  // split two ways over grid.y with fp32 slices and the reduction pass: 64 x 4096 x 11008 34.0 -> 27.6 us cold against the
+  // register-layout kernels below. The same split on wider weights loses (N = 11008: 23.0 -> 25.5 us, four ways 33.6),
+  // and at K = 4096 it changes nothing (14.6 -> 15.0).
+  const bool canSplitLds = a.N % 8 == 0 && mult8(p.sOm) && ptr16(p.out) && (!p.bias || ptr16(p.bias)) &&
+                           (!p.Cin || (p.sCn == 1 && mult8(p.sCm) && ptr16(p.Cin))) && rot == nullptr;
+  const bool narrowLongK = a.N >= 4096 && a.N < 5120 && a.M > 32 && a.K >= 8192 && a.K % (2 * kSkinnyLdsBK) == 0 && canSplitLds;
+  if ((a.N >= 5120 || (a.N >= 4096 && a.M > 16 && a.M <= 32) || narrowLongK) &&
       ((int64_t)(a.N - 1) * a.ldb + a.K) * (int64_t)sizeof(T) < ((int64_t)1 << 31) &&
       ((int64_t)(a.M - 1) * a.lda + a.K) * (int64_t)sizeof(T) < ((int64_t)1 << 31)) {
-    const int rounds = (a.N + 128 * cus - 1) / (128 * cus);
-    a.colsPerWg = (a.N + cus * rounds - 1) / (cus * rounds);
+    const int ways = narrowLongK ? 2 : 1;
+    const int wgs = std::max(1, cus / ways);
+    const int rounds = (a.N + 128 * wgs - 1) / (128 * wgs);
+    a.colsPerWg = (a.N + wgs * rounds - 1) / (wgs * rounds);
+    if (ways > 1) {
+      void* ws = nullptr;
+      AMD_TRY(requireWorkspace(ctx, (int64_t)ways * a.M * a.N * 4, &ws));
+      a.partial = static_cast<float*>(ws), a.kPerWg = a.K / ways;
+    }
     if (rot != nullptr) a.colsPerWg = (a.colsPerWg + 1) & ~1;  // even: the two columns of a rotary pair stay together
     if (handled) *handled = true;
     if (a.colsPerWg > 64) {

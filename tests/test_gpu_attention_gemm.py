@@ -279,7 +279,8 @@ def test_skinny_m_linear_and_addmm(ops, dev, dtype, m, n, k):
     form that stages both operands through LDS (columns dealt evenly over the CUs, up to 64 or 128 per workgroup,
     walking K in stages of 128 from a staggered start): one to four row groups, column shares that are no multiple
     of 16, a last workgroup with fewer columns, K of one, two, three and five stages (fewer than the ring holds)
-    up to 86."""
+    up to 86. Two cases (more than 32 rows, 4096 and 4104 columns, K of 8192 and 11008) take that form with K split two
+    ways over the grid and the reduction pass."""
     x = torch.randn(m, k, generator=g(50)).to(dtype)
     w = (torch.randn(n, k, generator=g(51)) * 0.05).to(dtype)
     b = torch.randn(n, generator=g(52)).to(dtype)
