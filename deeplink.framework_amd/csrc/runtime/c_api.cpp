@@ -303,6 +303,24 @@ int dipuAmdCachingResetPeakStats(int device) {
     if (!Runtime::get().useRaw()) Runtime::get().caching(device)->resetPeakStats();
   });
 }
+namespace {
+void copyTrace(const std::vector<TraceEntry>& t, dipuAmdTraceEntry* entries, uint64_t capacity, uint64_t* count) {
+  *count = t.size();
+  for (size_t i = 0; i < t.size() && i < capacity; ++i)
+    entries[i] = dipuAmdTraceEntry{t[i].action, 0, t[i].addr, t[i].size, t[i].stream};
+}
+}  // namespace
+int dipuAmdCachingRecordHistory(int device, int enabled, uint64_t max_entries) {
+  return guarded([&] {
+    if (!Runtime::get().useRaw()) Runtime::get().caching(device)->recordHistory(enabled != 0, max_entries);
+  });
+}
+int dipuAmdCachingTrace(int device, dipuAmdTraceEntry* entries, uint64_t capacity, uint64_t* count) {
+  return guarded([&] {
+    *count = 0;
+    if (!Runtime::get().useRaw()) copyTrace(Runtime::get().caching(device)->trace(), entries, capacity, count);
+  });
+}
 int dipuAmdCachingHostMalloc(void** p, size_t n) { return guarded([&] { *p = Runtime::get().host.malloc(n); }); }
 int dipuAmdCachingHostFree(void* p) { return guarded([&] { Runtime::get().host.free(p); }); }
 int dipuAmdCachingHostRecordStream(void* p, void* stream) {
@@ -389,6 +407,12 @@ int dipuAmdSimAllocatorEmptyCache(void* handle) {
 }
 int dipuAmdSimAllocatorStats(void* handle, dipuAmdMemoryStats* stats) {
   return guarded([&] { fillStats(static_cast<SimAllocator*>(handle)->alloc->stats(), stats); });
+}
+int dipuAmdSimAllocatorRecordHistory(void* handle, int enabled, uint64_t max_entries) {
+  return guarded([&] { static_cast<SimAllocator*>(handle)->alloc->recordHistory(enabled != 0, max_entries); });
+}
+int dipuAmdSimAllocatorTrace(void* handle, dipuAmdTraceEntry* entries, uint64_t capacity, uint64_t* count) {
+  return guarded([&] { copyTrace(static_cast<SimAllocator*>(handle)->alloc->trace(), entries, capacity, count); });
 }
 int dipuAmdSimAllocatorCompleteEvents(void* handle, void* stream) {
   return guarded([&] {

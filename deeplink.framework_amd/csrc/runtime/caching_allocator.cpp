@@ -99,6 +99,35 @@ DeviceCachingAllocator::~DeviceCachingAllocator() {
 }
 
 // ---------------------------------------------------------------- malloc ----
+void DeviceCachingAllocator::recordHistory(bool enabled, size_t maxEntries) {
+  std::lock_guard<std::recursive_mutex> lock(mutex_);
+  recordHistory_ = enabled;
+  traceMax_ = std::max<size_t>(1, maxEntries);
+  traceNext_ = 0;
+  trace_.clear();
+}
+
+void DeviceCachingAllocator::recordTrace(int action, int64_t addr, size_t size, StreamHandle stream) const {
+  if (!recordHistory_) return;
+  auto* self = const_cast<DeviceCachingAllocator*>(this);
+  const TraceEntry e{action, addr, size, stream};
+  if (trace_.size() < traceMax_) {
+    trace_.push_back(e);
+  } else {  // full: the oldest entry is overwritten
+    trace_[traceNext_] = e;
+    self->traceNext_ = (traceNext_ + 1) % traceMax_;
+  }
+}
+
+std::vector<TraceEntry> DeviceCachingAllocator::trace() const {
+  std::lock_guard<std::recursive_mutex> lock(mutex_);
+  std::vector<TraceEntry> out;
+  out.reserve(trace_.size());
+  out.insert(out.end(), trace_.begin() + static_cast<std::ptrdiff_t>(traceNext_), trace_.end());
+  out.insert(out.end(), trace_.begin(), trace_.begin() + static_cast<std::ptrdiff_t>(traceNext_));
+  return out;
+}
+
 bool DeviceCachingAllocator::shouldSplit(const Block* block, size_t size) const {
   size_t remaining = block->size - size;
   if (block->pool->isSmall) return remaining >= kMinBlockSize;
@@ -183,6 +212,7 @@ bool DeviceCachingAllocator::mapBlock(Block* toMap, size_t size) {
   pool.blocks.insert(toMap);
   totalReserved_ += ms;
   stats_.reservedBytes.add(static_cast<int64_t>(ms));
+  recordTrace(TraceEntry::SEGMENT_MAP, reinterpret_cast<int64_t>(mp), ms, toMap->stream);
   return true;
 }
 
@@ -242,6 +272,7 @@ void DeviceCachingAllocator::unmapBlock(Block* block) {
   pool.unmapped.insert(block);
   totalReserved_ -= us;
   stats_.reservedBytes.add(-static_cast<int64_t>(us));
+  recordTrace(TraceEntry::SEGMENT_UNMAP, reinterpret_cast<int64_t>(up), us, block->stream);
 }
 
 void DeviceCachingAllocator::releaseExpandable(Block* block) {
@@ -270,6 +301,7 @@ bool DeviceCachingAllocator::allocBlock(BlockPool& pool, size_t size, size_t all
   totalReserved_ += allocSize;
   stats_.segment.add(1);
   stats_.reservedBytes.add(static_cast<int64_t>(allocSize));
+  recordTrace(TraceEntry::SEGMENT_ALLOC, reinterpret_cast<int64_t>(p), allocSize, stream);
   *out = b;
   return true;
 }
@@ -313,6 +345,7 @@ void* DeviceCachingAllocator::malloc(size_t origSize, StreamHandle stream) {
     }
     if (!ok) {
       ++stats_.numOoms;
+      recordTrace(TraceEntry::OOM, static_cast<int64_t>(allocSize), origSize, stream);
       std::ostringstream os;
       os << "HIP out of memory. Tried to allocate " << allocSize << " bytes (request " << origSize << "). "
          << stats_.allocatedBytes.current << " bytes allocated, " << stats_.reservedBytes.current
@@ -355,6 +388,7 @@ void* DeviceCachingAllocator::malloc(size_t origSize, StreamHandle stream) {
   stats_.activeBlocks.add(1);
   stats_.activeBytes.add(static_cast<int64_t>(block->size));
   stats_.requestedBytes.add(static_cast<int64_t>(origSize));
+  recordTrace(TraceEntry::ALLOC, reinterpret_cast<int64_t>(block->ptr), origSize, block->stream);
   return block->ptr;
 }
 
@@ -370,6 +404,7 @@ void DeviceCachingAllocator::free(void* ptr) {
   stats_.allocation.add(-1);
   stats_.allocatedBytes.add(-static_cast<int64_t>(block->size));
   stats_.requestedBytes.add(-static_cast<int64_t>(block->requested));
+  recordTrace(TraceEntry::FREE_REQUESTED, reinterpret_cast<int64_t>(block->ptr), block->requested, block->stream);
   if (!block->streamUses.empty()) {
     insertEvents(block);  // reuse waits until every recorded stream has passed this point
   } else {
@@ -396,6 +431,7 @@ size_t DeviceCachingAllocator::tryMerge(Block* dst, Block* src, BlockPool& pool)
 
 void DeviceCachingAllocator::freeBlock(Block* block) {
   size_t origSize = block->size;
+  recordTrace(TraceEntry::FREE_COMPLETED, reinterpret_cast<int64_t>(block->ptr), block->requested, block->stream);
   BlockPool& pool = *block->pool;
   int64_t netInactiveBlocks = 0, netInactiveBytes = 0;
   Block* neighbours[2] = {block->prev, block->next};
@@ -473,6 +509,7 @@ void DeviceCachingAllocator::synchronizeAndFreeEvents() {
 
 // --------------------------------------------------------------- release ----
 void DeviceCachingAllocator::releaseBlock(Block* block) {
+  recordTrace(TraceEntry::SEGMENT_FREE, reinterpret_cast<int64_t>(block->ptr), block->size, block->stream);
   backend_.freeDevice(block->ptr);
   ++stats_.numDeviceFree;
   totalReserved_ -= block->size;
@@ -611,6 +648,9 @@ std::vector<SegmentInfo> DeviceCachingAllocator::snapshot() const {
     }
     out.push_back(s);
   }
+  size_t active = 0;
+  for (const SegmentInfo& si : out) active += si.activeSize;
+  recordTrace(TraceEntry::SNAPSHOT, 0, active, nullptr);
   return out;
 }
 

@@ -125,6 +125,25 @@ struct Block {
   bool isSplit() const { return prev != nullptr || next != nullptr; }
 };
 
+// One step of the allocator's history (DIPUCachingDeviceAllocator.h:134-164, without the Python stack context).
+struct TraceEntry {
+  enum Action {
+    ALLOC = 0,           // a request served (addr, requested size)
+    FREE_REQUESTED = 1,  // free() called
+    FREE_COMPLETED = 2,  // the block actually went back to the pool (after the events of recordStream, if any)
+    SEGMENT_ALLOC = 3,   // memory taken from the device
+    SEGMENT_FREE = 4,    // memory given back to the device
+    SEGMENT_MAP = 5,     // expandable segments: part of a range mapped
+    SEGMENT_UNMAP = 6,   // expandable segments: part of a range unmapped
+    SNAPSHOT = 7,        // snapshot() called (size = active bytes)
+    OOM = 8              // OutOfMemory thrown (addr = bytes the request would have taken from the device)
+  };
+  int action;
+  int64_t addr;
+  size_t size;
+  StreamHandle stream;
+};
+
 struct SegmentInfo {
   void* address;
   size_t totalSize, allocatedSize, activeSize;
@@ -151,6 +170,10 @@ class DeviceAllocator {
   virtual void processEvents() = 0;
   virtual DeviceStats stats() const = 0;
   virtual void resetPeakStats() = 0;
+  // History of the allocator's steps; only the TORCH algorithm keeps one (the others ignore the switch).
+  virtual void recordHistory(bool /*enabled*/, size_t /*maxEntries*/) {}
+  virtual bool isHistoryEnabled() const { return false; }
+  virtual std::vector<TraceEntry> trace() const { return {}; }
 };
 
 class DeviceCachingAllocator : public DeviceAllocator {
@@ -175,9 +198,18 @@ class DeviceCachingAllocator : public DeviceAllocator {
   void resetPeakStats() override;
   std::vector<SegmentInfo> snapshot() const;
   size_t blockSize(void* ptr) const;  // rounded size of a live allocation (0 if unknown)
+  // History of the allocator's steps (DIPUCachingDeviceAllocator.cpp:555-566, 1017-1027): a ring of the last maxEntries
+  // entries, cleared whenever it is switched; trace() returns them oldest first.
+  void recordHistory(bool enabled, size_t maxEntries) override;
+  bool isHistoryEnabled() const override { return recordHistory_; }
+  std::vector<TraceEntry> trace() const override;
 
  private:
   bool cacheOnly_ = false;  // set for the duration of mallocFromCache (under mutex_)
+  bool recordHistory_ = false;
+  size_t traceMax_ = 1, traceNext_ = 0;
+  mutable std::vector<TraceEntry> trace_;
+  void recordTrace(int action, int64_t addr, size_t size, StreamHandle stream) const;
   Block* getFreeBlock(BlockPool& pool, size_t size, StreamHandle stream);
   bool allocBlock(BlockPool& pool, size_t size, size_t allocSize, StreamHandle stream, Block** out);
   Block* findExpandableBlock(BlockPool& pool, size_t size, StreamHandle stream);

@@ -245,6 +245,33 @@ def cachingStats(dev=-1):
     return s.as_dict()
 
 
+TRACE_ACTIONS = ("ALLOC", "FREE_REQUESTED", "FREE_COMPLETED", "SEGMENT_ALLOC", "SEGMENT_FREE", "SEGMENT_MAP",
+                 "SEGMENT_UNMAP", "SNAPSHOT", "OOM")   # DIPUCachingDeviceAllocator.h:135-153
+
+
+class TraceEntry(ctypes.Structure):
+    _fields_ = [("action", ctypes.c_int32), ("reserved", ctypes.c_int32), ("addr", ctypes.c_int64),
+                ("size", c_uint64), ("stream", c_void_p)]
+
+
+def _read_trace(fn, *head):
+    n = c_uint64()
+    _check(fn(*head, None, c_uint64(0), byref(n)))
+    buf = (TraceEntry * max(1, n.value))()
+    _check(fn(*head, buf, c_uint64(n.value), byref(n)))
+    return [{"action": TRACE_ACTIONS[e.action], "addr": e.addr, "size": e.size, "stream": e.stream or 0}
+            for e in buf[:min(n.value, len(buf))]]
+
+
+def cachingRecordHistory(enabled, max_entries=2 ** 20, dev=-1):
+    """torch_dipu's _dipu_record_memory_history: keep the last max_entries steps of the TORCH allocator."""
+    _check(_rt().dipuAmdCachingRecordHistory(c_int(dev), c_int(int(bool(enabled))), c_uint64(max_entries)))
+
+
+def cachingTrace(dev=-1):
+    return _read_trace(_rt().dipuAmdCachingTrace, c_int(dev))
+
+
 def cachingHostMalloc(n):
     p = c_void_p()
     _check(_rt().dipuAmdCachingHostMalloc(byref(p), c_size_t(n)))
@@ -320,6 +347,12 @@ class SimAllocator:
         s = MemoryStats()
         _check(_rt().dipuAmdSimAllocatorStats(self.h, byref(s)))
         return s.as_dict()
+
+    def record_history(self, enabled, max_entries=2 ** 20):
+        _check(_rt().dipuAmdSimAllocatorRecordHistory(self.h, c_int(int(bool(enabled))), c_uint64(max_entries)))
+
+    def trace(self):
+        return _read_trace(_rt().dipuAmdSimAllocatorTrace, self.h)
 
     def backend_usage(self):
         b, n = c_uint64(), c_uint64()

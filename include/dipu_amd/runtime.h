@@ -94,6 +94,21 @@ DIPU_AMD_API int dipuAmdCachingRecordStream(void* p, void* stream);
 DIPU_AMD_API int dipuAmdCachingEmptyCache(void);
 DIPU_AMD_API int dipuAmdCachingStats(int device, dipuAmdMemoryStats* stats);
 DIPU_AMD_API int dipuAmdCachingResetPeakStats(int device);
+/* History of the TORCH allocator's steps: recordHistory / trace of DIPUCachingDeviceAllocator.cpp:555-566, 1017-1027,
+ * entries of DIPUCachingDeviceAllocator.h:134-164 without the Python stack context. A ring of the last max_entries
+ * steps, cleared whenever it is switched. action: 0 ALLOC, 1 FREE_REQUESTED, 2 FREE_COMPLETED, 3 SEGMENT_ALLOC,
+ * 4 SEGMENT_FREE, 5 SEGMENT_MAP, 6 SEGMENT_UNMAP, 7 SNAPSHOT (size = active bytes), 8 OOM (addr = bytes the request
+ * would have taken from the device). Trace copies at most `capacity` entries, oldest first, and reports how many the
+ * ring holds in *count. The RAW, BF and BS algorithms keep no history: the switch is ignored and *count is 0. */
+typedef struct dipuAmdTraceEntry {
+  int32_t action;
+  int32_t reserved;
+  int64_t addr;
+  uint64_t size;
+  void* stream;
+} dipuAmdTraceEntry;
+DIPU_AMD_API int dipuAmdCachingRecordHistory(int device, int enabled, uint64_t max_entries);
+DIPU_AMD_API int dipuAmdCachingTrace(int device, dipuAmdTraceEntry* entries, uint64_t capacity, uint64_t* count);
 /* pinned host cache: power-of-two sized, runtime/core/allocator/DIPUCachingHostAllocator.cpp:99-123,238 */
 DIPU_AMD_API int dipuAmdCachingHostMalloc(void** p, size_t nbytes);
 DIPU_AMD_API int dipuAmdCachingHostFree(void* p);
@@ -142,6 +157,8 @@ DIPU_AMD_API int dipuAmdSimAllocatorFree(void* handle, void* p);
 DIPU_AMD_API int dipuAmdSimAllocatorRecordStream(void* handle, void* p, void* stream);
 DIPU_AMD_API int dipuAmdSimAllocatorEmptyCache(void* handle);
 DIPU_AMD_API int dipuAmdSimAllocatorStats(void* handle, dipuAmdMemoryStats* stats);
+DIPU_AMD_API int dipuAmdSimAllocatorRecordHistory(void* handle, int enabled, uint64_t max_entries);
+DIPU_AMD_API int dipuAmdSimAllocatorTrace(void* handle, dipuAmdTraceEntry* entries, uint64_t capacity, uint64_t* count);
 /* events recorded so far on `stream` (all streams when null) become ready */
 DIPU_AMD_API int dipuAmdSimAllocatorCompleteEvents(void* handle, void* stream);
 DIPU_AMD_API int dipuAmdSimAllocatorBackendUsage(void* handle, uint64_t* bytes_in_use, uint64_t* live_segments);

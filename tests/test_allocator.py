@@ -15,8 +15,8 @@ MiB = 1 << 20
 def sim(pkg):
     made = []
 
-    def make(capacity=8 << 30, conf=""):
-        a = pkg.runtime.SimAllocator(capacity, conf)
+    def make(capacity=8 << 30, conf="", **kw):
+        a = pkg.runtime.SimAllocator(capacity, conf, **kw)
         made.append(a)
         return a
 
@@ -158,6 +158,63 @@ def test_cache_only_request_queries_no_event(sim):
     a.complete_events(s2)
     q = a.malloc(8192, s1)                      # the next ordinary request sees the event and reuses p
     assert q == p
+
+
+def test_history_records_each_step_in_order(pkg, sim):
+    # recordHistory / trace (DIPUCachingDeviceAllocator.cpp:555-566, 1017-1027): every step, oldest first
+    a = sim(capacity=64 * MiB)
+    assert a.trace() == []
+    p0 = a.malloc(4096)                         # before the switch: not recorded
+    a.record_history(True, 64)
+    s1, s2 = 0x1000, 0x2000
+    p = a.malloc(3000, s1)                      # a new 2 MiB segment on s1
+    a.record_stream(p, s2)
+    a.free(p)                                   # requested now, completed when s2's event is seen
+    a.complete_events(s2)
+    q = a.malloc(30 * MiB, s1)
+    with pytest.raises(pkg.runtime.RuntimeError_, match="out of memory"):
+        a.malloc(60 * MiB, s1)                  # the ladder gives the cached segment back, then fails
+    steps = [(e["action"], e["addr"], e["size"], e["stream"]) for e in a.trace()]
+    assert steps == [
+        ("SEGMENT_ALLOC", p, 2 * MiB, s1), ("ALLOC", p, 3000, s1),
+        ("FREE_REQUESTED", p, 3000, s1), ("FREE_COMPLETED", p, 3000, s1),
+        ("SEGMENT_ALLOC", q, 30 * MiB, s1), ("ALLOC", q, 30 * MiB, s1),
+        ("SEGMENT_FREE", p, 2 * MiB, s1), ("OOM", 60 * MiB, 60 * MiB, s1),
+    ]
+    a.record_history(False)                     # switching clears the ring and stops recording
+    a.free(q)
+    a.free(p0)
+    assert a.trace() == []
+
+
+def test_history_ring_keeps_the_newest_entries(sim):
+    a = sim()
+    a.record_history(True, 5)
+    ptrs = [a.malloc(512 * (i + 1)) for i in range(4)]   # SEGMENT_ALLOC + 4 ALLOC
+    for p in ptrs:
+        a.free(p)                                        # 4 x (FREE_REQUESTED, FREE_COMPLETED)
+    t = a.trace()
+    assert len(t) == 5
+    assert [e["action"] for e in t] == ["FREE_COMPLETED", "FREE_REQUESTED", "FREE_COMPLETED", "FREE_REQUESTED", "FREE_COMPLETED"]
+    assert [e["addr"] for e in t] == [ptrs[1], ptrs[2], ptrs[2], ptrs[3], ptrs[3]]
+    assert [e["size"] for e in t] == [1024, 1536, 1536, 2048, 2048]
+
+
+def test_history_of_expandable_segments_and_other_algorithms(sim):
+    a = sim(conf="expandable_segments:True")
+    a.record_history(True, 32)
+    p = a.malloc(3 * MiB)
+    a.free(p)
+    a.empty_cache()
+    acts = [e["action"] for e in a.trace()]
+    assert acts[0] == "SEGMENT_MAP" and acts[-1] == "SEGMENT_UNMAP"
+    assert acts.count("ALLOC") == 1 and "SEGMENT_ALLOC" not in acts
+    mapped = sum(e["size"] for e in a.trace() if e["action"] == "SEGMENT_MAP")
+    assert mapped >= 3 * MiB and mapped == sum(e["size"] for e in a.trace() if e["action"] == "SEGMENT_UNMAP")
+    b = sim(algorithm="BF")                     # BF and BS keep no history
+    b.record_history(True, 8)
+    b.free(b.malloc(4096))
+    assert b.trace() == []
 
 
 def test_oom_ladder_releases_cache_then_raises(pkg, sim):

@@ -118,6 +118,22 @@ def test_caching_allocator_on_device(rt):
     assert rt.cachingHostMalloc(1024) == hp                # power-of-two block reused after its event
 
 
+def test_caching_allocator_history_on_device(rt):
+    # torch_dipu's _dipu_record_memory_history: DIPUCachingDeviceAllocator.cpp:555-566, 1017-1027
+    rt.cachingEmptyCache()
+    rt.cachingRecordHistory(True, 16)
+    stream = rt.getDefaultStream()
+    p = rt.cachingMalloc(48 << 20, stream)
+    rt.cachingFree(p)
+    rt.cachingEmptyCache()
+    steps = [(e["action"], e["addr"], e["size"], e["stream"]) for e in rt.cachingTrace()]
+    rt.cachingRecordHistory(False)
+    assert steps == [("SEGMENT_ALLOC", p, 48 << 20, stream), ("ALLOC", p, 48 << 20, stream),
+                     ("FREE_REQUESTED", p, 48 << 20, stream), ("FREE_COMPLETED", p, 48 << 20, stream),
+                     ("SEGMENT_FREE", p, 48 << 20, stream)]
+    assert rt.cachingTrace() == []
+
+
 def test_context_workspace_lifetime(pkg, ops, dev):
     # workspace requested by the impl library lives until the context closes
     # (diopirt_impl.h:19-26), then returns to the caching allocator
