@@ -34,7 +34,7 @@ MFMA_BF16_PEAK_TF = 2500.0   # MI355X dense bf16, published
 # a counter cannot be read from inside this process, so the figure is carried here as measured, with the commit
 # whose kernels the counters were taken on (it does not move when the kernel does; re-take it after a GEMM change).
 GEMM_TRAFFIC_BYTES_PER_LAUNCH = 1_391_000_000
-GEMM_TRAFFIC_MEASURED_AT = "47aa3ca"
+GEMM_TRAFFIC_MEASURED_AT = "6dad182"
 
 
 def parse():
@@ -45,6 +45,8 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-ops", action="store_true", help="skip the per-op HBM microbenchmarks")
     ap.add_argument("--only-layer", action="store_true", help="alias for --no-cpu --no-ops")
+    ap.add_argument("--warm-ms", type=float, default=None, help="device work on an op before it is timed, in ms (default 25); "
+                    "0 keeps a counter-collecting run short")
     ap.add_argument("--gemm", metavar="M,N,K", help="profiling aid: time only diopiLinear on [M,K] x [N,K]^T (bf16 unless --gemm-dtype says otherwise) "
                     "(activations N(0,1), weights N(0,0.02)) for --steps launches and print one JSON line")
     ap.add_argument("--gemm-dtype", choices=["bf16", "fp16", "fp32"], default="bf16", help="with --gemm: the operand dtype")
@@ -655,6 +657,9 @@ def main():
     args = parse()
     if args.only_layer:
         args.no_cpu = args.no_ops = True
+    if args.warm_ms is not None:
+        global WARM_MS
+        WARM_MS = args.warm_ms
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this build has no multi-GPU path (got --gpus {args.gpus}). "
               "Run with --gpus 1.", file=sys.stderr)

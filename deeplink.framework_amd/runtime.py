@@ -264,7 +264,7 @@ def _read_trace(fn, *head):
 
 
 def cachingRecordHistory(enabled, max_entries=2 ** 20, dev=-1):
-    """torch_dipu's _dipu_record_memory_history: keep the last max_entries steps of the TORCH allocator."""
+    """recordHistory of the TORCH allocator (DIPUCachingDeviceAllocator.cpp:555-566): keep its last max_entries steps."""
     _check(_rt().dipuAmdCachingRecordHistory(c_int(dev), c_int(int(bool(enabled))), c_uint64(max_entries)))
 
 

@@ -119,7 +119,7 @@ def test_caching_allocator_on_device(rt):
 
 
 def test_caching_allocator_history_on_device(rt):
-    # torch_dipu's _dipu_record_memory_history: DIPUCachingDeviceAllocator.cpp:555-566, 1017-1027
+    # recordHistory / trace of the TORCH allocator: DIPUCachingDeviceAllocator.cpp:555-566, 1017-1027
     rt.cachingEmptyCache()
     rt.cachingRecordHistory(True, 16)
     stream = rt.getDefaultStream()
