@@ -109,13 +109,12 @@ void DeviceCachingAllocator::recordHistory(bool enabled, size_t maxEntries) {
 
 void DeviceCachingAllocator::recordTrace(int action, int64_t addr, size_t size, StreamHandle stream) const {
   if (!recordHistory_) return;
-  auto* self = const_cast<DeviceCachingAllocator*>(this);
   const TraceEntry e{action, addr, size, stream};
   if (trace_.size() < traceMax_) {
     trace_.push_back(e);
   } else {  // full: the oldest entry is overwritten
     trace_[traceNext_] = e;
-    self->traceNext_ = (traceNext_ + 1) % traceMax_;
+    traceNext_ = (traceNext_ + 1) % traceMax_;
   }
 }
 

@@ -207,7 +207,8 @@ class DeviceCachingAllocator : public DeviceAllocator {
  private:
   bool cacheOnly_ = false;  // set for the duration of mallocFromCache (under mutex_)
   bool recordHistory_ = false;
-  size_t traceMax_ = 1, traceNext_ = 0;
+  size_t traceMax_ = 1;
+  mutable size_t traceNext_ = 0;           // the ring is also written by const members (snapshot records itself)
   mutable std::vector<TraceEntry> trace_;
   void recordTrace(int action, int64_t addr, size_t size, StreamHandle stream) const;
   Block* getFreeBlock(BlockPool& pool, size_t size, StreamHandle stream);
