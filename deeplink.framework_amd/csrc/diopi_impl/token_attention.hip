@@ -22,9 +22,9 @@
 //     (2 + 2 wave-loads, 4 KiB per wave) and the slot indices of iteration i + 2 are in flight,
 //     so neither the row latency nor the index -> address dependency is exposed. A deeper queue is
 //     slower, not faster: 4 + 4 loads per wave measured 458 us where 2 + 2 take 432 (8 + 8: 509);
-//   * a workgroup = 4 waves owns a chunk of the sequence (split-KV, chunks of at least 512
-//     tokens and at most 64 per sequence); states are merged by wave butterflies, then through
-//     LDS, then across chunks by a small lane-parallel second kernel.
+//   * a workgroup = 4 waves owns a chunk of the sequence (split-KV: chunks of 512 tokens, shorter ones, down to 64,
+//     when there would otherwise be too few workgroups for the chip, at most 256 per sequence); states are merged by
+//     wave butterflies, then through LDS, then across chunks by a small lane-parallel second kernel.
 //
 // Head rows of 128, 256 or 512 bytes at 16-byte aligned strides take the kernels above; any other head size or
 // alignment (up to 1024 elements) takes the generic kernels at the end: one workgroup per (sequence, head), 256 tokens
@@ -40,7 +40,10 @@ constexpr float kLog2eTA = 1.4426950408889634f;
 constexpr int kTaWaves = 4;
 constexpr int kTaUnroll = 2;
 constexpr int kTaChunk = 512;  // tokens of one sequence handled by one workgroup (grows for very long sequences)
-constexpr int kTaMaxSplit = 64; // the merge step handles one split per lane
+constexpr int kTaMaxSplit = 256;  // decodeMergeWideKernel holds four splits' weights per lane (decodeMergeKernel: one, up to 64 splits)
+constexpr int kTaMinChunk = 128;  // shorter chunks cost more in prologues, partial results and merging than they gain ...
+constexpr int kTaTinyChunk = 64;  // ... unless even those leave CUs without a workgroup
+constexpr int kTaWgsPerCu = 8;    // workgroups per CU the chunk length aims for
 
 __device__ __forceinline__ int64_t ldIndex(const void* p, int64_t i, bool is64) {
   return is64 ? reinterpret_cast<const int64_t*>(p)[i] : static_cast<int64_t>(reinterpret_cast<const int32_t*>(p)[i]);
@@ -270,6 +273,75 @@ __global__ __launch_bounds__(256) void decodeMergeKernel(T* __restrict__ out, co
   for (int k = 0; k < kMaxPerLane; ++k) {
     const int e = lane + 64 * k;
     if (e < d) out[pair * d + e] = static_cast<T>(acc[k]);
+  }
+}
+
+// The same merge for 65 to 256 splits (few sequences with long contexts, cut fine to fill the chip): one workgroup per
+// (b, h). Every wave works out the weights of all splits (lane s holds splits s, s + 64, s + 128, s + 192), then wave w
+// combines splits w, w + 4, ... and the four sums meet in LDS.
+template <typename T>
+__global__ __launch_bounds__(256) void decodeMergeWideKernel(T* __restrict__ out, const float* __restrict__ partial,
+                                                              const void* bLen, bool len64, int heads, int d, int nsplit,
+                                                              int chunk) {
+  constexpr int kBatch = 8, kMaxPerLane = 4, kPerLane = kTaMaxSplit / 64;  // d <= 256
+  __shared__ float red[4][64 * kMaxPerLane];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t pair = blockIdx.x;
+  const int b = (int)(pair / heads);
+  const int row = 2 + d;
+  const float* src = partial + pair * nsplit * row;
+  const int len = (int)ldIndex(bLen, b, len64);
+  const int used = len <= 0 ? 1 : min(nsplit, (len + chunk - 1) / chunk);
+  float ms[kPerLane], ls[kPerLane], wgt[kPerLane];
+  float m = -INFINITY;
+#pragma unroll
+  for (int k = 0; k < kPerLane; ++k) {
+    const int sp = lane + 64 * k;
+    ms[k] = sp < used ? src[sp * row] : -INFINITY;  // splits that hold no tokens were never written
+    ls[k] = sp < used ? src[sp * row + 1] : 0.f;
+    m = fmaxf(m, ms[k]);
+  }
+  m = waveMax(m);
+  float lsum = 0.f;
+#pragma unroll
+  for (int k = 0; k < kPerLane; ++k) {
+    wgt[k] = ms[k] == -INFINITY ? 0.f : exp2f(ms[k] - m);
+    lsum += ls[k] * wgt[k];
+  }
+  const float l = waveSum(lsum);
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  float acc[kMaxPerLane] = {0.f, 0.f, 0.f, 0.f};
+  for (int s0 = wave; s0 < used; s0 += 4 * kBatch) {
+    float v[kBatch][kMaxPerLane];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const float* r = src + (int64_t)min(s0 + 4 * u, nsplit - 1) * row + 2;
+#pragma unroll
+      for (int k = 0; k < kMaxPerLane; ++k) {
+        const int e = lane + 64 * k;
+        v[u][k] = e < d ? r[e] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int sp = s0 + 4 * u, owner = sp >> 6;  // wave-uniform
+      float w = wgt[0];
+#pragma unroll
+      for (int k = 1; k < kPerLane; ++k) w = owner == k ? wgt[k] : w;
+      w = __shfl(w, sp & 63, 64) * inv;
+#pragma unroll
+      for (int k = 0; k < kMaxPerLane; ++k) acc[k] += sp < used ? w * v[u][k] : 0.f;
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < kMaxPerLane; ++k) red[wave][lane + 64 * k] = acc[k];
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int k = 0; k < kMaxPerLane; ++k) {
+      const int e = lane + 64 * k;
+      if (e < d) out[pair * d + e] = static_cast<T>(red[0][e] + red[1][e] + red[2][e] + red[3][e]);
+    }
   }
 }
 
@@ -722,6 +794,25 @@ static diopiError_t decodeAttention(diopiContextHandle_t ctx, diopiTensorHandle_
     AMD_LAUNCH_CHECK();
     return diopiSuccess;
   }
+  const int64_t bytes = t.q.shape[2] * t.q.itemsize;
+  // The lane groups of a wave take consecutive heads of one token when the head count allows it: a wave load is then
+  // one contiguous piece of a slot (1 KiB) instead of head rows of four different slots (431 -> 421 us at batch 64,
+  // 32 heads x 128, 156 043 cached tokens).
+  const int tpw = (int)(64 / std::max<int64_t>(1, bytes / 16));
+  const bool hiw = (bytes == 128 || bytes == 256 || bytes == 512) && a.heads % tpw == 0;
+  // A workgroup walks its chunk with two loads per wave in flight, so the rate comes from the number of workgroups a
+  // CU holds at once. Few sequences or short ones are cut into smaller chunks until there are about kTaWgsPerCu
+  // workgroups per CU; large batches keep the 512-token chunks, whose partial results are fewer. Measured (us, 32 heads
+  // x 128, bf16, with 512-token chunks -> with these): 1 x 2048 tokens 72 -> 20, 1 x 32768 130 -> 96, 8 x 4096 130 -> 91,
+  // 4 x (100 .. 16384) 123 -> 86, 64 x (256 .. 512) 101 -> 80; 64 x (512 .. 4096) and 256 x (1024 .. 2048) keep their chunks.
+  {
+    const int64_t groups = (hiw ? a.heads / tpw : a.heads) * batch, cus = computeUnits(), len = std::max(maxInputLen, 1);
+    const int64_t wantSplits = std::max<int64_t>(1, ceilDiv(kTaWgsPerCu * cus, groups));
+    const int64_t fine = ceilDiv(ceilDiv(len, wantSplits), 64) * 64;
+    const int64_t capped = ceilDiv(ceilDiv(len, (int64_t)kTaMaxSplit), 64) * 64;  // at most kTaMaxSplit chunks
+    const int64_t shortest = groups * ceilDiv(len, (int64_t)kTaMinChunk) < cus ? kTaTinyChunk : kTaMinChunk;
+    a.chunk = (int)std::max(std::max(capped, shortest), std::min<int64_t>(a.chunk, fine));
+  }
   a.nsplit = (int)std::max<int64_t>(1, ceilDiv(maxInputLen, a.chunk));
   AMD_CHECK(batch <= 65535 && a.nsplit <= 65535, "token attention: batch %ld / splits %d exceed the grid limits", (long)batch,
             a.nsplit);
@@ -742,12 +833,6 @@ static diopiError_t decodeAttention(diopiContextHandle_t ctx, diopiTensorHandle_
       partial = static_cast<float*>(ws);
     }
   }
-  const int64_t bytes = t.q.shape[2] * t.q.itemsize;
-  // The lane groups of a wave take consecutive heads of one token when the head count allows it: a wave load is then
-  // one contiguous piece of a slot (1 KiB) instead of head rows of four different slots (431 -> 421 us at batch 64,
-  // 32 heads x 128, 156 043 cached tokens).
-  const int tpw = (int)(64 / std::max<int64_t>(1, bytes / 16));
-  const bool hiw = (bytes == 128 || bytes == 256 || bytes == 512) && a.heads % tpw == 0;
   dim3 grid(hiw ? a.heads / tpw : a.heads, a.nsplit, (unsigned)batch), block(kTaWaves * 64);
 #define DECODE_CALL(T, LPT)                                                                                               \
   if (hiw) hipLaunchKernelGGL((decodeSplitKernel<T, LPT, true>), grid, block, 0, stream, a, out.ptr<T>(), partial);       \
@@ -755,7 +840,16 @@ static diopiError_t decodeAttention(diopiContextHandle_t ctx, diopiTensorHandle_
   TA_DISPATCH(t.q.dtype, bytes, DECODE_CALL);
 #undef DECODE_CALL
   AMD_LAUNCH_CHECK();
-  if (a.nsplit > 1) {
+  if (a.nsplit > 64) {
+    const int64_t pairs = batch * a.heads;
+    AMD_CHECK(a.nsplit <= kTaMaxSplit && a.d <= 256, "token attention: %d splits of head size %d cannot be merged", a.nsplit, a.d);
+#define MERGE_WIDE_CALL(T, LPT)                                                                                              \
+  hipLaunchKernelGGL((decodeMergeWideKernel<T>), dim3((unsigned)pairs), dim3(256), 0, stream, out.ptr<T>(), partial, a.bLen, \
+                     a.len64, a.heads, a.d, a.nsplit, a.chunk)
+    TA_DISPATCH(t.q.dtype, bytes, MERGE_WIDE_CALL);
+#undef MERGE_WIDE_CALL
+    AMD_LAUNCH_CHECK();
+  } else if (a.nsplit > 1) {
     int64_t pairs = batch * a.heads;
     dim3 mgrid((unsigned)ceilDiv(pairs, 4)), mblock(256);
 #define MERGE_CALL(T, LPT)                                                                                       \

@@ -100,8 +100,9 @@ def test_paged_decode_step_at_batch_64(ops, dev, pkg):
 
 @pytest.mark.parametrize("lens", [[32768, 700], [32769, 1], [40000, 33000, 5], [5000, 4097, 4096, 513]])
 def test_token_attention_long_sequences(ops, dev, lens):
-    """64 splits of exactly 512 tokens, one token more (the chunk grows to 576), 40 000 tokens, and 9-10 splits (two
-    batches of the merge kernel). Slots are drawn with repetition from a small pool."""
+    """Few sequences, so the chunks are short: 256 splits of exactly 128 tokens, one token more (the chunk grows to 192),
+    40 000 tokens (all three merged by the kernel for more than 64 splits), and 40 splits (five batches of the merge
+    kernel for up to 64). Slots are drawn with repetition from a small pool."""
     heads, kvh, d, slots = 4, 2, 128, 8192
     batch, width = len(lens), max(lens)
     kp = torch.randn(slots, kvh, d, generator=g(50)).bfloat16()
@@ -123,6 +124,27 @@ def test_token_attention_long_sequences(ops, dev, lens):
     out2 = torch.empty_like(got)
     ops.token_softmax_reducev(att, vp.to(dev), out2, *args)
     assert_half(out2, want)
+
+
+@pytest.mark.parametrize("lens", [[2048], [9000, 8000, 77], [130] * 16])
+def test_token_attention_few_sequences_at_32_heads(ops, dev, lens):
+    """Small batches at the 7B head count: the chunk length follows the number of workgroups the chip needs (64-token
+    chunks for one 2048-token sequence, 128-token chunks and 71 splits for the second case, and two chunks each, of
+    128 and 2 tokens, for the third)."""
+    heads, d, slots = 32, 128, 4096
+    batch, width = len(lens), max(lens)
+    kp = torch.randn(slots, heads, d, generator=g(70)).bfloat16()
+    vp = torch.randn(slots, heads, d, generator=g(71)).bfloat16()
+    q = torch.randn(batch, heads, d, generator=g(72)).bfloat16()
+    b_loc = torch.zeros(batch, width, dtype=torch.int32)
+    for b, n in enumerate(lens):
+        b_loc[b, width - n:] = torch.randint(0, slots, (n,), generator=g(73 + b), dtype=torch.int32)
+    ln = torch.tensor(lens, dtype=torch.int32)
+    st = torch.zeros(batch, dtype=torch.int32)
+    st[1:] = torch.cumsum(ln, 0)[:-1]
+    want = oracle.token_attention(q.float(), kp.float(), vp.float(), b_loc, ln, width)
+    got = ops.token_decode_attention(q.to(dev), kp.to(dev), vp.to(dev), b_loc.to(dev), st.to(dev), ln.to(dev), width)
+    assert_half(got, want)
 
 
 def test_token_attention_length_beyond_the_table_is_cut(ops, dev):

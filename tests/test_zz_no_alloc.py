@@ -54,7 +54,7 @@ def test_no_alloc_decode_attention_requests_no_workspace_and_rejects_oversize(op
         assert rt.cachingStats()["allocations"] == before["allocations"] + 1   # the allocating entry point's workspace
     torch.cuda.synchronize()
     scope.close()
-    # 64 sequences x 32 heads x 64 splits x 130 floats = 68 MB of partial results: beyond the 32 MiB the library holds
+    # 64 sequences x 32 heads x 79 splits x 130 floats = 84 MB of partial results: beyond the 32 MiB the library holds
     big_loc = torch.zeros(64, 40000, dtype=torch.int32, device=dev)
     q = torch.zeros(64, 32, 128, dtype=torch.bfloat16, device=dev)
     pool = torch.zeros(64, 32, 128, dtype=torch.bfloat16, device=dev)
