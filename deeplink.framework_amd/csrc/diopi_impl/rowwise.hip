@@ -9,7 +9,10 @@
 // next row's loads in flight while the current one is reduced, and keeps its slice of the
 // RMSNorm weight in registers.
 //
-// Generic path: one workgroup per row, LDS-staged block reduction, rows of any length;
+// Short rows (at most 32 vectors) share a wave, 2 to 8 rows at a time; rows longer than a wave's registers (up to 8192
+// vectors) take a workgroup per row with the row packed in the threads' registers.
+//
+// Generic path: one workgroup per row, LDS-staged block reduction, rows of any length or alignment;
 // softmax over a non-last dim walks the reduced dim with a stride (one lane per column).
 //
 // Semantics: softmax as at::softmax on CPU (dipu/torch_dipu/csrc_dipu/aten/ops/CustomFallbackFunctions.hpp:466-474);
@@ -171,6 +174,106 @@ __global__ __launch_bounds__(256) void rowWaveKernel(T* __restrict__ out, const 
   }  // persistent row loop
 }
 
+// ------------------------------------------------- several short rows per wave ---
+// Rows of at most 32 vectors (256 elements of a 16-bit type): a wave-per-row kernel would leave most lanes without a
+// vector. Here LPR lanes share a row, a wave takes 64 / LPR rows at a time, one vector per lane, and the reductions are
+// butterflies within the LPR lanes. Four such row groups per iteration keep four loads per lane in flight.
+template <int LPR>
+__device__ __forceinline__ float groupReduce(float v, bool isMax) {
+#pragma unroll
+  for (int o = LPR / 2; o >= 1; o >>= 1) {
+    const float other = __shfl_xor(v, o, 64);
+    v = isMax ? fmaxf(v, other) : v + other;
+  }
+  return v;
+}
+
+template <typename T, int LPR, int OP, typename WT>
+__global__ __launch_bounds__(256) void rowSubWaveKernel(T* __restrict__ out, const T* __restrict__ in,
+                                                         const WT* __restrict__ weight, const WT* __restrict__ bias,
+                                                         float* __restrict__ invRmsOut, int64_t rows, int cols,
+                                                         int64_t inRowStride, int64_t outRowStride, float eps) {
+  using V = typename Vec16<T>::type;
+  using WV = typename Vec16<WT>::type;
+  constexpr int N = Vec16<T>::N, WN = Vec16<WT>::N, WPER = (N + WN - 1) / WN;
+  constexpr int RPW = 64 / LPR, U = 4;
+  const int lane = threadIdx.x & 63, sub = lane % LPR, r = lane / LPR;
+  const bool active = sub < cols / N;
+  float w[N], b[N];
+#pragma unroll
+  for (int j = 0; j < N; ++j) w[j] = 1.f, b[j] = 0.f;
+  if (OP == kRowRmsNorm && active) {
+#pragma unroll
+    for (int p = 0; p < WPER; ++p) {
+      if (weight != nullptr) {
+        const WV wv = reinterpret_cast<const WV*>(weight)[sub * WPER + p];
+#pragma unroll
+        for (int j = 0; j < WN && p * WN + j < N; ++j) w[p * WN + j] = static_cast<float>(wv[j]);
+      }
+      if (bias != nullptr) {
+        const WV bv = reinterpret_cast<const WV*>(bias)[sub * WPER + p];
+#pragma unroll
+        for (int j = 0; j < WN && p * WN + j < N; ++j) b[p * WN + j] = static_cast<float>(bv[j]);
+      }
+    }
+  }
+  const int64_t nWaves = (int64_t)gridDim.x * 4, step = nWaves * RPW * U;
+  for (int64_t base = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * RPW * U; base < rows; base += step) {
+    V x[U];
+    bool ok[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t row = base + u * RPW + r;
+      ok[u] = active && row < rows;
+      if (ok[u]) x[u] = __builtin_nontemporal_load(reinterpret_cast<const V*>(in + row * inRowStride) + sub);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t row = base + u * RPW + r;
+      float f[N];
+      V v;
+      if constexpr (OP == kRowSoftmax) {
+        float m = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+          f[j] = ok[u] ? static_cast<float>(x[u][j]) : -INFINITY;
+          m = fmaxf(m, f[j]);
+        }
+        m = groupReduce<LPR>(m, true);
+        const float mScaled = (m == -INFINITY) ? 0.f : m * kLog2e;  // all -inf row -> nan like the CPU kernel
+        float sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+          f[j] = ok[u] ? __builtin_amdgcn_exp2f(fmaf(f[j], kLog2e, -mScaled)) : 0.f;
+          sum += f[j];
+        }
+        sum = groupReduce<LPR>(sum, false);
+        const float inv = 1.f / sum;
+#pragma unroll
+        for (int j = 0; j < N; ++j) v[j] = static_cast<T>(f[j] * inv);
+      } else {
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+          f[j] = ok[u] ? static_cast<float>(x[u][j]) : 0.f;
+          ss += f[j] * f[j];
+        }
+        ss = groupReduce<LPR>(ss, false);
+        const float inv = 1.0f / sqrtf(ss / (float)cols + eps);
+        if (invRmsOut != nullptr && sub == 0 && row < rows) invRmsOut[row] = inv;
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+          float t = f[j] * inv;
+          if (weight != nullptr) t *= w[j];
+          if (bias != nullptr) t += b[j];
+          v[j] = static_cast<T>(t);
+        }
+      }
+      if (ok[u]) __builtin_nontemporal_store(v, reinterpret_cast<V*>(out + row * outRowStride) + sub);
+    }
+  }
+}
+
 // --------------------------------------------------------- block-per-row ----
 __device__ __forceinline__ float blockReduce(float v, bool isMax, float* smem) {
   v = isMax ? waveMax(v) : waveSum(v);
@@ -234,6 +337,117 @@ __global__ __launch_bounds__(256) void rowBlockKernel(T* out, const T* in, const
       if (weight != nullptr) v *= static_cast<float>(weight[c]);
       if (bias != nullptr) v += static_cast<float>(bias[c]);
       dst[c] = static_cast<T>(v);
+    }
+  }
+}
+
+// Rows too long for one wave's registers (more than 1024 vectors), 16-byte aligned: a workgroup per row, every thread
+// keeps NVT vectors of the row packed in registers, so the row still makes one trip from and one trip to memory;
+// the two reductions of a row go through LDS. Workgroups walk the rows with a stride.
+template <typename T, int NVT, int OP, typename WT>
+__global__ __launch_bounds__(256) void rowBlockVecKernel(T* __restrict__ out, const T* __restrict__ in,
+                                                          const WT* __restrict__ weight, const WT* __restrict__ bias,
+                                                          float* __restrict__ invRmsOut, int64_t rows, int cols,
+                                                          int64_t inRowStride, int64_t outRowStride, float eps) {
+  using V = typename Vec16<T>::type;
+  using WV = typename Vec16<WT>::type;
+  constexpr int N = Vec16<T>::N, WN = Vec16<WT>::N, WPER = (N + WN - 1) / WN;
+  __shared__ float red[8];
+  const int nvec = cols / N, tid = threadIdx.x;
+  // RMSNorm: this thread's pieces of the weight stay in registers for all the rows of the workgroup when they fit
+  // next to the row
+  constexpr bool kEarly = OP == kRowRmsNorm && NVT * WPER <= 16;
+  WV wEarly[kEarly ? NVT * WPER : 1];
+  if constexpr (kEarly) {
+    if (weight != nullptr) {
+#pragma unroll
+      for (int i = 0; i < NVT; ++i)
+        if (tid + 256 * i < nvec) {
+#pragma unroll
+          for (int p = 0; p < WPER; ++p) wEarly[i * WPER + p] = reinterpret_cast<const WV*>(weight)[(tid + 256 * i) * WPER + p];
+        }
+    }
+  }
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const V* src = reinterpret_cast<const V*>(in + row * inRowStride);
+    V* dst = reinterpret_cast<V*>(out + row * outRowStride);
+    V x[NVT];
+#pragma unroll
+    for (int i = 0; i < NVT; ++i)
+      if (tid + 256 * i < nvec) x[i] = __builtin_nontemporal_load(src + tid + 256 * i);
+    if constexpr (OP == kRowSoftmax) {
+      float m = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < NVT; ++i)
+        if (tid + 256 * i < nvec) {
+#pragma unroll
+          for (int j = 0; j < N; ++j) m = fmaxf(m, static_cast<float>(x[i][j]));
+        }
+      m = blockReduce(m, true, red);
+      const float mScaled = (m == -INFINITY) ? 0.f : m * kLog2e;
+      float sum = 0.f;
+#pragma unroll
+      for (int i = 0; i < NVT; ++i)
+        if (tid + 256 * i < nvec) {
+#pragma unroll
+          for (int j = 0; j < N; ++j) sum += __builtin_amdgcn_exp2f(fmaf(static_cast<float>(x[i][j]), kLog2e, -mScaled));
+        }
+      sum = blockReduce(sum, false, red);
+      const float inv = 1.f / sum;
+#pragma unroll
+      for (int i = 0; i < NVT; ++i)
+        if (tid + 256 * i < nvec) {
+          V v;
+#pragma unroll
+          for (int j = 0; j < N; ++j)
+            v[j] = static_cast<T>(__builtin_amdgcn_exp2f(fmaf(static_cast<float>(x[i][j]), kLog2e, -mScaled)) * inv);
+          __builtin_nontemporal_store(v, dst + tid + 256 * i);
+        }
+    } else {
+      float ss = 0.f;
+#pragma unroll
+      for (int i = 0; i < NVT; ++i)
+        if (tid + 256 * i < nvec) {
+#pragma unroll
+          for (int j = 0; j < N; ++j) {
+            const float f = static_cast<float>(x[i][j]);
+            ss += f * f;
+          }
+        }
+      ss = blockReduce(ss, false, red);
+      const float inv = 1.0f / sqrtf(ss / (float)cols + eps);
+      if (invRmsOut != nullptr && tid == 0) invRmsOut[row] = inv;
+#pragma unroll
+      for (int i = 0; i < NVT; ++i) {
+        const int idx = tid + 256 * i;
+        if (idx < nvec) {
+          float w[N], b[N];
+#pragma unroll
+          for (int p = 0; p < WPER; ++p) {
+            if (weight != nullptr) {
+              WV wv;
+              if constexpr (kEarly) wv = wEarly[i * WPER + p];
+              else wv = reinterpret_cast<const WV*>(weight)[idx * WPER + p];
+#pragma unroll
+              for (int j = 0; j < WN && p * WN + j < N; ++j) w[p * WN + j] = static_cast<float>(wv[j]);
+            }
+            if (bias != nullptr) {
+              const WV bv = reinterpret_cast<const WV*>(bias)[idx * WPER + p];
+#pragma unroll
+              for (int j = 0; j < WN && p * WN + j < N; ++j) b[p * WN + j] = static_cast<float>(bv[j]);
+            }
+          }
+          V v;
+#pragma unroll
+          for (int j = 0; j < N; ++j) {
+            float t = static_cast<float>(x[i][j]) * inv;
+            if (weight != nullptr) t *= w[j];
+            if (bias != nullptr) t += b[j];
+            v[j] = static_cast<T>(t);
+          }
+          __builtin_nontemporal_store(v, dst + idx);
+        }
+      }
     }
   }
 }
@@ -331,7 +545,19 @@ static diopiError_t launchRows(hipStream_t stream, T* out, const T* in, const WT
                                float eps, bool vectorOk) {
   constexpr int N = Vec16<T>::N;
   if (rows == 0 || cols == 0) return diopiSuccess;
-  if (vectorOk && cols % N == 0 && cols / N <= 64 * 16) {
+  if (vectorOk && cols % N == 0 && cols / N <= 32 && rows >= 16) {
+    const int nvec = (int)(cols / N), lpr = nvec <= 8 ? 8 : (nvec <= 16 ? 16 : 32);
+    // 16 waves per CU, every wave 4 row groups of 64 / lpr rows per iteration
+    const int64_t groups = ceilDiv(rows, (int64_t)(64 / lpr) * 4);
+    dim3 grid((unsigned)std::min<int64_t>(ceilDiv(groups, 4), (int64_t)computeUnits() * 4)), block(256);
+#define SUB_LAUNCH(LPR)                                                                                               \
+  hipLaunchKernelGGL((rowSubWaveKernel<T, LPR, OP, WT>), grid, block, 0, stream, out, in, weight, bias, invRms, rows, \
+                     (int)cols, inStride, outStride, eps)
+    if (lpr == 8) SUB_LAUNCH(8);
+    else if (lpr == 16) SUB_LAUNCH(16);
+    else SUB_LAUNCH(32);
+#undef SUB_LAUNCH
+  } else if (vectorOk && cols % N == 0 && cols / N <= 64 * 16) {
     int nvec = (int)(cols / N);
     int nv = (nvec + 63) / 64;
     // persistent waves: the kernels hold 16 waves per CU (4 per SIMD, <= 128 registers); give every
@@ -348,6 +574,16 @@ static diopiError_t launchRows(hipStream_t stream, T* out, const T* in, const WT
     else if (nv <= 8) ROW_LAUNCH(8);
     else ROW_LAUNCH(16);
 #undef ROW_LAUNCH
+  } else if (vectorOk && cols % N == 0 && cols / N <= 256 * 32) {
+    const int nvt = (int)ceilDiv(cols / N, 256);
+    dim3 grid((unsigned)std::min<int64_t>(rows, (int64_t)computeUnits() * 8)), block(256);
+#define BLOCK_LAUNCH(NVT)                                                                                               \
+  hipLaunchKernelGGL((rowBlockVecKernel<T, NVT, OP, WT>), grid, block, 0, stream, out, in, weight, bias, invRms, rows, \
+                     (int)cols, inStride, outStride, eps)
+    if (nvt <= 8) BLOCK_LAUNCH(8);
+    else if (nvt <= 16) BLOCK_LAUNCH(16);
+    else BLOCK_LAUNCH(32);
+#undef BLOCK_LAUNCH
   } else {
     int stage = cols <= 12288 ? (int)cols : 0;  // 48 KiB of fp32 staging
     size_t lds = (8 + (size_t)stage) * sizeof(float);

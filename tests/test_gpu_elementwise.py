@@ -192,6 +192,32 @@ def test_softmax(ops, dev, dtype):
         assert_close(got.nan_to_num(0.0), want.nan_to_num(0.0))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_softmax_and_rms_norm_short_and_long_rows(ops, dev, dtype):
+    """Rows that share a wave (a few vectors each, ragged row counts) and rows longer than one wave holds (a workgroup
+    per row, up to 65536 16-bit elements), with masked entries and one fully masked row in the softmax."""
+    for rows, cols in [(1000, 64), (101, 8), (17, 24), (4099, 128), (33, 256), (300, 11008), (40, 32000), (3, 65536)]:
+        x = (torch.randn(rows, cols, generator=g(140)) * 3).to(dtype)
+        x[torch.rand(rows, cols, generator=g(141)) < 0.05] = float("-inf")
+        x[:, 0] = 0.5
+        x[rows // 2].fill_(float("-inf"))
+        got, want = ops.softmax(x.to(dev), -1).cpu(), oracle.softmax(x.double() if dtype == torch.float32 else x, -1).to(dtype)
+        assert torch.equal(got.isnan(), want.isnan()), (rows, cols)
+        assert_close(got.nan_to_num(0.0), want.nan_to_num(0.0))
+        xr = torch.randn(rows, cols, generator=g(142)).to(dtype)
+        w = (1 + 0.1 * torch.randn(cols, generator=g(143))).to(dtype)
+        bvec = (0.1 * torch.randn(cols, generator=g(144))).to(dtype)
+        inv = torch.empty(rows, dtype=torch.float32, device=dev)
+        gotn = ops.rms_norm(xr.to(dev), w.to(dev), 1e-5, bias=bvec.to(dev), inv_rms=inv)
+        wantn = oracle.rms_norm(xr.float(), w.float(), 1e-5) + bvec.float()
+        if dtype == torch.float32:
+            assert_fp32(gotn, wantn)
+        else:
+            assert_half(gotn, wantn)
+            assert_half(ops.rms_norm(xr.to(dev), w.float().to(dev), 1e-5), oracle.rms_norm(xr.float(), w.float(), 1e-5))
+        assert_fp32(inv, torch.rsqrt(xr.float().pow(2).mean(-1) + 1e-5), rel=1e-5)
+
+
 def test_broadcast_rows_groups_and_mixed_dtypes(ops, dev):
     """The 8-columns-per-lane path: a bias row, a per-row scale, a table shared by every head ([b, 1, s, d] against
     [b, h, s, d]), operands of different floating dtypes, an in-place form, and a column slice as destination."""
