@@ -557,6 +557,18 @@ static diopiError_t launchRows(hipStream_t stream, T* out, const T* in, const WT
     else if (lpr == 16) SUB_LAUNCH(16);
     else SUB_LAUNCH(32);
 #undef SUB_LAUNCH
+  } else if (vectorOk && cols % N == 0 && cols / N >= 256 && cols / N <= 64 * 16 && rows * 4 <= computeUnits()) {
+    // A handful of long rows (the norms of a decode step): a workgroup per row shortens the chain load - reduce - store
+    // that a single wave walks with eight vectors per lane.
+    const int nvt = (int)ceilDiv(cols / N, 256);
+    dim3 grid((unsigned)rows), block(256);
+#define FEW_LAUNCH(NVT)                                                                                                \
+  hipLaunchKernelGGL((rowBlockVecKernel<T, NVT, OP, WT>), grid, block, 0, stream, out, in, weight, bias, invRms, rows, \
+                     (int)cols, inStride, outStride, eps)
+    if (nvt <= 1) FEW_LAUNCH(1);
+    else if (nvt <= 2) FEW_LAUNCH(2);
+    else FEW_LAUNCH(4);
+#undef FEW_LAUNCH
   } else if (vectorOk && cols % N == 0 && cols / N <= 64 * 16) {
     int nvec = (int)(cols / N);
     int nv = (nvec + 63) / 64;

@@ -281,7 +281,7 @@ def test_softmax_rows_sum_to_one_at_full_size(ops, dev):
 
 @pytest.mark.parametrize("dtype,eps", [(torch.float32, 1e-6), (torch.bfloat16, 1e-5), (torch.float16, 1e-5)])
 def test_rms_norm(ops, dev, dtype, eps):
-    for shape in [(2, 128, 512), (512, 4096), (3, 100), (4, 20000)]:
+    for shape in [(2, 128, 512), (512, 4096), (3, 100), (4, 20000), (8, 4096), (64, 8192), (1, 2048)]:
         x = torch.randn(shape, generator=g(21)).to(dtype)
         w = (1 + 0.1 * torch.randn(shape[-1], generator=g(22))).to(dtype)
         want32 = oracle.rms_norm(x.float(), w.float(), eps)
