@@ -2130,24 +2130,28 @@ static diopiError_t launchSkinnyForShape(diopiContextHandle_t ctx, hipStream_t s
   // 52.9 -> 33.6, 55.7 -> 36.0. At N = 4096 (16 columns per workgroup: the activations are four times the weight
   // bytes on the way into a CU) only 17 to 32 rows gain (14.4 -> 12.7); one row loses (9.1 -> 11.0), and so does
   // everything narrower.
-  // A 4096-wide weight with a long K at 33 to 64 rows (the down projection of a decode step) takes this form too, K
-  // split two ways over grid.y with fp32 slices and the reduction pass: 64 x 4096 x 11008 34.0 -> 27.6 us cold against the
-  // register-layout kernels below. The same split on wider weights loses (N = 11008: 23.0 -> 25.5 us, four ways 33.6),
-  // and at K = 4096 it changes nothing (14.6 -> 15.0).
+  // A 4096-wide weight (the o and down projections of a decode step) takes this form too with K split over grid.y, fp32
+  // slices and the reduction pass: with K of 8192 and more at any row count, two slices up to 16 rows and four beyond
+  // (us cold at K = 11008 against the register-layout kernels below: 1 row 23.9 -> 19.2, 16 rows 28.3 -> 20.3, 32 rows
+  // 27.5 -> 21.6, 64 rows 34.0 -> 24.5 (27.7 with two slices); 64 x 4096 x 14336 34.2 -> 28.5). At K = 4096 two slices are
+  // within the noise of what the other routes do (32 rows 12.4 -> 11.5 .. 12.3, 64 rows 14.5 -> 13.8 .. 14.8) and one row
+  // loses (7.7 -> 10.0). The same split on wider weights loses (N = 11008: 23.0 -> 25.5 us, four ways 33.6).
   const bool canSplitLds = a.N % 8 == 0 && mult8(p.sOm) && ptr16(p.out) && (!p.bias || ptr16(p.bias)) &&
                            (!p.Cin || (p.sCn == 1 && mult8(p.sCm) && ptr16(p.Cin))) && rot == nullptr;
-  const bool narrowLongK = a.N >= 4096 && a.N < 5120 && a.M > 32 && a.K >= 8192 && a.K % (2 * kSkinnyLdsBK) == 0 && canSplitLds;
+  const bool narrow = a.N >= 4096 && a.N < 5120 && a.K % kSkinnyLdsBK == 0 && canSplitLds;
+  const int narrowWays = narrow && a.K >= 8192 ? (a.M <= 16 ? 2 : 4) : 1;
+  const bool narrowLongK = narrowWays > 1;
   if ((a.N >= 5120 || (a.N >= 4096 && a.M > 16 && a.M <= 32) || narrowLongK) &&
       ((int64_t)(a.N - 1) * a.ldb + a.K) * (int64_t)sizeof(T) < ((int64_t)1 << 31) &&
       ((int64_t)(a.M - 1) * a.lda + a.K) * (int64_t)sizeof(T) < ((int64_t)1 << 31)) {
-    const int ways = narrowLongK ? 2 : 1;
+    const int ways = narrowWays;
     const int wgs = std::max(1, cus / ways);
     const int rounds = (a.N + 128 * wgs - 1) / (128 * wgs);
     a.colsPerWg = (a.N + wgs * rounds - 1) / (wgs * rounds);
     if (ways > 1) {
       void* ws = nullptr;
       AMD_TRY(requireWorkspace(ctx, (int64_t)ways * a.M * a.N * 4, &ws));
-      a.partial = static_cast<float*>(ws), a.kPerWg = a.K / ways;
+      a.partial = static_cast<float*>(ws), a.kPerWg = ceilDiv(a.K / kSkinnyLdsBK, ways) * kSkinnyLdsBK;  // whole stages
     }
     if (rot != nullptr) a.colsPerWg = (a.colsPerWg + 1) & ~1;  // even: the two columns of a rotary pair stay together
     if (handled) *handled = true;
