@@ -1890,14 +1890,28 @@ template <typename T>
 __global__ __launch_bounds__(256) void splitKReduceKernel(MfmaArgs g, int splits) {
   using Frag = typename MfmaOp<T>::Frag;
   const int groups = g.N / 8;
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= (int64_t)g.M * groups) return;
   const int row = (int)(idx / groups), col = (int)(idx - (int64_t)row * groups) * 8;
   const float* src = g.partial + (int64_t)row * g.N + col;
+  // four slices' pieces are requested together (a loop of one load and one add per slice walks the slices one memory
+  // round trip at a time); the additions keep the slice order
   f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = lo;
-  for (int sp = 0; sp < splits; ++sp) {
-    lo += *reinterpret_cast<const f32x4*>(src + (int64_t)sp * g.M * g.N);
-    hi += *reinterpret_cast<const f32x4*>(src + (int64_t)sp * g.M * g.N + 4);
+  const int64_t slice = (int64_t)g.M * g.N;
+  int sp = 0;
+  for (; sp + 4 <= splits; sp += 4) {
+    f32x4 l4[4], h4[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      l4[u] = *reinterpret_cast<const f32x4*>(src + (sp + u) * slice);
+      h4[u] = *reinterpret_cast<const f32x4*>(src + (sp + u) * slice + 4);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) lo += l4[u], hi += h4[u];
+  }
+  for (; sp < splits; ++sp) {
+    lo += *reinterpret_cast<const f32x4*>(src + sp * slice);
+    hi += *reinterpret_cast<const f32x4*>(src + sp * slice + 4);
   }
   const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   const T* cin = reinterpret_cast<const T*>(g.Cin);
@@ -1913,6 +1927,14 @@ __global__ __launch_bounds__(256) void splitKReduceKernel(MfmaArgs g, int splits
     o[e] = static_cast<T>(x);
   }
   *reinterpret_cast<Frag*>(reinterpret_cast<T*>(g.out) + (int64_t)row * g.ldo + col) = o;
+}
+
+// Small reductions (decode-sized products: a few tens of thousands of lanes) go out as single waves, so that they spread
+// over more CUs than they would fill workgroups of four.
+template <typename T>
+static void launchSplitKReduce(hipStream_t stream, const MfmaArgs& g, int splits, int64_t items) {
+  const int threads = items <= 65536 ? 64 : 256;
+  hipLaunchKernelGGL(splitKReduceKernel<T>, dim3((unsigned)ceilDiv(items, (int64_t)threads)), dim3(threads), 0, stream, g, splits);
 }
 
 // How many ways to split K so that a problem with few 128 x 128 tiles still fills the chip (two workgroups per CU):
@@ -1990,7 +2012,7 @@ static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p
   AMD_LAUNCH_CHECK();
   if (EPI == kEpiPartial) {
     const int64_t items = p.M * (p.N / 8);
-    hipLaunchKernelGGL(splitKReduceKernel<T>, dim3((unsigned)ceilDiv(items, 256)), dim3(256), 0, stream, g, splits);
+    launchSplitKReduce<T>(stream, g, splits, items);
     AMD_LAUNCH_CHECK();
   }
   return diopiSuccess;
@@ -2030,7 +2052,7 @@ static diopiError_t launchMfmaPipelined128(hipStream_t stream, const GemmProblem
   AMD_LAUNCH_CHECK();
   if (EPI == kEpiPartial) {
     const int64_t items = p.M * (p.N / 8);
-    hipLaunchKernelGGL(splitKReduceKernel<T>, dim3((unsigned)ceilDiv(items, 256)), dim3(256), 0, stream, g, splits);
+    launchSplitKReduce<T>(stream, g, splits, items);
     AMD_LAUNCH_CHECK();
   }
   return diopiSuccess;
@@ -2053,8 +2075,7 @@ static diopiError_t launchSkinny(hipStream_t stream, const SkinnyArgs& a) {
     g.out = a.out, g.Cin = a.Cin, g.bias = a.bias, g.partial = a.partial;
     g.ldo = a.ldo, g.sCm = a.sCm, g.sCn = a.sCn;
     g.M = a.M, g.N = a.N, g.K = a.K, g.alpha = a.alpha, g.beta = a.beta;
-    hipLaunchKernelGGL(splitKReduceKernel<T>, dim3((unsigned)ceilDiv((int64_t)a.M * (a.N / 8), 256)), dim3(256), 0, stream, g,
-                       splits);
+    launchSplitKReduce<T>(stream, g, splits, (int64_t)a.M * (a.N / 8));
     AMD_LAUNCH_CHECK();
   }
   return diopiSuccess;
@@ -2074,8 +2095,7 @@ static diopiError_t launchSkinnyLds(hipStream_t stream, const SkinnyArgs& a) {
     g.out = a.out, g.Cin = a.Cin, g.bias = a.bias, g.partial = a.partial;
     g.ldo = a.ldo, g.sCm = a.sCm, g.sCn = a.sCn;
     g.M = a.M, g.N = a.N, g.K = a.K, g.alpha = a.alpha, g.beta = a.beta;
-    hipLaunchKernelGGL(splitKReduceKernel<T>, dim3((unsigned)ceilDiv((int64_t)a.M * (a.N / 8), 256)), dim3(256), 0, stream, g,
-                       splits);
+    launchSplitKReduce<T>(stream, g, splits, (int64_t)a.M * (a.N / 8));
     AMD_LAUNCH_CHECK();
   }
   return diopiSuccess;
@@ -2095,8 +2115,7 @@ static diopiError_t launchSkinnyWide(hipStream_t stream, const SkinnyArgs& a) {
     g.out = a.out, g.Cin = a.Cin, g.bias = a.bias, g.partial = a.partial;
     g.ldo = a.ldo, g.sCm = a.sCm, g.sCn = a.sCn;
     g.M = a.M, g.N = a.N, g.K = a.K, g.alpha = a.alpha, g.beta = a.beta;
-    hipLaunchKernelGGL(splitKReduceKernel<T>, dim3((unsigned)ceilDiv((int64_t)a.M * (a.N / 8), 256)), dim3(256), 0, stream, g,
-                       splits);
+    launchSplitKReduce<T>(stream, g, splits, (int64_t)a.M * (a.N / 8));
     AMD_LAUNCH_CHECK();
   }
   return diopiSuccess;
