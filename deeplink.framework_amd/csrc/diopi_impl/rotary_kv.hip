@@ -526,6 +526,20 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiIndexPutInp(
     AMD_TRY(stridedCopy(stream, one, expanded));
     cval = expanded;
   }
+  // Whole rows of the leading dim replaced by rows of the same dtype (how a KV cache is written through index_put):
+  // the byte mover of diopiDestIndexCopyKV, a workgroup per row with the widest vector the rows allow, instead of an
+  // element per lane through a lossless carrier (8192 rows of 8 KiB: 94 -> 24 us). Negative indices wrap and rows out
+  // of range are dropped, as in the generic form.
+  if (!accumulate && nIdx == 1 && cval.dtype == in.dtype && valRowStride == inner && inner * in.itemsize >= 512 &&
+      rows <= 0x7fffffff) {
+    KvScatterArgs a;
+    a.pool[0].out = in.data, a.pool[0].src = cval.data, a.pool[0].slots = in.shape[0];
+    a.pool[0].outRowStrideVecs = in.stride[0] * in.itemsize, a.pool[0].srcRowStrideVecs = inner * in.itemsize;
+    a.pool[1] = a.pool[0];
+    a.destLoc = idx[0].data, a.tokens = rows;
+    return idt == diopi_dtype_int64 ? launchDestCopy<int64_t>(stream, a, 1, inner * in.itemsize)
+                                    : launchDestCopy<int32_t>(stream, a, 1, inner * in.itemsize);
+  }
   IndexTables tab;
   for (int i = 0; i < kMaxDims; ++i) tab.ptrs[i] = nullptr, tab.sizes[i] = 1, tab.strides[i] = 0;
   for (int64_t i = 0; i < nIdx; ++i) {

@@ -461,3 +461,16 @@ def test_index_put(ops, dev):
     got = pool.clone().to(dev)
     ops.index_put_(got, [loc.to(dev)], rows.to(dev))
     assert_exact(got, oracle.index_put_(pool.clone(), [loc], rows))
+    # the same with rows long enough for the whole-row byte mover (8 KiB, 520 bytes and 1000 bytes a row), negative
+    # indices, both index types, and a value dtype that differs from the pool's (which takes the element form)
+    for shape, dt in [((300, 32, 128), torch.bfloat16), ((64, 130), torch.float32), ((50, 5, 100), torch.float16)]:
+        pool = torch.randn(shape, generator=g(44)).to(dt)
+        loc = torch.tensor([5, -1, 17, 0, -shape[0] + 1, 33, 2])
+        rows = torch.randn(len(loc), *shape[1:], generator=g(45)).to(dt)
+        for idt in (torch.int64, torch.int32):
+            got = pool.clone().to(dev)
+            ops.index_put_(got, [loc.to(idt).to(dev)], rows.to(dev))
+            assert_exact(got, oracle.index_put_(pool.clone(), [loc], rows))
+        got = pool.clone().to(dev)
+        ops.index_put_(got, [loc.to(dev)], rows.float().to(dev))
+        assert_exact(got, oracle.index_put_(pool.clone(), [loc], rows))
