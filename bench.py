@@ -516,6 +516,18 @@ def op_microbench(pkg, torch, dev, rt, stream, with_cpu=True):
         mil = int(pd["max_input_len"])
         res[-2]["cpu"] = cpu_op(torch, dev, lambda q, kp, vp, loc, ln: oracle.token_attention(q, kp, vp, loc, ln, mil),
                                 (g["q"], g["k_pool"], g["v_pool"], g["b_loc"], g["b_seq_len"]), warm=1, runs=3)
+    # the two-call form of the same attention, which is what the reference's yaml binds: scores [heads, tokens] in fp32 to
+    # memory, then softmax and the sum over V from them
+    att = torch.empty(32, L, dtype=torch.float32, device=dev)
+    a1 = Prepared(pkg, "diopiTokenAttentionInference", att, g["q"], g["k_pool"], g["b_loc"], g["b_start_loc"], g["b_seq_len"],
+                  int(g["max_input_len"]))
+    a2 = Prepared(pkg, "diopiTokenSoftmaxReduceVInference", out, att, g["v_pool"], g["b_loc"], g["b_start_loc"], g["b_seq_len"],
+                  int(g["max_input_len"]), 0)
+    p_a1, p_a2 = time_ops_stats(rt, stream, [a1, a2], 30, 6)
+    half_bytes = L * 8192 + L * idx_b + L * 32 * 4 + 64 * 32 * 128 * 2
+    res.append(hbm_row("diopiTokenAttentionInference", f"batch 64, 32x128, sum(len)={L}, fp32 scores", half_bytes, None, p_a1))
+    res.append(hbm_row("diopiTokenSoftmaxReduceVInference", f"batch 64, 32x128, sum(len)={L}, fp32 scores", half_bytes, None, p_a2))
+    del att
     res.append(decode_layer_step(pkg, torch, dev, rt, stream, g))
     del g, pd
     # int8 weight-only linear: weights rotate through 8 copies (360 MB) for the cold figure

@@ -26,6 +26,10 @@
 //     when there would otherwise be too few workgroups for the chip, at most 256 per sequence); states are merged by
 //     wave butterflies, then through LDS, then across chunks by a small lane-parallel second kernel.
 //
+// The two halves of the two-call form (scores to memory, then softmax and the sum over V from stored scores) are the same
+// streaming kernel with the other half of the work compiled out: 588 -> 462 us for both at batch 64 with 156 000 cached
+// tokens, and the second half no longer walks a long sequence with one workgroup (1 x 32768 tokens: 1709 -> 60 us).
+//
 // Head rows of 128, 256 or 512 bytes at 16-byte aligned strides take the kernels above; any other head size or
 // alignment (up to 1024 elements) takes the generic kernels at the end: one workgroup per (sequence, head), 256 tokens
 // at a time, one token's dot product per thread and P.V with the threads over d. A correctness path.
@@ -64,6 +68,8 @@ struct TaArgs {
   int64_t slots;
   int heads, kvHeads, d, maxLen, nsplit, chunk;
   float scaleLog2e;  // log2(e) / sqrt(d)
+  const void* logits;  // two-call form: scores [heads, total_tokens], row h at logits + h * logitsHeadStride (elements)
+  int64_t logitsHeadStride;
 };
 
 // Merge (m, l, acc) of another online-softmax stream into this one.
@@ -79,13 +85,23 @@ __device__ __forceinline__ void mergeState(float& m, float& l, float (&acc)[E], 
   m = mn;
 }
 
-// T: bf16_t / half_t (8 per 16 B) or float (4 per 16 B). LPT lanes cover one head row.
-template <typename T, int LPT, bool HIW>
+// The three things the streaming kernel below can do with a chunk of a sequence: the whole decode attention (scores,
+// online softmax and the sum over V), only the scores (first half of the two-call form: att[h, start_b + t]), or the
+// softmax and the sum over V from scores computed earlier (second half of the two-call form).
+enum TaMode { kTaFused = 0, kTaLogitsOut = 1, kTaReduceV = 2 };
+
+// T: bf16_t / half_t (8 per 16 B) or float (4 per 16 B). LPT lanes cover one head row. LT: the type of the scores in
+// memory (the two-call modes).
+template <typename T, int LPT, bool HIW, int MODE = kTaFused, typename LT = float>
 __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* __restrict__ out,
                                                                      float* __restrict__ partial) {
   using V = typename Vec16<T>::type;
   constexpr int N = Vec16<T>::N;
   constexpr int TPW = 64 / LPT;  // tokens per wave-wide load
+  constexpr bool kNeedK = MODE != kTaReduceV, kNeedV = MODE != kTaLogitsOut;
+  // rows per wave in flight: 2 K + 2 V in the fused mode; 4 K when only scores are produced; 2 V (and their stored scores)
+  // in the second half of the two-call form, where 4 measured slower (306 against 234 us at batch 64, 156 000 tokens)
+  constexpr int UNR = MODE == kTaLogitsOut ? 2 * kTaUnroll : kTaUnroll;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int sub = lane % LPT, grp = lane / LPT;
   // HIW: the lane groups of a wave take TPW consecutive heads of the same token (a wave load is TPW head rows, contiguous
@@ -93,71 +109,91 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   const int h = HIW ? blockIdx.x * TPW + grp : blockIdx.x, split = blockIdx.y, b = blockIdx.z;
   const int len = min(max((int)ldIndex(a.bLen, b, a.len64), 0), a.maxLen);  // a length beyond the table's width is cut to it
   const int begin = split * a.chunk;
-  if (begin >= len && !(split == 0)) return;  // nothing to do; split 0 still writes zeros for len == 0
+  if (begin >= len && !(split == 0 && MODE != kTaLogitsOut)) return;  // nothing to do; split 0 still writes zeros for len == 0
   const int end = min(len, begin + a.chunk);
   const int kvh = h / (a.heads / a.kvHeads);
   const int64_t locBase = (int64_t)b * a.locRowStride + (a.maxLen - len);
+  // the scores of this lane's head for the tokens of sequence b (two-call modes)
+  LT* scores = nullptr;
+  if constexpr (MODE != kTaFused)
+    scores = static_cast<LT*>(const_cast<void*>(a.logits)) + h * a.logitsHeadStride + ldIndex(a.bStart, b, a.start64);
 
   float qf[N];
-  {
+  if constexpr (kNeedK) {
+    // scores leave the kernel in natural units, inside it they are in units of log2
+    const float qScale = MODE == kTaLogitsOut ? a.scaleLog2e / kLog2eTA : a.scaleLog2e;
     V qv = *reinterpret_cast<const V*>(reinterpret_cast<const T*>(a.q) + b * a.qBatchStride + h * a.qHeadStride + sub * N);
 #pragma unroll
-    for (int e = 0; e < N; ++e) qf[e] = static_cast<float>(qv[e]) * a.scaleLog2e;
+    for (int e = 0; e < N; ++e) qf[e] = static_cast<float>(qv[e]) * qScale;
   }
-  const T* kBase = reinterpret_cast<const T*>(a.k) + kvh * a.kHeadStride + sub * N;
-  const T* vBase = reinterpret_cast<const T*>(a.v) + kvh * a.vHeadStride + sub * N;
+  const T* kBase = kNeedK ? reinterpret_cast<const T*>(a.k) + kvh * a.kHeadStride + sub * N : nullptr;
+  const T* vBase = kNeedV ? reinterpret_cast<const T*>(a.v) + kvh * a.vHeadStride + sub * N : nullptr;
 
   float m = -INFINITY, l = 0.f, acc[N];
 #pragma unroll
   for (int e = 0; e < N; ++e) acc[e] = 0.f;
 
   constexpr int TPI = HIW ? 1 : TPW;  // tokens per wave-wide load
-  constexpr int STEP = kTaWaves * kTaUnroll * TPI;  // tokens per workgroup iteration
+  constexpr int STEP = kTaWaves * UNR * TPI;  // tokens per workgroup iteration
   // Two-deep software pipeline: while the rows of iteration i are being reduced, the K/V rows
   // of iteration i+1 and the slot indices of iteration i+2 are already in flight.
-  int64_t slot[kTaUnroll];
-  V kr[kTaUnroll], vr[kTaUnroll], kn[kTaUnroll], vn[kTaUnroll];
-  bool ok[kTaUnroll], okn[kTaUnroll];
+  int64_t slot[UNR];
+  int slotTok[UNR];  // the token each slot index belongs to (the stored scores are addressed by it)
+  V kr[UNR], vr[UNR], kn[UNR], vn[UNR];
+  float lr[UNR], ln[UNR];  // stored scores of the rows (kTaReduceV)
+  bool ok[UNR], okn[UNR];
   auto loadSlots = [&](int it) {
-    int t0 = it + wave * kTaUnroll * TPI + (HIW ? 0 : grp);
+    int t0 = it + wave * UNR * TPI + (HIW ? 0 : grp);
 #pragma unroll
-    for (int u = 0; u < kTaUnroll; ++u) {
+    for (int u = 0; u < UNR; ++u) {
       int t = t0 + u * TPI;
+      slotTok[u] = t;
       slot[u] = t < end ? ldIndex(a.bLoc, locBase + t, a.loc64) : -1;
     }
   };
-  auto loadRows = [&](V (&kk)[kTaUnroll], V (&vv)[kTaUnroll], bool (&okk)[kTaUnroll]) {
+  auto loadRows = [&](V (&kk)[UNR], V (&vv)[UNR], float (&lg)[UNR], bool (&okk)[UNR]) {
 #pragma unroll
-    for (int u = 0; u < kTaUnroll; ++u) {
+    for (int u = 0; u < UNR; ++u) {
       okk[u] = slot[u] >= 0 && slot[u] < a.slots;  // slots outside the pool are skipped, never dereferenced
       int64_t s = okk[u] ? slot[u] : 0;
-      kk[u] = __builtin_nontemporal_load(reinterpret_cast<const V*>(kBase + s * a.kSlotStride));
-      vv[u] = __builtin_nontemporal_load(reinterpret_cast<const V*>(vBase + s * a.vSlotStride));
+      if constexpr (kNeedK) kk[u] = __builtin_nontemporal_load(reinterpret_cast<const V*>(kBase + s * a.kSlotStride));
+      if constexpr (kNeedV) vv[u] = __builtin_nontemporal_load(reinterpret_cast<const V*>(vBase + s * a.vSlotStride));
+      if constexpr (MODE == kTaReduceV) lg[u] = okk[u] ? static_cast<float>(scores[slotTok[u]]) * kLog2eTA : -INFINITY;
     }
   };
   loadSlots(begin);
-  loadRows(kr, vr, ok);
+  loadRows(kr, vr, lr, ok);
   loadSlots(begin + STEP);
   for (int it = begin; it < end; it += STEP) {
-    loadRows(kn, vn, okn);        // rows of the next iteration (all masked past the end)
+    loadRows(kn, vn, ln, okn);    // rows of the next iteration (all masked past the end)
     loadSlots(it + 2 * STEP);     // indices of the one after
-    float sc[kTaUnroll];
+    float sc[UNR];
     float mn = m;
 #pragma unroll
-    for (int u = 0; u < kTaUnroll; ++u) {
-      float d = 0.f;
+    for (int u = 0; u < UNR; ++u) {
+      if constexpr (kNeedK) {
+        float d = 0.f;
 #pragma unroll
-      for (int e = 0; e < N; ++e) d += qf[e] * static_cast<float>(kr[u][e]);
+        for (int e = 0; e < N; ++e) d += qf[e] * static_cast<float>(kr[u][e]);
 #pragma unroll
-      for (int off = LPT / 2; off > 0; off >>= 1) d += __shfl_xor(d, off, 64);
-      sc[u] = ok[u] ? d : -INFINITY;
+        for (int off = LPT / 2; off > 0; off >>= 1) d += __shfl_xor(d, off, 64);
+        sc[u] = ok[u] ? d : -INFINITY;
+      } else {
+        sc[u] = lr[u];
+      }
       mn = fmaxf(mn, sc[u]);
     }
-    if (mn != -INFINITY) {
-      float corr = __builtin_amdgcn_exp2f(m - mn);  // m == -inf gives 0, acc and l are 0 then anyway
-      float p[kTaUnroll], ps = 0.f;
+    if constexpr (MODE == kTaLogitsOut) {
 #pragma unroll
-      for (int u = 0; u < kTaUnroll; ++u) {
+      for (int u = 0; u < UNR; ++u) {
+        const int t = it + wave * UNR * TPI + (HIW ? 0 : grp) + u * TPI;
+        if (sub == 0 && t < end) scores[t] = static_cast<LT>(sc[u]);
+      }
+    } else if (mn != -INFINITY) {
+      float corr = __builtin_amdgcn_exp2f(m - mn);  // m == -inf gives 0, acc and l are 0 then anyway
+      float p[UNR], ps = 0.f;
+#pragma unroll
+      for (int u = 0; u < UNR; ++u) {
         p[u] = __builtin_amdgcn_exp2f(sc[u] - mn);
         ps += p[u];
       }
@@ -166,14 +202,15 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
       for (int e = 0; e < N; ++e) {
         float s = acc[e] * corr;
 #pragma unroll
-        for (int u = 0; u < kTaUnroll; ++u) s += p[u] * static_cast<float>(vr[u][e]);
+        for (int u = 0; u < UNR; ++u) s += p[u] * static_cast<float>(vr[u][e]);
         acc[e] = s;
       }
       m = mn;
     }
 #pragma unroll
-    for (int u = 0; u < kTaUnroll; ++u) kr[u] = kn[u], vr[u] = vn[u], ok[u] = okn[u];
+    for (int u = 0; u < UNR; ++u) kr[u] = kn[u], vr[u] = vn[u], lr[u] = ln[u], ok[u] = okn[u];
   }
+  if constexpr (MODE == kTaLogitsOut) return;
 
   // merge the TPW lane groups of the wave (each holds other tokens of the same head)
   if (!HIW)
@@ -342,137 +379,6 @@ __global__ __launch_bounds__(256) void decodeMergeWideKernel(T* __restrict__ out
       const int e = lane + 64 * k;
       if (e < d) out[pair * d + e] = static_cast<T>(red[0][e] + red[1][e] + red[2][e] + red[3][e]);
     }
-  }
-}
-
-// ------------------------------------------------- two-call form, first half --
-// att[h, start_b + t] = q[b,h,:] . k[slot_t,h,:] / sqrt(d); a workgroup covers 256*? tokens
-template <typename T, int LPT, typename OT>
-__global__ __launch_bounds__(256) void tokenLogitsKernel(TaArgs a, OT* __restrict__ att, int64_t attHeadStride) {
-  using V = typename Vec16<T>::type;
-  constexpr int N = Vec16<T>::N;
-  constexpr int TPW = 64 / LPT;
-  const int h = blockIdx.x, b = blockIdx.z;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int sub = lane % LPT, grp = lane / LPT;
-  const int len = min(max((int)ldIndex(a.bLen, b, a.len64), 0), a.maxLen);  // a length beyond the table's width is cut to it
-  const int64_t start = ldIndex(a.bStart, b, a.start64);
-  const int begin = blockIdx.y * a.chunk;
-  if (begin >= len) return;
-  const int end = min(len, begin + a.chunk);
-  const int kvh = h / (a.heads / a.kvHeads);
-  const int64_t locBase = (int64_t)b * a.locRowStride + (a.maxLen - len);
-  float qf[N];
-  {
-    V qv = *reinterpret_cast<const V*>(reinterpret_cast<const T*>(a.q) + b * a.qBatchStride + h * a.qHeadStride + sub * N);
-#pragma unroll
-    for (int e = 0; e < N; ++e) qf[e] = static_cast<float>(qv[e]);
-  }
-  const T* kBase = reinterpret_cast<const T*>(a.k) + kvh * a.kHeadStride + sub * N;
-  const float scale = a.scaleLog2e / kLog2eTA;
-  constexpr int STEP = 4 * kTaUnroll * TPW;
-  for (int it = begin; it < end; it += STEP) {
-    int t0 = it + wave * kTaUnroll * TPW + grp;
-    V kr[kTaUnroll];
-    bool ok[kTaUnroll];
-#pragma unroll
-    for (int u = 0; u < kTaUnroll; ++u) {
-      int t = t0 + u * TPW;
-      int64_t s = t < end ? ldIndex(a.bLoc, locBase + t, a.loc64) : -1;
-      ok[u] = s >= 0 && s < a.slots;
-      kr[u] = *reinterpret_cast<const V*>(kBase + (ok[u] ? s : 0) * a.kSlotStride);
-    }
-#pragma unroll
-    for (int u = 0; u < kTaUnroll; ++u) {
-      float d = 0.f;
-#pragma unroll
-      for (int e = 0; e < N; ++e) d += qf[e] * static_cast<float>(kr[u][e]);
-#pragma unroll
-      for (int off = LPT / 2; off > 0; off >>= 1) d += __shfl_xor(d, off, 64);
-      int t = t0 + u * TPW;
-      if (sub == 0 && t < end) att[h * attHeadStride + start + t] = static_cast<OT>(ok[u] ? d * scale : -INFINITY);
-    }
-  }
-}
-
-// ------------------------------------------------ two-call form, second half --
-// out[b,h,:] = softmax(logics[h, start_b : start_b+len]) . v[slots]; one workgroup per (b,h)
-template <typename T, int LPT, typename LT>
-__global__ __launch_bounds__(256) void softmaxReduceVKernel(TaArgs a, T* __restrict__ out,
-                                                             const LT* __restrict__ logics, int64_t logHeadStride) {
-  using V = typename Vec16<T>::type;
-  constexpr int N = Vec16<T>::N;
-  constexpr int TPW = 64 / LPT;
-  const int h = blockIdx.x, b = blockIdx.z;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int sub = lane % LPT, grp = lane / LPT;
-  const int len = min(max((int)ldIndex(a.bLen, b, a.len64), 0), a.maxLen);  // a length beyond the table's width is cut to it
-  const int64_t start = ldIndex(a.bStart, b, a.start64);
-  const int kvh = h / (a.heads / a.kvHeads);
-  const int64_t locBase = (int64_t)b * a.locRowStride + (a.maxLen - len);
-  const LT* lg = logics + h * logHeadStride + start;
-  __shared__ float red[4][2 + LPT * N];
-  __shared__ float bcast[2];
-  // pass 1: row max and sum of exp over the logits
-  float m = -INFINITY;
-  for (int t = threadIdx.x; t < len; t += 256) m = fmaxf(m, static_cast<float>(lg[t]));
-  m = waveMax(m);
-  if (lane == 0) red[wave][0] = m;
-  __syncthreads();
-  m = fmaxf(fmaxf(red[0][0], red[1][0]), fmaxf(red[2][0], red[3][0]));
-  __syncthreads();
-  const float mS = (m == -INFINITY) ? 0.f : m * kLog2eTA;
-  float s = 0.f;
-  for (int t = threadIdx.x; t < len; t += 256) s += exp2f(static_cast<float>(lg[t]) * kLog2eTA - mS);
-  s = waveSum(s);
-  if (lane == 0) red[wave][1] = s;
-  __syncthreads();
-  if (threadIdx.x == 0) bcast[0] = red[0][1] + red[1][1] + red[2][1] + red[3][1];
-  __syncthreads();
-  const float inv = bcast[0] > 0.f ? 1.f / bcast[0] : 0.f;
-  // pass 2: stream V
-  const T* vBase = reinterpret_cast<const T*>(a.v) + kvh * a.vHeadStride + sub * N;
-  float acc[N];
-#pragma unroll
-  for (int e = 0; e < N; ++e) acc[e] = 0.f;
-  constexpr int STEP = 4 * kTaUnroll * TPW;
-  for (int it = 0; it < len; it += STEP) {
-    int t0 = it + wave * kTaUnroll * TPW + grp;
-    V vr[kTaUnroll];
-    float p[kTaUnroll];
-#pragma unroll
-    for (int u = 0; u < kTaUnroll; ++u) {
-      int t = t0 + u * TPW;
-      int64_t sl = t < len ? ldIndex(a.bLoc, locBase + t, a.loc64) : -1;
-      bool ok = sl >= 0 && sl < a.slots;
-      vr[u] = *reinterpret_cast<const V*>(vBase + (ok ? sl : 0) * a.vSlotStride);
-      p[u] = ok ? exp2f(static_cast<float>(lg[t]) * kLog2eTA - mS) : 0.f;
-    }
-#pragma unroll
-    for (int e = 0; e < N; ++e) {
-#pragma unroll
-      for (int u = 0; u < kTaUnroll; ++u) acc[e] += p[u] * static_cast<float>(vr[u][e]);
-    }
-  }
-#pragma unroll
-  for (int off = LPT; off < 64; off <<= 1) {
-#pragma unroll
-    for (int e = 0; e < N; ++e) acc[e] += __shfl_xor(acc[e], off, 64);
-  }
-  __syncthreads();
-  if (grp == 0) {
-#pragma unroll
-    for (int e = 0; e < N; ++e) red[wave][2 + sub * N + e] = acc[e];
-  }
-  __syncthreads();
-  if (wave == 0 && grp == 0) {
-    V o;
-#pragma unroll
-    for (int e = 0; e < N; ++e) {
-      float r = red[0][2 + sub * N + e] + red[1][2 + sub * N + e] + red[2][2 + sub * N + e] + red[3][2 + sub * N + e];
-      o[e] = static_cast<T>(r * inv);
-    }
-    *reinterpret_cast<V*>(out + ((int64_t)b * a.heads + h) * a.d + sub * N) = o;
   }
 }
 
@@ -700,11 +606,27 @@ static diopiError_t fillArgs(const TaViews& t, bool needK, bool needV, int maxLe
   a->d = (int)q.shape[2];
   a->maxLen = maxLen;
   a->nsplit = 1;
+  a->logits = nullptr, a->logitsHeadStride = 0;
   // at most kTaMaxSplit chunks per sequence; chunks stay a multiple of 64 tokens
   a->chunk = kTaChunk;
   if ((int64_t)maxLen > (int64_t)kTaChunk * kTaMaxSplit) a->chunk = (int)(ceilDiv(ceilDiv(maxLen, kTaMaxSplit), 64) * 64);
   a->scaleLog2e = kLog2eTA / sqrtf((float)q.shape[2]);
   return diopiSuccess;
+}
+
+// Chunk length of the split over a sequence for the streaming kernels (decodeSplitKernel in its three modes).
+static void chooseChunk(TaArgs* a, int64_t groupsPerSeq, int64_t batch, int maxInputLen) {
+  // A workgroup walks its chunk with two loads per wave in flight, so the rate comes from the number of workgroups a
+  // CU holds at once. Few sequences or short ones are cut into smaller chunks until there are about kTaWgsPerCu
+  // workgroups per CU; large batches keep the 512-token chunks, whose partial results are fewer. Measured (us, 32 heads
+  // x 128, bf16, with 512-token chunks -> with these): 1 x 2048 tokens 72 -> 20, 1 x 32768 130 -> 96, 8 x 4096 130 -> 91,
+  // 4 x (100 .. 16384) 123 -> 86, 64 x (256 .. 512) 101 -> 80; 64 x (512 .. 4096) and 256 x (1024 .. 2048) keep their chunks.
+  const int64_t groups = groupsPerSeq * batch, cus = computeUnits(), len = std::max(maxInputLen, 1);
+  const int64_t wantSplits = std::max<int64_t>(1, ceilDiv(kTaWgsPerCu * cus, groups));
+  const int64_t fine = ceilDiv(ceilDiv(len, wantSplits), 64) * 64;
+  const int64_t capped = ceilDiv(ceilDiv(len, (int64_t)kTaMaxSplit), 64) * 64;  // at most kTaMaxSplit chunks
+  const int64_t shortest = groups * ceilDiv(len, (int64_t)kTaMinChunk) < cus ? kTaTinyChunk : kTaMinChunk;
+  a->chunk = (int)std::max(std::max(capped, shortest), std::min<int64_t>(a->chunk, fine));
 }
 
 #define TA_DISPATCH(DTYPE, BYTES, CALL)                                                        \
@@ -759,6 +681,77 @@ static diopiError_t decodeScratch(float** out) {
 using namespace amd;
 
 // staticScratch: partial results go to the library's own device array instead of workspace from the context.
+// Launches decodeSplitKernel in one of its modes over (head groups, chunks, sequences) and, for the modes that produce
+// the attention output, merges the chunks. scoresF32: the stored scores of the two-call modes are float32 (else T).
+template <int MODE>
+static diopiError_t streamChunks(diopiContextHandle_t ctx, hipStream_t stream, TaArgs a, diopiDtype_t dtype, int64_t bytes,
+                                 int64_t batch, int maxInputLen, void* outPtr, bool scoresF32, bool staticScratch,
+                                 float* ownScratch) {
+  // The lane groups of a wave take consecutive heads of one token when the head count allows it: a wave load is then
+  // one contiguous piece of a slot (1 KiB) instead of head rows of four different slots (431 -> 421 us at batch 64,
+  // 32 heads x 128, 156 043 cached tokens).
+  const int tpw = (int)(64 / std::max<int64_t>(1, bytes / 16));
+  // (the two-call modes keep four tokens of one head per wave load: their stored scores are then four consecutive
+  // floats of a row instead of one float in each of four rows; second half at batch 64, 156 000 tokens: 326 -> 234 us)
+  const bool hiw = MODE == kTaFused && (bytes == 128 || bytes == 256 || bytes == 512) && a.heads % tpw == 0;
+  chooseChunk(&a, hiw ? a.heads / tpw : a.heads, batch, maxInputLen);
+  a.nsplit = (int)std::max<int64_t>(1, ceilDiv(maxInputLen, a.chunk));
+  AMD_CHECK(batch <= 65535 && a.nsplit <= 65535, "token attention: batch %ld / splits %d exceed the grid limits", (long)batch,
+            a.nsplit);
+  float* partial = nullptr;
+  if (MODE != kTaLogitsOut && a.nsplit > 1) {
+    const int64_t need = (int64_t)batch * a.heads * a.nsplit * (2 + a.d) * (int64_t)sizeof(float);
+    if (staticScratch) {
+      AMD_CHECK(need <= kDecodeScratchBytes,
+                "token attention: batch %ld x %d heads x %d splits of %d tokens needs %ld bytes of partial results, the "
+                "entry point that allocates nothing holds %ld; use diopiTokenDecodeAttentionInference",
+                (long)batch, a.heads, a.nsplit, a.chunk, (long)need, (long)kDecodeScratchBytes);
+      // Nothing has to start at zero: the split kernel writes every (max, sum, acc) row the merge kernel uses, and
+      // rows of splits that hold no tokens are read but discarded by a select.
+      partial = ownScratch;
+    } else {
+      void* ws = nullptr;
+      AMD_TRY(requireWorkspace(ctx, need, &ws));
+      partial = static_cast<float*>(ws);
+    }
+  }
+  dim3 grid(hiw ? a.heads / tpw : a.heads, a.nsplit, (unsigned)batch), block(kTaWaves * 64);
+#define STREAM_CALL_AS(T, LPT, LT)                                                                                                   \
+  if (hiw) hipLaunchKernelGGL((decodeSplitKernel<T, LPT, true, MODE, LT>), grid, block, 0, stream, a, static_cast<T*>(outPtr), partial); \
+  else hipLaunchKernelGGL((decodeSplitKernel<T, LPT, false, MODE, LT>), grid, block, 0, stream, a, static_cast<T*>(outPtr), partial)
+#define STREAM_CALL(T, LPT)                                \
+  if (MODE == kTaFused || scoresF32) {                     \
+    STREAM_CALL_AS(T, LPT, float);                         \
+  } else {                                                 \
+    STREAM_CALL_AS(T, LPT, T);                             \
+  }
+  TA_DISPATCH(dtype, bytes, STREAM_CALL);
+#undef STREAM_CALL
+#undef STREAM_CALL_AS
+  AMD_LAUNCH_CHECK();
+  if (MODE == kTaLogitsOut) return diopiSuccess;
+  if (a.nsplit > 64) {
+    const int64_t pairs = batch * a.heads;
+    AMD_CHECK(a.nsplit <= kTaMaxSplit && a.d <= 256, "token attention: %d splits of head size %d cannot be merged", a.nsplit, a.d);
+#define MERGE_WIDE_CALL(T, LPT)                                                                                                      \
+  hipLaunchKernelGGL((decodeMergeWideKernel<T>), dim3((unsigned)pairs), dim3(256), 0, stream, static_cast<T*>(outPtr), partial, a.bLen, \
+                     a.len64, a.heads, a.d, a.nsplit, a.chunk)
+    TA_DISPATCH(dtype, bytes, MERGE_WIDE_CALL);
+#undef MERGE_WIDE_CALL
+    AMD_LAUNCH_CHECK();
+  } else if (a.nsplit > 1) {
+    int64_t pairs = batch * a.heads;
+    dim3 mgrid((unsigned)ceilDiv(pairs, 4)), mblock(256);
+#define MERGE_CALL(T, LPT)                                                                                                     \
+  hipLaunchKernelGGL((decodeMergeKernel<T>), mgrid, mblock, 0, stream, static_cast<T*>(outPtr), partial, a.bLen, a.len64, pairs, \
+                     a.heads, a.d, a.nsplit, a.chunk)
+    TA_DISPATCH(dtype, bytes, MERGE_CALL);
+#undef MERGE_CALL
+    AMD_LAUNCH_CHECK();
+  }
+  return diopiSuccess;
+}
+
 static diopiError_t decodeAttention(diopiContextHandle_t ctx, diopiTensorHandle_t outH, diopiConstTensorHandle_t qH,
                                     diopiConstTensorHandle_t kH, diopiConstTensorHandle_t vH, diopiConstTensorHandle_t locH,
                                     diopiConstTensorHandle_t startH, diopiConstTensorHandle_t lenH, int maxInputLen,
@@ -794,72 +787,8 @@ static diopiError_t decodeAttention(diopiContextHandle_t ctx, diopiTensorHandle_
     AMD_LAUNCH_CHECK();
     return diopiSuccess;
   }
-  const int64_t bytes = t.q.shape[2] * t.q.itemsize;
-  // The lane groups of a wave take consecutive heads of one token when the head count allows it: a wave load is then
-  // one contiguous piece of a slot (1 KiB) instead of head rows of four different slots (431 -> 421 us at batch 64,
-  // 32 heads x 128, 156 043 cached tokens).
-  const int tpw = (int)(64 / std::max<int64_t>(1, bytes / 16));
-  const bool hiw = (bytes == 128 || bytes == 256 || bytes == 512) && a.heads % tpw == 0;
-  // A workgroup walks its chunk with two loads per wave in flight, so the rate comes from the number of workgroups a
-  // CU holds at once. Few sequences or short ones are cut into smaller chunks until there are about kTaWgsPerCu
-  // workgroups per CU; large batches keep the 512-token chunks, whose partial results are fewer. Measured (us, 32 heads
-  // x 128, bf16, with 512-token chunks -> with these): 1 x 2048 tokens 72 -> 20, 1 x 32768 130 -> 96, 8 x 4096 130 -> 91,
-  // 4 x (100 .. 16384) 123 -> 86, 64 x (256 .. 512) 101 -> 80; 64 x (512 .. 4096) and 256 x (1024 .. 2048) keep their chunks.
-  {
-    const int64_t groups = (hiw ? a.heads / tpw : a.heads) * batch, cus = computeUnits(), len = std::max(maxInputLen, 1);
-    const int64_t wantSplits = std::max<int64_t>(1, ceilDiv(kTaWgsPerCu * cus, groups));
-    const int64_t fine = ceilDiv(ceilDiv(len, wantSplits), 64) * 64;
-    const int64_t capped = ceilDiv(ceilDiv(len, (int64_t)kTaMaxSplit), 64) * 64;  // at most kTaMaxSplit chunks
-    const int64_t shortest = groups * ceilDiv(len, (int64_t)kTaMinChunk) < cus ? kTaTinyChunk : kTaMinChunk;
-    a.chunk = (int)std::max(std::max(capped, shortest), std::min<int64_t>(a.chunk, fine));
-  }
-  a.nsplit = (int)std::max<int64_t>(1, ceilDiv(maxInputLen, a.chunk));
-  AMD_CHECK(batch <= 65535 && a.nsplit <= 65535, "token attention: batch %ld / splits %d exceed the grid limits", (long)batch,
-            a.nsplit);
-  float* partial = nullptr;
-  if (a.nsplit > 1) {
-    const int64_t need = (int64_t)batch * a.heads * a.nsplit * (2 + a.d) * (int64_t)sizeof(float);
-    if (staticScratch) {
-      AMD_CHECK(need <= kDecodeScratchBytes,
-                "token attention: batch %ld x %d heads x %d splits of %d tokens needs %ld bytes of partial results, the "
-                "entry point that allocates nothing holds %ld; use diopiTokenDecodeAttentionInference",
-                (long)batch, a.heads, a.nsplit, a.chunk, (long)need, (long)kDecodeScratchBytes);
-      // Nothing has to start at zero: the split kernel writes every (max, sum, acc) row the merge kernel uses, and
-      // rows of splits that hold no tokens are read but discarded by a select.
-      partial = ownScratch;
-    } else {
-      void* ws = nullptr;
-      AMD_TRY(requireWorkspace(ctx, need, &ws));
-      partial = static_cast<float*>(ws);
-    }
-  }
-  dim3 grid(hiw ? a.heads / tpw : a.heads, a.nsplit, (unsigned)batch), block(kTaWaves * 64);
-#define DECODE_CALL(T, LPT)                                                                                               \
-  if (hiw) hipLaunchKernelGGL((decodeSplitKernel<T, LPT, true>), grid, block, 0, stream, a, out.ptr<T>(), partial);       \
-  else hipLaunchKernelGGL((decodeSplitKernel<T, LPT, false>), grid, block, 0, stream, a, out.ptr<T>(), partial)
-  TA_DISPATCH(t.q.dtype, bytes, DECODE_CALL);
-#undef DECODE_CALL
-  AMD_LAUNCH_CHECK();
-  if (a.nsplit > 64) {
-    const int64_t pairs = batch * a.heads;
-    AMD_CHECK(a.nsplit <= kTaMaxSplit && a.d <= 256, "token attention: %d splits of head size %d cannot be merged", a.nsplit, a.d);
-#define MERGE_WIDE_CALL(T, LPT)                                                                                              \
-  hipLaunchKernelGGL((decodeMergeWideKernel<T>), dim3((unsigned)pairs), dim3(256), 0, stream, out.ptr<T>(), partial, a.bLen, \
-                     a.len64, a.heads, a.d, a.nsplit, a.chunk)
-    TA_DISPATCH(t.q.dtype, bytes, MERGE_WIDE_CALL);
-#undef MERGE_WIDE_CALL
-    AMD_LAUNCH_CHECK();
-  } else if (a.nsplit > 1) {
-    int64_t pairs = batch * a.heads;
-    dim3 mgrid((unsigned)ceilDiv(pairs, 4)), mblock(256);
-#define MERGE_CALL(T, LPT)                                                                                       \
-  hipLaunchKernelGGL((decodeMergeKernel<T>), mgrid, mblock, 0, stream, out.ptr<T>(), partial, a.bLen, a.len64, pairs, \
-                     a.heads, a.d, a.nsplit, a.chunk)
-    TA_DISPATCH(t.q.dtype, bytes, MERGE_CALL);
-#undef MERGE_CALL
-    AMD_LAUNCH_CHECK();
-  }
-  return diopiSuccess;
+  return streamChunks<kTaFused>(ctx, stream, a, t.q.dtype, t.q.shape[2] * t.q.itemsize, batch, maxInputLen, out.data, true,
+                                staticScratch, ownScratch);
 }
 
 extern "C" __attribute__((visibility("default"))) diopiError_t diopiTokenDecodeAttentionInference(
@@ -917,19 +846,9 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiTokenAttenti
     AMD_LAUNCH_CHECK();
     return diopiSuccess;
   }
-  if (att.dtype == diopi_dtype_float32) {
-#define LOGIT_CALL(T, LPT) \
-  hipLaunchKernelGGL((tokenLogitsKernel<T, LPT, float>), grid, block, 0, stream, a, att.ptr<float>(), att.stride[0])
-    TA_DISPATCH(t.q.dtype, bytes, LOGIT_CALL);
-#undef LOGIT_CALL
-  } else {
-#define LOGIT_CALL(T, LPT) \
-  hipLaunchKernelGGL((tokenLogitsKernel<T, LPT, T>), grid, block, 0, stream, a, att.ptr<T>(), att.stride[0])
-    TA_DISPATCH(t.q.dtype, bytes, LOGIT_CALL);
-#undef LOGIT_CALL
-  }
-  AMD_LAUNCH_CHECK();
-  return diopiSuccess;
+  a.logits = att.data, a.logitsHeadStride = att.stride[0];
+  return streamChunks<kTaLogitsOut>(ctx, stream, a, t.q.dtype, bytes, batch, maxInputLen, nullptr,
+                                    att.dtype == diopi_dtype_float32, false, nullptr);
 }
 
 extern "C" __attribute__((visibility("default"))) diopiError_t diopiTokenSoftmaxReduceVInference(
@@ -974,17 +893,7 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiTokenSoftmax
     AMD_LAUNCH_CHECK();
     return diopiSuccess;
   }
-  if (lg.dtype == diopi_dtype_float32) {
-#define RV_CALL(T, LPT) \
-  hipLaunchKernelGGL((softmaxReduceVKernel<T, LPT, float>), grid, block, 0, stream, a, out.ptr<T>(), lg.ptr<float>(), lg.stride[0])
-    TA_DISPATCH(out.dtype, bytes, RV_CALL);
-#undef RV_CALL
-  } else {
-#define RV_CALL(T, LPT) \
-  hipLaunchKernelGGL((softmaxReduceVKernel<T, LPT, T>), grid, block, 0, stream, a, out.ptr<T>(), lg.ptr<T>(), lg.stride[0])
-    TA_DISPATCH(out.dtype, bytes, RV_CALL);
-#undef RV_CALL
-  }
-  AMD_LAUNCH_CHECK();
-  return diopiSuccess;
+  a.logits = lg.data, a.logitsHeadStride = lg.stride[0];
+  return streamChunks<kTaReduceV>(ctx, stream, a, out.dtype, bytes, batch, maxInputLen, out.data,
+                                  lg.dtype == diopi_dtype_float32, false, nullptr);
 }
