@@ -380,16 +380,26 @@ template <typename T, int D>
 __global__ __launch_bounds__(256, 2) void contextAttnMfmaKernel(CaArgs a, int numQBlocks, int numSeq) {
   const int pairs = (numQBlocks + 1) / 2, hb = a.heads * numSeq;
   const int flat = (int)blockIdx.x;
-  int headSeq, pair;
-  if ((hb & 7) == 0) {
+  int h, b, pair;
+  if ((a.heads & 7) == 0) {
+    // every sequence's heads are dealt over the 8 XCDs, a contiguous eighth of them each, so that a batch of unequal
+    // sequences loads the XCDs alike (with whole sequences per XCD, one long sequence among short ones kept a single
+    // XCD busy: 4096 + 12 x 340 tokens 843 us against 146 for 4 x 2048, which is the same work)
+    const int xcd = flat & 7, idx = flat >> 3, perXcd = a.heads >> 3;
+    const int hs = idx / pairs;
+    pair = idx - hs * pairs;
+    b = hs / perXcd;
+    h = xcd * perXcd + (hs - b * perXcd);
+  } else if ((hb & 7) == 0) {
     const int xcd = flat & 7, idx = flat >> 3;
-    headSeq = xcd * (hb >> 3) + idx / pairs;
+    const int headSeq = xcd * (hb >> 3) + idx / pairs;
     pair = idx % pairs;
+    h = headSeq % a.heads, b = headSeq / a.heads;
   } else {
-    headSeq = flat / pairs;
+    const int headSeq = flat / pairs;
     pair = flat % pairs;
+    h = headSeq % a.heads, b = headSeq / a.heads;
   }
-  const int h = headSeq % a.heads, b = headSeq / a.heads;
   const int heavy = numQBlocks - 1 - pair, light = pair;
   for (int pass = 0; pass < 2; ++pass) {
     if (pass == 1) {
