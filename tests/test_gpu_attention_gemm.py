@@ -433,13 +433,14 @@ def test_context_attention_uniform_keys_give_running_mean_at_length_2048(ops, de
     run_mean = torch.cumsum(v.float(), 0) / torch.arange(1, n + 1).view(-1, 1, 1)
     assert_half(got, run_mean)
 
-def test_context_attention_long_ragged_batch_paired_blocks(ops, dev):
-    """Ragged sequences up to 2048 tokens with grouped-query heads: exercises the heavy + light query-block pairing
-    (odd and even block counts, sequences shorter than the longest one) and the workgroup decoding used when
-    heads x sequences is a multiple of 8."""
-    lens = [1000, 2048, 517]
-    heads, kvh, d = 8, 2, 128
-    starts = [0, 1000, 3048]
+@pytest.mark.parametrize("heads,kvh,lens", [(8, 2, [1000, 2048, 517]), (16, 16, [1300, 90, 700]), (4, 4, [900, 1100]),
+                                            (4, 2, [600, 1025, 130])])
+def test_context_attention_long_ragged_batch_paired_blocks(ops, dev, heads, kvh, lens):
+    """Ragged sequences up to 2048 tokens: exercises the heavy + light query-block pairing (odd and even block counts,
+    sequences shorter than the longest one) and the three ways a workgroup finds its (sequence, head): a head count
+    that is a multiple of 8 (one or two heads of every sequence per XCD), heads x sequences a multiple of 8, neither."""
+    d = 128
+    starts = [sum(lens[:i]) for i in range(len(lens))]
     total = sum(lens)
     q = torch.randn(total, heads, d, generator=g(27)).bfloat16()
     k = torch.randn(total, kvh, d, generator=g(28)).bfloat16()
