@@ -538,6 +538,189 @@ __global__ __launch_bounds__(256) void rowMeanKernel(T* out, const T* in, int64_
   if (lane == 0) out[row] = static_cast<T>(s / (float)cols);
 }
 
+// Sums over the middle dim of a dense [outer, R, inner] tensor, inner > 1 (a mean over leading dims: the kept elements
+// lie next to each other). A workgroup owns lpr VEC adjacent columns of one `outer` (lpr lanes per row, a power of two
+// up to 64, so a wave load covers 64 / lpr rows of a narrow tensor) and one share of the R rows; its four waves take
+// turns at the rows of the share with one VEC-wide load per lane (whole 1 KiB pieces of a row when VEC fills 16 bytes
+// and lpr is 64), two loads ahead, and meet in LDS. With one share per column (partial == nullptr) the mean goes
+// straight to `out`; otherwise the fp32 sums of share s go to partial[(o * shares + s) * inner + c] and
+// finishMeanKernel adds them up. [8192, 4096] bf16 over dim 0: 13 + 4 us, against 50 us as a transposing copy followed
+// by row means; all of it (one row of 33 M elements, rowShareSumKernel): 12 + 4 us.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void columnSumKernel(T* __restrict__ out, float* __restrict__ partial,
+                                                       const T* __restrict__ in, int64_t R, int64_t inner,
+                                                       int64_t rowsPerShare, int shares, int colTiles, int lpr, float scale) {
+  __shared__ float red[4][64 * VEC];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int rpw = 64 / lpr, sub = lane / lpr, cl = lane & (lpr - 1);  // rows per wave load, this lane's row and column piece
+  const int64_t flat = blockIdx.x;
+  const int tile = (int)(flat % colTiles);
+  const int share = (int)((flat / colTiles) % shares);
+  const int64_t o = flat / ((int64_t)colTiles * shares);
+  const int64_t c0 = ((int64_t)tile * lpr + cl) * VEC;
+  const int64_t r0 = (int64_t)share * rowsPerShare, r1 = min(R, r0 + rowsPerShare);
+  float s[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) s[j] = 0.f;
+  if (c0 < inner) {  // inner is a multiple of VEC: a lane's columns are all live or all past the end
+    const T* src = in + (o * R) * inner + c0;
+    struct alignas(sizeof(T) * VEC) Piece { T v[VEC]; };
+    const int step = 4 * rpw;
+    int64_t r = r0 + wave * rpw + sub;
+    for (; r + step < r1; r += 2 * step) {
+      const Piece a = *reinterpret_cast<const Piece*>(src + r * inner);
+      const Piece b = *reinterpret_cast<const Piece*>(src + (r + step) * inner);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) s[j] += static_cast<float>(a.v[j]) + static_cast<float>(b.v[j]);
+    }
+    if (r < r1) {
+      const Piece a = *reinterpret_cast<const Piece*>(src + r * inner);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) s[j] += static_cast<float>(a.v[j]);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) red[wave][lane * VEC + j] = s[j];
+  __syncthreads();
+  // thread t finishes columns t, t + 256, ... of the tile: four waves times rpw rows of lanes each
+  for (int c = threadIdx.x; c < lpr * VEC; c += 256) {
+    const int64_t col = (int64_t)tile * lpr * VEC + c;
+    if (col >= inner) break;
+    float v = 0.f;
+    for (int q = 0; q < rpw; ++q) {
+      const int at = q * lpr * VEC + c;
+      v += red[0][at] + red[1][at] + red[2][at] + red[3][at];
+    }
+    if (partial) partial[(o * shares + share) * inner + col] = v;
+    else out[o * inner + col] = static_cast<T>(v * scale);
+  }
+}
+
+// Sums of one share of each dense row, for a few very long rows (a mean over everything is one row): workgroup
+// (row, share) adds its piece of the row with 16-byte loads where the piece allows and writes one fp32 sum.
+template <typename T>
+__global__ __launch_bounds__(256) void rowShareSumKernel(float* __restrict__ partial, const T* __restrict__ in,
+                                                         int64_t cols, int64_t colsPerShare, int shares) {
+  __shared__ float red[4];
+  using V = typename Vec16<T>::type;
+  constexpr int N = Vec16<T>::N;
+  const int64_t row = blockIdx.x / shares;
+  const int share = (int)(blockIdx.x % shares);
+  const int64_t c0 = min(cols, (int64_t)share * colsPerShare), c1 = min(cols, c0 + colsPerShare);
+  const T* src = in + row * cols;
+  float s = 0.f;
+  int64_t c = c0;
+  if ((reinterpret_cast<uintptr_t>(src + c0) & 15) == 0) {
+    const int64_t nvec = (c1 - c0) / N;
+    const V* vs = reinterpret_cast<const V*>(src + c0);
+    for (int64_t v = threadIdx.x; v < nvec; v += 256) {
+      const V x = vs[v];
+#pragma unroll
+      for (int j = 0; j < N; ++j) s += static_cast<float>(x[j]);
+    }
+    c = c0 + nvec * N;
+  }
+  for (c += threadIdx.x; c < c1; c += 256) s += static_cast<float>(src[c]);
+  s = waveSum(s);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) partial[blockIdx.x] = red[0] + red[1] + red[2] + red[3];
+}
+
+// out[o, c] = scale * sum over s of partial[(o * shares + s) * inner + c]. A workgroup takes cpb adjacent columns (a
+// power of two, at most 64) of one o; its 256 threads split the shares 256 / cpb ways and meet in LDS. (One thread
+// per output walking the shares one after the other took 60 us for 256 shares of 4096 columns, 64 columns per
+// workgroup with 64 shares per thread 12 us.)
+template <typename T>
+__global__ __launch_bounds__(256) void finishMeanKernel(T* __restrict__ out, const float* __restrict__ partial,
+                                                        int64_t inner, int shares, int cpb, int colBlocks, float scale) {
+  __shared__ float red[256];
+  const int c = threadIdx.x & (cpb - 1), kg = threadIdx.x / cpb, kgs = 256 / cpb;
+  const int64_t o = blockIdx.x / colBlocks;
+  const int64_t col = (int64_t)(blockIdx.x % colBlocks) * cpb + c;
+  float s = 0.f;
+  if (col < inner) {
+    const float* p = partial + (o * shares) * inner + col;
+    for (int k = kg; k < shares; k += kgs) s += p[(int64_t)k * inner];
+  }
+  red[threadIdx.x] = s;
+  __syncthreads();
+  for (int stride = 128; stride >= cpb; stride >>= 1) {
+    if ((int)threadIdx.x < stride) red[threadIdx.x] += red[threadIdx.x + stride];
+    __syncthreads();
+  }
+  if ((int)threadIdx.x < cpb && col < inner) out[o * inner + col] = static_cast<T>(red[threadIdx.x] * scale);
+}
+
+template <typename T>
+static void launchFinishMean(hipStream_t stream, T* out, const float* partial, int64_t outer, int64_t inner, int shares,
+                             float scale) {
+  // about eight shares per thread: many shares want few columns per workgroup (and so more workgroups)
+  int cpb = 1;
+  while (cpb < 64 && cpb * 2 <= inner && cpb * 2 * shares <= 2048) cpb *= 2;
+  const int64_t colBlocks = ceilDiv(inner, (int64_t)cpb);
+  hipLaunchKernelGGL(finishMeanKernel<T>, dim3((unsigned)(outer * colBlocks)), dim3(256), 0, stream, out, partial, inner,
+                     shares, cpb, (int)colBlocks, scale);
+}
+
+template <typename T>
+static diopiError_t launchColumnMean(diopiContextHandle_t ctx, hipStream_t stream, T* out, const T* in, int64_t outer,
+                                     int64_t R, int64_t inner) {
+  constexpr int N = Vec16<T>::N;
+  const bool vec = inner % N == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0;
+  const int64_t pieces = vec ? inner / N : inner;  // per row
+  int lpr = 1;
+  while (lpr < 64 && lpr < pieces) lpr *= 2;
+  const int64_t colTiles = ceilDiv(pieces, (int64_t)lpr);
+  const int rowsPerPass = 4 * (64 / lpr);  // of the four waves together
+  // two workgroups per CU where the rows allow, no share under sixteen passes (two to sixteen per CU and four to
+  // sixteen passes all read 12.9 - 14.5 us on [8192, 4096] bf16; fewer shares leave less for the second kernel)
+  const int64_t want = ceilDiv((int64_t)computeUnits() * 2, outer * colTiles);
+  const int shares = (int)std::max<int64_t>(1, std::min<int64_t>(want, R / (16 * rowsPerPass)));
+  const int64_t rowsPerShare = ceilDiv(R, (int64_t)shares);
+  const int64_t wgs = outer * colTiles * shares;
+  AMD_CHECK(wgs <= INT32_MAX && colTiles <= INT32_MAX, "diopiMean: %ld workgroups", (long)wgs);
+  float* partial = nullptr;
+  if (shares > 1) {
+    void* ws = nullptr;
+    AMD_TRY(requireWorkspace(ctx, outer * shares * inner * 4, &ws));
+    partial = static_cast<float*>(ws);
+  }
+  const float scale = 1.f / (float)R;
+  if (vec)
+    hipLaunchKernelGGL((columnSumKernel<T, N>), dim3((unsigned)wgs), dim3(256), 0, stream, out, partial, in, R, inner,
+                       rowsPerShare, shares, (int)colTiles, lpr, scale);
+  else
+    hipLaunchKernelGGL((columnSumKernel<T, 1>), dim3((unsigned)wgs), dim3(256), 0, stream, out, partial, in, R, inner,
+                       rowsPerShare, shares, (int)colTiles, lpr, scale);
+  AMD_LAUNCH_CHECK();
+  if (partial) {
+    launchFinishMean<T>(stream, out, partial, outer, inner, shares, scale);
+    AMD_LAUNCH_CHECK();
+  }
+  return diopiSuccess;
+}
+
+// A few rows far longer than a wave's worth: shares of each row summed by separate workgroups, then added up.
+template <typename T>
+static diopiError_t launchLongRowMean(diopiContextHandle_t ctx, hipStream_t stream, T* out, const T* in, int64_t rows,
+                                      int64_t cols) {
+  constexpr int N = Vec16<T>::N;
+  const int64_t want = ceilDiv((int64_t)computeUnits() * 8, rows);
+  const int shares = (int)std::max<int64_t>(1, std::min<int64_t>(want, cols / 4096));
+  // whole vectors per share, so every share of an aligned row starts aligned
+  const int64_t colsPerShare = ceilDiv(ceilDiv(cols, (int64_t)shares), (int64_t)N) * N;
+  void* ws = nullptr;
+  AMD_TRY(requireWorkspace(ctx, rows * shares * 4, &ws));
+  float* partial = static_cast<float*>(ws);
+  hipLaunchKernelGGL(rowShareSumKernel<T>, dim3((unsigned)(rows * shares)), dim3(256), 0, stream, partial, in, cols,
+                     colsPerShare, shares);
+  AMD_LAUNCH_CHECK();
+  launchFinishMean<T>(stream, out, partial, rows, 1, shares, 1.f / (float)cols);
+  AMD_LAUNCH_CHECK();
+  return diopiSuccess;
+}
+
 // ------------------------------------------------------------- dispatch ------
 template <typename T, int OP, typename WT>
 static diopiError_t launchRows(hipStream_t stream, T* out, const T* in, const WT* weight, const WT* bias,
@@ -791,8 +974,10 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiRMSNorm(
   return diopiSuccess;
 }
 
-// mean over `dims`: the kept dims are moved to the front (a strided view), made dense,
-// and each row of prod(reduced) elements is averaged by one wave.
+// mean over `dims`. Reduced dims that lie next to each other in a dense input with kept dims after them are summed
+// down the columns where they lie; otherwise the kept dims are moved to the front (a strided view, made dense if it
+// is not) and each row of prod(reduced) elements is averaged by one wave, or by many workgroups when the rows are few
+// and long.
 extern "C" __attribute__((visibility("default"))) diopiError_t diopiMean(diopiContextHandle_t ctx,
                                                                          diopiTensorHandle_t outH,
                                                                          diopiConstTensorHandle_t inH,
@@ -824,14 +1009,39 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiMean(diopiCo
     if (reduced[d]) perm.shape[w] = in.shape[d], perm.stride[w] = in.stride[d], cols *= in.shape[d], ++w;
   AMD_CHECK(out.numel == rows, "diopiMean: output has %ld elements, expected %ld", (long)out.numel, (long)rows);
   if (rows == 0) return diopiSuccess;
-  TensorView cin;
-  AMD_TRY(makeContiguous(ctx, stream, perm, &cin));
   TensorView cout = out;
   bool outTemp = !out.isContiguous();
   if (outTemp) {
     diopiTensorHandle_t th;
     AMD_TRY(requireTensor(ctx, out.shape, out.ndim, out.dtype, &th, &cout));
   }
+  // The reduced dims of a dense input next to each other, kept dims after them: [outer, R, inner] summed over R where
+  // it lies (no transposing copy).
+  int firstRed = -1, lastRed = -1, nRed = 0;
+  for (int d = 0; d < in.ndim; ++d)
+    if (reduced[d]) firstRed = firstRed < 0 ? d : firstRed, lastRed = d, ++nRed;
+  const bool oneRun = nRed > 0 && lastRed - firstRed + 1 == nRed && in.isContiguous() && cols > 0;
+  int64_t inner = 1;
+  for (int d = lastRed + 1; oneRun && d < in.ndim; ++d) inner *= in.shape[d];
+#define MEAN_BY_DTYPE(CALL)                                                           \
+  switch (in.dtype) {                                                                 \
+    case diopi_dtype_bfloat16: { using T = bf16_t; AMD_TRY(CALL); break; }            \
+    case diopi_dtype_float16: { using T = half_t; AMD_TRY(CALL); break; }             \
+    default: { using T = float; AMD_TRY(CALL); break; }                               \
+  }
+  if (oneRun && inner > 1) {
+    MEAN_BY_DTYPE((launchColumnMean<T>(ctx, stream, cout.ptr<T>(), in.ptr<T>(), rows / inner, cols, inner)));
+    if (outTemp) AMD_TRY(stridedCopy(stream, cout, out));
+    return diopiSuccess;
+  }
+  TensorView cin;
+  AMD_TRY(makeContiguous(ctx, stream, perm, &cin));
+  if (rows * 4 <= computeUnits() && cols >= 65536) {
+    MEAN_BY_DTYPE((launchLongRowMean<T>(ctx, stream, cout.ptr<T>(), cin.ptr<T>(), rows, cols)));
+    if (outTemp) AMD_TRY(stridedCopy(stream, cout, out));
+    return diopiSuccess;
+  }
+#undef MEAN_BY_DTYPE
   dim3 grid((unsigned)ceilDiv(rows, 4)), block(256);
   switch (in.dtype) {
     case diopi_dtype_bfloat16:

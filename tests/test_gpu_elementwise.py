@@ -171,6 +171,25 @@ def test_copy_cast_cat_mean(ops, dev):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_mean_over_leading_dims_and_of_long_rows(ops, dev, dtype):
+    # kept dims after the reduced ones (sums down the columns, rows shared out over workgroups or not), ragged and
+    # unaligned widths, and a few rows far longer than a wave's worth (a mean over everything is one such row)
+    cases = [((6, 7, 64), [0]), ((6, 7, 64), [1]), ((5, 300, 24), [0, 1]), ((1000, 520), [0]), ((700, 3, 1031), [0]),
+             ((4, 513, 8), [1]), ((2, 4100, 1536), [1]), ((3, 70001), [-1]), ((300, 1000), [0, 1]), ((2, 131072), [1])]
+    for i, (shape, dims) in enumerate(cases):
+        x = torch.randn(shape, generator=g(170 + i)).to(dtype)
+        want = x.float().mean(dims)
+        for keep in (False, True):
+            got = ops.mean(x.to(dev), dims, keepdim=keep)
+            assert got.dtype == dtype and tuple(got.shape) == tuple(x.mean(dims, keepdim=keep).shape)
+            tol = 1e-5 if dtype == torch.float32 else 4e-3   # the result rounded to 16 bits
+            err = (got.cpu().float().reshape(want.shape) - want).abs()
+            assert bool((err <= tol * (1 + want.abs())).all()), (shape, dims, float(err.max()))
+    base = torch.randn(64, 48, generator=g(190)).to(dtype)   # a strided view still goes through the dense copy
+    assert (ops.mean(base.to(dev)[::2, 1:33], [0]).cpu().float() - base[::2, 1:33].float().mean(0)).abs().max() < 4e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_softmax(ops, dev, dtype):
     # shapes of dipu/tests/python/unittests/test_softmax.py:41-70 (dim 0 there), plus row softmax
     for shape, dim in [((256, 1000), 0), ((32, 48, 1024), 0), ((64, 4096), -1), ((2, 8, 128, 128), -1),
