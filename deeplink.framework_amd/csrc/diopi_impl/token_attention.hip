@@ -85,6 +85,26 @@ __device__ __forceinline__ void mergeState(float& m, float& l, float (&acc)[E], 
   m = mn;
 }
 
+// Sum over the LPT (8, 16 or 32) adjacent lanes that share a head row, left in all of them. The steps within a row of 16
+// lanes are lane permutations folded into the additions (quad swaps, then the mirror images within 8 and within 16,
+// which pair every lane with one that holds the other half of the sum): no trips through the LDS crossbar. Decode
+// attention at batch 64 (156 000 cached tokens): 373.7 -> 371.6 us; at batch 256: 1054 -> 1046 us.
+template <int CTRL>
+__device__ __forceinline__ float addPermuted(float v) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false);
+  return v + __builtin_bit_cast(float, moved);
+}
+template <int LPT>
+__device__ __forceinline__ float headRowSum(float v) {
+  static_assert(LPT == 8 || LPT == 16 || LPT == 32, "a head row is shared by 8, 16 or 32 lanes");
+  v = addPermuted<0xB1>(v);   // quad_perm [1, 0, 3, 2]
+  v = addPermuted<0x4E>(v);   // quad_perm [2, 3, 0, 1]
+  v = addPermuted<0x141>(v);  // row_half_mirror
+  if (LPT >= 16) v = addPermuted<0x140>(v);  // row_mirror
+  if (LPT >= 32) v += __shfl_xor(v, 16, 64);
+  return v;
+}
+
 // The three things the streaming kernel below can do with a chunk of a sequence: the whole decode attention (scores,
 // online softmax and the sum over V), only the scores (first half of the two-call form: att[h, start_b + t]), or the
 // softmax and the sum over V from scores computed earlier (second half of the two-call form).
@@ -99,9 +119,9 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   constexpr int N = Vec16<T>::N;
   constexpr int TPW = 64 / LPT;  // tokens per wave-wide load
   constexpr bool kNeedK = MODE != kTaReduceV, kNeedV = MODE != kTaLogitsOut;
-  // rows per wave in flight: 2 K + 2 V in the fused mode; 4 K when only scores are produced; 2 V (and their stored scores)
-  // in the second half of the two-call form, where 4 measured slower (306 against 234 us at batch 64, 156 000 tokens)
-  constexpr int UNR = MODE == kTaLogitsOut ? 2 * kTaUnroll : kTaUnroll;
+  // rows per wave in flight: 2 K + 2 V in the fused mode, 2 K or 2 V in the halves of the two-call form (at batch 64,
+  // 156 000 tokens: scores 215 us with 2, 219 with 4, 229 with 6; second half 204 with 2, 212 with 3, 221 with 4)
+  constexpr int UNR = kTaUnroll;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int sub = lane % LPT, grp = lane / LPT;
   // HIW: the lane groups of a wave take TPW consecutive heads of the same token (a wave load is TPW head rows, contiguous
@@ -118,6 +138,19 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   if constexpr (MODE != kTaFused)
     scores = static_cast<LT*>(const_cast<void*>(a.logits)) + h * a.logitsHeadStride + ldIndex(a.bStart, b, a.start64);
 
+  // Two-call modes: the scores of the chunk pass through LDS, so memory sees them as whole rows of the chunk (one
+  // coalesced read before the walk, one coalesced write after it) instead of four floats per wave and row on the way
+  // (at batch 64, 156 000 tokens: scores 225 -> 219 us, second half 234 -> 205 us). Chunks longer than the buffer
+  // (sequences past 131 072 tokens) keep the direct accesses.
+  constexpr int kLdsScores = 1024;
+  __shared__ float sbuf[MODE != kTaFused ? kLdsScores : 1];
+  const bool useLds = MODE != kTaFused && a.chunk <= kLdsScores;
+  if constexpr (MODE == kTaReduceV) {
+    if (useLds) {
+      for (int i = threadIdx.x; i < end - begin; i += kTaWaves * 64) sbuf[i] = static_cast<float>(scores[begin + i]) * kLog2eTA;
+      __syncthreads();
+    }
+  }
   float qf[N];
   if constexpr (kNeedK) {
     // scores leave the kernel in natural units, inside it they are in units of log2
@@ -158,7 +191,8 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
       int64_t s = okk[u] ? slot[u] : 0;
       if constexpr (kNeedK) kk[u] = __builtin_nontemporal_load(reinterpret_cast<const V*>(kBase + s * a.kSlotStride));
       if constexpr (kNeedV) vv[u] = __builtin_nontemporal_load(reinterpret_cast<const V*>(vBase + s * a.vSlotStride));
-      if constexpr (MODE == kTaReduceV) lg[u] = okk[u] ? static_cast<float>(scores[slotTok[u]]) * kLog2eTA : -INFINITY;
+      if constexpr (MODE == kTaReduceV)
+        lg[u] = !okk[u] ? -INFINITY : (useLds ? sbuf[slotTok[u] - begin] : static_cast<float>(scores[slotTok[u]]) * kLog2eTA);
     }
   };
   loadSlots(begin);
@@ -175,8 +209,7 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
         float d = 0.f;
 #pragma unroll
         for (int e = 0; e < N; ++e) d += qf[e] * static_cast<float>(kr[u][e]);
-#pragma unroll
-        for (int off = LPT / 2; off > 0; off >>= 1) d += __shfl_xor(d, off, 64);
+        d = headRowSum<LPT>(d);
         sc[u] = ok[u] ? d : -INFINITY;
       } else {
         sc[u] = lr[u];
@@ -187,7 +220,10 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
 #pragma unroll
       for (int u = 0; u < UNR; ++u) {
         const int t = it + wave * UNR * TPI + (HIW ? 0 : grp) + u * TPI;
-        if (sub == 0 && t < end) scores[t] = static_cast<LT>(sc[u]);
+        if (sub == 0 && t < end) {
+          if (useLds) sbuf[t - begin] = sc[u];
+          else scores[t] = static_cast<LT>(sc[u]);
+        }
       }
     } else if (mn != -INFINITY) {
       float corr = __builtin_amdgcn_exp2f(m - mn);  // m == -inf gives 0, acc and l are 0 then anyway
@@ -210,7 +246,13 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
 #pragma unroll
     for (int u = 0; u < UNR; ++u) kr[u] = kn[u], vr[u] = vn[u], lr[u] = ln[u], ok[u] = okn[u];
   }
-  if constexpr (MODE == kTaLogitsOut) return;
+  if constexpr (MODE == kTaLogitsOut) {
+    if (useLds) {
+      __syncthreads();
+      for (int i = threadIdx.x; i < end - begin; i += kTaWaves * 64) scores[begin + i] = static_cast<LT>(sbuf[i]);
+    }
+    return;
+  }
 
   // merge the TPW lane groups of the wave (each holds other tokens of the same head)
   if (!HIW)
@@ -691,8 +733,9 @@ static diopiError_t streamChunks(diopiContextHandle_t ctx, hipStream_t stream, T
   // one contiguous piece of a slot (1 KiB) instead of head rows of four different slots (431 -> 421 us at batch 64,
   // 32 heads x 128, 156 043 cached tokens).
   const int tpw = (int)(64 / std::max<int64_t>(1, bytes / 16));
-  // (the two-call modes keep four tokens of one head per wave load: their stored scores are then four consecutive
-  // floats of a row instead of one float in each of four rows; second half at batch 64, 156 000 tokens: 326 -> 234 us)
+  // (the two-call modes keep four tokens of one head per wave load and a workgroup per head: at batch 64, 156 000
+  // tokens, with the chunk's scores staged in LDS either way, four heads per workgroup read 244 against 219 us for the
+  // scores and 238 against 205 us for the second half)
   const bool hiw = MODE == kTaFused && (bytes == 128 || bytes == 256 || bytes == 512) && a.heads % tpw == 0;
   chooseChunk(&a, hiw ? a.heads / tpw : a.heads, batch, maxInputLen);
   a.nsplit = (int)std::max<int64_t>(1, ceilDiv(maxInputLen, a.chunk));
