@@ -203,15 +203,33 @@ struct Vec16 {  // 16 bytes of T
   typedef T type __attribute__((ext_vector_type(16 / sizeof(T))));
 };
 
+// Reductions over the 64 lanes of a wave, the result in every lane. All lanes of the wave must be active. Within a
+// row of 16 lanes the steps are lane permutations folded into the arithmetic instruction (quad swaps, then the mirror
+// images within 8 and within 16 lanes, which pair every lane with one that holds the other half of the partial
+// result); the four rows are then read out of lanes 0, 16, 32 and 48 and combined the same way by every lane. No
+// trips through the LDS crossbar, which a shuffle by lane index takes once per step.
+template <int CTRL>
+__device__ __forceinline__ float lanePermuted(float v) {  // the value of the lane CTRL pairs this one with
+  const int bits = __builtin_bit_cast(int, v);
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(bits, bits, CTRL, 0xf, 0xf, false));
+}
+constexpr int kDppQuadSwap1 = 0xB1, kDppQuadSwap2 = 0x4E, kDppHalfMirror = 0x141, kDppMirror = 0x140;
+__device__ __forceinline__ float rowOfWave(float v, int row) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16 * row));
+}
 __device__ __forceinline__ float waveSum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-  return v;
+  v += lanePermuted<kDppQuadSwap1>(v);
+  v += lanePermuted<kDppQuadSwap2>(v);
+  v += lanePermuted<kDppHalfMirror>(v);
+  v += lanePermuted<kDppMirror>(v);
+  return (rowOfWave(v, 0) + rowOfWave(v, 1)) + (rowOfWave(v, 2) + rowOfWave(v, 3));
 }
 __device__ __forceinline__ float waveMax(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-  return v;
+  v = fmaxf(v, lanePermuted<kDppQuadSwap1>(v));
+  v = fmaxf(v, lanePermuted<kDppQuadSwap2>(v));
+  v = fmaxf(v, lanePermuted<kDppHalfMirror>(v));
+  v = fmaxf(v, lanePermuted<kDppMirror>(v));
+  return fmaxf(fmaxf(rowOfWave(v, 0), rowOfWave(v, 1)), fmaxf(rowOfWave(v, 2), rowOfWave(v, 3)));
 }
 
 __device__ __forceinline__ bool isFloatDtypeDev(int dt) {

@@ -180,11 +180,13 @@ __global__ __launch_bounds__(256) void rowWaveKernel(T* __restrict__ out, const 
 // butterflies within the LPR lanes. Four such row groups per iteration keep four loads per lane in flight.
 template <int LPR>
 __device__ __forceinline__ float groupReduce(float v, bool isMax) {
-#pragma unroll
-  for (int o = LPR / 2; o >= 1; o >>= 1) {
-    const float other = __shfl_xor(v, o, 64);
-    v = isMax ? fmaxf(v, other) : v + other;
-  }
+  // within a row of 16 lanes: permutations folded into the arithmetic (see waveSum); 32 lanes: one shuffle more
+  auto step = [&](float other) { v = isMax ? fmaxf(v, other) : v + other; };
+  step(lanePermuted<kDppQuadSwap1>(v));
+  step(lanePermuted<kDppQuadSwap2>(v));
+  step(lanePermuted<kDppHalfMirror>(v));
+  if (LPR >= 16) step(lanePermuted<kDppMirror>(v));
+  if (LPR >= 32) step(__shfl_xor(v, 16, 64));
   return v;
 }
 

@@ -85,22 +85,16 @@ __device__ __forceinline__ void mergeState(float& m, float& l, float (&acc)[E], 
   m = mn;
 }
 
-// Sum over the LPT (8, 16 or 32) adjacent lanes that share a head row, left in all of them. The steps within a row of 16
-// lanes are lane permutations folded into the additions (quad swaps, then the mirror images within 8 and within 16,
-// which pair every lane with one that holds the other half of the sum): no trips through the LDS crossbar. Decode
+// Sum over the LPT (8, 16 or 32) adjacent lanes that share a head row, left in all of them: within a row of 16 lanes
+// the steps are lane permutations folded into the additions (see waveSum), no trips through the LDS crossbar. Decode
 // attention at batch 64 (156 000 cached tokens): 373.7 -> 371.6 us; at batch 256: 1054 -> 1046 us.
-template <int CTRL>
-__device__ __forceinline__ float addPermuted(float v) {
-  const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false);
-  return v + __builtin_bit_cast(float, moved);
-}
 template <int LPT>
 __device__ __forceinline__ float headRowSum(float v) {
   static_assert(LPT == 8 || LPT == 16 || LPT == 32, "a head row is shared by 8, 16 or 32 lanes");
-  v = addPermuted<0xB1>(v);   // quad_perm [1, 0, 3, 2]
-  v = addPermuted<0x4E>(v);   // quad_perm [2, 3, 0, 1]
-  v = addPermuted<0x141>(v);  // row_half_mirror
-  if (LPT >= 16) v = addPermuted<0x140>(v);  // row_mirror
+  v += lanePermuted<kDppQuadSwap1>(v);
+  v += lanePermuted<kDppQuadSwap2>(v);
+  v += lanePermuted<kDppHalfMirror>(v);
+  if (LPT >= 16) v += lanePermuted<kDppMirror>(v);
   if (LPT >= 32) v += __shfl_xor(v, 16, 64);
   return v;
 }
