@@ -139,6 +139,22 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   constexpr int kLdsScores = 1024;
   __shared__ float sbuf[MODE != kTaFused ? kLdsScores : 1];
   const bool useLds = MODE != kTaFused && a.chunk <= kLdsScores;
+  // The slot indices of a 512-token chunk take the same way in those modes: one coalesced read of the chunk's piece of
+  // b_loc, then the walk finds its slots in LDS instead of asking memory for one index per wave and row (indices
+  // outside the pool are stored as -1): scores 216 -> 209 us, second half 205 -> 199 us at batch 64; 621 -> 595 and
+  // 565 -> 549 us at batch 256 (8 x 4096 tokens, one round of workgroups: 48.5 -> 50.4 us). Not for the shorter chunks
+  // of small batches, where the wait for the whole piece before the first row is requested weighs more, and not for
+  // the fused mode, whose time moves by a few percent either way with anything that shifts the tail of the grid
+  // (batch 64: 371 -> 392 us, batch 256: 1045 -> 1022 us, 8 x 4096: 90.6 -> 96.7 us).
+  __shared__ int sidx[MODE != kTaFused ? kLdsScores : 1];
+  const bool idxInLds = MODE != kTaFused && a.chunk >= kTaChunk && a.chunk <= kLdsScores && a.slots <= 0x7fffffff;
+  if (idxInLds) {
+    for (int i = threadIdx.x; i < end - begin; i += kTaWaves * 64) {
+      const int64_t s = ldIndex(a.bLoc, locBase + begin + i, a.loc64);
+      sidx[i] = s >= 0 && s < a.slots ? (int)s : -1;
+    }
+    if (!(MODE == kTaReduceV && useLds)) __syncthreads();  // (that mode's barrier below publishes both)
+  }
   if constexpr (MODE == kTaReduceV) {
     if (useLds) {
       for (int i = threadIdx.x; i < end - begin; i += kTaWaves * 64) sbuf[i] = static_cast<float>(scores[begin + i]) * kLog2eTA;
@@ -175,7 +191,7 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
     for (int u = 0; u < UNR; ++u) {
       int t = t0 + u * TPI;
       slotTok[u] = t;
-      slot[u] = t < end ? ldIndex(a.bLoc, locBase + t, a.loc64) : -1;
+      slot[u] = t >= end ? -1 : (idxInLds ? (int64_t)sidx[t - begin] : ldIndex(a.bLoc, locBase + t, a.loc64));
     }
   };
   auto loadRows = [&](V (&kk)[UNR], V (&vv)[UNR], float (&lg)[UNR], bool (&okk)[UNR]) {
