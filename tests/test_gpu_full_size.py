@@ -147,6 +147,56 @@ def test_token_attention_few_sequences_at_32_heads(ops, dev, lens):
     assert_half(got, want)
 
 
+@pytest.mark.parametrize("score_dtype,idt", [(torch.float32, torch.int64), (torch.bfloat16, torch.int32)])
+def test_token_attention_two_call_at_512_token_chunks(ops, dev, score_dtype, idt):
+    """64 sequences of 2048..2600 tokens at 8 heads keep the 512-token chunks, whose scores and slot indices the two-call
+    kernels stage per chunk. 64-bit and 32-bit tables, fp32 and 16-bit score tensors, and table entries that point
+    outside the pool: their scores are -inf and they take no part in the softmax, as in the fused form."""
+    heads, d, slots, batch = 8, 128, 16384, 64
+    lens = torch.randint(2048, 2601, (batch,), generator=g(80))
+    width, total = int(lens.max()), int(lens.sum())
+    kp = torch.randn(slots, heads, d, generator=g(81)).bfloat16()
+    vp = torch.randn(slots, heads, d, generator=g(82)).bfloat16()
+    q = torch.randn(batch, heads, d, generator=g(83)).bfloat16()
+    b_loc = torch.zeros(batch, width, dtype=idt)
+    for b in range(batch):
+        n = int(lens[b])
+        b_loc[b, width - n:] = torch.randint(0, slots, (n,), generator=g(84 + b)).to(idt)
+    ln = lens.to(idt)
+    st = torch.zeros(batch, dtype=idt)
+    st[1:] = torch.cumsum(ln, 0)[:-1]
+    want_att = oracle.token_logits(q, kp, b_loc, st, ln, width, total)
+    # entries outside the pool, in the first, a middle and the last chunk of a few sequences
+    bad = [(0, 0, -1), (0, 700, slots), (3, 1500, slots + 12345), (17, int(lens[17]) - 1, -7), (63, 511, 1 << 30), (63, 512, -slots)]
+    dead = torch.zeros(total, dtype=torch.bool)
+    for b, t, val in bad:
+        b_loc[b, width - int(lens[b]) + t] = val
+        dead[int(st[b]) + t] = True
+    want_att[:, dead] = float("-inf")
+    args = (b_loc.to(dev), st.to(dev), ln.to(dev), width)
+    att = torch.zeros(heads, total, dtype=score_dtype, device=dev)
+    ops.token_attention(q.to(dev), kp.to(dev), att, *args)
+    live = ~dead
+    assert bool(torch.isneginf(att.cpu()[:, dead]).all())
+    if score_dtype == torch.float32:
+        assert_fp32(att.cpu()[:, live], want_att[:, live], rel=1e-5)
+    else:
+        assert_half(att.cpu()[:, live], want_att[:, live])
+    # the second half from the scores the first half stored: softmax over each sequence's live tokens, times V
+    stored = att.cpu().float()
+    want = torch.zeros(batch, heads, d)
+    for b in range(batch):
+        n, s0 = int(lens[b]), int(st[b])
+        sl = b_loc[b, width - n:].long().clamp(0, slots - 1)
+        prob = torch.softmax(stored[:, s0:s0 + n], dim=-1)            # -inf scores weigh nothing
+        want[b] = torch.einsum("hn,nhd->hd", prob, vp[sl].float())
+    out = torch.empty(batch, heads, d, dtype=torch.bfloat16, device=dev)
+    ops.token_softmax_reducev(att, vp.to(dev), out, *args)
+    assert_half(out, want)
+    fused = ops.token_decode_attention(q.to(dev), kp.to(dev), vp.to(dev), *args)
+    assert_half(fused, want)
+
+
 def test_token_attention_length_beyond_the_table_is_cut(ops, dev):
     """b_seq_len larger than max_input_len reads the table row's max_input_len columns and nothing before it."""
     heads, d, slots, width = 4, 128, 256, 600
