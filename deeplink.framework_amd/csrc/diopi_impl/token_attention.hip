@@ -99,16 +99,37 @@ __device__ __forceinline__ float headRowSum(float v) {
   return v;
 }
 
+// c + a[0] b[0] + a[1] b[1] for two packed 16-bit pairs, in one instruction (fp32 accumulation).
+template <typename T>
+__device__ __forceinline__ float dotPair(uint32_t a, uint32_t b, float c) {
+  static_assert(sizeof(T) == 2, "packed pairs of 16-bit elements");
+  if constexpr (std::is_same<T, bf16_t>::value) {
+    typedef __bf16 Pair __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(Pair, a), __builtin_bit_cast(Pair, b), c, false);
+  } else {
+    typedef _Float16 Pair __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(Pair, a), __builtin_bit_cast(Pair, b), c, false);
+  }
+}
+template <typename T>
+__device__ __forceinline__ uint32_t packPair(float lo, float hi) {
+  const T l = static_cast<T>(lo), h = static_cast<T>(hi);
+  return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
+}
+
 // The three things the streaming kernel below can do with a chunk of a sequence: the whole decode attention (scores,
 // online softmax and the sum over V), only the scores (first half of the two-call form: att[h, start_b + t]), or the
 // softmax and the sum over V from scores computed earlier (second half of the two-call form).
 enum TaMode { kTaFused = 0, kTaLogitsOut = 1, kTaReduceV = 2 };
 
 // T: bf16_t / half_t (8 per 16 B) or float (4 per 16 B). LPT lanes cover one head row. LT: the type of the scores in
-// memory (the two-call modes).
-template <typename T, int LPT, bool HIW, int MODE = kTaFused, typename LT = float>
+// memory (the two-call modes). QPK: query heads that share this workgroup's K/V head and are all served from one read
+// of its rows (grouped-query layouts; 1 otherwise). With QPK > 1 blockIdx.x counts (group of QPK query heads, K/V
+// head) pairs, the K/V head fastest, so the groups of one K/V head run on the same XCD and find its rows in that L2.
+template <typename T, int LPT, bool HIW, int MODE = kTaFused, typename LT = float, int QPK = 1>
 __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* __restrict__ out,
                                                                      float* __restrict__ partial) {
+  static_assert(QPK == 1 || !HIW, "several query heads per lane group: the lane groups of a wave take tokens, not heads");
   using V = typename Vec16<T>::type;
   constexpr int N = Vec16<T>::N;
   constexpr int TPW = 64 / LPT;  // tokens per wave-wide load
@@ -120,14 +141,22 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   const int sub = lane % LPT, grp = lane / LPT;
   // HIW: the lane groups of a wave take TPW consecutive heads of the same token (a wave load is TPW head rows, contiguous
   // in a slot) instead of TPW tokens of one head
-  const int h = HIW ? blockIdx.x * TPW + grp : blockIdx.x, split = blockIdx.y, b = blockIdx.z;
+  const int split = blockIdx.y, b = blockIdx.z;
+  const int perKv = a.heads / a.kvHeads;
+  int h, kvh;  // h: this lane group's (first) query head
+  if constexpr (QPK == 1) {
+    h = HIW ? blockIdx.x * TPW + grp : blockIdx.x;
+    kvh = h / perKv;
+  } else {
+    kvh = blockIdx.x % a.kvHeads;
+    h = kvh * perKv + (blockIdx.x / a.kvHeads) * QPK;
+  }
   const int len = min(max((int)ldIndex(a.bLen, b, a.len64), 0), a.maxLen);  // a length beyond the table's width is cut to it
   const int begin = split * a.chunk;
   if (begin >= len && !(split == 0 && MODE != kTaLogitsOut)) return;  // nothing to do; split 0 still writes zeros for len == 0
   const int end = min(len, begin + a.chunk);
-  const int kvh = h / (a.heads / a.kvHeads);
   const int64_t locBase = (int64_t)b * a.locRowStride + (a.maxLen - len);
-  // the scores of this lane's head for the tokens of sequence b (two-call modes)
+  // the scores of this lane's (first) head for the tokens of sequence b (two-call modes); head h + j is j rows further
   LT* scores = nullptr;
   if constexpr (MODE != kTaFused)
     scores = static_cast<LT*>(const_cast<void*>(a.logits)) + h * a.logitsHeadStride + ldIndex(a.bStart, b, a.start64);
@@ -137,7 +166,7 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   // (at batch 64, 156 000 tokens: scores 225 -> 219 us, second half 234 -> 205 us). Chunks longer than the buffer
   // (sequences past 131 072 tokens) keep the direct accesses.
   constexpr int kLdsScores = 1024;
-  __shared__ float sbuf[MODE != kTaFused ? kLdsScores : 1];
+  __shared__ float sbuf[MODE != kTaFused ? QPK * kLdsScores : 1];
   const bool useLds = MODE != kTaFused && a.chunk <= kLdsScores;
   // The slot indices of a 512-token chunk take the same way in those modes: one coalesced read of the chunk's piece of
   // b_loc, then the walk finds its slots in LDS instead of asking memory for one index per wave and row (indices
@@ -157,24 +186,47 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   }
   if constexpr (MODE == kTaReduceV) {
     if (useLds) {
-      for (int i = threadIdx.x; i < end - begin; i += kTaWaves * 64) sbuf[i] = static_cast<float>(scores[begin + i]) * kLog2eTA;
+#pragma unroll
+      for (int j = 0; j < QPK; ++j)
+        for (int i = threadIdx.x; i < end - begin; i += kTaWaves * 64)
+          sbuf[j * kLdsScores + i] = static_cast<float>(scores[j * a.logitsHeadStride + begin + i]) * kLog2eTA;
       __syncthreads();
     }
   }
-  float qf[N];
+  // Several query heads on 16-bit rows: the products are taken two at a time on the packed pairs as they come from
+  // memory (q.k: a pair of q against a pair of k; p.v: the probabilities of the two rows in flight, rounded to 16
+  // bits, against the two rows' values of one element), which halves the arithmetic instructions and needs no
+  // conversions of K and V. 32 query heads on 8 K/V heads, batch 64 x (512..4096), fused: 184 -> 157 us (147 -> 110
+  // registers, three -> four waves per SIMD); batch 256 x (1024..2048): 484 -> 413 us.
+  constexpr bool kPairs = QPK > 1 && sizeof(T) == 2 && UNR == 2;
+  // scores leave the kernel in natural units, inside it they are in units of log2
+  const float qScale = MODE == kTaLogitsOut ? a.scaleLog2e / kLog2eTA : a.scaleLog2e;
+  float qf[kPairs ? 1 : QPK][N];
+  uint32_t qp[kPairs ? QPK : 1][4];
   if constexpr (kNeedK) {
-    // scores leave the kernel in natural units, inside it they are in units of log2
-    const float qScale = MODE == kTaLogitsOut ? a.scaleLog2e / kLog2eTA : a.scaleLog2e;
-    V qv = *reinterpret_cast<const V*>(reinterpret_cast<const T*>(a.q) + b * a.qBatchStride + h * a.qHeadStride + sub * N);
 #pragma unroll
-    for (int e = 0; e < N; ++e) qf[e] = static_cast<float>(qv[e]) * qScale;
+    for (int j = 0; j < QPK; ++j) {
+      V qv = *reinterpret_cast<const V*>(reinterpret_cast<const T*>(a.q) + b * a.qBatchStride + (h + j) * a.qHeadStride + sub * N);
+      if constexpr (kPairs) {
+        const u32x4 raw = __builtin_bit_cast(u32x4, qv);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) qp[j][c] = raw[c];
+      } else {
+#pragma unroll
+        for (int e = 0; e < N; ++e) qf[j][e] = static_cast<float>(qv[e]) * qScale;
+      }
+    }
   }
   const T* kBase = kNeedK ? reinterpret_cast<const T*>(a.k) + kvh * a.kHeadStride + sub * N : nullptr;
   const T* vBase = kNeedV ? reinterpret_cast<const T*>(a.v) + kvh * a.vHeadStride + sub * N : nullptr;
 
-  float m = -INFINITY, l = 0.f, acc[N];
+  float m[QPK], l[QPK], acc[QPK][N];
 #pragma unroll
-  for (int e = 0; e < N; ++e) acc[e] = 0.f;
+  for (int j = 0; j < QPK; ++j) {
+    m[j] = -INFINITY, l[j] = 0.f;
+#pragma unroll
+    for (int e = 0; e < N; ++e) acc[j][e] = 0.f;
+  }
 
   constexpr int TPI = HIW ? 1 : TPW;  // tokens per wave-wide load
   constexpr int STEP = kTaWaves * UNR * TPI;  // tokens per workgroup iteration
@@ -183,7 +235,7 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   int64_t slot[UNR];
   int slotTok[UNR];  // the token each slot index belongs to (the stored scores are addressed by it)
   V kr[UNR], vr[UNR], kn[UNR], vn[UNR];
-  float lr[UNR], ln[UNR];  // stored scores of the rows (kTaReduceV)
+  float lr[QPK][UNR], ln[QPK][UNR];  // stored scores of the rows (kTaReduceV)
   bool ok[UNR], okn[UNR];
   auto loadSlots = [&](int it) {
     int t0 = it + wave * UNR * TPI + (HIW ? 0 : grp);
@@ -194,15 +246,20 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
       slot[u] = t >= end ? -1 : (idxInLds ? (int64_t)sidx[t - begin] : ldIndex(a.bLoc, locBase + t, a.loc64));
     }
   };
-  auto loadRows = [&](V (&kk)[UNR], V (&vv)[UNR], float (&lg)[UNR], bool (&okk)[UNR]) {
+  auto loadRows = [&](V (&kk)[UNR], V (&vv)[UNR], float (&lg)[QPK][UNR], bool (&okk)[UNR]) {
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
       okk[u] = slot[u] >= 0 && slot[u] < a.slots;  // slots outside the pool are skipped, never dereferenced
       int64_t s = okk[u] ? slot[u] : 0;
       if constexpr (kNeedK) kk[u] = __builtin_nontemporal_load(reinterpret_cast<const V*>(kBase + s * a.kSlotStride));
       if constexpr (kNeedV) vv[u] = __builtin_nontemporal_load(reinterpret_cast<const V*>(vBase + s * a.vSlotStride));
-      if constexpr (MODE == kTaReduceV)
-        lg[u] = !okk[u] ? -INFINITY : (useLds ? sbuf[slotTok[u] - begin] : static_cast<float>(scores[slotTok[u]]) * kLog2eTA);
+      if constexpr (MODE == kTaReduceV) {
+#pragma unroll
+        for (int j = 0; j < QPK; ++j)
+          lg[j][u] = !okk[u] ? -INFINITY
+                             : (useLds ? sbuf[j * kLdsScores + slotTok[u] - begin]
+                                       : static_cast<float>(scores[j * a.logitsHeadStride + slotTok[u]]) * kLog2eTA);
+      }
     }
   };
   loadSlots(begin);
@@ -211,55 +268,98 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   for (int it = begin; it < end; it += STEP) {
     loadRows(kn, vn, ln, okn);    // rows of the next iteration (all masked past the end)
     loadSlots(it + 2 * STEP);     // indices of the one after
-    float sc[UNR];
-    float mn = m;
+    float kf[kNeedK && QPK > 1 && !kPairs ? UNR : 1][N];  // several query heads on fp32 rows: the K rows are converted once
+    if constexpr (kNeedK && QPK > 1 && !kPairs) {
+#pragma unroll
+      for (int u = 0; u < UNR; ++u)
+#pragma unroll
+        for (int e = 0; e < N; ++e) kf[u][e] = static_cast<float>(kr[u][e]);
+    }
+    // kPairs: element 2 c and 2 c + 1 of the two V rows, regrouped as (row 0, row 1) pairs of one element each
+    uint32_t vlo[kPairs && kNeedV ? 4 : 1], vhi[kPairs && kNeedV ? 4 : 1];
+    if constexpr (kPairs && kNeedV) {
+      const u32x4 r0 = __builtin_bit_cast(u32x4, vr[0]), r1 = __builtin_bit_cast(u32x4, vr[1]);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        vlo[c] = __builtin_amdgcn_perm(r1[c], r0[c], 0x05040100u);
+        vhi[c] = __builtin_amdgcn_perm(r1[c], r0[c], 0x07060302u);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < QPK; ++j) {
+      float sc[UNR];
+      float mn = m[j];
+#pragma unroll
+      for (int u = 0; u < UNR; ++u) {
+        if constexpr (kNeedK) {
+          float d = 0.f;
+          if constexpr (kPairs) {
+            const u32x4 kraw = __builtin_bit_cast(u32x4, kr[u]);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) d = dotPair<T>(qp[j][c], kraw[c], d);
+            d = headRowSum<LPT>(d) * qScale;
+          } else {
+#pragma unroll
+            for (int e = 0; e < N; ++e) d += qf[j][e] * (QPK > 1 ? kf[u][e] : static_cast<float>(kr[u][e]));
+            d = headRowSum<LPT>(d);
+          }
+          sc[u] = ok[u] ? d : -INFINITY;
+        } else {
+          sc[u] = lr[j][u];
+        }
+        mn = fmaxf(mn, sc[u]);
+      }
+      if constexpr (MODE == kTaLogitsOut) {
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+          const int t = it + wave * UNR * TPI + (HIW ? 0 : grp) + u * TPI;
+          if (sub == 0 && t < end) {
+            if (useLds) sbuf[j * kLdsScores + t - begin] = sc[u];
+            else scores[j * a.logitsHeadStride + t] = static_cast<LT>(sc[u]);
+          }
+        }
+      } else if (mn != -INFINITY) {
+        float corr = __builtin_amdgcn_exp2f(m[j] - mn);  // m == -inf gives 0, acc and l are 0 then anyway
+        float p[UNR], ps = 0.f;
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+          p[u] = __builtin_amdgcn_exp2f(sc[u] - mn);
+          ps += p[u];
+        }
+        l[j] = l[j] * corr + ps;
+        if constexpr (kPairs) {
+          const uint32_t pp = packPair<T>(p[0], p[UNR - 1]);
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            acc[j][2 * c] = dotPair<T>(pp, vlo[c], acc[j][2 * c] * corr);
+            acc[j][2 * c + 1] = dotPair<T>(pp, vhi[c], acc[j][2 * c + 1] * corr);
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < N; ++e) {
+            float s = acc[j][e] * corr;
+#pragma unroll
+            for (int u = 0; u < UNR; ++u) s += p[u] * static_cast<float>(vr[u][e]);
+            acc[j][e] = s;
+          }
+        }
+        m[j] = mn;
+      }
+    }
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
-      if constexpr (kNeedK) {
-        float d = 0.f;
+      kr[u] = kn[u], vr[u] = vn[u], ok[u] = okn[u];
 #pragma unroll
-        for (int e = 0; e < N; ++e) d += qf[e] * static_cast<float>(kr[u][e]);
-        d = headRowSum<LPT>(d);
-        sc[u] = ok[u] ? d : -INFINITY;
-      } else {
-        sc[u] = lr[u];
-      }
-      mn = fmaxf(mn, sc[u]);
+      for (int j = 0; j < QPK; ++j) lr[j][u] = ln[j][u];
     }
-    if constexpr (MODE == kTaLogitsOut) {
-#pragma unroll
-      for (int u = 0; u < UNR; ++u) {
-        const int t = it + wave * UNR * TPI + (HIW ? 0 : grp) + u * TPI;
-        if (sub == 0 && t < end) {
-          if (useLds) sbuf[t - begin] = sc[u];
-          else scores[t] = static_cast<LT>(sc[u]);
-        }
-      }
-    } else if (mn != -INFINITY) {
-      float corr = __builtin_amdgcn_exp2f(m - mn);  // m == -inf gives 0, acc and l are 0 then anyway
-      float p[UNR], ps = 0.f;
-#pragma unroll
-      for (int u = 0; u < UNR; ++u) {
-        p[u] = __builtin_amdgcn_exp2f(sc[u] - mn);
-        ps += p[u];
-      }
-      l = l * corr + ps;
-#pragma unroll
-      for (int e = 0; e < N; ++e) {
-        float s = acc[e] * corr;
-#pragma unroll
-        for (int u = 0; u < UNR; ++u) s += p[u] * static_cast<float>(vr[u][e]);
-        acc[e] = s;
-      }
-      m = mn;
-    }
-#pragma unroll
-    for (int u = 0; u < UNR; ++u) kr[u] = kn[u], vr[u] = vn[u], lr[u] = ln[u], ok[u] = okn[u];
   }
   if constexpr (MODE == kTaLogitsOut) {
     if (useLds) {
       __syncthreads();
-      for (int i = threadIdx.x; i < end - begin; i += kTaWaves * 64) scores[begin + i] = static_cast<LT>(sbuf[i]);
+#pragma unroll
+      for (int j = 0; j < QPK; ++j)
+        for (int i = threadIdx.x; i < end - begin; i += kTaWaves * 64)
+          scores[j * a.logitsHeadStride + begin + i] = static_cast<LT>(sbuf[j * kLdsScores + i]);
     }
     return;
   }
@@ -267,41 +367,47 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   // merge the TPW lane groups of the wave (each holds other tokens of the same head)
   if (!HIW)
 #pragma unroll
-  for (int off = LPT; off < 64; off <<= 1) {
-    float m2 = __shfl_xor(m, off, 64), l2 = __shfl_xor(l, off, 64), acc2[N];
+  for (int j = 0; j < QPK; ++j)
 #pragma unroll
-    for (int e = 0; e < N; ++e) acc2[e] = __shfl_xor(acc[e], off, 64);
-    mergeState<N>(m, l, acc, m2, l2, acc2);
+  for (int off = LPT; off < 64; off <<= 1) {
+    float m2 = __shfl_xor(m[j], off, 64), l2 = __shfl_xor(l[j], off, 64), acc2[N];
+#pragma unroll
+    for (int e = 0; e < N; ++e) acc2[e] = __shfl_xor(acc[j][e], off, 64);
+    mergeState<N>(m[j], l[j], acc[j], m2, l2, acc2);
   }
-  // merge the waves through LDS: [wave][2 + LPT*N]
+  // merge the waves through LDS: [wave][2 + LPT*N], one query head after the other
   constexpr int RG = HIW ? TPW : 1;  // lane groups with a state of their own
   const int rg = HIW ? grp : 0;
   __shared__ float red[kTaWaves][RG][2 + LPT * N];
-  if (HIW || grp == 0) {
-    if (sub == 0) red[wave][rg][0] = m, red[wave][rg][1] = l;
 #pragma unroll
-    for (int e = 0; e < N; ++e) red[wave][rg][2 + sub * N + e] = acc[e];
-  }
-  __syncthreads();
-  if (wave == 0 && (HIW || grp == 0)) {
+  for (int j = 0; j < QPK; ++j) {
+    if (j > 0) __syncthreads();  // wave 0 has read the previous head's states
+    if (HIW || grp == 0) {
+      if (sub == 0) red[wave][rg][0] = m[j], red[wave][rg][1] = l[j];
 #pragma unroll
-    for (int w = 1; w < kTaWaves; ++w) {
-      float acc2[N];
-#pragma unroll
-      for (int e = 0; e < N; ++e) acc2[e] = red[w][rg][2 + sub * N + e];
-      mergeState<N>(m, l, acc, red[w][rg][0], red[w][rg][1], acc2);
+      for (int e = 0; e < N; ++e) red[wave][rg][2 + sub * N + e] = acc[j][e];
     }
-    if (a.nsplit == 1) {
-      float inv = l > 0.f ? 1.f / l : 0.f;
-      V o;
+    __syncthreads();
+    if (wave == 0 && (HIW || grp == 0)) {
 #pragma unroll
-      for (int e = 0; e < N; ++e) o[e] = static_cast<T>(acc[e] * inv);
-      *reinterpret_cast<V*>(out + ((int64_t)b * a.heads + h) * a.d + sub * N) = o;
-    } else {
-      float* dst = partial + (((int64_t)b * a.heads + h) * a.nsplit + split) * (2 + a.d);
-      if (sub == 0) dst[0] = m, dst[1] = l;
+      for (int w = 1; w < kTaWaves; ++w) {
+        float acc2[N];
 #pragma unroll
-      for (int e = 0; e < N; ++e) dst[2 + sub * N + e] = acc[e];
+        for (int e = 0; e < N; ++e) acc2[e] = red[w][rg][2 + sub * N + e];
+        mergeState<N>(m[j], l[j], acc[j], red[w][rg][0], red[w][rg][1], acc2);
+      }
+      if (a.nsplit == 1) {
+        float inv = l[j] > 0.f ? 1.f / l[j] : 0.f;
+        V o;
+#pragma unroll
+        for (int e = 0; e < N; ++e) o[e] = static_cast<T>(acc[j][e] * inv);
+        *reinterpret_cast<V*>(out + ((int64_t)b * a.heads + h + j) * a.d + sub * N) = o;
+      } else {
+        float* dst = partial + (((int64_t)b * a.heads + h + j) * a.nsplit + split) * (2 + a.d);
+        if (sub == 0) dst[0] = m[j], dst[1] = l[j];
+#pragma unroll
+        for (int e = 0; e < N; ++e) dst[2 + sub * N + e] = acc[j][e];
+      }
     }
   }
 }
@@ -746,8 +852,16 @@ static diopiError_t streamChunks(diopiContextHandle_t ctx, hipStream_t stream, T
   // (the two-call modes keep four tokens of one head per wave load and a workgroup per head: at batch 64, 156 000
   // tokens, with the chunk's scores staged in LDS either way, four heads per workgroup read 244 against 219 us for the
   // scores and 238 against 205 us for the second half)
-  const bool hiw = MODE == kTaFused && (bytes == 128 || bytes == 256 || bytes == 512) && a.heads % tpw == 0;
-  chooseChunk(&a, hiw ? a.heads / tpw : a.heads, batch, maxInputLen);
+  // Grouped-query layouts: one read of a K/V row serves four (or two) of the query heads that share it, with their
+  // softmax states side by side in the lane group's registers; more sharers than that are dealt over several
+  // workgroups that run on the same XCD. At batch 64 x (512..4096) tokens, 32 query heads on 8 K/V heads (every query
+  // head used to read the rows for itself): fused 236 -> 157 us, scores 214 -> 74 us, second half 205 -> 106 us; 64
+  // query heads on 8: 405 -> 240 us fused. A sharing factor that is odd keeps the one-head-per-read form.
+  const int perKv = a.heads / a.kvHeads;
+  const int qpk = perKv % 4 == 0 ? 4 : (perKv % 2 == 0 ? 2 : 1);
+  const bool hiw = qpk == 1 && MODE == kTaFused && (bytes == 128 || bytes == 256 || bytes == 512) && a.heads % tpw == 0;
+  const int groupsPerSeq = qpk > 1 ? a.kvHeads * (perKv / qpk) : (hiw ? a.heads / tpw : a.heads);
+  chooseChunk(&a, groupsPerSeq, batch, maxInputLen);
   a.nsplit = (int)std::max<int64_t>(1, ceilDiv(maxInputLen, a.chunk));
   AMD_CHECK(batch <= 65535 && a.nsplit <= 65535, "token attention: batch %ld / splits %d exceed the grid limits", (long)batch,
             a.nsplit);
@@ -768,9 +882,11 @@ static diopiError_t streamChunks(diopiContextHandle_t ctx, hipStream_t stream, T
       partial = static_cast<float*>(ws);
     }
   }
-  dim3 grid(hiw ? a.heads / tpw : a.heads, a.nsplit, (unsigned)batch), block(kTaWaves * 64);
+  dim3 grid((unsigned)groupsPerSeq, a.nsplit, (unsigned)batch), block(kTaWaves * 64);
 #define STREAM_CALL_AS(T, LPT, LT)                                                                                                   \
-  if (hiw) hipLaunchKernelGGL((decodeSplitKernel<T, LPT, true, MODE, LT>), grid, block, 0, stream, a, static_cast<T*>(outPtr), partial); \
+  if (qpk == 4) hipLaunchKernelGGL((decodeSplitKernel<T, LPT, false, MODE, LT, 4>), grid, block, 0, stream, a, static_cast<T*>(outPtr), partial); \
+  else if (qpk == 2) hipLaunchKernelGGL((decodeSplitKernel<T, LPT, false, MODE, LT, 2>), grid, block, 0, stream, a, static_cast<T*>(outPtr), partial); \
+  else if (hiw) hipLaunchKernelGGL((decodeSplitKernel<T, LPT, true, MODE, LT>), grid, block, 0, stream, a, static_cast<T*>(outPtr), partial); \
   else hipLaunchKernelGGL((decodeSplitKernel<T, LPT, false, MODE, LT>), grid, block, 0, stream, a, static_cast<T*>(outPtr), partial)
 #define STREAM_CALL(T, LPT)                                \
   if (MODE == kTaFused || scoresF32) {                     \

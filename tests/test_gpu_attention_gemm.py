@@ -511,8 +511,7 @@ def test_token_attention_any_head_size(ops, dev, pkg, dtype, d, kvh, rep):
 
 @pytest.mark.parametrize("heads,kvh", [(8, 2), (6, 3)])
 def test_token_attention_len_one_and_gqa(ops, dev, heads, kvh):
-    """Grouped-query decode: 8 heads (a wave's lane groups take four consecutive heads of one token) and 6 heads (not a
-    multiple of four: the lane groups take four tokens of one head)."""
+    """Grouped-query decode: four query heads per K/V head (served from one read of its rows) and two."""
     slots, d = 64, 128
     kp = torch.randn(slots, kvh, d, generator=g(30)).bfloat16()
     vp = torch.randn(slots, kvh, d, generator=g(31)).bfloat16()
@@ -529,6 +528,42 @@ def test_token_attention_len_one_and_gqa(ops, dev, heads, kvh):
     # a single cached token: the output is that token's V row for the mapped kv head
     assert_exact(got[0].cpu(), vp[17].repeat_interleave(heads // kvh, dim=0))
     assert_exact(got[2].cpu(), vp[63].repeat_interleave(heads // kvh, dim=0))
+
+
+@pytest.mark.parametrize("heads,kvh,dtype,d,idt", [
+    (32, 8, torch.bfloat16, 128, torch.int32),    # four query heads per K/V row read, products on packed pairs
+    (16, 8, torch.float16, 64, torch.int64),      # two per read, 8 lanes per head row
+    (64, 8, torch.bfloat16, 128, torch.int32),    # eight sharers: two workgroups of four per K/V head
+    (8, 1, torch.float32, 64, torch.int32),       # one K/V head for all; fp32 rows take the unpacked arithmetic
+    (8, 2, torch.float16, 256, torch.int32),      # 32 lanes per head row
+    (12, 4, torch.bfloat16, 128, torch.int32),    # three sharers: every query head reads the rows for itself
+])
+def test_token_attention_grouped_query_layouts(ops, dev, heads, kvh, dtype, d, idt):
+    """Fused and two-call decode attention with fewer K/V heads than query heads, over sequences of 1 to 1500 tokens
+    (one to several chunks, ragged ends), against the oracle's repeat-interleaved K/V."""
+    slots = 4096
+    lens = [1, 1500, 777, 64, 513, 130, 1024]
+    batch, width, total = len(lens), max(lens), sum(lens)
+    kp = torch.randn(slots, kvh, d, generator=g(90)).to(dtype)
+    vp = torch.randn(slots, kvh, d, generator=g(91)).to(dtype)
+    q = torch.randn(batch, heads, d, generator=g(92)).to(dtype)
+    b_loc = torch.zeros(batch, width, dtype=idt)
+    for b, n in enumerate(lens):
+        b_loc[b, width - n:] = torch.randint(0, slots, (n,), generator=g(93 + b)).to(idt)
+    ln = torch.tensor(lens, dtype=idt)
+    st = torch.zeros(batch, dtype=idt)
+    st[1:] = torch.cumsum(ln, 0)[:-1]
+    want = oracle.token_attention(q.float(), kp.float(), vp.float(), b_loc, ln, width)
+    chk = assert_fp32 if dtype == torch.float32 else assert_half
+    args = (b_loc.to(dev), st.to(dev), ln.to(dev), width)
+    got = ops.token_decode_attention(q.to(dev), kp.to(dev), vp.to(dev), *args)
+    chk(got, want)
+    att = torch.zeros(heads, total, dtype=torch.float32, device=dev)
+    ops.token_attention(q.to(dev), kp.to(dev), att, *args)
+    assert_fp32(att, oracle.token_logits(q, kp, b_loc, st, ln, width, total), rel=1e-5)
+    out2 = torch.empty_like(got)
+    ops.token_softmax_reducev(att, vp.to(dev), out2, *args)
+    chk(out2, want)
 
 
 # ------------------------------------------------------------------ int8 weight-only linear
