@@ -141,7 +141,11 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   const int sub = lane % LPT, grp = lane / LPT;
   // HIW: the lane groups of a wave take TPW consecutive heads of the same token (a wave load is TPW head rows, contiguous
   // in a slot) instead of TPW tokens of one head
-  const int split = blockIdx.y, b = blockIdx.z;
+  // Dispatch order: the chunk index is the slowest grid dimension and runs backwards, so the ragged part of the work
+  // (the last, partly filled chunk of every sequence and the chunks only long sequences have) is handed out first and
+  // the launch ends on whole chunks that finish together. Against sequence-major order, batch 64 x (512..4096):
+  // 410.7 -> 406.8 us; 32 x (100..8192): 332 -> 323; 256 x (1024..2048): 1040 -> 1025, and with 8 K/V heads 413 -> 361.
+  const int split = (int)gridDim.z - 1 - (int)blockIdx.z, b = blockIdx.y;
   const int perKv = a.heads / a.kvHeads;
   int h, kvh;  // h: this lane group's (first) query head
   if constexpr (QPK == 1) {
@@ -882,7 +886,7 @@ static diopiError_t streamChunks(diopiContextHandle_t ctx, hipStream_t stream, T
       partial = static_cast<float*>(ws);
     }
   }
-  dim3 grid((unsigned)groupsPerSeq, a.nsplit, (unsigned)batch), block(kTaWaves * 64);
+  dim3 grid((unsigned)groupsPerSeq, (unsigned)batch, a.nsplit), block(kTaWaves * 64);
 #define STREAM_CALL_AS(T, LPT, LT)                                                                                                   \
   if (qpk == 4) hipLaunchKernelGGL((decodeSplitKernel<T, LPT, false, MODE, LT, 4>), grid, block, 0, stream, a, static_cast<T*>(outPtr), partial); \
   else if (qpk == 2) hipLaunchKernelGGL((decodeSplitKernel<T, LPT, false, MODE, LT, 2>), grid, block, 0, stream, a, static_cast<T*>(outPtr), partial); \
