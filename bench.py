@@ -528,6 +528,14 @@ def op_microbench(pkg, torch, dev, rt, stream, with_cpu=True):
     res.append(hbm_row("diopiTokenAttentionInference", f"batch 64, 32x128, sum(len)={L}, fp32 scores", half_bytes, None, p_a1))
     res.append(hbm_row("diopiTokenSoftmaxReduceVInference", f"batch 64, 32x128, sum(len)={L}, fp32 scores", half_bytes, None, p_a2))
     del att
+    # the same sequences over a pool with 8 K/V heads for the 32 query heads (a grouped-query layout: the pool is a view of
+    # the first 8 heads of the same slots, so a row read serves four query heads)
+    k8, v8 = g["k_pool"][:, :8], g["v_pool"][:, :8]
+    a8 = Prepared(pkg, "diopiTokenDecodeAttentionInference", out, g["q"], k8, v8, g["b_loc"], g["b_start_loc"], g["b_seq_len"],
+                  int(g["max_input_len"]))
+    p_a8 = time_ops_stats(rt, stream, [a8], 30, 6)[0]
+    res.append(hbm_row("diopiTokenDecodeAttentionInference", f"batch 64, 32 query heads on 8 K/V heads x 128, sum(len)={L}",
+                       L * 8 * 128 * 2 * 2 + L * idx_b + 2 * 64 * 32 * 128 * 2, None, p_a8))
     res.append(decode_layer_step(pkg, torch, dev, rt, stream, g))
     del g, pd
     # int8 weight-only linear: weights rotate through 8 copies (360 MB) for the cold figure
