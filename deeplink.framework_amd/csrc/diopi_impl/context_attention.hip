@@ -410,6 +410,23 @@ __global__ __launch_bounds__(256, 2) void contextAttnMfmaKernel(CaArgs a, int nu
   }
 }
 
+// The same blocks one per workgroup, the heaviest first, for launches whose pairs would leave CUs without work or with
+// twice their share (a single prompt of a few hundred tokens; a few sequences whose pairs are a little more than one
+// per CU). The dispatcher hands a free CU the heaviest block left, so the load evens out the way a longest-job-first
+// list does, and a short prompt has twice the workgroups. The blocks of one head are no longer neighbours in time
+// and share less in L2, which is why launches whose pairs already fill the chip evenly keep the paired form. Measured
+// (us, 32 heads x 128, bf16, pairs -> this): 1 x 256 tokens 14.6 -> 9.1, 1 x 512 19.1 -> 13.6, 1 x 1024 28.0 -> 22.8,
+// 3 x 700 30.9 -> 24.4, 1 x 3000 89.7 -> 84.9; against it: 1 x 2048 46.8 -> 51.0, 32 x 512 134 -> 155, 8 x 1000 88 -> 103.
+template <typename T, int D>
+__global__ __launch_bounds__(256, 2) void contextAttnSingleBlockKernel(CaArgs a, int numQBlocks, int numSeq) {
+  const int flat = (int)blockIdx.x;
+  const int xcd = flat & 7, idx = flat >> 3, perXcd = a.heads >> 3;  // the head count is a multiple of 8
+  const int hsPerXcd = perXcd * numSeq;
+  const int rank = idx / hsPerXcd, hs = idx - rank * hsPerXcd;
+  const int b = hs / perXcd, h = xcd * perXcd + (hs - b * perXcd);
+  contextAttnBlock<T, D>(a, numQBlocks - 1 - rank, h, b);
+}
+
 // One workgroup per (query token, head): scores to LDS, softmax, then P.V with lanes over d.
 template <typename T>
 __global__ __launch_bounds__(256) void contextAttnScalarKernel(CaArgs a, int maxLen) {
@@ -465,6 +482,18 @@ static diopiError_t launchCaMfma(hipStream_t stream, const CaArgs& a, int maxLen
   const int numQBlocks = (int)ceilDiv(maxLen, kCaBQ);
   const int64_t blocks = (int64_t)((numQBlocks + 1) / 2) * a.heads * batch;
   AMD_CHECK(blocks < ((int64_t)1 << 31), "context attention: grid limits exceeded");
+  // Busiest CU's load in units of one key-block column of a query block (block i costs i + 1): pairs of numQBlocks + 1
+  // dealt round-robin, against single blocks handed out heaviest first (the mean load, or the heaviest block alone).
+  const int64_t cus = computeUnits(), hb = (int64_t)a.heads * batch;
+  const int64_t pairedLoad = ceilDiv(blocks, cus) * (numQBlocks + 1);
+  const int64_t singleLoad = std::max<int64_t>(ceilDiv(hb * numQBlocks * (numQBlocks + 1) / 2, cus), numQBlocks);
+  if ((a.heads & 7) == 0 && numQBlocks > 1 && singleLoad * 11 < pairedLoad * 10 && hb * numQBlocks < ((int64_t)1 << 31)) {
+    AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&contextAttnSingleBlockKernel<T, D>), (int)lds));
+    hipLaunchKernelGGL((contextAttnSingleBlockKernel<T, D>), dim3((unsigned)(hb * numQBlocks)), dim3(256), lds, stream, a, numQBlocks,
+                       (int)batch);
+    AMD_LAUNCH_CHECK();
+    return diopiSuccess;
+  }
   hipLaunchKernelGGL((contextAttnMfmaKernel<T, D>), dim3((unsigned)blocks), dim3(256), lds, stream, a, numQBlocks, (int)batch);
   AMD_LAUNCH_CHECK();
   return diopiSuccess;

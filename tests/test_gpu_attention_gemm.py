@@ -451,6 +451,23 @@ def test_context_attention_long_ragged_batch_paired_blocks(ops, dev, heads, kvh,
     assert_half(got, want)
 
 
+@pytest.mark.parametrize("heads,kvh,d,dtype,lens", [(32, 32, 128, torch.bfloat16, [512]), (8, 2, 128, torch.bfloat16, [1000]),
+                                                    (16, 4, 64, torch.float16, [700, 129, 5]), (8, 8, 128, torch.float16, [257, 256, 255, 1])])
+def test_context_attention_one_query_block_per_workgroup(ops, dev, heads, kvh, d, dtype, lens):
+    """Launches too small for the paired schedule to fill the chip evenly: every 128-query block is a workgroup of its
+    own, heaviest first (a single short prompt; a few ragged sequences; block counts of 4, 8, 6 and 3)."""
+    starts = [sum(lens[:i]) for i in range(len(lens))]
+    total = sum(lens)
+    q = torch.randn(total, heads, d, generator=g(40)).to(dtype)
+    k = torch.randn(total, kvh, d, generator=g(41)).to(dtype)
+    v = torch.randn(total, kvh, d, generator=g(42)).to(dtype)
+    st, ln = torch.tensor(starts, dtype=torch.int32), torch.tensor(lens, dtype=torch.int32)
+    want = oracle.context_attention(q.float(), k.float(), v.float(), st, ln)
+    got = ops.context_attention(q.to(dev), k.to(dev), v.to(dev), st.to(dev), ln.to(dev), max(lens))
+    assert_half(got, want)
+    assert_exact(got[starts[-1]].cpu(), v[starts[-1]].repeat_interleave(heads // kvh, dim=0))   # a sequence's first query sees one key
+
+
 # ------------------------------------------------------------------ decode attention
 @pytest.mark.parametrize("dtype,d,idt", [(torch.bfloat16, 128, torch.int32), (torch.float16, 64, torch.int64),
                                           (torch.float32, 64, torch.int32), (torch.bfloat16, 256, torch.int32)])
