@@ -70,6 +70,7 @@ struct TaArgs {
   float scaleLog2e;  // log2(e) / sqrt(d)
   const void* logits;  // two-call form: scores [heads, total_tokens], row h at logits + h * logitsHeadStride (elements)
   int64_t logitsHeadStride;
+  int qGroups;  // grouped-query layouts: workgroups that share the query heads of one K/V head between them
 };
 
 // Merge (m, l, acc) of another online-softmax stream into this one.
@@ -147,14 +148,19 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   // 410.7 -> 406.8 us; 32 x (100..8192): 332 -> 323; 256 x (1024..2048): 1040 -> 1025, and with 8 K/V heads 413 -> 361.
   const int split = (int)gridDim.z - 1 - (int)blockIdx.z, b = blockIdx.y;
   const int perKv = a.heads / a.kvHeads;
-  int h, kvh;  // h: this lane group's (first) query head
+  int h, kvh, nq = 1;  // h: this lane group's (first) query head; nq: how many it serves (at most QPK)
   if constexpr (QPK == 1) {
     h = HIW ? blockIdx.x * TPW + grp : blockIdx.x;
     kvh = h / perKv;
   } else {
+    // the perKv sharers of a K/V head are dealt over qGroups workgroups as evenly as they go (7 = 4 + 3); a group
+    // short of QPK heads computes its last head again in the spare places and stores nothing from them
     kvh = blockIdx.x % a.kvHeads;
-    h = kvh * perKv + (blockIdx.x / a.kvHeads) * QPK;
+    const int g = blockIdx.x / a.kvHeads, base = perKv / a.qGroups, rem = perKv % a.qGroups;
+    h = kvh * perKv + g * base + min(g, rem);
+    nq = base + (g < rem ? 1 : 0);
   }
+  auto headOf = [&](int j) { return QPK == 1 ? 0 : min(j, nq - 1); };  // offset of place j's head from h
   const int len = min(max((int)ldIndex(a.bLen, b, a.len64), 0), a.maxLen);  // a length beyond the table's width is cut to it
   const int begin = split * a.chunk;
   if (begin >= len && !(split == 0 && MODE != kTaLogitsOut)) return;  // nothing to do; split 0 still writes zeros for len == 0
@@ -193,7 +199,7 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
 #pragma unroll
       for (int j = 0; j < QPK; ++j)
         for (int i = threadIdx.x; i < end - begin; i += kTaWaves * 64)
-          sbuf[j * kLdsScores + i] = static_cast<float>(scores[j * a.logitsHeadStride + begin + i]) * kLog2eTA;
+          sbuf[j * kLdsScores + i] = static_cast<float>(scores[headOf(j) * a.logitsHeadStride + begin + i]) * kLog2eTA;
       __syncthreads();
     }
   }
@@ -210,7 +216,7 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   if constexpr (kNeedK) {
 #pragma unroll
     for (int j = 0; j < QPK; ++j) {
-      V qv = *reinterpret_cast<const V*>(reinterpret_cast<const T*>(a.q) + b * a.qBatchStride + (h + j) * a.qHeadStride + sub * N);
+      V qv = *reinterpret_cast<const V*>(reinterpret_cast<const T*>(a.q) + b * a.qBatchStride + (h + headOf(j)) * a.qHeadStride + sub * N);
       if constexpr (kPairs) {
         const u32x4 raw = __builtin_bit_cast(u32x4, qv);
 #pragma unroll
@@ -262,7 +268,7 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
         for (int j = 0; j < QPK; ++j)
           lg[j][u] = !okk[u] ? -INFINITY
                              : (useLds ? sbuf[j * kLdsScores + slotTok[u] - begin]
-                                       : static_cast<float>(scores[j * a.logitsHeadStride + slotTok[u]]) * kLog2eTA);
+                                       : static_cast<float>(scores[headOf(j) * a.logitsHeadStride + slotTok[u]]) * kLog2eTA);
       }
     }
   };
@@ -319,7 +325,7 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
           const int t = it + wave * UNR * TPI + (HIW ? 0 : grp) + u * TPI;
           if (sub == 0 && t < end) {
             if (useLds) sbuf[j * kLdsScores + t - begin] = sc[u];
-            else scores[j * a.logitsHeadStride + t] = static_cast<LT>(sc[u]);
+            else if (j < nq) scores[j * a.logitsHeadStride + t] = static_cast<LT>(sc[u]);
           }
         }
       } else if (mn != -INFINITY) {
@@ -362,8 +368,9 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
       __syncthreads();
 #pragma unroll
       for (int j = 0; j < QPK; ++j)
-        for (int i = threadIdx.x; i < end - begin; i += kTaWaves * 64)
-          scores[j * a.logitsHeadStride + begin + i] = static_cast<LT>(sbuf[j * kLdsScores + i]);
+        if (j < nq)
+          for (int i = threadIdx.x; i < end - begin; i += kTaWaves * 64)
+            scores[j * a.logitsHeadStride + begin + i] = static_cast<LT>(sbuf[j * kLdsScores + i]);
     }
     return;
   }
@@ -392,7 +399,7 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
       for (int e = 0; e < N; ++e) red[wave][rg][2 + sub * N + e] = acc[j][e];
     }
     __syncthreads();
-    if (wave == 0 && (HIW || grp == 0)) {
+    if (wave == 0 && (HIW || grp == 0) && j < nq) {
 #pragma unroll
       for (int w = 1; w < kTaWaves; ++w) {
         float acc2[N];
@@ -768,7 +775,7 @@ static diopiError_t fillArgs(const TaViews& t, bool needK, bool needV, int maxLe
   a->d = (int)q.shape[2];
   a->maxLen = maxLen;
   a->nsplit = 1;
-  a->logits = nullptr, a->logitsHeadStride = 0;
+  a->logits = nullptr, a->logitsHeadStride = 0, a->qGroups = 1;
   // at most kTaMaxSplit chunks per sequence; chunks stay a multiple of 64 tokens
   a->chunk = kTaChunk;
   if ((int64_t)maxLen > (int64_t)kTaChunk * kTaMaxSplit) a->chunk = (int)(ceilDiv(ceilDiv(maxLen, kTaMaxSplit), 64) * 64);
@@ -860,11 +867,13 @@ static diopiError_t streamChunks(diopiContextHandle_t ctx, hipStream_t stream, T
   // softmax states side by side in the lane group's registers; more sharers than that are dealt over several
   // workgroups that run on the same XCD. At batch 64 x (512..4096) tokens, 32 query heads on 8 K/V heads (every query
   // head used to read the rows for itself): fused 236 -> 157 us, scores 214 -> 74 us, second half 205 -> 106 us; 64
-  // query heads on 8: 405 -> 240 us fused. A sharing factor that is odd keeps the one-head-per-read form.
+  // query heads on 8: 405 -> 240 us fused. Sharing factors that are no multiple of four are dealt over the workgroups
+  // as evenly as they go (28 query heads on 4 K/V heads: 4 + 3 per K/V head).
   const int perKv = a.heads / a.kvHeads;
-  const int qpk = perKv % 4 == 0 ? 4 : (perKv % 2 == 0 ? 2 : 1);
+  const int qpk = perKv >= 3 ? 4 : perKv;  // 1, 2 or 4 query heads per read
+  a.qGroups = (perKv + qpk - 1) / qpk;
   const bool hiw = qpk == 1 && MODE == kTaFused && (bytes == 128 || bytes == 256 || bytes == 512) && a.heads % tpw == 0;
-  const int groupsPerSeq = qpk > 1 ? a.kvHeads * (perKv / qpk) : (hiw ? a.heads / tpw : a.heads);
+  const int groupsPerSeq = qpk > 1 ? a.kvHeads * a.qGroups : (hiw ? a.heads / tpw : a.heads);
   chooseChunk(&a, groupsPerSeq, batch, maxInputLen);
   a.nsplit = (int)std::max<int64_t>(1, ceilDiv(maxInputLen, a.chunk));
   AMD_CHECK(batch <= 65535 && a.nsplit <= 65535, "token attention: batch %ld / splits %d exceed the grid limits", (long)batch,

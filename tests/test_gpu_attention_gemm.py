@@ -553,7 +553,9 @@ def test_token_attention_len_one_and_gqa(ops, dev, heads, kvh):
     (64, 8, torch.bfloat16, 128, torch.int32),    # eight sharers: two workgroups of four per K/V head
     (8, 1, torch.float32, 64, torch.int32),       # one K/V head for all; fp32 rows take the unpacked arithmetic
     (8, 2, torch.float16, 256, torch.int32),      # 32 lanes per head row
-    (12, 4, torch.bfloat16, 128, torch.int32),    # three sharers: every query head reads the rows for itself
+    (12, 4, torch.bfloat16, 128, torch.int32),    # three sharers in a group with four places
+    (28, 4, torch.bfloat16, 128, torch.int64),    # seven sharers: a group of four and a group of three per K/V head
+    (10, 2, torch.float16, 128, torch.int32),     # five: three and two
 ])
 def test_token_attention_grouped_query_layouts(ops, dev, heads, kvh, dtype, d, idt):
     """Fused and two-call decode attention with fewer K/V heads than query heads, over sequences of 1 to 1500 tokens
