@@ -71,6 +71,7 @@ struct TaArgs {
   const void* logits;  // two-call form: scores [heads, total_tokens], row h at logits + h * logitsHeadStride (elements)
   int64_t logitsHeadStride;
   int qGroups;  // grouped-query layouts: workgroups that share the query heads of one K/V head between them
+  int batch;    // sequences (the grouped-query kernels decode a one-dimensional grid)
 };
 
 // Merge (m, l, acc) of another online-softmax stream into this one.
@@ -125,8 +126,8 @@ enum TaMode { kTaFused = 0, kTaLogitsOut = 1, kTaReduceV = 2 };
 
 // T: bf16_t / half_t (8 per 16 B) or float (4 per 16 B). LPT lanes cover one head row. LT: the type of the scores in
 // memory (the two-call modes). QPK: query heads that share this workgroup's K/V head and are all served from one read
-// of its rows (grouped-query layouts; 1 otherwise). With QPK > 1 blockIdx.x counts (group of QPK query heads, K/V
-// head) pairs, the K/V head fastest, so the groups of one K/V head run on the same XCD and find its rows in that L2.
+// of its rows (grouped-query layouts; 1 otherwise). With QPK > 1 the grid is one-dimensional and decoded so that the
+// workgroups that share a K/V head's rows run next to each other on one XCD.
 template <typename T, int LPT, bool HIW, int MODE = kTaFused, typename LT = float, int QPK = 1>
 __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* __restrict__ out,
                                                                      float* __restrict__ partial) {
@@ -146,17 +147,26 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   // (the last, partly filled chunk of every sequence and the chunks only long sequences have) is handed out first and
   // the launch ends on whole chunks that finish together. Against sequence-major order, batch 64 x (512..4096):
   // 410.7 -> 406.8 us; 32 x (100..8192): 332 -> 323; 256 x (1024..2048): 1040 -> 1025, and with 8 K/V heads 413 -> 361.
-  const int split = (int)gridDim.z - 1 - (int)blockIdx.z, b = blockIdx.y;
+  int split = (int)gridDim.z - 1 - (int)blockIdx.z, b = blockIdx.y;
   const int perKv = a.heads / a.kvHeads;
   int h, kvh, nq = 1;  // h: this lane group's (first) query head; nq: how many it serves (at most QPK)
   if constexpr (QPK == 1) {
     h = HIW ? blockIdx.x * TPW + grp : blockIdx.x;
     kvh = h / perKv;
   } else {
-    // the perKv sharers of a K/V head are dealt over qGroups workgroups as evenly as they go (7 = 4 + 3); a group
+    // One-dimensional grid. A unit is a (K/V head, sequence, chunk); its qGroups workgroups read the same rows, so they
+    // get consecutive places on one XCD (workgroup ids go round the 8 XCDs) and find the rows in that L2 after the
+    // first of them has fetched them. Units go round the XCDs in the order the three-dimensional grid has: K/V head
+    // fastest, then sequence, chunks from the last to the first.
+    const int f = blockIdx.x, idx = f >> 3;
+    const int g = idx % a.qGroups, u = (idx / a.qGroups) * 8 + (f & 7);
+    if (u >= a.kvHeads * a.batch * a.nsplit) return;  // the grid is rounded up to whole rounds of the XCDs
+    kvh = u % a.kvHeads;
+    const int rest = u / a.kvHeads;
+    b = rest % a.batch, split = a.nsplit - 1 - rest / a.batch;
+    // the perKv sharers of a K/V head are dealt over the qGroups workgroups as evenly as they go (7 = 4 + 3); a group
     // short of QPK heads computes its last head again in the spare places and stores nothing from them
-    kvh = blockIdx.x % a.kvHeads;
-    const int g = blockIdx.x / a.kvHeads, base = perKv / a.qGroups, rem = perKv % a.qGroups;
+    const int base = perKv / a.qGroups, rem = perKv % a.qGroups;
     h = kvh * perKv + g * base + min(g, rem);
     nq = base + (g < rem ? 1 : 0);
   }
@@ -775,7 +785,7 @@ static diopiError_t fillArgs(const TaViews& t, bool needK, bool needV, int maxLe
   a->d = (int)q.shape[2];
   a->maxLen = maxLen;
   a->nsplit = 1;
-  a->logits = nullptr, a->logitsHeadStride = 0, a->qGroups = 1;
+  a->logits = nullptr, a->logitsHeadStride = 0, a->qGroups = 1, a->batch = (int)q.shape[0];
   // at most kTaMaxSplit chunks per sequence; chunks stay a multiple of 64 tokens
   a->chunk = kTaChunk;
   if ((int64_t)maxLen > (int64_t)kTaChunk * kTaMaxSplit) a->chunk = (int)(ceilDiv(ceilDiv(maxLen, kTaMaxSplit), 64) * 64);
@@ -896,6 +906,11 @@ static diopiError_t streamChunks(diopiContextHandle_t ctx, hipStream_t stream, T
     }
   }
   dim3 grid((unsigned)groupsPerSeq, (unsigned)batch, a.nsplit), block(kTaWaves * 64);
+  if (qpk > 1) {
+    const int64_t units = (int64_t)a.kvHeads * batch * a.nsplit, wgs = ceilDiv(units, (int64_t)8) * 8 * a.qGroups;
+    AMD_CHECK(wgs < ((int64_t)1 << 31), "token attention: %ld workgroups exceed the grid limits", (long)wgs);
+    grid = dim3((unsigned)wgs, 1, 1);
+  }
 #define STREAM_CALL_AS(T, LPT, LT)                                                                                                   \
   if (qpk == 4) hipLaunchKernelGGL((decodeSplitKernel<T, LPT, false, MODE, LT, 4>), grid, block, 0, stream, a, static_cast<T*>(outPtr), partial); \
   else if (qpk == 2) hipLaunchKernelGGL((decodeSplitKernel<T, LPT, false, MODE, LT, 2>), grid, block, 0, stream, a, static_cast<T*>(outPtr), partial); \
