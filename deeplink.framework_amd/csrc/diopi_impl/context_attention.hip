@@ -420,10 +420,19 @@ __global__ __launch_bounds__(256, 2) void contextAttnMfmaKernel(CaArgs a, int nu
 template <typename T, int D>
 __global__ __launch_bounds__(256, 2) void contextAttnSingleBlockKernel(CaArgs a, int numQBlocks, int numSeq) {
   const int flat = (int)blockIdx.x;
-  const int xcd = flat & 7, idx = flat >> 3, perXcd = a.heads >> 3;  // the head count is a multiple of 8
-  const int hsPerXcd = perXcd * numSeq;
-  const int rank = idx / hsPerXcd, hs = idx - rank * hsPerXcd;
-  const int b = hs / perXcd, h = xcd * perXcd + (hs - b * perXcd);
+  int rank, b, h;
+  if ((a.heads & 7) == 0) {  // a contiguous eighth of every sequence's heads per XCD, as in the paired form
+    const int xcd = flat & 7, idx = flat >> 3, perXcd = a.heads >> 3;
+    const int hsPerXcd = perXcd * numSeq;
+    rank = idx / hsPerXcd;
+    const int hs = idx - rank * hsPerXcd;
+    b = hs / perXcd, h = xcd * perXcd + (hs - b * perXcd);
+  } else {
+    const int hb = a.heads * numSeq;
+    rank = flat / hb;
+    const int hs = flat - rank * hb;
+    b = hs / a.heads, h = hs - b * a.heads;
+  }
   contextAttnBlock<T, D>(a, numQBlocks - 1 - rank, h, b);
 }
 
@@ -487,7 +496,7 @@ static diopiError_t launchCaMfma(hipStream_t stream, const CaArgs& a, int maxLen
   const int64_t cus = computeUnits(), hb = (int64_t)a.heads * batch;
   const int64_t pairedLoad = ceilDiv(blocks, cus) * (numQBlocks + 1);
   const int64_t singleLoad = std::max<int64_t>(ceilDiv(hb * numQBlocks * (numQBlocks + 1) / 2, cus), numQBlocks);
-  if ((a.heads & 7) == 0 && numQBlocks > 1 && singleLoad * 11 < pairedLoad * 10 && hb * numQBlocks < ((int64_t)1 << 31)) {
+  if (numQBlocks > 1 && singleLoad * 11 < pairedLoad * 10 && hb * numQBlocks < ((int64_t)1 << 31)) {
     AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&contextAttnSingleBlockKernel<T, D>), (int)lds));
     hipLaunchKernelGGL((contextAttnSingleBlockKernel<T, D>), dim3((unsigned)(hb * numQBlocks)), dim3(256), lds, stream, a, numQBlocks,
                        (int)batch);

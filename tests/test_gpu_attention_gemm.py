@@ -452,7 +452,8 @@ def test_context_attention_long_ragged_batch_paired_blocks(ops, dev, heads, kvh,
 
 
 @pytest.mark.parametrize("heads,kvh,d,dtype,lens", [(32, 32, 128, torch.bfloat16, [512]), (8, 2, 128, torch.bfloat16, [1000]),
-                                                    (16, 4, 64, torch.float16, [700, 129, 5]), (8, 8, 128, torch.float16, [257, 256, 255, 1])])
+                                                    (16, 4, 64, torch.float16, [700, 129, 5]), (8, 8, 128, torch.float16, [257, 256, 255, 1]),
+                                                    (28, 4, 128, torch.bfloat16, [600]), (6, 3, 64, torch.bfloat16, [300, 1025])])
 def test_context_attention_one_query_block_per_workgroup(ops, dev, heads, kvh, d, dtype, lens):
     """Launches too small for the paired schedule to fill the chip evenly: every 128-query block is a workgroup of its
     own, heaviest first (a single short prompt; a few ragged sequences; block counts of 4, 8, 6 and 3)."""
