@@ -584,6 +584,13 @@ def test_token_attention_grouped_query_layouts(ops, dev, heads, kvh, dtype, d, i
     out2 = torch.empty_like(got)
     ops.token_softmax_reducev(att, vp.to(dev), out2, *args)
     chk(out2, want)
+    if dtype != torch.float32:   # scores kept in the 16-bit dtype between the two calls
+        att16 = torch.zeros(heads, total, dtype=dtype, device=dev)
+        ops.token_attention(q.to(dev), kp.to(dev), att16, *args)
+        assert_half(att16, oracle.token_logits(q, kp, b_loc, st, ln, width, total))
+        out3 = torch.empty_like(got)
+        ops.token_softmax_reducev(att16, vp.to(dev), out3, *args)
+        assert_half(out3, want, rel=3e-2, abs_=2e-2)   # softmax of scores rounded to 8 (11) bits
 
 
 # ------------------------------------------------------------------ int8 weight-only linear
