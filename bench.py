@@ -50,6 +50,8 @@ def parse():
     ap.add_argument("--gemm", metavar="M,N,K", help="profiling aid: time only diopiLinear on [M,K] x [N,K]^T (bf16 unless --gemm-dtype says otherwise) "
                     "(activations N(0,1), weights N(0,0.02)) for --steps launches and print one JSON line")
     ap.add_argument("--gemm-dtype", choices=["bf16", "fp16", "fp32"], default="bf16", help="with --gemm: the operand dtype")
+    ap.add_argument("--decode-attention", type=int, metavar="KV_HEADS", default=0, help="profiling aid: time only the fused decode "
+                    "attention of the paged workload (batch 64, 32 query heads x 128) on a pool with KV_HEADS K/V heads")
     ap.add_argument("--attention", action="store_true", help="profiling aid: time only the prefill attention of the "
                     "layer workload (batch 4 x seq 2048, 32 heads x 128, bf16) for --steps launches")
     return ap.parse_args()
@@ -589,6 +591,19 @@ def single_kernel(pkg, torch, dev, rt, stream, args):
         call = Prepared(pkg, "diopiLinear", out, a, w, None)
         label = f"diopiLinear {args.gemm_dtype} {m}x{n}x{k}"
         work, unit = 2.0 * m * n * k / 1e12, "TFLOP/s"
+    elif args.decode_attention:
+        kvh = args.decode_attention
+        pd = pkg.workloads.paged_decode(seed=0, fill_pool=False)
+        gdev = {k: (v.to(dev) if hasattr(v, "to") else v) for k, v in pd.items()}
+        kp, vp = gdev["k_pool"][:, :kvh], gdev["v_pool"][:, :kvh]   # views of the first KV_HEADS heads of every slot
+        gdev["k_pool"].normal_()
+        gdev["v_pool"].normal_()
+        out = torch.empty_like(gdev["q"])
+        call = Prepared(pkg, "diopiTokenDecodeAttentionInference", out, gdev["q"], kp, vp, gdev["b_loc"], gdev["b_start_loc"],
+                        gdev["b_seq_len"], int(gdev["max_input_len"]))
+        L = int(pd["b_seq_len"].sum())
+        work = (L * kvh * 128 * 2 * 2 + L * pd["b_loc"].element_size() + 2 * 64 * 32 * 128 * 2) / 1e12
+        unit, label = "TB/s", f"decode attention bf16 batch 64, 32 query heads on {kvh} K/V heads x 128, sum(len)={L}"
     else:
         b, s, h, hd = 4, 2048, 32, 128
         g = torch.Generator().manual_seed(0)
@@ -694,7 +709,7 @@ def main():
     dev = torch.device("cuda:0")
     rt = pkg.runtime
     stream = torch.cuda.current_stream().cuda_stream
-    if args.gemm or args.attention:
+    if args.gemm or args.attention or args.decode_attention:
         single_kernel(pkg, torch, dev, rt, stream, args)
         return
 
