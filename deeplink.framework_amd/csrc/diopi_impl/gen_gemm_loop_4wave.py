@@ -28,6 +28,9 @@ the power limit, where the cycles saved come back as a lower clock (1.59 against
 count when the clock is not what limits it.
 Fragment reads are issued in the order the MFMAs need them (B0, A0..A7, B1..B7; the MFMAs run B-major) and LDS
 returns them in order, so the wait before an MFMA is a count of younger reads that may still be outstanding.
+Within a k-step the A fragments are walked forth for even B fragments and back for odd ones, so consecutive MFMAs
+always share one operand (with A0..A7 restarted for every B, both operands change at each turn). At the power limit
+that is measurable: 8192 x 4096 x 12288 550.4 -> 545.9 us, x 22016 985.9 -> 978.2 us, same box, same results bit for bit.
 Measured and not used: K tiles of 32 in a four-stage ring (loads three tiles ahead) is 10 % slower, because a tile
 load then fetches 64-byte row pieces, twice the cache lines per byte; issuing the loads twice as densely (to gain
 slack) stalls the wave at issue. The same tile out of v_mfma_f32_32x32x16 (4 x 4 blocks per wave, four 16-wide k-steps,
@@ -106,10 +109,11 @@ def tile(out, s, loads, next_tile, next_output=False):
             after[65 + 3 * r].append(("read0", r))
     for m in range(128):
         ks, mm = divmod(m, 64)
-        j, i = divmod(mm, 8)
+        j, pos = divmod(mm, 8)
+        i = pos if j % 2 == 0 else 7 - pos                 # A fragments back and forth: one operand changes per MFMA
         if m == 0:
             out.append("s_waitcnt lgkmcnt(7)")             # B0, A0..A7 of buffer 0 (read during the previous k-step 1)
-        elif ks == 0 and i == 0 and j >= 1 and m <= B1_SLOT:
+        elif ks == 0 and pos == 0 and j >= 1 and m <= B1_SLOT:
             # B_j of buffer 0: 7 - j reads of its set are younger, and so are this tile's reads issued so far
             out.append(f"s_waitcnt lgkmcnt({min(7 - j + min(m, 16), 15)})")
         if m == 64 and next_tile:                          # B2; the last K tile has no successor to wait for
