@@ -303,7 +303,13 @@ struct MfmaOp16<half_t> {
 // multiplies K tiles [s * kTilesPerSplit, ...) and stores its fp32 accumulators to partial[s], to be summed and
 // given the linear epilogue by splitKReduceKernel; kEpiRotary is acc + bias followed by the interleaved rotary
 // embedding on the leading rotCols columns (the q and k heads of a stacked QKV projection).
-enum PipeEpilogue { kEpiLinear = 0, kEpiSiluMul = 1, kEpiPartial = 2, kEpiRotary = 3 };
+// kEpiRotaryUniform is kEpiRotary for the usual case, no bias and a rotated width that is a multiple of 32 columns:
+// whether a lane's 32-column piece is rotated is then the same for the whole wave. It is an instantiation of its own
+// because the one-wave-per-SIMD kernel has no register to spare for a second path next to the general one.
+// kEpiRotaryLds (4-wave kernel only) is kEpiRotaryUniform for 16-bit tables and heads of 128 columns with the table
+// entries of an output tile's first four fragment rows waiting in LDS when the epilogue starts (see rotaryTablesToLds).
+enum PipeEpilogue { kEpiLinear = 0, kEpiSiluMul = 1, kEpiPartial = 2, kEpiRotary = 3, kEpiRotaryUniform = 4, kEpiRotaryLds = 5 };
+constexpr int kRotaryLdsBytes = 32768;  // behind the two K-tile stages of the 4-wave kernel: 128 rows x (64 cos | 64 sin) x 2 bytes
 
 // The vector epilogue of the 256 x 256 kernels: a wave's TM x TN fragments of 16 x 16 (v_mfma_f32_16x16x32 with the
 // weight fragment first, so lane (frow = l & 15, kq = l >> 4) holds columns 4 kq .. 4 kq + 3 of row frow of every
@@ -321,9 +327,42 @@ enum PipeEpilogue { kEpiLinear = 0, kEpiSiluMul = 1, kEpiPartial = 2, kEpiRotary
 // piece also waits for every store before it, so the pieces of four fragment rows are requested
 // together before the first store of the four (one exposed round trip per four rows instead of one per
 // row), and without an addend there is no load (and no wait) in the stream.
+// The rotary epilogue's table entries are what it waits for: with the loads answered by constants the launch is as
+// long as a plain linear's, with them it was 26 - 37 us longer (8192 x 4096 x 12288; 15 - 21 us now), because a wave that asks for a
+// batch of entries has nothing else to do until L2 answers, and with one wave per SIMD nobody else has either. So the
+// workgroup copies the cosines and sines of the first four fragment rows of both row halves of its output tile
+// (2 x 64 rows of 64 entries each, 16 KiB + 16 KiB) straight into LDS before the last K tiles run: the copies are
+// over when the epilogue starts, and the entries of the other four rows are requested from memory at that point and
+// arrive while the first four are worked through. Wave w copies table rows 32 w .. 32 w + 31 of that region (row
+// r: row half r / 64, fragment row (r % 64) / 16, row in fragment r % 16): four copy instructions of 8 rows x 128
+// bytes for the cosines and four for the sines. The caller waits for its own copies and meets the other waves at a
+// barrier before the epilogue reads.
+template <typename T>
+__device__ __forceinline__ void rotaryTablesToLds(const MfmaArgs& g, int tileRow0, int wave, int lane, unsigned ldsTab) {
+  int tableRows = g.rotTableRows;
+  asm volatile("" : "+s"(tableRows));  // (a division by a run-time value: its set-up is not to be kept across the K loop)
+  const int64_t bytes = (int64_t)tableRows * 64 * (int64_t)sizeof(T);
+  auto descriptor = [&](const void* base) {
+    uint64_t p = reinterpret_cast<uint64_t>(base);
+    asm volatile("" : "+s"(p));  // built here, per call: eight scalar registers that must not stay live across the K loop
+    u32x4 d = {(uint32_t)p, (uint32_t)(p >> 32) & 0xffffu, (uint32_t)bytes, 0x00020000u};
+    return d;
+  };
+  const u32x4 rsCos = descriptor(g.rotCos), rsSin = descriptor(g.rotSin);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int r = wave * 32 + q * 8 + (lane >> 3);
+    const int row = tileRow0 + (r >> 6) * 128 + ((r >> 4) & 3) * 16 + (r & 15);
+    const int voff = row < g.M ? ((row % tableRows) * 64 + (lane & 7) * 8) * (int)sizeof(T) : (int)0x80000000u;
+    const unsigned to = ldsTab + (unsigned)(wave * 32 + q * 8) * 128u;
+    loadToLds16(rsCos, voff, 0, to);
+    loadToLds16(rsSin, voff, 0, to + 16384u);
+  }
+}
+
 template <typename T, int EPI, int TM, int TN, typename AccRow>
 __device__ __forceinline__ void vectorEpilogue(const MfmaArgs& g, T* out, const T* cin, const T* bias, int row0, int colBase,
-                                               int frow, int kq, AccRow&& accRow) {
+                                               int frow, int kq, AccRow&& accRow, unsigned ldsTab = 0) {
   using Frag = typename MfmaOp<T>::Frag;
   static_assert(TM % 4 == 0 && TN % 4 == 0, "rows are handled four at a time, columns in pairs of fragments");
   const int cperm = (kq & 1) * 16 + (kq >> 1) * 8;
@@ -371,7 +410,7 @@ __device__ __forceinline__ void vectorEpilogue(const MfmaArgs& g, T* out, const 
         put(i, hb, o);
       }
     });
-  } else if constexpr (EPI == kEpiRotary) {
+  } else if constexpr (EPI == kEpiRotary || EPI == kEpiRotaryUniform || EPI == kEpiRotaryLds) {
     // A lane's 8 consecutive columns are 4 adjacent pairs of one head; their angles are 4 consecutive table
     // entries of the lane's row. Pieces at or past rotCols (the v heads) pass through with cos = 1, sin = 0.
     // the two divisors are made opaque so that the set-up of the divisions by them is done here, per call, and not
@@ -406,6 +445,126 @@ __device__ __forceinline__ void vectorEpilogue(const MfmaArgs& g, T* out, const 
     float cs[4][TN / 2][4], sn[4][TN / 2][4];
     // a wave whose columns all lie at or past rotCols (v heads) asks for no table entries at all
     const bool anyRot = __builtin_amdgcn_readfirstlane(colBase) < g.rotCols;
+    if constexpr (EPI == kEpiRotaryLds) {
+      // Fragment rows 0 - 3 find their entries in LDS (rotaryTablesToLds); those of rows 4 - 7 are requested now, before
+      // anything is stored, and land while rows 0 - 3 are rotated and stored.
+      static_assert(TM == 8, "four fragment rows from LDS, four from memory");
+      bool rotU[TN / 2];
+#pragma unroll
+      for (int jp = 0; jp < TN / 2; ++jp) rotU[jp] = __builtin_amdgcn_readfirstlane(colBase) + jp * 32 < g.rotCols;
+      const float sign = g.rotSinSign;
+      u32x2 craw[4][TN / 2], sraw[4][TN / 2];
+      if (anyRot) {
+#pragma unroll
+        for (int i = 4; i < 8; ++i) {
+          const int row = row0 + i * 16 + frow;
+#pragma unroll
+          for (int jp = 0; jp < TN / 2; ++jp) {
+            if (!rotU[jp]) continue;
+            const int off = row < g.M ? ((row % tableRows) * half + pair0[jp]) * tsz : kOutside;
+            craw[i - 4][jp] = __builtin_amdgcn_raw_buffer_load_b64(rsCos, off, 0, 0);
+            sraw[i - 4][jp] = __builtin_amdgcn_raw_buffer_load_b64(rsSin, off, 0, 0);
+          }
+        }
+      }
+      typedef __attribute__((address_space(3))) const u32x2* LdsPair;
+      const unsigned tabRow = ldsTab + (unsigned)((((row0 >> 7) & 1) * 64 + frow) * 128);
+      staticFor<TM>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        f32x4 a[TN];
+        accRow(ic, a);
+#pragma unroll
+        for (int jp = 0; jp < TN / 2; ++jp) {
+          f32x4 x0 = a[2 * jp], x1 = a[2 * jp + 1];
+          swapPair(x0, x1);
+          const float v[8] = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+          Frag o;
+          if (rotU[jp]) {
+            u32x2 cr, sr;
+            if constexpr (i < 4) {
+              const unsigned at = tabRow + (unsigned)(i * 16 * 128 + pair0[jp] * 2);
+              cr = *(LdsPair)(uintptr_t)at;
+              sr = *(LdsPair)(uintptr_t)(at + 16384u);
+            } else {
+              cr = craw[i - 4][jp], sr = sraw[i - 4][jp];
+            }
+            typedef T T4 __attribute__((ext_vector_type(4)));
+            const T4 c4 = __builtin_bit_cast(T4, cr), s4 = __builtin_bit_cast(T4, sr);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float c = static_cast<float>(c4[e]), sv = static_cast<float>(s4[e]) * sign;
+              o[2 * e] = static_cast<T>(v[2 * e] * c - v[2 * e + 1] * sv);
+              o[2 * e + 1] = static_cast<T>(v[2 * e] * sv + v[2 * e + 1] * c);
+            }
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = static_cast<T>(v[e]);
+          }
+          put(i, jp, o);
+        }
+      });
+    } else if constexpr (EPI == kEpiRotaryUniform) {
+      // The choice per 32-column piece is a branch instead of selects in every lane, the pieces of the v heads are
+      // converted and stored like a plain linear's, no zero bias is added, and the sine's sign is applied once, where the
+      // table entries are converted: 52 vector instructions per 8 outputs become 36 for rotated pieces and 8 for the
+      // others. (No faster for that: what the rotary epilogue waits for is its table entries, see rotaryTablesToLds.)
+      bool rotU[TN / 2];
+#pragma unroll
+      for (int jp = 0; jp < TN / 2; ++jp) rotU[jp] = __builtin_amdgcn_readfirstlane(colBase) + jp * 32 < g.rotCols;
+      const float sign = g.rotSinSign;
+      auto fetchU = [&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        if (!anyRot) return;
+        const int row = row0 + i * 16 + frow;
+#pragma unroll
+        for (int jp = 0; jp < TN / 2; ++jp) {
+          if (!rotU[jp]) continue;
+          const int off = row < g.M ? ((row % tableRows) * half + pair0[jp]) * tsz : kOutside;
+          if (g.rotTableF32) {
+            const u32x4 c4 = __builtin_amdgcn_raw_buffer_load_b128(rsCos, off, 0, 0);
+            const u32x4 s4 = __builtin_amdgcn_raw_buffer_load_b128(rsSin, off, 0, 0);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) cs[i % 4][jp][e] = __uint_as_float(c4[e]), sn[i % 4][jp][e] = __uint_as_float(s4[e]) * sign;
+          } else {
+            typedef T T4 __attribute__((ext_vector_type(4)));
+            const T4 c4 = __builtin_bit_cast(T4, __builtin_amdgcn_raw_buffer_load_b64(rsCos, off, 0, 0));
+            const T4 s4 = __builtin_bit_cast(T4, __builtin_amdgcn_raw_buffer_load_b64(rsSin, off, 0, 0));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) cs[i % 4][jp][e] = static_cast<float>(c4[e]), sn[i % 4][jp][e] = static_cast<float>(s4[e]) * sign;
+          }
+        }
+      };
+      staticFor<TM>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        if constexpr (i % 4 == 0) {
+          fetchU(std::integral_constant<int, i>{});
+          fetchU(std::integral_constant<int, i + 1>{});
+          fetchU(std::integral_constant<int, i + 2>{});
+          fetchU(std::integral_constant<int, i + 3>{});
+        }
+        f32x4 a[TN];
+        accRow(ic, a);
+#pragma unroll
+        for (int jp = 0; jp < TN / 2; ++jp) {
+          f32x4 x0 = a[2 * jp], x1 = a[2 * jp + 1];
+          swapPair(x0, x1);
+          const float v[8] = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+          Frag o;
+          if (rotU[jp]) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float c = cs[i % 4][jp][e], sv = sn[i % 4][jp][e];
+              o[2 * e] = static_cast<T>(v[2 * e] * c - v[2 * e + 1] * sv);
+              o[2 * e + 1] = static_cast<T>(v[2 * e] * sv + v[2 * e + 1] * c);
+            }
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = static_cast<T>(v[e]);
+          }
+          put(i, jp, o);
+        }
+      });
+    } else {
     auto fetch = [&](auto ic) {
       constexpr int i = decltype(ic)::value;
       if (!anyRot) return;
@@ -454,6 +613,7 @@ __device__ __forceinline__ void vectorEpilogue(const MfmaArgs& g, T* out, const 
         put(i, jp, o);
       }
     });
+    }
   } else {
     float bv[TN / 2][8];
 #pragma unroll
@@ -820,7 +980,7 @@ __global__ __launch_bounds__(TILE == 256 ? kPipeThreads : 256, TILE == 256 ? 1 :
 // offsets, the epilogue's conversions and address arithmetic) must therefore fit the other 128 ordinary registers
 // and touch no accumulation register, and nothing may spill: a reload would also stall behind the tile loads in
 // flight. build.py compiles this file with the resource-usage remark and fails when any instantiation reports
-// scratch or spills; tests/test_gpu_attention_gemm.py runs every instantiation by name on exact inputs.
+// scratch or spilled vector registers; tests/test_gpu_attention_gemm.py runs every instantiation by name on exact inputs.
 #include "gemm_loop_4wave.inc"
 
 // Sixteen consecutive accumulation registers a[R .. R + 15] as four fragments, in one statement: the reads issue back
@@ -943,6 +1103,11 @@ __global__ __launch_bounds__(256) void gemmMfma4WaveKernel(MfmaArgs g) {
     else
       GEMM4W_RUN(PROLOGUE_LOADED);
     for (int p = 1; p < pairs; ++p) GEMM4W_RUN(BODY);
+    // (rotary tables through LDS: this output tile's entries are copied now, behind every tile load of its K loop; tiles
+    // of v heads need none; the decision is the same for the whole workgroup)
+    if constexpr (EPI == kEpiRotaryLds) {
+      if (tn * BN < g.rotCols) rotaryTablesToLds<T>(g, tm * BM, waveS, laneNow(), base + 131072u);
+    }
     const int next = pid + (int)gridDim.x;
     int ntm = 0, ntn = 0;
     if (next < total) {
@@ -952,6 +1117,14 @@ __global__ __launch_bounds__(256) void gemmMfma4WaveKernel(MfmaArgs g) {
       GEMM4W_RUN(TAIL_NEXT);
     } else {
       GEMM4W_RUN(TAIL);
+    }
+    if constexpr (EPI == kEpiRotaryLds) {
+      if (tn * BN < g.rotCols) {
+        // this wave's table copies are older than the 32 tile loads the tail issued for the next output tile (if any)
+        if (next < total) __builtin_amdgcn_s_waitcnt(0x0f70 | (32 & 15) | ((32 >> 4) << 14));
+        else __builtin_amdgcn_s_waitcnt(0x0f70);
+        __builtin_amdgcn_s_barrier();
+      }
     }
     // one fragment row at a time out of the accumulation registers, which the compiler does not know to be live:
     // the epilogue stays far below the 256 ordinary registers, so it never borrows them
@@ -966,7 +1139,7 @@ __global__ __launch_bounds__(256) void gemmMfma4WaveKernel(MfmaArgs g) {
       accRegisters16<32 * i + 16>(hi);
 #pragma unroll
       for (int j = 0; j < 4; ++j) row[j] = lo[j], row[4 + j] = hi[j];
-    });
+    }, base + 131072u);
     if (next >= total) break;
     pid = next, tm = ntm, tn = ntn, first = false;
   }
@@ -1976,11 +2149,13 @@ static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p
   g.vecEpilogue = p.N % 8 == 0 && p.sOm % 8 == 0 && p.sOb % 8 == 0 && al16(p.out) && span32 &&
                   (!p.Cin || (p.sCn == 1 && p.sCm % 8 == 0 && p.sCb % 8 == 0 && al16(p.Cin))) && (!p.bias || al16(p.bias));
   constexpr size_t lds = 2 * (size_t)(256 + 256) * kBK * sizeof(T);
-  AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmMfmaPipelinedKernel<T, EPI>), (int)lds));
+  if constexpr (EPI != kEpiRotaryLds) AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmMfmaPipelinedKernel<T, EPI>), (int)lds));
   g.partial = partial;
   g.kTilesPerSplit = kTilesPerSplit;
-  if (EPI == kEpiRotary) {
+  if (EPI == kEpiRotary || EPI == kEpiRotaryUniform || EPI == kEpiRotaryLds) {
     AMD_CHECK(rot && g.vecEpilogue && !p.Cin && p.alpha == 1.f, "rotary epilogue: needs tables, the vector epilogue and no addend");
+    if (EPI != kEpiRotary) AMD_CHECK(!p.bias && rot->cols % 32 == 0, "rotary epilogue: the uniform form takes no bias and whole 32-column pieces");
+    if (EPI == kEpiRotaryLds) AMD_CHECK(!rot->tableF32 && rot->headDim == 128, "rotary epilogue: tables through LDS are 16-bit, for heads of 128");
     g.rotCos = rot->cosT, g.rotSin = rot->sinT, g.rotCols = rot->cols, g.rotHeadDim = rot->headDim, g.rotTableRows = rot->tableRows;
     g.rotTableF32 = rot->tableF32, g.rotSinSign = rot->sinSign;
   }
@@ -1999,15 +2174,20 @@ static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p
   if constexpr (EPI != kEpiPartial) {
     // the 4-wave kernel: an even number of K tiles, 16-byte epilogue pieces, lane offsets that fit 31 bits
     if (g.vecEpilogue && p.K % (2 * kBK) == 0 && p.M * p.sAm * 2 < (int64_t(1) << 31) && p.N * p.sBn * 2 < (int64_t(1) << 31)) {
-      AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmMfma4WaveKernel<T, EPI>), (int)lds));
+      constexpr size_t lds4 = lds + (EPI == kEpiRotaryLds ? kRotaryLdsBytes : 0);  // (160 KiB with the rotary tables: all of a CU's)
+      AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmMfma4WaveKernel<T, EPI>), (int)lds4));
       // one workgroup per CU (its LDS ring takes most of a CU's), each walking its share of the tiles
       const int resident = computeUnits() / 8 * 8;
       if (resident >= 8 && (int)grid.x > resident) grid.x = (unsigned)resident;
-      hipLaunchKernelGGL((gemmMfma4WaveKernel<T, EPI>), grid, dim3(256), lds, stream, g);
+      hipLaunchKernelGGL((gemmMfma4WaveKernel<T, EPI>), grid, dim3(256), lds4, stream, g);
       AMD_LAUNCH_CHECK();
       return diopiSuccess;
     }
   }
+  if constexpr (EPI == kEpiRotaryLds) {
+    setLastError("rotary epilogue: the form with tables in LDS exists for the 4-wave kernel only");
+    return diopiErrorOccurred;
+  } else {
   hipLaunchKernelGGL((gemmMfmaPipelinedKernel<T, EPI>), grid, dim3(kPipeThreads), lds, stream, g);
   AMD_LAUNCH_CHECK();
   if (EPI == kEpiPartial) {
@@ -2016,6 +2196,7 @@ static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p
     AMD_LAUNCH_CHECK();
   }
   return diopiSuccess;
+  }
 }
 
 // The 128 x 128 form of the pipelined kernel (4 waves, two workgroups per CU): linear epilogue, or fp32 partial
@@ -2840,8 +3021,18 @@ GEMM_EXPORT diopiError_t diopiLinearRotary(diopiContextHandle_t ctx, diopiTensor
     RotaryEpilogue r;
     r.cosT = cc.data, r.sinT = cs.data, r.cols = (int)rotaryCols, r.headDim = (int)headDim, r.tableRows = (int)tableRows;
     r.tableF32 = cc.dtype == diopi_dtype_float32, r.sinSign = conj ? -1.f : 1.f;
-    AMD_TRY(p.dtype == diopi_dtype_bfloat16 ? (launchMfmaPipelined<bf16_t, kEpiRotary>(stream, p, nullptr, 1, 0, &r))
-                                            : (launchMfmaPipelined<half_t, kEpiRotary>(stream, p, nullptr, 1, 0, &r)));
+    // (what launchMfmaPipelined asks of a problem before it takes the 4-wave kernel, whose LDS has room for the tables)
+    const bool fourWave = k % (2 * kBK) == 0 && n % 8 == 0 && ptr16(p.out) && p.M * k * 2 < (int64_t(1) << 31) && n * k * 2 < (int64_t(1) << 31) &&
+                          (p.M - 1) * n * 2 + n * 2 < (int64_t(1) << 31);
+    if (!p.bias && r.cols % 32 == 0 && !r.tableF32 && r.headDim == 128 && fourWave)
+      AMD_TRY(p.dtype == diopi_dtype_bfloat16 ? (launchMfmaPipelined<bf16_t, kEpiRotaryLds>(stream, p, nullptr, 1, 0, &r))
+                                              : (launchMfmaPipelined<half_t, kEpiRotaryLds>(stream, p, nullptr, 1, 0, &r)));
+    else if (!p.bias && r.cols % 32 == 0)
+      AMD_TRY(p.dtype == diopi_dtype_bfloat16 ? (launchMfmaPipelined<bf16_t, kEpiRotaryUniform>(stream, p, nullptr, 1, 0, &r))
+                                              : (launchMfmaPipelined<half_t, kEpiRotaryUniform>(stream, p, nullptr, 1, 0, &r)));
+    else
+      AMD_TRY(p.dtype == diopi_dtype_bfloat16 ? (launchMfmaPipelined<bf16_t, kEpiRotary>(stream, p, nullptr, 1, 0, &r))
+                                              : (launchMfmaPipelined<half_t, kEpiRotary>(stream, p, nullptr, 1, 0, &r)));
   } else {
     // decode-sized: the weight-streaming kernel that stages both operands through LDS rotates its sums
     bool fused = false;

@@ -21,6 +21,9 @@ def test_scratch_guard_reads_the_resource_usage_remarks():
     spilled = clean.replace("ScratchSize [bytes/lane]: 0", "ScratchSize [bytes/lane]: 52").replace("VGPRs Spill: 0", "VGPRs Spill: 13")
     bad = b.scratch_users(spilled, ("gemmMfma4WaveKernel",))
     assert len(bad) == 2 and "ScratchSize" in bad[0] and "VGPRs Spill: 13" in bad[1]
+    # scalar registers parked in lanes of a vector register are not scratch
+    lanes = clean.replace("SGPRs Spill: 0", "SGPRs Spill: 2")
+    assert b.scratch_users(lanes, ("gemmMfma4WaveKernel",)) == []
     # another kernel's scratch is not this guard's business
     other = spilled.replace("gemmMfma4WaveKernel", "gemmFmaKernel")
     assert b.scratch_users(other, ("gemmMfma4WaveKernel",)) == []

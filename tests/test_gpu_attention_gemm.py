@@ -189,16 +189,21 @@ def test_second_operand_read_in_place_as_k_by_n(ops, dev, dtype, batch, m, k, n)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("epilogue", ["linear", "bias", "addend", "rotary", "silu_mul"])
+@pytest.mark.parametrize("epilogue", ["linear", "bias", "addend", "rotary", "rotary_bias", "rotary_conj", "rotary_f32_tables",
+                                      "rotary_ragged_rows", "silu_mul"])
 def test_four_wave_gemm_every_instantiation_exact(ops, dev, dtype, epilogue):
-    """Every instantiation of the 4-wave large-tile kernel (two dtypes x plain, bias, addend, rotary and gated
-    epilogues) by name, on a problem of 288 tiles of 256 x 256 so that every workgroup walks at least one tile after
+    """Every instantiation of the 4-wave large-tile kernel (two dtypes x plain, bias, addend, rotary without a bias and
+    with 16-bit tables (the form whose table entries wait in LDS; also with the conjugate rotation and with rows that
+    end inside the last tile), rotary with fp32 tables (the wave-uniform form), rotary with a bias (the general form)
+    and gated epilogues) by name, on a problem of 288 tiles of 256 x 256 so that every workgroup walks at least one tile after
     its first (the path that requests the next tile's operands before the epilogue) and K = 256 (a prologue, one loop
     body and the tail). The kernel keeps its accumulators and operand fragments in registers the compiler only knows
     as clobbered: a change of register allocation around the loop would show here. Activations are one-hot rows, so
     every product is one weight element and the expected result is exact."""
     g0 = g(77)
     m, n, k = 8192, 2304, 256
+    if epilogue == "rotary_ragged_rows":
+        m -= 64                                         # 31 whole tile rows and 192 rows of the last one
     cols = torch.randint(0, k, (m,), generator=g0)
     x = torch.zeros(m, k, dtype=dtype)
     x[torch.arange(m), cols] = 1
@@ -224,12 +229,18 @@ def test_four_wave_gemm_every_instantiation_exact(ops, dev, dtype, epilogue):
         hd, rows = 128, 64
         e = torch.randint(-3, 1, (rows, hd // 2), generator=g0).float()
         sg = torch.randint(0, 2, (rows, hd // 2), generator=g0).float() * 2 - 1
-        cos, sin = (2.0 ** e).to(dtype), (sg * 2.0 ** (e - 1)).to(dtype)
+        tdt = torch.float32 if epilogue == "rotary_f32_tables" else dtype
+        cos, sin = (2.0 ** e).to(tdt), (sg * 2.0 ** (e - 1)).to(tdt)
         rot = n - 2 * hd                                # the last two heads pass through, like v
-        got = ops.linear_rotary(x.to(dev), w.to(dev), cos.to(dev), sin.to(dev), rot, hd, interleaved=True)
+        conj = epilogue == "rotary_conj"
+        b = (torch.randint(-4, 5, (n,), generator=g0).float() / 4).to(dtype) if epilogue == "rotary_bias" else None
+        got = ops.linear_rotary(x.to(dev), w.to(dev), cos.to(dev), sin.to(dev), rot, hd, None if b is None else b.to(dev),
+                                conj=conj, interleaved=True)
+        if b is not None:
+            sel = sel + b.float()                       # quarters added to 8- or 11-bit values: exact in fp32
         v = sel.clone().reshape(m, n // hd, hd // 2, 2)
         cf = cos.float()[torch.arange(m) % rows][:, None, :]
-        sf = sin.float()[torch.arange(m) % rows][:, None, :]
+        sf = sin.float()[torch.arange(m) % rows][:, None, :] * (-1.0 if conj else 1.0)
         out = torch.stack([v[..., 0] * cf - v[..., 1] * sf, v[..., 0] * sf + v[..., 1] * cf], dim=-1)
         out[:, rot // hd:] = v[:, rot // hd:]
         assert_exact(got, out.reshape(m, n).to(dtype))
