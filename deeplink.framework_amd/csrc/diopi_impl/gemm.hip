@@ -308,7 +308,10 @@ struct MfmaOp16<half_t> {
 // because the one-wave-per-SIMD kernel has no register to spare for a second path next to the general one.
 // kEpiRotaryLds (4-wave kernel only) is kEpiRotaryUniform for 16-bit tables and heads of 128 columns with the table
 // entries of an output tile's first four fragment rows waiting in LDS when the epilogue starts (see rotaryTablesToLds).
-enum PipeEpilogue { kEpiLinear = 0, kEpiSiluMul = 1, kEpiPartial = 2, kEpiRotary = 3, kEpiRotaryUniform = 4, kEpiRotaryLds = 5 };
+// kEpiAddendLds (4-wave kernel only) is kEpiLinear with an addend whose pieces for an output tile's first two fragment
+// rows wait in LDS when the epilogue starts (see addendToLds).
+enum PipeEpilogue { kEpiLinear = 0, kEpiSiluMul = 1, kEpiPartial = 2, kEpiRotary = 3, kEpiRotaryUniform = 4, kEpiRotaryLds = 5, kEpiAddendLds = 6 };
+constexpr int kAddendLdsBytes = 32768;  // behind the two K-tile stages of the 4-wave kernel: 4 waves x 32 rows x 128 columns x 2 bytes
 constexpr int kRotaryLdsBytes = 32768;  // behind the two K-tile stages of the 4-wave kernel: 128 rows x (64 cos | 64 sin) x 2 bytes
 
 // The vector epilogue of the 256 x 256 kernels: a wave's TM x TN fragments of 16 x 16 (v_mfma_f32_16x16x32 with the
@@ -357,6 +360,29 @@ __device__ __forceinline__ void rotaryTablesToLds(const MfmaArgs& g, int tileRow
     const unsigned to = ldsTab + (unsigned)(wave * 32 + q * 8) * 128u;
     loadToLds16(rsCos, voff, 0, to);
     loadToLds16(rsSin, voff, 0, to + 16384u);
+  }
+}
+
+// The addend of the linear epilogue is waited for in the same way: a wave that asks for the pieces of four fragment
+// rows has nothing to do until they arrive, twice per output tile. The 32 KiB behind the K-tile stages hold a quarter
+// of a tile's addend, so every wave copies the addend of its own first two fragment rows (32 rows of 128 columns,
+// 8 KiB) there before the last K tiles run, asks for the other six rows' pieces when the epilogue starts and works
+// through the two rows in LDS while those are on their way: one shortened wait per tile instead of two whole ones.
+// A copy instruction takes 4 rows of 256 bytes; the 16-byte piece p of local row r lies in slot p ^ (r & 15) of its
+// row (the swizzle is applied to the global address), so that the 16 lanes which read one piece index of 16
+// consecutive rows touch every bank once. A wave reads only what it copied itself: it waits for its own copies, and
+// no barrier is needed.
+template <typename T>
+__device__ __forceinline__ void addendToLds(const MfmaArgs& g, const T* cin, int waveRow0, int waveCol0, int lane, unsigned ldsDst) {
+  uint64_t p = reinterpret_cast<uint64_t>(cin);
+  asm volatile("" : "+s"(p));  // the descriptor is built here, per call: its registers must not stay live across the K loop
+  const u32x4 rsC = {(uint32_t)p, (uint32_t)(p >> 32) & 0xffffu, (uint32_t)(((int64_t)(g.M - 1) * g.sCm + g.N) * (int64_t)sizeof(T)), 0x00020000u};
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    const int r = q * 4 + (lane >> 4);
+    const int row = waveRow0 + r, col = waveCol0 + (((lane & 15) ^ (r & 15)) << 3);
+    const int voff = row < g.M && col < g.N ? (int)(((int64_t)row * g.sCm + col) * (int64_t)sizeof(T)) : (int)0x80000000u;
+    loadToLds16(rsC, voff, 0, ldsDst + (unsigned)q * 1024u);
   }
 }
 
@@ -614,6 +640,57 @@ __device__ __forceinline__ void vectorEpilogue(const MfmaArgs& g, T* out, const 
       }
     });
     }
+  } else if constexpr (EPI == kEpiAddendLds) {
+    // ldsTab is this wave's own 8 KiB: the addend of fragment rows 0 and 1 (addendToLds). The pieces of rows 2 - 7 are
+    // requested now, before anything is stored, and land while rows 0 and 1 are worked through.
+    static_assert(TM == 8 && TN == 8, "two fragment rows from LDS, six from memory, 128 columns per wave");
+    float zero = 0.f;  // (produced here: a zero kept from before the K loop would occupy a register across it)
+    asm volatile("" : "+v"(zero));
+    float bv[TN / 2][8];
+#pragma unroll
+    for (int jp = 0; jp < TN / 2; ++jp) {
+      const int col = min(col0 + jp * 32, g.N - 8);
+      Frag b8;
+      if (bias) b8 = *reinterpret_cast<const Frag*>(bias + col);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) bv[jp][e] = bias ? static_cast<float>(b8[e]) : zero;
+    }
+    const __amdgpu_buffer_rsrc_t rsC = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<T*>(cin), 0, (int)(((int64_t)(g.M - 1) * g.sCm + g.N) * sizeof(T)), 0x00020000);
+    u32x4 cv[TM - 2][TN / 2];
+#pragma unroll
+    for (int i = 2; i < TM; ++i) {
+#pragma unroll
+      for (int jp = 0; jp < TN / 2; ++jp) cv[i - 2][jp] = __builtin_amdgcn_raw_buffer_load_b128(rsC, offsetOf(i, jp, g.sCm), 0, 0);
+    }
+    typedef __attribute__((address_space(3))) const u32x4* LdsQuad;
+    const unsigned ldsRow = ldsTab + (unsigned)frow * 256u;
+    const int piece0 = (kq & 1) * 2 + (kq >> 1);  // this lane's 8 columns of a 32-column pair, as a piece index
+    staticFor<TM>([&](auto ic) {
+      constexpr int i = decltype(ic)::value;
+      f32x4 a[TN];
+      accRow(ic, a);
+#pragma unroll
+      for (int jp = 0; jp < TN / 2; ++jp) {
+        f32x4 x0 = a[2 * jp], x1 = a[2 * jp + 1];
+        swapPair(x0, x1);
+        const float v[8] = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+        u32x4 craw;
+        if constexpr (i < 2)
+          craw = *(LdsQuad)(uintptr_t)(ldsRow + (unsigned)(i * 16 * 256) + (unsigned)(((piece0 + 4 * jp) ^ frow) << 4));
+        else
+          craw = cv[i - 2][jp];
+        const Frag c8 = __builtin_bit_cast(Frag, craw);
+        Frag o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float x = v[e] * g.alpha + bv[jp][e];
+          x += g.beta * static_cast<float>(c8[e]);
+          o[e] = static_cast<T>(x);
+        }
+        put(i, jp, o);
+      }
+    });
   } else {
     float bv[TN / 2][8];
 #pragma unroll
@@ -1108,6 +1185,9 @@ __global__ __launch_bounds__(256) void gemmMfma4WaveKernel(MfmaArgs g) {
     if constexpr (EPI == kEpiRotaryLds) {
       if (tn * BN < g.rotCols) rotaryTablesToLds<T>(g, tm * BM, waveS, laneNow(), base + 131072u);
     }
+    // (addend through LDS: every wave copies the addend of its own first two fragment rows, likewise behind the tile loads)
+    if constexpr (EPI == kEpiAddendLds)
+      addendToLds<T>(g, cin, tm * BM + (waveS >> 1) * WM, tn * BN + (waveS & 1) * WN, laneNow(), base + 131072u + (unsigned)waveS * 8192u);
     const int next = pid + (int)gridDim.x;
     int ntm = 0, ntn = 0;
     if (next < total) {
@@ -1126,6 +1206,11 @@ __global__ __launch_bounds__(256) void gemmMfma4WaveKernel(MfmaArgs g) {
         __builtin_amdgcn_s_barrier();
       }
     }
+    if constexpr (EPI == kEpiAddendLds) {
+      // (a wave reads back only its own copies: no barrier)
+      if (next < total) __builtin_amdgcn_s_waitcnt(0x0f70 | (32 & 15) | ((32 >> 4) << 14));
+      else __builtin_amdgcn_s_waitcnt(0x0f70);
+    }
     // one fragment row at a time out of the accumulation registers, which the compiler does not know to be live:
     // the epilogue stays far below the 256 ordinary registers, so it never borrows them
     // The lane's position is asked for again here: otherwise every lane-dependent value of the epilogue that does not
@@ -1139,7 +1224,7 @@ __global__ __launch_bounds__(256) void gemmMfma4WaveKernel(MfmaArgs g) {
       accRegisters16<32 * i + 16>(hi);
 #pragma unroll
       for (int j = 0; j < 4; ++j) row[j] = lo[j], row[4 + j] = hi[j];
-    }, base + 131072u);
+    }, base + 131072u + (EPI == kEpiAddendLds ? (unsigned)waveS * 8192u : 0u));
     if (next >= total) break;
     pid = next, tm = ntm, tn = ntn, first = false;
   }
@@ -2174,11 +2259,21 @@ static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p
   if constexpr (EPI != kEpiPartial) {
     // the 4-wave kernel: an even number of K tiles, 16-byte epilogue pieces, lane offsets that fit 31 bits
     if (g.vecEpilogue && p.K % (2 * kBK) == 0 && p.M * p.sAm * 2 < (int64_t(1) << 31) && p.N * p.sBn * 2 < (int64_t(1) << 31)) {
-      constexpr size_t lds4 = lds + (EPI == kEpiRotaryLds ? kRotaryLdsBytes : 0);  // (160 KiB with the rotary tables: all of a CU's)
-      AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmMfma4WaveKernel<T, EPI>), (int)lds4));
       // one workgroup per CU (its LDS ring takes most of a CU's), each walking its share of the tiles
       const int resident = computeUnits() / 8 * 8;
       if (resident >= 8 && (int)grid.x > resident) grid.x = (unsigned)resident;
+      if constexpr (EPI == kEpiLinear) {
+        if (p.Cin) {
+          // with an addend: the form that finds a quarter of each tile's addend in LDS (160 KiB: all of a CU's)
+          constexpr size_t ldsAddend = lds + kAddendLdsBytes;
+          AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmMfma4WaveKernel<T, kEpiAddendLds>), (int)ldsAddend));
+          hipLaunchKernelGGL((gemmMfma4WaveKernel<T, kEpiAddendLds>), grid, dim3(256), ldsAddend, stream, g);
+          AMD_LAUNCH_CHECK();
+          return diopiSuccess;
+        }
+      }
+      constexpr size_t lds4 = lds + (EPI == kEpiRotaryLds ? kRotaryLdsBytes : 0);  // (160 KiB with the rotary tables: all of a CU's)
+      AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmMfma4WaveKernel<T, EPI>), (int)lds4));
       hipLaunchKernelGGL((gemmMfma4WaveKernel<T, EPI>), grid, dim3(256), lds4, stream, g);
       AMD_LAUNCH_CHECK();
       return diopiSuccess;

@@ -189,10 +189,12 @@ def test_second_operand_read_in_place_as_k_by_n(ops, dev, dtype, batch, m, k, n)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("epilogue", ["linear", "bias", "addend", "rotary", "rotary_bias", "rotary_conj", "rotary_f32_tables",
-                                      "rotary_ragged_rows", "silu_mul"])
+@pytest.mark.parametrize("epilogue", ["linear", "bias", "addend", "addend_ragged", "addend_in_place_scaled", "rotary", "rotary_bias",
+                                      "rotary_conj", "rotary_f32_tables", "rotary_ragged_rows", "silu_mul"])
 def test_four_wave_gemm_every_instantiation_exact(ops, dev, dtype, epilogue):
-    """Every instantiation of the 4-wave large-tile kernel (two dtypes x plain, bias, addend, rotary without a bias and
+    """Every instantiation of the 4-wave large-tile kernel (two dtypes x plain, bias, addend (the form that finds a quarter of
+    each tile's addend in LDS; also with rows and columns that end inside the last tiles and an addend with a longer row
+    pitch, and with the output written over the addend under alpha and beta), rotary without a bias and
     with 16-bit tables (the form whose table entries wait in LDS; also with the conjugate rotation and with rows that
     end inside the last tile), rotary with fp32 tables (the wave-uniform form), rotary with a bias (the general form)
     and gated epilogues) by name, on a problem of 288 tiles of 256 x 256 so that every workgroup walks at least one tile after
@@ -202,8 +204,10 @@ def test_four_wave_gemm_every_instantiation_exact(ops, dev, dtype, epilogue):
     every product is one weight element and the expected result is exact."""
     g0 = g(77)
     m, n, k = 8192, 2304, 256
-    if epilogue == "rotary_ragged_rows":
+    if epilogue in ("rotary_ragged_rows", "addend_ragged"):
         m -= 64                                         # 31 whole tile rows and 192 rows of the last one
+    if epilogue == "addend_ragged":
+        n -= 40                                         # 8 whole tile columns and 216 columns of the last one
     cols = torch.randint(0, k, (m,), generator=g0)
     x = torch.zeros(m, k, dtype=dtype)
     x[torch.arange(m), cols] = 1
@@ -224,6 +228,16 @@ def test_four_wave_gemm_every_instantiation_exact(ops, dev, dtype, epilogue):
     elif epilogue == "addend":
         c = torch.randn(m, n, generator=g0).to(dtype)
         assert_exact(ops.addmm(c.to(dev), x.to(dev), w.to(dev).t()), (c.float() + sel).to(dtype))
+    elif epilogue == "addend_ragged":
+        wide = torch.randn(m, n + 24, generator=g0).to(dtype)      # the addend is a column slice: its rows are 24 elements apart
+        got = ops.addmm(wide.to(dev)[:, 8:8 + n], x.to(dev), w.to(dev).t())
+        assert_exact(got, (wide[:, 8:8 + n].float() + sel).to(dtype))
+    elif epilogue == "addend_in_place_scaled":
+        c = torch.randn(m, n, generator=g0).to(dtype)
+        dc = c.to(dev)
+        got = ops.addmm(dc, x.to(dev), w.to(dev).t(), beta=0.5, alpha=2, out=dc)     # powers of two: still one rounding
+        assert got.data_ptr() == dc.data_ptr()
+        assert_exact(got, (0.5 * c.float() + 2 * sel).to(dtype))
     else:
         # tables of signed powers of two: each rotated value is a sum of two exactly scaled terms, rounded once
         hd, rows = 128, 64
