@@ -189,12 +189,12 @@ def test_second_operand_read_in_place_as_k_by_n(ops, dev, dtype, batch, m, k, n)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("epilogue", ["linear", "bias", "addend", "addend_ragged", "addend_in_place_scaled", "rotary", "rotary_bias",
-                                      "rotary_conj", "rotary_f32_tables", "rotary_ragged_rows", "silu_mul"])
+@pytest.mark.parametrize("epilogue", ["linear", "bias", "addend", "addend_ragged", "addend_in_place_scaled", "addend_batched", "rotary",
+                                      "rotary_bias", "rotary_conj", "rotary_f32_tables", "rotary_ragged_rows", "silu_mul"])
 def test_four_wave_gemm_every_instantiation_exact(ops, dev, dtype, epilogue):
     """Every instantiation of the 4-wave large-tile kernel (two dtypes x plain, bias, addend (the form that finds a quarter of
     each tile's addend in LDS; also with rows and columns that end inside the last tiles and an addend with a longer row
-    pitch, and with the output written over the addend under alpha and beta), rotary without a bias and
+    pitch, with the output written over the addend under alpha and beta, and batched), rotary without a bias and
     with 16-bit tables (the form whose table entries wait in LDS; also with the conjugate rotation and with rows that
     end inside the last tile), rotary with fp32 tables (the wave-uniform form), rotary with a bias (the general form)
     and gated epilogues) by name, on a problem of 288 tiles of 256 x 256 so that every workgroup walks at least one tile after
@@ -232,6 +232,13 @@ def test_four_wave_gemm_every_instantiation_exact(ops, dev, dtype, epilogue):
         wide = torch.randn(m, n + 24, generator=g0).to(dtype)      # the addend is a column slice: its rows are 24 elements apart
         got = ops.addmm(wide.to(dev)[:, 8:8 + n], x.to(dev), w.to(dev).t())
         assert_exact(got, (wide[:, 8:8 + n].float() + sel).to(dtype))
+    elif epilogue == "addend_batched":
+        # two batches of the same problem through baddbmm: the addend and the output of batch 1 lie a batch stride further on
+        c = torch.randn(2, m, n, generator=g0).to(dtype)
+        x2 = torch.stack([x, x.flip(0)])
+        sel2 = torch.stack([sel, sel.flip(0)])
+        got = ops.baddbmm(c.to(dev), x2.to(dev), w.to(dev).t().unsqueeze(0).expand(2, k, n))
+        assert_exact(got, (c.float() + sel2).to(dtype))
     elif epilogue == "addend_in_place_scaled":
         c = torch.randn(m, n, generator=g0).to(dtype)
         dc = c.to(dev)
