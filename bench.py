@@ -399,25 +399,31 @@ def decode_layer_step(pkg, torch, dev, rt, stream, g):
     want = out.clone()
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        # Recording may not allocate device memory, so the capture stream's workspace cache is filled first: passes
-        # that hold all their workspace, like the recording will, until one finds everything in the cache (the pass
-        # after it starts from the same cache and makes the same choices).
-        for _ in range(6):
-            before = pkg.runtime.cachingStats()["num_device_malloc"]
-            warm = calls(True)
-            for c in warm:
+
+    def record(layers):
+        """The step's calls recorded `layers` times over into one graph (a model records all its layers into one)."""
+        with torch.cuda.stream(side):
+            # Recording may not allocate device memory, so the capture stream's workspace cache is filled first: passes
+            # that hold all their workspace, like the recording will, until one finds everything in the cache (the pass
+            # after it starts from the same cache and makes the same choices).
+            for _ in range(6):
+                before = pkg.runtime.cachingStats()["num_device_malloc"]
+                warm = [c for _ in range(layers) for c in calls(True)]
+                for c in warm:
+                    c()
+                side.synchronize()
+                for c in warm:
+                    c.close()
+                if pkg.runtime.cachingStats()["num_device_malloc"] == before:
+                    break
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            recorded = [c for _ in range(layers) for c in calls(True)]
+            for c in recorded:
                 c()
-            side.synchronize()
-            for c in warm:
-                c.close()
-            if pkg.runtime.cachingStats()["num_device_malloc"] == before:
-                break
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph, stream=side):
-        recorded = calls(True)
-        for c in recorded:
-            c()
+        return graph, recorded
+
+    graph, recorded = record(1)
     out.zero_()
     (t_graph,) = time_ops(rt, stream, [graph.replay], 30, 6)
     torch.cuda.synchronize()
@@ -425,8 +431,20 @@ def decode_layer_step(pkg, torch, dev, rt, stream, g):
     del graph
     for c in recorded:
         c.close()
+    # hipGraphLaunch itself takes a few microseconds between two replays, which a one-layer graph pays per layer and a
+    # model's graph once per step: the same eight calls recorded eight times over, per layer
+    layers = 8
+    graph, recorded = record(layers)
+    out.zero_()
+    (t_deep,) = time_ops(rt, stream, [graph.replay], 8, 3)
+    torch.cuda.synchronize()
+    same = same and bool(torch.equal(out, want))
+    del graph
+    for c in recorded:
+        c.close()
     return {"op": "decode layer step, 8 DIOPI calls", "workload": "7B-shaped layer, batch 64, paged KV as above",
             "us_eager_launches": round(t_eager, 2), "us_hip_graph_replay": round(t_graph, 2),
+            "us_per_layer_in_a_graph_of_8_layers": round(t_deep / layers, 2),
             "tokens_per_s_graph": round(B / (t_graph * 1e-6), 1), "replay_equals_eager": same}
 
 
