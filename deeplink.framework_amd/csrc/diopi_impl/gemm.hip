@@ -90,6 +90,8 @@ struct MfmaArgs {
   int rotCols = 0, rotHeadDim = 0, rotTableRows = 1;
   bool rotTableF32 = false;
   float rotSinSign = 1.f;
+  const void* colScale = nullptr;  // kEpiColScale: N values of dtype colScaleDtype
+  int colScaleDtype = 0;
 };
 
 constexpr int kBK = 64;  // K elements per LDS tile (128-byte rows)
@@ -308,9 +310,11 @@ struct MfmaOp16<half_t> {
 // because the one-wave-per-SIMD kernel has no register to spare for a second path next to the general one.
 // kEpiRotaryLds (4-wave kernel only) is kEpiRotaryUniform for 16-bit tables and heads of 128 columns with the table
 // entries of an output tile's first four fragment rows waiting in LDS when the epilogue starts (see rotaryTablesToLds).
+// kEpiColScale (4-wave kernel only): out = alpha * sum * colScale[column], no addend, no bias (int8 weights expanded to
+// the activation type, the channel scale applied to the fp32 sum).
 // kEpiAddendLds (4-wave kernel only) is kEpiLinear with an addend whose pieces for an output tile's first two fragment
 // rows wait in LDS when the epilogue starts (see addendToLds).
-enum PipeEpilogue { kEpiLinear = 0, kEpiSiluMul = 1, kEpiPartial = 2, kEpiRotary = 3, kEpiRotaryUniform = 4, kEpiRotaryLds = 5, kEpiAddendLds = 6 };
+enum PipeEpilogue { kEpiLinear = 0, kEpiSiluMul = 1, kEpiPartial = 2, kEpiRotary = 3, kEpiRotaryUniform = 4, kEpiRotaryLds = 5, kEpiAddendLds = 6, kEpiColScale = 7 };
 constexpr int kAddendLdsBytes = 32768;  // behind the two K-tile stages of the 4-wave kernel: 4 waves x 32 rows x 128 columns x 2 bytes
 constexpr int kRotaryLdsBytes = 32768;  // behind the two K-tile stages of the 4-wave kernel: 128 rows x (64 cos | 64 sin) x 2 bytes
 
@@ -640,6 +644,29 @@ __device__ __forceinline__ void vectorEpilogue(const MfmaArgs& g, T* out, const 
       }
     });
     }
+  } else if constexpr (EPI == kEpiColScale) {
+    float sv[TN / 2][8];
+#pragma unroll
+    for (int jp = 0; jp < TN / 2; ++jp) {
+      const int col = min(col0 + jp * 32, g.N - 8);  // N % 8 == 0 here; a clamped piece is never stored
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sv[jp][e] = loadAs<float>(g.colScale, col + e, g.colScaleDtype) * g.alpha;
+    }
+    staticFor<TM>([&](auto ic) {
+      constexpr int i = decltype(ic)::value;
+      f32x4 a[TN];
+      accRow(ic, a);
+#pragma unroll
+      for (int jp = 0; jp < TN / 2; ++jp) {
+        f32x4 x0 = a[2 * jp], x1 = a[2 * jp + 1];
+        swapPair(x0, x1);
+        const float v[8] = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+        Frag o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = static_cast<T>(v[e] * sv[jp][e]);
+        put(i, jp, o);
+      }
+    });
   } else if constexpr (EPI == kEpiAddendLds) {
     // ldsTab is this wave's own 8 KiB: the addend of fragment rows 0 and 1 (addendToLds). The pieces of rows 2 - 7 are
     // requested now, before anything is stored, and land while rows 0 and 1 are worked through.
@@ -2227,6 +2254,7 @@ static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p
   g.M = (int)p.M, g.N = (int)p.N, g.K = (int)p.K;
   g.tilesM = (int)ceilDiv(p.M, 256), g.tilesN = (int)ceilDiv(p.N, 256);
   g.alpha = p.alpha, g.beta = p.beta;
+  g.colScale = p.colScale, g.colScaleDtype = (int)p.colScaleDtype;
   auto al16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
   // the vector epilogue addresses one batch of the output and of the addend with 32-bit byte offsets
   const bool span32 = ((p.M - 1) * p.sOm + p.N) * (int64_t)sizeof(T) < (int64_t(1) << 31) &&
@@ -2234,7 +2262,8 @@ static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p
   g.vecEpilogue = p.N % 8 == 0 && p.sOm % 8 == 0 && p.sOb % 8 == 0 && al16(p.out) && span32 &&
                   (!p.Cin || (p.sCn == 1 && p.sCm % 8 == 0 && p.sCb % 8 == 0 && al16(p.Cin))) && (!p.bias || al16(p.bias));
   constexpr size_t lds = 2 * (size_t)(256 + 256) * kBK * sizeof(T);
-  if constexpr (EPI != kEpiRotaryLds) AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmMfmaPipelinedKernel<T, EPI>), (int)lds));
+  if constexpr (EPI != kEpiRotaryLds && EPI != kEpiColScale) AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&gemmMfmaPipelinedKernel<T, EPI>), (int)lds));
+  if (EPI == kEpiColScale) AMD_CHECK(p.colScale && g.vecEpilogue && !p.Cin && !p.bias, "column scale epilogue: needs the scale, the vector epilogue and neither addend nor bias");
   g.partial = partial;
   g.kTilesPerSplit = kTilesPerSplit;
   if (EPI == kEpiRotary || EPI == kEpiRotaryUniform || EPI == kEpiRotaryLds) {
@@ -2281,6 +2310,9 @@ static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p
   }
   if constexpr (EPI == kEpiRotaryLds) {
     setLastError("rotary epilogue: the form with tables in LDS exists for the 4-wave kernel only");
+    return diopiErrorOccurred;
+  } else if constexpr (EPI == kEpiColScale) {
+    setLastError("column scale epilogue: exists for the 4-wave kernel only (see gemmAppliesColumnScale)");
     return diopiErrorOccurred;
   } else {
   hipLaunchKernelGGL((gemmMfmaPipelinedKernel<T, EPI>), grid, dim3(kPipeThreads), lds, stream, g);
@@ -2544,6 +2576,19 @@ diopiError_t transposeCopy(hipStream_t stream, void* dst, const void* src, int i
   return launchTranspose<uint32_t>(stream, dst, src, batch, rows, cols, sRow, sCol, sBatch);
 }
 
+bool gemmAppliesColumnScale(const GemmProblem& p) {
+  // the conditions under which runGemm below reaches the 4-wave kernel without touching the operands
+  const bool half = p.dtype == diopi_dtype_bfloat16 || p.dtype == diopi_dtype_float16;
+  if (!half || p.batch != 1 || p.Cin || p.bias || p.K <= 0 || p.M >= (int64_t(1) << 31) || p.N >= (int64_t(1) << 31)) return false;
+  if (p.sAk != 1 || !mult8(p.sAm) || !ptr16(p.A) || p.sBk != 1 || !mult8(p.sBn) || !ptr16(p.B)) return false;
+  if (p.M <= kSkinnyMaxM) return false;
+  const bool big = ceilDiv(p.M, 256) * ceilDiv(p.N, 256) >= 144 && p.N > 128 && p.K > 2 * kBK;
+  const bool fits2g = ((p.M - 1) * p.sAm + p.K) * 2 < (int64_t(1) << 31) && ((p.N - 1) * p.sBn + p.K) * 2 < (int64_t(1) << 31);
+  if (!big || p.K % (2 * kBK) != 0 || !fits2g) return false;
+  const bool vec = p.N % 8 == 0 && p.sOm % 8 == 0 && ptr16(p.out) && ((p.M - 1) * p.sOm + p.N) * 2 < (int64_t(1) << 31);
+  return vec && p.M * p.sAm * 2 < (int64_t(1) << 31) && p.N * p.sBn * 2 < (int64_t(1) << 31);
+}
+
 diopiError_t runGemm(diopiContextHandle_t ctx, hipStream_t stream, GemmProblem p) {
   if (p.batch == 0 || p.M == 0 || p.N == 0) return diopiSuccess;
   AMD_CHECK(p.batch <= 65535, "gemm: batch %ld exceeds the grid limit", (long)p.batch);
@@ -2589,9 +2634,13 @@ diopiError_t runGemm(diopiContextHandle_t ctx, hipStream_t stream, GemmProblem p
     const bool big = ceilDiv(p.M, 256) * ceilDiv(p.N, 256) * p.batch >= 144 && p.N > 128 && p.K > 2 * kBK;
     const bool fits2g = bT || (((p.M - 1) * p.sAm + p.K) * 2 < (int64_t(1) << 31) && ((p.N - 1) * p.sBn + p.K) * 2 < (int64_t(1) << 31));
     if (big && p.K % kBK == 0 && p.K >= 2 * kBK && fits2g) {
+      if (p.colScale)
+        return p.dtype == diopi_dtype_bfloat16 ? launchMfmaPipelined<bf16_t, kEpiColScale>(stream, p)
+                                               : launchMfmaPipelined<half_t, kEpiColScale>(stream, p);
       return p.dtype == diopi_dtype_bfloat16 ? launchMfmaPipelined<bf16_t>(stream, p, nullptr, 1, 0, nullptr, bT)
                                              : launchMfmaPipelined<half_t>(stream, p, nullptr, 1, 0, nullptr, bT);
     }
+    AMD_CHECK(!p.colScale, "gemm: a column scale was set on a problem gemmAppliesColumnScale does not accept");
     // In between (too few 256 x 256 tiles for the chip, too many rows for the weight-streaming kernel): the same
     // large-tile kernel with K split over grid.y, fp32 partial products in workspace and a reduction pass.
     // In between (too few 256 x 256 tiles for the chip, too many rows for the weight-streaming kernels): the 128 x 128

@@ -23,9 +23,17 @@ struct GemmProblem {
   int64_t sCb = 0, sCm = 0, sCn = 0;
   const void* bias = nullptr;
   float alpha = 1.f, beta = 0.f;
+  // out[m, n] = alpha * sum * colScale[n], one rounding: N values of colScaleDtype (fp16 / bf16 / fp32). Only for
+  // problems gemmAppliesColumnScale accepts (no addend, no bias).
+  const void* colScale = nullptr;
+  diopiDtype_t colScaleDtype = diopi_dtype_float32;
 };
 
 diopiError_t runGemm(diopiContextHandle_t ctx, hipStream_t stream, GemmProblem p);
+
+// Whether runGemm would send p to the kernel whose epilogue can multiply every column by a scale of its own (the
+// 4-wave large-tile kernel): the caller sets colScale only then, and applies the scale in a pass of its own otherwise.
+bool gemmAppliesColumnScale(const GemmProblem& p);
 
 // diopiRotaryEmbedding on views (rotary_kv.hip): out and x of shape [..., heads, head_dim], strided views allowed.
 diopiError_t runRotary(diopiContextHandle_t ctx, hipStream_t stream, const TensorView& out, const TensorView& x,

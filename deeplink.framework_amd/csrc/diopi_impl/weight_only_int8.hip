@@ -451,8 +451,10 @@ __global__ __launch_bounds__(256) void w8LinearScalarKernel(W8Args a) {
 // Many rows (prefill with int8 weights): the streaming kernels above read the weights once per 64 rows, which at 8192
 // rows is 128 times. From 129 rows on the weights are expanded once to the activation type (exact: an int8 fits its
 // mantissa), the dense GEMM multiplies with alpha = 1 / 128 (so that the unscaled sums stay far inside the range of
-// fp16), and one pass over the result applies the channel scale: 8192 x 11008 x 4096 2387 -> about 600 us.
-// The scale is applied to the rounded sum, not folded into the weights: a weight rounded with its scale puts noise of
+// fp16), and one pass over the result applies the channel scale: 8192 x 11008 x 4096 2387 -> about 600 us. Where the
+// product goes to the large-tile kernel, that kernel's epilogue multiplies the fp32 sums by the channel scale instead
+// (alpha = 1, one rounding, no pass over the result).
+// The scale is applied to the sum, not folded into the weights: a weight rounded with its scale puts noise of
 // the size of the largest terms on every output, which the small outputs of a long sum do not survive. For the same
 // reason a call with a bias stays with the streaming kernels: added after the sum has been rounded, a bias that nearly
 // cancels it leaves the rounding error of the sum on a result many times smaller.
@@ -558,11 +560,17 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiWeightOnlyIn
     p.B = expanded, p.sBn = K, p.sBk = 1;
     p.out = cout.data, p.sOm = N;
     p.alpha = kW8SumScale;
+    // where the product goes to the kernel that can scale every column in its epilogue, the channel scale meets the
+    // fp32 sum there: 8192 x 11008 x 4096 594 -> 544 us, 2048 rows 204 -> 183 us (the same products with 16-bit weights:
+    // 499 and 151 us; what remains above them is the expansion)
+    const bool scaleInEpilogue = gemmAppliesColumnScale(p);
+    if (scaleInEpilogue) p.alpha = 1.f, p.colScale = csc.data, p.colScaleDtype = csc.dtype;
 #define W8_MANY_ROWS(T)                                                                                                          \
   do {                                                                                                                           \
     hipLaunchKernelGGL(w8ExpandKernel<T>, egrid, dim3(256), 0, stream, static_cast<T*>(expanded), cw.ptr<int8_t>(), N, K, ldw);   \
     AMD_LAUNCH_CHECK();                                                                                                          \
     AMD_TRY(runGemm(ctx, stream, p));                                                                                            \
+    if (scaleInEpilogue) break;                                                                                                  \
     if (per == 8) hipLaunchKernelGGL((w8ScaleKernel<T, 8>), sgrid, dim3(256), 0, stream, cout.ptr<T>(), csc.data, (int)csc.dtype, M, N); \
     else hipLaunchKernelGGL((w8ScaleKernel<T, 1>), sgrid, dim3(256), 0, stream, cout.ptr<T>(), csc.data, (int)csc.dtype, M, N);   \
   } while (0)

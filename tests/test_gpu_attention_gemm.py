@@ -675,14 +675,18 @@ def test_weight_only_int8_linear_chunked_k_row_groups_and_tile_counts(ops, dev, 
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("m,k,n", [(129, 4096, 1000), (300, 1024 + 16, 520), (1024, 4096, 4096)])
+@pytest.mark.parametrize("m,k,n", [(129, 4096, 1000), (300, 1024 + 16, 520), (1024, 4096, 4096), (4608, 384, 4096),
+                                   (4568, 512, 4072)])
 def test_weight_only_int8_linear_many_rows(ops, dev, pkg, m, k, n, dtype):
     """From 129 rows on, without a bias, the weights are expanded once and the product goes to the dense GEMM, the
-    channel scale in a pass over the result: against the oracle, with a bias (the streaming kernels), and exactly on
-    one-hot rows, where the result is w * scale rounded once on either route."""
+    channel scale in a pass over the result or, where the product takes the large-tile kernel (the last two shapes:
+    288 tiles, the second with ragged last tiles), in that kernel's epilogue: against the oracle, with a bias (the
+    streaming kernels), with a float32 scale, and exactly on one-hot rows, where the result is w * scale rounded once
+    on every route."""
     w = pkg.workloads.int8_linear(seed=6, m=m, k=k, n=n, dtype=dtype)
     want = oracle.weight_only_int8_linear(w["x"], w["w"], w["scale"])
     assert_half(ops.weight_only_int8_linear(w["x"].to(dev), w["w"].to(dev), w["scale"].to(dev)), want)
+    assert_half(ops.weight_only_int8_linear(w["x"].to(dev), w["w"].to(dev), w["scale"].float().to(dev)), want)
     bias = torch.randn(n, generator=g(35)).to(dtype)
     assert_half(ops.weight_only_int8_linear(w["x"].to(dev), w["w"].to(dev), w["scale"].to(dev), bias.to(dev)), want + bias.float())
     assert_half(ops.weight_only_int8_linear(w["x"].to(dev), w["w"].to(dev), w["scale"].float().to(dev), bias.float().to(dev)),
