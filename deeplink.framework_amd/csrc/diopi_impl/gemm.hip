@@ -90,8 +90,10 @@ struct MfmaArgs {
   int rotCols = 0, rotHeadDim = 0, rotTableRows = 1;
   bool rotTableF32 = false;
   float rotSinSign = 1.f;
-  const void* colScale = nullptr;  // kEpiColScale: N values of dtype colScaleDtype
+  const void* colScale = nullptr;  // kEpiColScale: N values of dtype colScaleDtype, and optionally N of colBiasDtype to add
   int colScaleDtype = 0;
+  const void* colBias = nullptr;
+  int colBiasDtype = 0;
 };
 
 constexpr int kBK = 64;  // K elements per LDS tile (128-byte rows)
@@ -310,8 +312,8 @@ struct MfmaOp16<half_t> {
 // because the one-wave-per-SIMD kernel has no register to spare for a second path next to the general one.
 // kEpiRotaryLds (4-wave kernel only) is kEpiRotaryUniform for 16-bit tables and heads of 128 columns with the table
 // entries of an output tile's first four fragment rows waiting in LDS when the epilogue starts (see rotaryTablesToLds).
-// kEpiColScale (4-wave kernel only): out = alpha * sum * colScale[column], no addend, no bias (int8 weights expanded to
-// the activation type, the channel scale applied to the fp32 sum).
+// kEpiColScale (4-wave kernel only): out = alpha * sum * colScale[column] (+ colBias[column]), no addend (int8 weights
+// expanded to the activation type, the channel scale and the bias applied to the fp32 sum).
 // kEpiAddendLds (4-wave kernel only) is kEpiLinear with an addend whose pieces for an output tile's first two fragment
 // rows wait in LDS when the epilogue starts (see addendToLds).
 enum PipeEpilogue { kEpiLinear = 0, kEpiSiluMul = 1, kEpiPartial = 2, kEpiRotary = 3, kEpiRotaryUniform = 4, kEpiRotaryLds = 5, kEpiAddendLds = 6, kEpiColScale = 7 };
@@ -645,12 +647,15 @@ __device__ __forceinline__ void vectorEpilogue(const MfmaArgs& g, T* out, const 
     });
     }
   } else if constexpr (EPI == kEpiColScale) {
-    float sv[TN / 2][8];
+    float sv[TN / 2][8], bv[TN / 2][8];
 #pragma unroll
     for (int jp = 0; jp < TN / 2; ++jp) {
       const int col = min(col0 + jp * 32, g.N - 8);  // N % 8 == 0 here; a clamped piece is never stored
 #pragma unroll
-      for (int e = 0; e < 8; ++e) sv[jp][e] = loadAs<float>(g.colScale, col + e, g.colScaleDtype) * g.alpha;
+      for (int e = 0; e < 8; ++e) {
+        sv[jp][e] = loadAs<float>(g.colScale, col + e, g.colScaleDtype) * g.alpha;
+        bv[jp][e] = g.colBias ? loadAs<float>(g.colBias, col + e, g.colBiasDtype) : 0.f;
+      }
     }
     staticFor<TM>([&](auto ic) {
       constexpr int i = decltype(ic)::value;
@@ -663,7 +668,7 @@ __device__ __forceinline__ void vectorEpilogue(const MfmaArgs& g, T* out, const 
         const float v[8] = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
         Frag o;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) o[e] = static_cast<T>(v[e] * sv[jp][e]);
+        for (int e = 0; e < 8; ++e) o[e] = static_cast<T>(v[e] * sv[jp][e] + bv[jp][e]);
         put(i, jp, o);
       }
     });
@@ -2254,7 +2259,7 @@ static diopiError_t launchMfmaPipelined(hipStream_t stream, const GemmProblem& p
   g.M = (int)p.M, g.N = (int)p.N, g.K = (int)p.K;
   g.tilesM = (int)ceilDiv(p.M, 256), g.tilesN = (int)ceilDiv(p.N, 256);
   g.alpha = p.alpha, g.beta = p.beta;
-  g.colScale = p.colScale, g.colScaleDtype = (int)p.colScaleDtype;
+  g.colScale = p.colScale, g.colScaleDtype = (int)p.colScaleDtype, g.colBias = p.colBias, g.colBiasDtype = (int)p.colBiasDtype;
   auto al16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
   // the vector epilogue addresses one batch of the output and of the addend with 32-bit byte offsets
   const bool span32 = ((p.M - 1) * p.sOm + p.N) * (int64_t)sizeof(T) < (int64_t(1) << 31) &&

@@ -23,10 +23,12 @@ struct GemmProblem {
   int64_t sCb = 0, sCm = 0, sCn = 0;
   const void* bias = nullptr;
   float alpha = 1.f, beta = 0.f;
-  // out[m, n] = alpha * sum * colScale[n], one rounding: N values of colScaleDtype (fp16 / bf16 / fp32). Only for
-  // problems gemmAppliesColumnScale accepts (no addend, no bias).
+  // out[m, n] = alpha * sum * colScale[n] + colBias[n], one rounding: N values each of their own dtype (fp16 / bf16 /
+  // fp32), colBias optional. Only for problems gemmAppliesColumnScale accepts (no addend, no `bias`).
   const void* colScale = nullptr;
   diopiDtype_t colScaleDtype = diopi_dtype_float32;
+  const void* colBias = nullptr;
+  diopiDtype_t colBiasDtype = diopi_dtype_float32;
 };
 
 diopiError_t runGemm(diopiContextHandle_t ctx, hipStream_t stream, GemmProblem p);

@@ -456,8 +456,9 @@ __global__ __launch_bounds__(256) void w8LinearScalarKernel(W8Args a) {
 // (alpha = 1, one rounding, no pass over the result).
 // The scale is applied to the sum, not folded into the weights: a weight rounded with its scale puts noise of
 // the size of the largest terms on every output, which the small outputs of a long sum do not survive. For the same
-// reason a call with a bias stays with the streaming kernels: added after the sum has been rounded, a bias that nearly
-// cancels it leaves the rounding error of the sum on a result many times smaller.
+// reason a call with a bias takes this route only where the epilogue adds it to the fp32 sum, and stays with the
+// streaming kernels otherwise: added after the sum has been rounded, a bias that nearly cancels it leaves the
+// rounding error of the sum on a result many times smaller.
 template <typename T>
 __global__ __launch_bounds__(256) void w8ExpandKernel(T* __restrict__ dst, const int8_t* __restrict__ w, int64_t n, int64_t k,
                                                        int64_t ldw) {
@@ -546,7 +547,17 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiWeightOnlyIn
     diopiTensorHandle_t th;
     AMD_TRY(requireTensor(ctx, out.shape, out.ndim, out.dtype, &th, &cout));
   }
-  if (M >= kW8ExpandFromRows && !bias.defined() && K % 16 == 0 && cw.aligned16() && (N == 1 || cw.stride[0] % 16 == 0)) {
+  GemmProblem p;
+  p.dtype = in.dtype, p.batch = 1, p.M = M, p.N = N, p.K = K;
+  p.A = cin.data, p.sAm = K, p.sAk = 1;
+  p.B = cw.data, p.sBn = K, p.sBk = 1;  // (stands in for the expanded copy, which is aligned at least as well)
+  p.out = cout.data, p.sOm = N;
+  // where the product goes to the kernel that can scale every column in its epilogue, the channel scale (and a bias)
+  // meet the fp32 sum there: 8192 x 11008 x 4096 594 -> 544 us, 2048 rows 204 -> 183 us (the same products with 16-bit
+  // weights: 499 and 151 us; what remains above them is the expansion)
+  const bool manyRows = M >= kW8ExpandFromRows && K % 16 == 0 && cw.aligned16() && (N == 1 || cw.stride[0] % 16 == 0);
+  const bool scaleInEpilogue = manyRows && gemmAppliesColumnScale(p);
+  if (manyRows && (scaleInEpilogue || !bias.defined())) {
     void* expanded = nullptr;
     AMD_TRY(requireWorkspace(ctx, N * K * in.itemsize, &expanded));
     const int64_t pieces = N * (K / 16), ldw = N > 1 ? cw.stride[0] : K;
@@ -554,17 +565,12 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiWeightOnlyIn
     const dim3 egrid((unsigned)ceilDiv(pieces, (int64_t)256));
     const int per = N % 8 == 0 && cout.aligned16() ? 8 : 1;
     const dim3 sgrid((unsigned)ceilDiv(N / per, (int64_t)256), (unsigned)std::min<int64_t>(M, 2048));
-    GemmProblem p;
-    p.dtype = in.dtype, p.batch = 1, p.M = M, p.N = N, p.K = K;
-    p.A = cin.data, p.sAm = K, p.sAk = 1;
-    p.B = expanded, p.sBn = K, p.sBk = 1;
-    p.out = cout.data, p.sOm = N;
+    p.B = expanded;
     p.alpha = kW8SumScale;
-    // where the product goes to the kernel that can scale every column in its epilogue, the channel scale meets the
-    // fp32 sum there: 8192 x 11008 x 4096 594 -> 544 us, 2048 rows 204 -> 183 us (the same products with 16-bit weights:
-    // 499 and 151 us; what remains above them is the expansion)
-    const bool scaleInEpilogue = gemmAppliesColumnScale(p);
-    if (scaleInEpilogue) p.alpha = 1.f, p.colScale = csc.data, p.colScaleDtype = csc.dtype;
+    if (scaleInEpilogue) {
+      p.alpha = 1.f, p.colScale = csc.data, p.colScaleDtype = csc.dtype;
+      if (bias.defined()) p.colBias = cb.data, p.colBiasDtype = cb.dtype;
+    }
 #define W8_MANY_ROWS(T)                                                                                                          \
   do {                                                                                                                           \
     hipLaunchKernelGGL(w8ExpandKernel<T>, egrid, dim3(256), 0, stream, static_cast<T*>(expanded), cw.ptr<int8_t>(), N, K, ldw);   \

@@ -681,8 +681,8 @@ def test_weight_only_int8_linear_many_rows(ops, dev, pkg, m, k, n, dtype):
     """From 129 rows on, without a bias, the weights are expanded once and the product goes to the dense GEMM, the
     channel scale in a pass over the result or, where the product takes the large-tile kernel (the last two shapes:
     288 tiles, the second with ragged last tiles), in that kernel's epilogue: against the oracle, with a bias (the
-    streaming kernels), with a float32 scale, and exactly on one-hot rows, where the result is w * scale rounded once
-    on every route."""
+    streaming kernels, or that epilogue), with a float32 scale, and exactly on one-hot rows, where the result is
+    w * scale (+ bias) rounded once on every route."""
     w = pkg.workloads.int8_linear(seed=6, m=m, k=k, n=n, dtype=dtype)
     want = oracle.weight_only_int8_linear(w["x"], w["w"], w["scale"])
     assert_half(ops.weight_only_int8_linear(w["x"].to(dev), w["w"].to(dev), w["scale"].to(dev)), want)
@@ -696,6 +696,9 @@ def test_weight_only_int8_linear_many_rows(ops, dev, pkg, m, k, n, dtype):
     x[torch.arange(m), cols] = 1
     got = ops.weight_only_int8_linear(x.to(dev), w["w"].to(dev), w["scale"].to(dev))
     assert_exact(got, (w["w"][:, cols].float() * w["scale"].float()[:, None]).t().to(dtype))
+    # and with a bias: w * scale is exact in fp32, the bias is added there, one rounding on every route
+    got = ops.weight_only_int8_linear(x.to(dev), w["w"].to(dev), w["scale"].to(dev), bias.to(dev))
+    assert_exact(got, ((w["w"][:, cols].float() * w["scale"].float()[:, None]).t() + bias.float()).to(dtype))
 
 
 # ------------------------------------------------------------------ decoder block
