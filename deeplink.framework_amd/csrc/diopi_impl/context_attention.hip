@@ -80,10 +80,10 @@ struct CaMfma<half_t> {
 
 // XOR applied to the 16-byte chunk index of K row `key` in LDS; the patterns are the ones that
 // measure conflict-free for ds_read_b128 with 32 consecutive rows per half-wave: 256-byte rows
-// (d = 128) need key & 15, 128-byte rows (d = 64) need (key >> 1) & 7.
+// (d = 128; 512-byte rows alias the banks the same way) need key & 15, 128-byte rows (d = 64) need (key >> 1) & 7.
 template <int D>
 __device__ __forceinline__ int kSwizzle(int key) {
-  return D == 128 ? (key & 15) : ((key >> 1) & 7);
+  return D >= 128 ? (key & 15) : ((key >> 1) & 7);
 }
 
 // XOR applied to the 16-byte chunk index of V row `key` in LDS (a multiple of 4, so the 32 bytes a 16-lane
@@ -91,7 +91,7 @@ __device__ __forceinline__ int kSwizzle(int key) {
 // consecutive keys x 2 pieces of 32 bytes, which these patterns put on 8 different 32-byte bank groups.
 template <int D>
 __device__ __forceinline__ int vSwizzle(int key) {
-  return D == 128 ? 4 * (key & 3) : 4 * ((key >> 1) & 1);
+  return D >= 128 ? 4 * (key & 3) : 4 * ((key >> 1) & 1);
 }
 
 constexpr int kCaBQ = 128, kCaBKV = 64;
@@ -102,7 +102,10 @@ constexpr int kCaBQ = 128, kCaBKV = 64;
 constexpr float kCaRescaleStep = 8.0f;
 
 // One 128-query block of one (sequence, head): the whole flash-attention pass over its key tiles.
-template <typename T, int D>
+// D is the head size the tiles are laid out for (64, 128 or 256); with PART the tensors' own head size a.d is any
+// multiple of 8 below D: the pieces of a row at or past a.d are zeros in the Q fragments and in the K and V tiles (they add
+// nothing to a score and produce output columns that are not stored).
+template <typename T, int D, bool PART>
 __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, const int h, const int b) {
   using Frag = typename CaMfma<T>::Frag;
   using Half = typename CaMfma<T>::Half;
@@ -129,10 +132,17 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
 
   const int qi = q0 + wave * 32 + l31;      // this lane's query (column of S^T)
   const int qiC = min(qi, len - 1);          // rows past the sequence compute on the last row, never stored
+  const int dReal = PART ? a.d : D;  // (PART: a variant of its own, so that whole rows pay nothing for the tests below)
   Frag qf[KS];
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks)
-    qf[ks] = *reinterpret_cast<const Frag*>(qg + (int64_t)qiC * a.qTok + ks * 16 + half * 8);
+  for (int ks = 0; ks < KS; ++ks) {
+    if (ks * 16 + half * 8 < dReal) {
+      qf[ks] = *reinterpret_cast<const Frag*>(qg + (int64_t)qiC * a.qTok + ks * 16 + half * 8);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) qf[ks][e] = static_cast<T>(0.f);
+    }
+  }
 
   const int ntiles = (min(len, q0 + kCaBQ) + kCaBKV - 1) / kCaBKV;
   const int waveMaxQ = min(q0 + wave * 32 + 31, len - 1);
@@ -146,16 +156,18 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
 #pragma unroll
   for (int i = 0; i < NLD; ++i) {
     const int key = (i * 4 + wave) * RPL + lane / CPR, pc = lane % CPR;
-    kVoff[i] = (key * (int)a.kTok + ((pc ^ kSwizzle<D>(key)) << 3)) * (int)sizeof(T);
-    vVoff[i] = (key * (int)a.vTok + ((pc ^ vSwizzle<D>(key)) << 3)) * (int)sizeof(T);
+    const int kc = (pc ^ kSwizzle<D>(key)) << 3, vc = (pc ^ vSwizzle<D>(key)) << 3;  // first element of the piece
+    constexpr int kPastEnd = (int)0x80000000u;  // beyond every descriptor: the copy writes zeros
+    kVoff[i] = kc < dReal ? (key * (int)a.kTok + kc) * (int)sizeof(T) : kPastEnd;
+    vVoff[i] = vc < dReal ? (key * (int)a.vTok + vc) * (int)sizeof(T) : kPastEnd;
   }
   auto descriptor = [](const T* base, int64_t bytes) {
     const uint64_t p = reinterpret_cast<uint64_t>(base);
     u32x4 d = {(uint32_t)p, (uint32_t)(p >> 32) & 0xffffu, (uint32_t)bytes, 0x00020000u};
     return d;
   };
-  const u32x4 rsK = descriptor(kg, ((int64_t)(len - 1) * a.kTok + D) * sizeof(T));
-  const u32x4 rsV = descriptor(vg, ((int64_t)(len - 1) * a.vTok + D) * sizeof(T));
+  const u32x4 rsK = descriptor(kg, ((int64_t)(len - 1) * a.kTok + dReal) * sizeof(T));
+  const u32x4 rsV = descriptor(vg, ((int64_t)(len - 1) * a.vTok + dReal) * sizeof(T));
   const unsigned ldsK = (unsigned)(uintptr_t)sK, ldsV = (unsigned)(uintptr_t)sV;
 
   auto copyK = [&](int t, int stage) {
@@ -295,7 +307,7 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
         // keys 8 r + 4 half + 0..3 of the step: the order the P^T operand holds them in.
         const int trKey = half * 4 + ((lane & 15) >> 2);
         const int trChunk = ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1), trIn = (lane & 1) * 4;
-        const int vsw = D == 128 ? (trKey & 3) : ((trKey >> 1) & 1);  // vSwizzle<D>(key) / 4: the low bits of the d tile
+        const int vsw = D >= 128 ? (trKey & 3) : ((trKey >> 1) & 1);  // vSwizzle<D>(key) / 4: the low bits of the d tile
         const unsigned vCur = opaque((unsigned)(trKey * ROWB + (trChunk << 4) + trIn * 2 + (vsw << 6)) + ldsV0 + cur * kStageBytes);
         typedef __attribute__((address_space(3))) s16x4* LdsTr;
         auto vfrag = [&](int i) {
@@ -363,7 +375,7 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
     int chunk = lane + 64 * i;
     int row = chunk / CPR, c = chunk % CPR;
     int qrow = q0 + wave * 32 + row;
-    if (qrow < len) *reinterpret_cast<Frag*>(og + (int64_t)qrow * a.oTok + c * 8) = *reinterpret_cast<const Frag*>(sO + row * OS + c * 8);
+    if (qrow < len && c * 8 < dReal) *reinterpret_cast<Frag*>(og + (int64_t)qrow * a.oTok + c * 8) = *reinterpret_cast<const Frag*>(sO + row * OS + c * 8);
   }
 }
 
@@ -376,8 +388,8 @@ __device__ __forceinline__ void contextAttnBlock(const CaArgs& a, const int qb, 
 // grid is therefore one-dimensional and decoded so that all workgroups of one (sequence, head), and
 // of neighbouring heads (which share K/V under grouped-query attention), land on the same XCD next to
 // each other in time: a K/V tile is fetched from HBM once and then served from that L2.
-template <typename T, int D>
-__global__ __launch_bounds__(256, 2) void contextAttnMfmaKernel(CaArgs a, int numQBlocks, int numSeq) {
+template <typename T, int D, bool PART>
+__global__ __launch_bounds__(256, D > 128 ? 1 : 2) void contextAttnMfmaKernel(CaArgs a, int numQBlocks, int numSeq) {
   const int pairs = (numQBlocks + 1) / 2, hb = a.heads * numSeq;
   const int flat = (int)blockIdx.x;
   int h, b, pair;
@@ -406,7 +418,7 @@ __global__ __launch_bounds__(256, 2) void contextAttnMfmaKernel(CaArgs a, int nu
       if (light == heavy) break;
       __syncthreads();  // the first block's output staging aliases the K/V stages the second one fills
     }
-    contextAttnBlock<T, D>(a, pass == 0 ? heavy : light, h, b);
+    contextAttnBlock<T, D, PART>(a, pass == 0 ? heavy : light, h, b);
   }
 }
 
@@ -417,8 +429,8 @@ __global__ __launch_bounds__(256, 2) void contextAttnMfmaKernel(CaArgs a, int nu
 // and share less in L2, which is why launches whose pairs already fill the chip evenly keep the paired form. Measured
 // (us, 32 heads x 128, bf16, pairs -> this): 1 x 256 tokens 14.6 -> 9.1, 1 x 512 19.1 -> 13.6, 1 x 1024 28.0 -> 22.8,
 // 3 x 700 30.9 -> 24.4, 1 x 3000 89.7 -> 84.9; against it: 1 x 2048 46.8 -> 51.0, 32 x 512 134 -> 155, 8 x 1000 88 -> 103.
-template <typename T, int D>
-__global__ __launch_bounds__(256, 2) void contextAttnSingleBlockKernel(CaArgs a, int numQBlocks, int numSeq) {
+template <typename T, int D, bool PART>
+__global__ __launch_bounds__(256, D > 128 ? 1 : 2) void contextAttnSingleBlockKernel(CaArgs a, int numQBlocks, int numSeq) {
   const int flat = (int)blockIdx.x;
   int rank, b, h;
   if ((a.heads & 7) == 0) {  // a contiguous eighth of every sequence's heads per XCD, as in the paired form
@@ -433,7 +445,7 @@ __global__ __launch_bounds__(256, 2) void contextAttnSingleBlockKernel(CaArgs a,
     const int hs = flat - rank * hb;
     b = hs / a.heads, h = hs - b * a.heads;
   }
-  contextAttnBlock<T, D>(a, numQBlocks - 1 - rank, h, b);
+  contextAttnBlock<T, D, PART>(a, numQBlocks - 1 - rank, h, b);
 }
 
 // One workgroup per (query token, head): scores to LDS, softmax, then P.V with lanes over d.
@@ -483,11 +495,11 @@ __global__ __launch_bounds__(256) void contextAttnScalarKernel(CaArgs a, int max
   }
 }
 
-template <typename T, int D>
-static diopiError_t launchCaMfma(hipStream_t stream, const CaArgs& a, int maxLen, int64_t batch) {
+template <typename T, int D, bool PART>
+static diopiError_t launchCaMfmaAs(hipStream_t stream, const CaArgs& a, int maxLen, int64_t batch) {
   constexpr size_t lds = 2 * (size_t)(2 * kCaBKV * D) * sizeof(T);
   static_assert(lds >= 4 * 32 * (D + 8) * sizeof(T), "epilogue staging must fit in the tile buffers");
-  AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&contextAttnMfmaKernel<T, D>), (int)lds));
+  AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&contextAttnMfmaKernel<T, D, PART>), (int)lds));
   const int numQBlocks = (int)ceilDiv(maxLen, kCaBQ);
   const int64_t blocks = (int64_t)((numQBlocks + 1) / 2) * a.heads * batch;
   AMD_CHECK(blocks < ((int64_t)1 << 31), "context attention: grid limits exceeded");
@@ -497,15 +509,20 @@ static diopiError_t launchCaMfma(hipStream_t stream, const CaArgs& a, int maxLen
   const int64_t pairedLoad = ceilDiv(blocks, cus) * (numQBlocks + 1);
   const int64_t singleLoad = std::max<int64_t>(ceilDiv(hb * numQBlocks * (numQBlocks + 1) / 2, cus), numQBlocks);
   if (numQBlocks > 1 && singleLoad * 11 < pairedLoad * 10 && hb * numQBlocks < ((int64_t)1 << 31)) {
-    AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&contextAttnSingleBlockKernel<T, D>), (int)lds));
-    hipLaunchKernelGGL((contextAttnSingleBlockKernel<T, D>), dim3((unsigned)(hb * numQBlocks)), dim3(256), lds, stream, a, numQBlocks,
+    AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&contextAttnSingleBlockKernel<T, D, PART>), (int)lds));
+    hipLaunchKernelGGL((contextAttnSingleBlockKernel<T, D, PART>), dim3((unsigned)(hb * numQBlocks)), dim3(256), lds, stream, a, numQBlocks,
                        (int)batch);
     AMD_LAUNCH_CHECK();
     return diopiSuccess;
   }
-  hipLaunchKernelGGL((contextAttnMfmaKernel<T, D>), dim3((unsigned)blocks), dim3(256), lds, stream, a, numQBlocks, (int)batch);
+  hipLaunchKernelGGL((contextAttnMfmaKernel<T, D, PART>), dim3((unsigned)blocks), dim3(256), lds, stream, a, numQBlocks, (int)batch);
   AMD_LAUNCH_CHECK();
   return diopiSuccess;
+}
+
+template <typename T, int D>
+static diopiError_t launchCaMfma(hipStream_t stream, const CaArgs& a, int maxLen, int64_t batch) {
+  return a.d == D ? launchCaMfmaAs<T, D, false>(stream, a, maxLen, batch) : launchCaMfmaAs<T, D, true>(stream, a, maxLen, batch);
 }
 
 }  // namespace amd
@@ -567,11 +584,16 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiContextAtten
   diopiError_t err;
   // the MFMA kernel addresses K and V rows of one sequence with 32-bit byte offsets
   const bool fits32 = ((int64_t)maxInputLen + kCaBKV) * std::max(a.kTok, a.vTok) * (int64_t)q.itemsize < (int64_t)1 << 31;
-  if (half && (a.d == 64 || a.d == 128) && al(cq) && al(ck) && al(cv) && al(co) && fits32) {
+  // head sizes that are a multiple of 8 (whole 16-byte pieces) take the tile layout of the next of 64 / 128 / 256
+  if (half && a.d % 8 == 0 && a.d <= 256 && al(cq) && al(ck) && al(cv) && al(co) && fits32) {
     if (q.dtype == diopi_dtype_bfloat16)
-      err = a.d == 128 ? launchCaMfma<bf16_t, 128>(stream, a, maxInputLen, batch) : launchCaMfma<bf16_t, 64>(stream, a, maxInputLen, batch);
+      err = a.d <= 64    ? launchCaMfma<bf16_t, 64>(stream, a, maxInputLen, batch)
+            : a.d <= 128 ? launchCaMfma<bf16_t, 128>(stream, a, maxInputLen, batch)
+                         : launchCaMfma<bf16_t, 256>(stream, a, maxInputLen, batch);
     else
-      err = a.d == 128 ? launchCaMfma<half_t, 128>(stream, a, maxInputLen, batch) : launchCaMfma<half_t, 64>(stream, a, maxInputLen, batch);
+      err = a.d <= 64    ? launchCaMfma<half_t, 64>(stream, a, maxInputLen, batch)
+            : a.d <= 128 ? launchCaMfma<half_t, 128>(stream, a, maxInputLen, batch)
+                         : launchCaMfma<half_t, 256>(stream, a, maxInputLen, batch);
   } else {
     AMD_CHECK(maxInputLen <= 12000, "context attention: the scalar path supports sequences up to 12000 tokens, got %d", maxInputLen);
     AMD_CHECK(maxInputLen <= 65535, "context attention: grid limits exceeded");

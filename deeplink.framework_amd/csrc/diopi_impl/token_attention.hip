@@ -30,8 +30,9 @@
 // streaming kernel with the other half of the work compiled out: 588 -> 462 us for both at batch 64 with 156 000 cached
 // tokens, and the second half no longer walks a long sequence with one workgroup (1 x 32768 tokens: 1709 -> 60 us).
 //
-// Head rows of 128, 256 or 512 bytes at 16-byte aligned strides take the kernels above; any other head size or
-// alignment (up to 1024 elements) takes the generic kernels at the end: one workgroup per (sequence, head), 256 tokens
+// Head rows of whole 16-byte pieces up to 512 bytes at 16-byte aligned strides take the kernels above (rows of other
+// lengths than 128, 256 or 512 bytes on the lanes of the next of those, the lanes past the row's end masked); any
+// other head size or alignment (up to 1024 elements) takes the generic kernels at the end: one workgroup per (sequence, head), 256 tokens
 // at a time, one token's dot product per thread and P.V with the threads over d. A correctness path.
 #include <algorithm>
 #include <mutex>
@@ -128,7 +129,7 @@ enum TaMode { kTaFused = 0, kTaLogitsOut = 1, kTaReduceV = 2 };
 // memory (the two-call modes). QPK: query heads that share this workgroup's K/V head and are all served from one read
 // of its rows (grouped-query layouts; 1 otherwise). With QPK > 1 the grid is one-dimensional and decoded so that the
 // workgroups that share a K/V head's rows run next to each other on one XCD.
-template <typename T, int LPT, bool HIW, int MODE = kTaFused, typename LT = float, int QPK = 1>
+template <typename T, int LPT, bool HIW, int MODE = kTaFused, typename LT = float, int QPK = 1, bool PART = false>
 __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* __restrict__ out,
                                                                      float* __restrict__ partial) {
   static_assert(QPK == 1 || !HIW, "several query heads per lane group: the lane groups of a wave take tokens, not heads");
@@ -219,6 +220,12 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   // conversions of K and V. 32 query heads on 8 K/V heads, batch 64 x (512..4096), fused: 184 -> 157 us (147 -> 110
   // registers, three -> four waves per SIMD); batch 256 x (1024..2048): 484 -> 413 us.
   constexpr bool kPairs = QPK > 1 && sizeof(T) == 2 && UNR == 2;
+  // PART: a head row shorter than the LPT pieces the lane group spans (head sizes between the powers of two). The lanes
+  // past its end read the row's first piece instead (memory that exists), hold zeros for q, so that they add nothing
+  // to a score, and store nothing. (A variant of its own: with these selects in the kernel for whole rows the launch
+  // at batch 64 reads 377 us against 366.)
+  const bool live = !PART || sub * N < a.d;
+  const int subIn = PART ? (live ? sub : 0) : sub;
   // scores leave the kernel in natural units, inside it they are in units of log2
   const float qScale = MODE == kTaLogitsOut ? a.scaleLog2e / kLog2eTA : a.scaleLog2e;
   float qf[kPairs ? 1 : QPK][N];
@@ -226,19 +233,19 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   if constexpr (kNeedK) {
 #pragma unroll
     for (int j = 0; j < QPK; ++j) {
-      V qv = *reinterpret_cast<const V*>(reinterpret_cast<const T*>(a.q) + b * a.qBatchStride + (h + headOf(j)) * a.qHeadStride + sub * N);
+      V qv = *reinterpret_cast<const V*>(reinterpret_cast<const T*>(a.q) + b * a.qBatchStride + (h + headOf(j)) * a.qHeadStride + subIn * N);
       if constexpr (kPairs) {
         const u32x4 raw = __builtin_bit_cast(u32x4, qv);
 #pragma unroll
-        for (int c = 0; c < 4; ++c) qp[j][c] = raw[c];
+        for (int c = 0; c < 4; ++c) qp[j][c] = live ? raw[c] : 0u;
       } else {
 #pragma unroll
-        for (int e = 0; e < N; ++e) qf[j][e] = static_cast<float>(qv[e]) * qScale;
+        for (int e = 0; e < N; ++e) qf[j][e] = live ? static_cast<float>(qv[e]) * qScale : 0.f;
       }
     }
   }
-  const T* kBase = kNeedK ? reinterpret_cast<const T*>(a.k) + kvh * a.kHeadStride + sub * N : nullptr;
-  const T* vBase = kNeedV ? reinterpret_cast<const T*>(a.v) + kvh * a.vHeadStride + sub * N : nullptr;
+  const T* kBase = kNeedK ? reinterpret_cast<const T*>(a.k) + kvh * a.kHeadStride + subIn * N : nullptr;
+  const T* vBase = kNeedV ? reinterpret_cast<const T*>(a.v) + kvh * a.vHeadStride + subIn * N : nullptr;
 
   float m[QPK], l[QPK], acc[QPK][N];
 #pragma unroll
@@ -422,12 +429,14 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
         V o;
 #pragma unroll
         for (int e = 0; e < N; ++e) o[e] = static_cast<T>(acc[j][e] * inv);
-        *reinterpret_cast<V*>(out + ((int64_t)b * a.heads + h + j) * a.d + sub * N) = o;
+        if (live) *reinterpret_cast<V*>(out + ((int64_t)b * a.heads + h + j) * a.d + sub * N) = o;
       } else {
         float* dst = partial + (((int64_t)b * a.heads + h + j) * a.nsplit + split) * (2 + a.d);
         if (sub == 0) dst[0] = m[j], dst[1] = l[j];
+        if (live) {
 #pragma unroll
-        for (int e = 0; e < N; ++e) dst[2 + sub * N + e] = acc[j][e];
+          for (int e = 0; e < N; ++e) dst[2 + sub * N + e] = acc[j][e];
+        }
       }
     }
   }
@@ -756,7 +765,8 @@ static diopiError_t fillArgs(const TaViews& t, bool needK, bool needV, int maxLe
   AMD_CHECK(q.dtype == diopi_dtype_bfloat16 || q.dtype == diopi_dtype_float16 || q.dtype == diopi_dtype_float32,
             "token attention: unsupported dtype %s", dtypeName(q.dtype));
   const int64_t bytes = q.shape[2] * q.itemsize;
-  bool vector = (bytes == 128 || bytes == 256 || bytes == 512) && q.aligned16() && kv.aligned16() &&
+  // head rows of whole 16-byte pieces up to 512 bytes: the streaming kernels span them with 8, 16 or 32 lanes
+  bool vector = bytes % 16 == 0 && bytes >= 16 && bytes <= 512 && q.aligned16() && kv.aligned16() &&
                 (kv.stride[0] * kv.itemsize) % 16 == 0 && (kv.stride[1] * kv.itemsize) % 16 == 0 &&
                 (q.stride[0] * q.itemsize) % 16 == 0 && (q.stride[1] * q.itemsize) % 16 == 0;
   if (needK && needV)
@@ -866,6 +876,9 @@ template <int MODE>
 static diopiError_t streamChunks(diopiContextHandle_t ctx, hipStream_t stream, TaArgs a, diopiDtype_t dtype, int64_t bytes,
                                  int64_t batch, int maxInputLen, void* outPtr, bool scoresF32, bool staticScratch,
                                  float* ownScratch) {
+  // a head row is spanned by 8, 16 or 32 lanes of 16 bytes: the next of 128 / 256 / 512 bytes (the kernel masks the rest)
+  const bool partRows = bytes != 128 && bytes != 256 && bytes != 512;
+  bytes = bytes <= 128 ? 128 : bytes <= 256 ? 256 : 512;
   // The lane groups of a wave take consecutive heads of one token when the head count allows it: a wave load is then
   // one contiguous piece of a slot (1 KiB) instead of head rows of four different slots (431 -> 421 us at batch 64,
   // 32 heads x 128, 156 043 cached tokens).
@@ -911,11 +924,17 @@ static diopiError_t streamChunks(diopiContextHandle_t ctx, hipStream_t stream, T
     AMD_CHECK(wgs < ((int64_t)1 << 31), "token attention: %ld workgroups exceed the grid limits", (long)wgs);
     grid = dim3((unsigned)wgs, 1, 1);
   }
-#define STREAM_CALL_AS(T, LPT, LT)                                                                                                   \
-  if (qpk == 4) hipLaunchKernelGGL((decodeSplitKernel<T, LPT, false, MODE, LT, 4>), grid, block, 0, stream, a, static_cast<T*>(outPtr), partial); \
-  else if (qpk == 2) hipLaunchKernelGGL((decodeSplitKernel<T, LPT, false, MODE, LT, 2>), grid, block, 0, stream, a, static_cast<T*>(outPtr), partial); \
-  else if (hiw) hipLaunchKernelGGL((decodeSplitKernel<T, LPT, true, MODE, LT>), grid, block, 0, stream, a, static_cast<T*>(outPtr), partial); \
-  else hipLaunchKernelGGL((decodeSplitKernel<T, LPT, false, MODE, LT>), grid, block, 0, stream, a, static_cast<T*>(outPtr), partial)
+#define STREAM_CALL_PART(T, LPT, LT, PART)                                                                                           \
+  if (qpk == 4) hipLaunchKernelGGL((decodeSplitKernel<T, LPT, false, MODE, LT, 4, PART>), grid, block, 0, stream, a, static_cast<T*>(outPtr), partial); \
+  else if (qpk == 2) hipLaunchKernelGGL((decodeSplitKernel<T, LPT, false, MODE, LT, 2, PART>), grid, block, 0, stream, a, static_cast<T*>(outPtr), partial); \
+  else if (hiw) hipLaunchKernelGGL((decodeSplitKernel<T, LPT, true, MODE, LT, 1, PART>), grid, block, 0, stream, a, static_cast<T*>(outPtr), partial); \
+  else hipLaunchKernelGGL((decodeSplitKernel<T, LPT, false, MODE, LT, 1, PART>), grid, block, 0, stream, a, static_cast<T*>(outPtr), partial)
+#define STREAM_CALL_AS(T, LPT, LT)            \
+  if (partRows) {                             \
+    STREAM_CALL_PART(T, LPT, LT, true);       \
+  } else {                                    \
+    STREAM_CALL_PART(T, LPT, LT, false);      \
+  }
 #define STREAM_CALL(T, LPT)                                \
   if (MODE == kTaFused || scoresF32) {                     \
     STREAM_CALL_AS(T, LPT, float);                         \
@@ -925,6 +944,7 @@ static diopiError_t streamChunks(diopiContextHandle_t ctx, hipStream_t stream, T
   TA_DISPATCH(dtype, bytes, STREAM_CALL);
 #undef STREAM_CALL
 #undef STREAM_CALL_AS
+#undef STREAM_CALL_PART
   AMD_LAUNCH_CHECK();
   if (MODE == kTaLogitsOut) return diopiSuccess;
   if (a.nsplit > 64) {

@@ -501,6 +501,29 @@ def test_context_attention_one_query_block_per_workgroup(ops, dev, heads, kvh, d
     assert_exact(got[starts[-1]].cpu(), v[starts[-1]].repeat_interleave(heads // kvh, dim=0))   # a sequence's first query sees one key
 
 
+@pytest.mark.parametrize("heads,kvh,d,dtype,lens", [(8, 8, 96, torch.bfloat16, [300, 1, 130, 64, 333]), (8, 2, 80, torch.float16, [700, 129]),
+                                                    (4, 4, 40, torch.bfloat16, [200, 513]), (4, 2, 256, torch.bfloat16, [260, 900, 64]),
+                                                    (16, 16, 256, torch.float16, [1300, 2048, 517]), (8, 4, 192, torch.bfloat16, [1000]),
+                                                    (32, 8, 112, torch.bfloat16, [2048, 2048])])
+def test_context_attention_other_head_sizes_on_the_matrix_pipe(ops, dev, heads, kvh, d, dtype, lens):
+    """Head sizes that are a multiple of 8 other than 64 and 128 take the tile layout of the next of 64 / 128 / 256, the
+    pieces of a row past the head size read as zeros and never stored: sizes under 64, between 64 and 128, 256 itself
+    and one between 128 and 256; both schedules (pairs of query blocks and a block per workgroup), grouped K/V heads,
+    ragged batches. The neighbours of every row (the next head, the next token) hold other values, so a piece read past
+    the head size would show."""
+    starts = [sum(lens[:i]) for i in range(len(lens))]
+    total = sum(lens)
+    q = torch.randn(total, heads, d, generator=g(43)).to(dtype)
+    k = torch.randn(total, kvh, d, generator=g(44)).to(dtype)
+    v = torch.randn(total, kvh, d, generator=g(45)).to(dtype)
+    st, ln = torch.tensor(starts, dtype=torch.int32), torch.tensor(lens, dtype=torch.int32)
+    want = oracle.context_attention(q.float(), k.float(), v.float(), st, ln)
+    out = torch.full((total, heads, d), 7.0, dtype=dtype, device=dev)
+    got = ops.context_attention(q.to(dev), k.to(dev), v.to(dev), st.to(dev), ln.to(dev), max(lens), out=out)
+    assert_half(got, want)
+    assert_exact(got[starts[-1]].cpu(), v[starts[-1]].repeat_interleave(heads // kvh, dim=0))   # a sequence's first query sees one key
+
+
 # ------------------------------------------------------------------ decode attention
 @pytest.mark.parametrize("dtype,d,idt", [(torch.bfloat16, 128, torch.int32), (torch.float16, 64, torch.int64),
                                           (torch.float32, 64, torch.int32), (torch.bfloat16, 256, torch.int32)])
@@ -533,9 +556,10 @@ def test_token_attention_fused_and_two_call(ops, dev, pkg, dtype, d, idt):
 @pytest.mark.parametrize("dtype,d,kvh,rep", [(torch.bfloat16, 80, 4, 2), (torch.float16, 32, 2, 1), (torch.float32, 96, 1, 4),
                                              (torch.bfloat16, 40, 8, 1), (torch.float32, 300, 2, 1)])
 def test_token_attention_any_head_size(ops, dev, pkg, dtype, d, kvh, rep):
-    """Head rows that are not 128, 256 or 512 bytes long (or not 16-byte aligned: d = 40 in bf16 is 80 bytes) take
-    the generic kernels: the fused form, the entry point that allocates nothing and the two-call form against the
-    oracle (ext_ops.py:100-133), with a sequence of one token and one longer than a block of 256."""
+    """Head rows that are not 128, 256 or 512 bytes long: whole 16-byte pieces up to 512 bytes ride on the lanes of the
+    next of those sizes with the lanes past the row's end masked (160, 64, 384 and 80 bytes here), longer rows take the
+    generic kernels (1200 bytes): the fused form, the entry point that allocates nothing and the two-call form against
+    the oracle (ext_ops.py:100-133), with a sequence of one token and one longer than a block of 256."""
     heads = kvh * rep
     w = pkg.workloads.paged_decode(seed=11, batch=5, heads=kvh, head_dim=d, min_len=1, max_len=700, pool_slots=4096, dtype=dtype)
     w["b_seq_len"][0] = 1                                    # b_loc is right-aligned: the last column is the token
@@ -557,6 +581,28 @@ def test_token_attention_any_head_size(ops, dev, pkg, dtype, d, kvh, rep):
     out2 = torch.empty_like(got)
     ops.token_softmax_reducev(att, dv, out2, *args)
     chk(out2, want)
+
+
+@pytest.mark.parametrize("dtype,d,heads,kvh", [(torch.bfloat16, 96, 8, 8), (torch.float16, 112, 12, 4), (torch.bfloat16, 192, 4, 2),
+                                               (torch.bfloat16, 80, 5, 5)])
+def test_token_attention_masked_head_rows_over_split_sequences(ops, dev, pkg, dtype, d, heads, kvh):
+    """Head sizes between the powers of two at lengths that are split into chunks and merged, on a pool whose every slot
+    is in use (the lanes past a row's end must not reach past the pool's last row): four heads of a token per wave
+    load, four and two query heads per K/V head, and a head count that keeps a workgroup per head."""
+    w = pkg.workloads.paged_decode(seed=21, batch=9, heads=kvh, head_dim=d, min_len=700, max_len=3000, pool_slots=15285, dtype=dtype)   # exactly the tokens drawn
+    gq = torch.Generator().manual_seed(22)
+    q = torch.randn(9, heads, d, generator=gq).to(dtype)
+    want = oracle.token_attention(q.float(), w["k_pool"].float(), w["v_pool"].float(), w["b_loc"], w["b_seq_len"], w["max_input_len"])
+    dk, dv = w["k_pool"].to(dev), w["v_pool"].to(dev)
+    args = (w["b_loc"].to(dev), w["b_start_loc"].to(dev), w["b_seq_len"].to(dev), w["max_input_len"])
+    got = ops.token_decode_attention(q.to(dev), dk, dv, *args)
+    assert_half(got, want)
+    assert_exact(ops.token_decode_attention(q.to(dev), dk, dv, *args, no_alloc=True), got.cpu())
+    att = torch.zeros(heads, w["total_tokens"], dtype=torch.float32, device=dev)
+    ops.token_attention(q.to(dev), dk, att, *args)
+    out2 = torch.empty_like(got)
+    ops.token_softmax_reducev(att, dv, out2, *args)
+    assert_half(out2, want)
 
 
 @pytest.mark.parametrize("heads,kvh", [(8, 2), (6, 3)])
