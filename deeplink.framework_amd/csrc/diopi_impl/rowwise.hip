@@ -454,6 +454,99 @@ __global__ __launch_bounds__(256) void rowBlockVecKernel(T* __restrict__ out, co
   }
 }
 
+// Rows too long for a workgroup's registers (a softmax over a vocabulary of more than 65 536 entries), or long and not
+// 16-byte aligned: a workgroup of 1024 threads per row streams the row twice, the second time mostly out of the caches
+// the first pass filled. Pass one keeps a running maximum and a sum rescaled to it per thread (softmax) or the sum of
+// squares (RMSNorm); pass two writes. VEC: 16-byte pieces (cols a multiple of the vector, aligned rows), else single
+// elements.
+template <typename T, int OP, typename WT, bool VEC>
+__global__ __launch_bounds__(1024) void rowStreamKernel(T* __restrict__ out, const T* __restrict__ in,
+                                                         const WT* __restrict__ weight, const WT* __restrict__ bias,
+                                                         float* __restrict__ invRmsOut, int64_t rows, int64_t cols,
+                                                         int64_t inRowStride, int64_t outRowStride, float eps) {
+  using V = typename Vec16<T>::type;
+  constexpr int N = VEC ? Vec16<T>::N : 1;
+  __shared__ float red[16];
+  const int64_t pieces = cols / N;
+  auto load = [&](const T* src, int64_t i, float (&f)[N]) {
+    if constexpr (VEC) {
+      const V v = reinterpret_cast<const V*>(src)[i];
+#pragma unroll
+      for (int j = 0; j < N; ++j) f[j] = static_cast<float>(v[j]);
+    } else {
+      f[0] = static_cast<float>(src[i]);
+    }
+  };
+  auto store = [&](T* dst, int64_t i, const float (&f)[N]) {
+    if constexpr (VEC) {
+      V v;
+#pragma unroll
+      for (int j = 0; j < N; ++j) v[j] = static_cast<T>(f[j]);
+      __builtin_nontemporal_store(v, reinterpret_cast<V*>(dst) + i);
+    } else {
+      dst[i] = static_cast<T>(f[0]);
+    }
+  };
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const T* src = in + row * inRowStride;
+    T* dst = out + row * outRowStride;
+    if constexpr (OP == kRowSoftmax) {
+      float m = -INFINITY, sum = 0.f;  // in units of log2
+      for (int64_t i = threadIdx.x; i < pieces; i += 1024) {
+        float f[N];
+        load(src, i, f);
+        float pm = f[0];
+#pragma unroll
+        for (int j = 1; j < N; ++j) pm = fmaxf(pm, f[j]);
+        pm *= kLog2e;
+        if (pm > m) {
+          sum *= __builtin_amdgcn_exp2f(m - pm);  // (m = -inf: sum is still 0, and exp2(-inf) = 0)
+          m = pm;
+        }
+        if (m != -INFINITY) {
+#pragma unroll
+          for (int j = 0; j < N; ++j) sum += __builtin_amdgcn_exp2f(fmaf(f[j], kLog2e, -m));
+        }
+      }
+      const float rowMax = blockReduce(m, true, red);
+      const float mScaled = (rowMax == -INFINITY) ? 0.f : rowMax;  // all -inf row: the sum is 0 and every output 0 * inf = nan, like the CPU kernel
+      sum = (m == -INFINITY) ? 0.f : sum * __builtin_amdgcn_exp2f(m - mScaled);
+      const float total = blockReduce(sum, false, red);
+      const float inv = 1.f / total;
+      for (int64_t i = threadIdx.x; i < pieces; i += 1024) {
+        float f[N];
+        load(src, i, f);
+#pragma unroll
+        for (int j = 0; j < N; ++j) f[j] = __builtin_amdgcn_exp2f(fmaf(f[j], kLog2e, -mScaled)) * inv;
+        store(dst, i, f);
+      }
+    } else {
+      float ss = 0.f;
+      for (int64_t i = threadIdx.x; i < pieces; i += 1024) {
+        float f[N];
+        load(src, i, f);
+#pragma unroll
+        for (int j = 0; j < N; ++j) ss += f[j] * f[j];
+      }
+      ss = blockReduce(ss, false, red);
+      const float inv = 1.0f / sqrtf(ss / (float)cols + eps);
+      if (invRmsOut != nullptr && threadIdx.x == 0) invRmsOut[row] = inv;
+      for (int64_t i = threadIdx.x; i < pieces; i += 1024) {
+        float f[N];
+        load(src, i, f);
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+          float t = f[j] * inv;
+          if (weight != nullptr) t *= static_cast<float>(weight[i * N + j]);
+          if (bias != nullptr) t += static_cast<float>(bias[i * N + j]);
+          f[j] = t;
+        }
+        store(dst, i, f);
+      }
+    }
+  }
+}
+
 // softmax along a non-last dim of a dense tensor [outer, dim, inner]: one lane per
 // (outer, inner) column, lanes adjacent along `inner` so every step is coalesced.
 template <typename T>
@@ -781,8 +874,17 @@ static diopiError_t launchRows(hipStream_t stream, T* out, const T* in, const WT
     else if (nvt <= 16) BLOCK_LAUNCH(16);
     else BLOCK_LAUNCH(32);
 #undef BLOCK_LAUNCH
+  } else if (cols > 12288) {
+    // longer than the register and LDS forms hold: two streaming passes, in 16-byte pieces where the rows allow them
+    dim3 grid((unsigned)std::min<int64_t>(rows, (int64_t)computeUnits() * 2)), block(1024);
+    if (vectorOk && cols % N == 0)
+      hipLaunchKernelGGL((rowStreamKernel<T, OP, WT, true>), grid, block, 0, stream, out, in, weight, bias, invRms, rows, cols,
+                         inStride, outStride, eps);
+    else
+      hipLaunchKernelGGL((rowStreamKernel<T, OP, WT, false>), grid, block, 0, stream, out, in, weight, bias, invRms, rows, cols,
+                         inStride, outStride, eps);
   } else {
-    int stage = cols <= 12288 ? (int)cols : 0;  // 48 KiB of fp32 staging
+    int stage = (int)cols;  // at most 48 KiB of fp32 staging
     size_t lds = (8 + (size_t)stage) * sizeof(float);
     hipLaunchKernelGGL((rowBlockKernel<T, OP, WT>), dim3((unsigned)rows), dim3(256), lds, stream, out, in, weight,
                        bias, invRms, rows, cols, inStride, outStride, eps, stage);

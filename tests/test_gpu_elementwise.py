@@ -213,9 +213,12 @@ def test_softmax(ops, dev, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_softmax_and_rms_norm_short_and_long_rows(ops, dev, dtype):
-    """Rows that share a wave (a few vectors each, ragged row counts) and rows longer than one wave holds (a workgroup
-    per row, up to 65536 16-bit elements), with masked entries and one fully masked row in the softmax."""
-    for rows, cols in [(1000, 64), (101, 8), (17, 24), (4099, 128), (33, 256), (300, 11008), (40, 32000), (3, 65536)]:
+    """Rows that share a wave (a few vectors each, ragged row counts), rows longer than one wave holds (a workgroup
+    per row, up to 65536 16-bit elements) and rows longer than that or long and unaligned (two streaming passes:
+    vocabularies of 128256 and 50257 entries, 70001 columns), with masked entries and one fully masked row in the
+    softmax."""
+    for rows, cols in [(1000, 64), (101, 8), (17, 24), (4099, 128), (33, 256), (300, 11008), (40, 32000), (3, 65536),
+                       (5, 128256), (7, 50257), (3, 70001), (600, 16392)]:
         x = (torch.randn(rows, cols, generator=g(140)) * 3).to(dtype)
         x[torch.rand(rows, cols, generator=g(141)) < 0.05] = float("-inf")
         x[:, 0] = 0.5
