@@ -53,6 +53,11 @@ struct W8Args {
   int M, N, K;
   int scaleDtype, biasDtype;
   int colsPerWg;  // w8LinearLdsKernel: output channels per workgroup
+  // w8LinearLdsKernel with K split over gridDim.z: workgroup z multiplies stagesPerSlice stages of K from stage
+  // z * stagesPerSlice on and leaves its unscaled fp32 sums in partial[z][M][N] (w8SliceReduceKernel finishes);
+  // partial == nullptr: the whole K, the result scaled and stored
+  float* partial = nullptr;
+  int stagesPerSlice = 0;
 };
 
 // The four int8 of one dword as floats: one SDWA conversion per byte (left to itself the compiler shifts
@@ -222,7 +227,11 @@ __global__ __launch_bounds__(512) void w8LinearLdsKernel(W8Args a) {
   const int ci = wave & 3, kq = wave & 3, nb = wave >> 2;
   const int n0 = blockIdx.x * a.colsPerWg, nCols = min(a.colsPerWg, a.N - n0);
   const int m0 = blockIdx.y * 16 * G, rows = min(16 * G, a.M - m0);
-  const int nStages = a.K / BK;  // the host sends only K that are multiples of BK here
+  // the host sends only K that are multiples of BK here; with K split over gridDim.z this workgroup takes the stages
+  // from firstStage on (every slice holds at least one)
+  const int allStages = a.K / BK;
+  const int firstStage = a.partial ? (int)blockIdx.z * a.stagesPerSlice : 0;
+  const int nStages = a.partial ? min(a.stagesPerSlice, allStages - firstStage) : allStages;
   const int kStart = (int)((blockIdx.x * (unsigned)kW8LdsStagger) % (unsigned)nStages);
   auto descriptor = [](const void* base, int64_t bytes) {
     const uint64_t p = reinterpret_cast<uint64_t>(base);
@@ -254,7 +263,7 @@ __global__ __launch_bounds__(512) void w8LinearLdsKernel(W8Args a) {
   auto copyStage = [&](int c, int buf) {  // a stage past the end copies the last one again, into a buffer nobody reads any more
     int cc = min(c, nStages - 1) + kStart;
     if (cc >= nStages) cc -= nStages;
-    const int from = __builtin_amdgcn_readfirstlane(cc * BK * (copiesW ? 1 : (int)sizeof(T)));
+    const int from = __builtin_amdgcn_readfirstlane((firstStage + cc) * BK * (copiesW ? 1 : (int)sizeof(T)));
 #pragma unroll
     for (int i = 0; i < IPW; ++i)
       if (i < ipw) {
@@ -363,11 +372,35 @@ __global__ __launch_bounds__(512) void w8LinearLdsKernel(W8Args a) {
           float v = 0.f;
 #pragma unroll
           for (int k2 = 0; k2 < 4; ++k2) v += red[((((nb * 4 + k2) * G + gi) * NTP + j) * 4 + r) * 64 + lane];
-          out[(int64_t)(m0 + row) * a.ldo + n0 + lc] = static_cast<T>(v * sc[j] + bv[j]);
+          if (a.partial) a.partial[((int64_t)blockIdx.z * a.M + m0 + row) * a.N + n0 + lc] = v;
+          else out[(int64_t)(m0 + row) * a.ldo + n0 + lc] = static_cast<T>(v * sc[j] + bv[j]);
         }
       }
     }
   }
+}
+
+// out[m, n] = (sum over the K slices of partial[z][m][n]) * scale[n] + bias[n]: four consecutive channels per thread.
+template <typename T>
+__global__ __launch_bounds__(256) void w8SliceReduceKernel(W8Args a, int slices) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x, perRow = a.N / 4;
+  if (idx >= (int64_t)a.M * perRow) return;
+  const int64_t m = idx / perRow, n = (idx - m * perRow) * 4;
+  f32x4 v = *reinterpret_cast<const f32x4*>(a.partial + m * a.N + n);
+  for (int z = 1; z < slices; ++z) {
+    const f32x4 p = *reinterpret_cast<const f32x4*>(a.partial + ((int64_t)z * a.M + m) * a.N + n);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] += p[e];
+  }
+  typedef T T4 __attribute__((ext_vector_type(4)));
+  T4 o;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    float r = v[e] * loadAs<float>(a.scale, n + e, a.scaleDtype);
+    if (a.bias) r += loadAs<float>(a.bias, n + e, a.biasDtype);
+    o[e] = static_cast<T>(r);
+  }
+  *reinterpret_cast<T4*>(reinterpret_cast<T*>(a.out) + m * a.ldo + n) = o;
 }
 
 template <typename T, int G, int NTP, int BK, int WST, int XST>
@@ -376,9 +409,15 @@ static diopiError_t launchW8Lds(hipStream_t stream, const W8Args& a) {
   AMD_CHECK(a.colsPerWg >= 1 && a.colsPerWg <= BN, "int8 linear: %d channels per workgroup do not fit %d", a.colsPerWg, BN);
   const int lds = std::max((WST * BN + XST * G * 16 * (int)sizeof(T)) * BK, 8 * G * NTP * 4 * 64 * (int)sizeof(float));
   AMD_HIP(allowDynamicLds(reinterpret_cast<const void*>(&w8LinearLdsKernel<T, G, NTP, BK, WST, XST>), lds));
-  dim3 grid((unsigned)((a.N + a.colsPerWg - 1) / a.colsPerWg), (unsigned)((a.M + 16 * G - 1) / (16 * G)));
+  const int slices = a.partial ? (a.K / BK + a.stagesPerSlice - 1) / a.stagesPerSlice : 1;
+  dim3 grid((unsigned)((a.N + a.colsPerWg - 1) / a.colsPerWg), (unsigned)((a.M + 16 * G - 1) / (16 * G)), (unsigned)slices);
   hipLaunchKernelGGL((w8LinearLdsKernel<T, G, NTP, BK, WST, XST>), grid, dim3(512), lds, stream, a);
   AMD_LAUNCH_CHECK();
+  if (a.partial) {
+    const int64_t items = (int64_t)a.M * (a.N / 4);
+    hipLaunchKernelGGL(w8SliceReduceKernel<T>, dim3((unsigned)ceilDiv(items, (int64_t)256)), dim3(256), 0, stream, a, slices);
+    AMD_LAUNCH_CHECK();
+  }
   return diopiSuccess;
 }
 
@@ -409,9 +448,28 @@ static diopiError_t launchW8ForTiles(hipStream_t stream, const W8Args& a) {
   }
 }
 
+// K slices for a narrow weight at more than 16 rows, or with a long K (0: the call keeps the other forms): 64 channels per workgroup and
+// enough slices of whole 256-column stages to give every CU a workgroup, so that a workgroup stages only its slice of
+// the activations (with whole K per workgroup the activations, re-read by every workgroup, outweigh the weights:
+// 64 x 4096 x 14336 took 68 us against 28 for the same product with 16-bit weights).
+static int w8SlicesFor(const W8Args& a) {
+  if (a.M > 64 || a.N >= 6144 || a.N < 64 || a.N % 4 != 0 || a.K % 256 != 0 || a.K < (a.M <= 16 ? 8192 : 2048)) return 0;
+  if ((int64_t)(a.N - 1) * a.ldw + a.K >= ((int64_t)1 << 31) || a.ldo % 4 != 0) return 0;
+  const int wgs = (a.N + 63) / 64, stages = a.K / 256;
+  const int want = std::max(1, computeUnits() / wgs);
+  const int slices = std::min(std::min(want, stages / 2), 16);  // at least two stages per slice
+  return slices >= 2 ? slices : 0;
+}
+
 template <typename T>
 static diopiError_t launchW8ForShape(hipStream_t stream, const W8Args& a0) {
   W8Args a = a0;
+  if (a.partial) {  // the caller has asked w8SlicesFor and brought the workspace
+    a.colsPerWg = 64;
+    if (a.M <= 16) return launchW8Lds<T, 1, 2, 256, 4, 4>(stream, a);
+    if (a.M <= 32) return launchW8Lds<T, 2, 2, 256, 4, 3>(stream, a);
+    return launchW8Lds<T, 4, 2, 256, 4, 2>(stream, a);
+  }
   // Wide weights go through w8LinearLdsKernel, the channels dealt evenly over the CUs. Measured cold against the form
   // below at K = 4096 (us, 1 / 16 / 32 / 64 rows): N = 11008 11.0 -> 10.8, 12.9 -> 11.7, 17.0 -> 14.2, 23.1 -> 21.1;
   // N = 22016 22.0 -> 19.2, 26.8 -> 20.2. Both forms have about 10 us of floor at these sizes, so narrower weights
@@ -592,6 +650,15 @@ extern "C" __attribute__((visibility("default"))) diopiError_t diopiWeightOnlyIn
   a.ldx = K, a.ldw = N > 1 ? cw.stride[0] : K, a.ldo = N;
   a.M = (int)M, a.N = (int)N, a.K = (int)K;
   a.scaleDtype = csc.dtype, a.biasDtype = bias.defined() ? cb.dtype : diopi_dtype_float32;
+  if (const int slices = w8SlicesFor(a); slices > 0 && cin.aligned16() && cw.aligned16() && a.ldw % 16 == 0 && cout.aligned16() &&
+                                           (std::min<int64_t>(M, 64) * K + K) * 2 < (int64_t(1) << 31)) {
+    const int stages = (int)(K / 256);
+    a.stagesPerSlice = (stages + slices - 1) / slices;
+    const int used = (stages + a.stagesPerSlice - 1) / a.stagesPerSlice;  // every slice holds at least one stage
+    void* ws = nullptr;
+    AMD_TRY(requireWorkspace(ctx, (int64_t)used * M * N * (int64_t)sizeof(float), &ws));
+    a.partial = static_cast<float*>(ws);
+  }
   const bool fast = K % kW8Block == 0 && cin.aligned16() && cw.aligned16() && a.ldw % 16 == 0 && ceilDiv(M, 64) <= 65535 &&
                     (std::min<int64_t>(M, 64) * K + K) * 2 < (int64_t(1) << 31);
   if (fast) {

@@ -721,6 +721,24 @@ def test_weight_only_int8_linear_chunked_k_row_groups_and_tile_counts(ops, dev, 
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,k,n", [(64, 14336, 4096), (33, 4096, 4096), (17, 2048 + 256, 5120), (48, 11008, 4100), (64, 2048, 200)])
+def test_weight_only_int8_linear_narrow_weights_split_over_k(ops, dev, pkg, m, k, n, dtype):
+    """Narrow weights at 17 - 64 rows: K split over workgroups (4, 4, 3, 3 and 4 slices here, one with a shorter last
+    slice, two with a ragged last channel block), unscaled fp32 sums reduced by a second launch that applies scale and
+    bias: against the oracle, with a bias in float32, and exactly on one-hot rows."""
+    w = pkg.workloads.int8_linear(seed=8, m=m, k=k, n=n, dtype=dtype)
+    want = oracle.weight_only_int8_linear(w["x"], w["w"], w["scale"])
+    assert_half(ops.weight_only_int8_linear(w["x"].to(dev), w["w"].to(dev), w["scale"].to(dev)), want)
+    bias = torch.randn(n, generator=g(37))
+    assert_half(ops.weight_only_int8_linear(w["x"].to(dev), w["w"].to(dev), w["scale"].to(dev), bias.to(dev)), want + bias)
+    x = torch.zeros(m, k, dtype=dtype)
+    cols = torch.randint(0, k, (m,), generator=g(38))
+    x[torch.arange(m), cols] = 1
+    got = ops.weight_only_int8_linear(x.to(dev), w["w"].to(dev), w["scale"].to(dev))
+    assert_exact(got, (w["w"][:, cols].float() * w["scale"].float()[:, None]).t().to(dtype))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("m,k,n", [(129, 4096, 1000), (300, 1024 + 16, 520), (1024, 4096, 4096), (4608, 384, 4096),
                                    (4568, 512, 4072)])
 def test_weight_only_int8_linear_many_rows(ops, dev, pkg, m, k, n, dtype):
