@@ -448,12 +448,15 @@ static diopiError_t launchW8ForTiles(hipStream_t stream, const W8Args& a) {
   }
 }
 
-// K slices for a narrow weight at more than 16 rows, or with a long K (0: the call keeps the other forms): 64 channels per workgroup and
-// enough slices of whole 256-column stages to give every CU a workgroup, so that a workgroup stages only its slice of
-// the activations (with whole K per workgroup the activations, re-read by every workgroup, outweigh the weights:
-// 64 x 4096 x 14336 took 68 us against 28 for the same product with 16-bit weights).
+// K slices for a weight of fewer than 10240 channels at more than 16 rows, or with a long K (0: the call keeps the other
+// forms): 64 channels per workgroup and enough slices of whole 256-column stages to give every CU a workgroup, so that a
+// workgroup stages only its slice of the activations (with whole K per workgroup the activations, re-read by every
+// workgroup, outweigh the weights: 64 x 4096 x 14336 took 68 us against 28 for the same product with 16-bit weights;
+// 64 x 8192 x 28672 110 -> 73 us, 16 x 8192 x 8192 23.8 -> 16.9 us).
 static int w8SlicesFor(const W8Args& a) {
-  if (a.M > 64 || a.N >= 6144 || a.N < 64 || a.N % 4 != 0 || a.K % 256 != 0 || a.K < (a.M <= 16 ? 8192 : 2048)) return 0;
+  if (a.M > 64 || a.N >= 10240 || a.N < 64 || a.N % 4 != 0 || a.K % 256 != 0 || a.K < (a.M <= 16 ? 8192 : 2048)) return 0;
+  // (a few rows against a large weight of medium width stream well as they are: 1 x 8192 x 28672 35.6 us, 39.4 in slices)
+  if (a.M <= 4 && a.N >= 6144 && (int64_t)a.N * a.K >= ((int64_t)1 << 27)) return 0;
   if ((int64_t)(a.N - 1) * a.ldw + a.K >= ((int64_t)1 << 31) || a.ldo % 4 != 0) return 0;
   const int wgs = (a.N + 63) / 64, stages = a.K / 256;
   const int want = std::max(1, computeUnits() / wgs);

@@ -721,10 +721,11 @@ def test_weight_only_int8_linear_chunked_k_row_groups_and_tile_counts(ops, dev, 
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("m,k,n", [(64, 14336, 4096), (33, 4096, 4096), (17, 2048 + 256, 5120), (48, 11008, 4100), (64, 2048, 200)])
+@pytest.mark.parametrize("m,k,n", [(64, 14336, 4096), (33, 4096, 4096), (17, 2048 + 256, 5120), (48, 11008, 4100), (64, 2048, 200),
+                                   (4, 8192, 4096), (16, 8192, 8192)])
 def test_weight_only_int8_linear_narrow_weights_split_over_k(ops, dev, pkg, m, k, n, dtype):
-    """Narrow weights at 17 - 64 rows: K split over workgroups (4, 4, 3, 3 and 4 slices here, one with a shorter last
-    slice, two with a ragged last channel block), unscaled fp32 sums reduced by a second launch that applies scale and
+    """Weights of fewer than 10240 channels at 17 - 64 rows, or at fewer rows with K from 8192 on: K split over workgroups
+    (4, 4, 3, 3, 4, 4 and 2 slices here, one with a shorter last slice, two with a ragged last channel block), unscaled fp32 sums reduced by a second launch that applies scale and
     bias: against the oracle, with a bias in float32, and exactly on one-hot rows."""
     w = pkg.workloads.int8_linear(seed=8, m=m, k=k, n=n, dtype=dtype)
     want = oracle.weight_only_int8_linear(w["x"], w["w"], w["scale"])
