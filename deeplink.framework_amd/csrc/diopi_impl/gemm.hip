@@ -2470,7 +2470,11 @@ static diopiError_t launchSkinnyForShape(diopiContextHandle_t ctx, hipStream_t s
   // loses (7.7 -> 10.0). The same split on wider weights loses (N = 11008: 23.0 -> 25.5 us, four ways 33.6).
   const bool canSplitLds = a.N % 8 == 0 && mult8(p.sOm) && ptr16(p.out) && (!p.bias || ptr16(p.bias)) &&
                            (!p.Cin || (p.sCn == 1 && mult8(p.sCm) && ptr16(p.Cin))) && rot == nullptr;
-  const bool narrow = a.N >= 4096 && a.N < 5120 && a.K % kSkinnyLdsBK == 0 && canSplitLds;
+  // Weights of 5120 to 10239 rows take the K slices when K is at least twice their width (the down projections of
+  // larger models; us, 1 / 16 / 32 / 64 rows: 5120 x 13824 30.7 -> 23.7, 31.8 -> 25.4, 36.1 -> 29.1, 46.5 -> 33.4;
+  // 6144 x 16384 at 64 rows 55.7 -> 41.9; 8192 x 28672 at 64 rows 111.6 -> 95.2); a square 8192 x 8192 loses
+  // (one row 21.5 -> 27.8).
+  const bool narrow = a.N >= 4096 && (a.N < 5120 || (a.N < 10240 && a.K >= 2 * a.N)) && a.K % kSkinnyLdsBK == 0 && canSplitLds;
   const int narrowWays = narrow && a.K >= 8192 ? (a.M <= 16 ? 2 : 4) : 1;
   const bool narrowLongK = narrowWays > 1;
   if ((a.N >= 5120 || (a.N >= 4096 && a.M > 16 && a.M <= 32) || narrowLongK) &&
