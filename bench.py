@@ -34,7 +34,7 @@ MFMA_BF16_PEAK_TF = 2500.0   # MI355X dense bf16, published
 # a counter cannot be read from inside this process, so the figure is carried here as measured, with the commit
 # whose kernels the counters were taken on (it does not move when the kernel does; re-take it after a GEMM change).
 GEMM_TRAFFIC_BYTES_PER_LAUNCH = 1_391_000_000
-GEMM_TRAFFIC_MEASURED_AT = "ab5c488"
+GEMM_TRAFFIC_MEASURED_AT = "cd6aa83"
 
 
 def parse():
