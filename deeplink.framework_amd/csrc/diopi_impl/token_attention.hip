@@ -125,6 +125,16 @@ __device__ __forceinline__ uint32_t packPair(float lo, float hi) {
 // softmax and the sum over V from scores computed earlier (second half of the two-call form).
 enum TaMode { kTaFused = 0, kTaLogitsOut = 1, kTaReduceV = 2 };
 
+// The value lane J of every aligned group of four lanes holds, in all four (one DPP move; every lane active).
+template <int J>
+__device__ __forceinline__ uint32_t quadBroadcast(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, J * 0x55, 0xf, 0xf, false);
+}
+template <int J>
+__device__ __forceinline__ float quadBroadcast(float v) {
+  return __builtin_bit_cast(float, quadBroadcast<J>(__builtin_bit_cast(uint32_t, v)));
+}
+
 // T: bf16_t / half_t (8 per 16 B) or float (4 per 16 B). LPT lanes cover one head row. LT: the type of the scores in
 // memory (the two-call modes). QPK: query heads that share this workgroup's K/V head and are all served from one read
 // of its rows (grouped-query layouts; 1 otherwise). With QPK > 1 the grid is one-dimensional and decoded so that the
@@ -247,6 +257,8 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
   const T* kBase = kNeedK ? reinterpret_cast<const T*>(a.k) + kvh * a.kHeadStride + subIn * N : nullptr;
   const T* vBase = kNeedV ? reinterpret_cast<const T*>(a.v) + kvh * a.vHeadStride + subIn * N : nullptr;
 
+  constexpr bool kShared = QPK == 4 && kPairs && MODE == kTaFused;
+  float mOwn = -INFINITY, lOwn = 0.f;  // kShared: the state of head (sub & 3), see the loop
   float m[QPK], l[QPK], acc[QPK][N];
 #pragma unroll
   for (int j = 0; j < QPK; ++j) {
@@ -312,6 +324,46 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
         vhi[c] = __builtin_amdgcn_perm(r1[c], r0[c], 0x07060302u);
       }
     }
+    // kShared: four query heads on 16-bit rows in the fused mode. Every lane of a lane group holds the scores of all
+    // four heads after the row sums, so the softmax update of head i is done by lanes i, i + 4, ... alone (their own
+    // running maximum and sum: mOwn, lOwn) and the factors reach the other lanes by one quad broadcast each: three
+    // exponentials per lane and pair of rows instead of twelve. The same arithmetic per head as the loop below.
+    if constexpr (kShared) {
+      float scAll[QPK][UNR];
+#pragma unroll
+      for (int j = 0; j < QPK; ++j)
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+          const u32x4 kraw = __builtin_bit_cast(u32x4, kr[u]);
+          float d = 0.f;
+#pragma unroll
+          for (int c = 0; c < 4; ++c) d = dotPair<T>(qp[j][c], kraw[c], d);
+          d = headRowSum<LPT>(d) * qScale;
+          scAll[j][u] = ok[u] ? d : -INFINITY;
+        }
+      const int own = sub & 3;
+      float my[UNR];
+#pragma unroll
+      for (int u = 0; u < UNR; ++u)
+        my[u] = own == 0 ? scAll[0][u] : (own == 1 ? scAll[1][u] : (own == 2 ? scAll[2][u] : scAll[3][u]));
+      const float mn = fmaxf(mOwn, fmaxf(my[0], my[UNR - 1]));
+      const bool any = mn != -INFINITY;
+      const float corr = any ? __builtin_amdgcn_exp2f(mOwn - mn) : 1.f;  // mOwn == -inf gives 0: acc and l are 0 then anyway
+      const float p0 = any ? __builtin_amdgcn_exp2f(my[0] - mn) : 0.f, p1 = any ? __builtin_amdgcn_exp2f(my[UNR - 1] - mn) : 0.f;
+      lOwn = lOwn * corr + (p0 + p1);
+      mOwn = mn;
+      const uint32_t ppOwn = packPair<T>(p0, p1);
+      staticFor<QPK>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        const float cj = quadBroadcast<j>(corr);
+        const uint32_t pp = quadBroadcast<j>(ppOwn);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          acc[j][2 * c] = dotPair<T>(pp, vlo[c], acc[j][2 * c] * cj);
+          acc[j][2 * c + 1] = dotPair<T>(pp, vhi[c], acc[j][2 * c + 1] * cj);
+        }
+      });
+    } else {
 #pragma unroll
     for (int j = 0; j < QPK; ++j) {
       float sc[UNR];
@@ -373,12 +425,20 @@ __global__ __launch_bounds__(kTaWaves * 64) void decodeSplitKernel(TaArgs a, T* 
         m[j] = mn;
       }
     }
+    }
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
       kr[u] = kn[u], vr[u] = vn[u], ok[u] = okn[u];
 #pragma unroll
       for (int j = 0; j < QPK; ++j) lr[j][u] = ln[j][u];
     }
+  }
+  if constexpr (kShared) {  // every lane gets the four heads' maxima and sums back for the merges below
+    staticFor<QPK>([&](auto jc) {
+      constexpr int j = decltype(jc)::value;
+      m[j] = quadBroadcast<j>(mOwn);
+      l[j] = quadBroadcast<j>(lOwn);
+    });
   }
   if constexpr (MODE == kTaLogitsOut) {
     if (useLds) {
