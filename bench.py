@@ -50,6 +50,8 @@ def parse():
     ap.add_argument("--gemm", metavar="M,N,K", help="profiling aid: time only diopiLinear on [M,K] x [N,K]^T (bf16 unless --gemm-dtype says otherwise) "
                     "(activations N(0,1), weights N(0,0.02)) for --steps launches and print one JSON line")
     ap.add_argument("--gemm-dtype", choices=["bf16", "fp16", "fp32"], default="bf16", help="with --gemm: the operand dtype")
+    ap.add_argument("--int8", metavar="M,N,K", help="profiling aid: time only diopiWeightOnlyInt8Linear on bf16 [M,K] x int8 [N,K]^T "
+                    "with a bf16 scale per channel for --steps launches and print one JSON line")
     ap.add_argument("--decode-attention", type=int, metavar="KV_HEADS", default=0, help="profiling aid: time only the fused decode "
                     "attention of the paged workload (batch 64, 32 query heads x 128) on a pool with KV_HEADS K/V heads")
     ap.add_argument("--attention", action="store_true", help="profiling aid: time only the prefill attention of the "
@@ -609,6 +611,16 @@ def single_kernel(pkg, torch, dev, rt, stream, args):
         call = Prepared(pkg, "diopiLinear", out, a, w, None)
         label = f"diopiLinear {args.gemm_dtype} {m}x{n}x{k}"
         work, unit = 2.0 * m * n * k / 1e12, "TFLOP/s"
+    elif args.int8:
+        m, n, k = (int(v) for v in args.int8.split(","))
+        g = torch.Generator().manual_seed(0)
+        a = torch.randn(m, k, generator=g).bfloat16().to(dev)
+        w = torch.randint(-127, 128, (n, k), generator=g, dtype=torch.int8).to(dev)
+        sc = (torch.rand(n, generator=g) * 0.01).bfloat16().to(dev)
+        out = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+        call = Prepared(pkg, "diopiWeightOnlyInt8Linear", out, a, w, sc, None)
+        label = f"diopiWeightOnlyInt8Linear bf16 x int8 {m}x{n}x{k}"
+        work, unit = (n * k + 2 * n + 2 * m * k + 2 * m * n) / 1e12, "TB/s"
     elif args.decode_attention:
         kvh = args.decode_attention
         pd = pkg.workloads.paged_decode(seed=0, fill_pool=False)
@@ -727,7 +739,7 @@ def main():
     dev = torch.device("cuda:0")
     rt = pkg.runtime
     stream = torch.cuda.current_stream().cuda_stream
-    if args.gemm or args.attention or args.decode_attention:
+    if args.gemm or args.int8 or args.attention or args.decode_attention:
         single_kernel(pkg, torch, dev, rt, stream, args)
         return
 
